@@ -1,0 +1,148 @@
+/*
+ * libnnueft — sparse feature transformer of nnue-pytorch for AMD Instinct MI355X (gfx950).
+ *
+ * C ABI.  Every pointer is a DEVICE pointer owned by the caller unless stated otherwise; the
+ * library never allocates, frees or retains memory.  `stream` is a hipStream_t passed as void*
+ * (NULL = the default stream); all work is enqueued on it and the call returns without waiting.
+ * The library keeps no global state and may be called from several host threads.
+ *
+ * Return value: 0 on success, a negative NNUEFT_E_* code for a rejected argument, or a positive
+ * hipError_t when a launch failed.  nnueft_error_string() describes either.
+ *
+ * Shapes and names follow the reference (paths relative to the nnue-pytorch checkout):
+ *   B  batch size (positions)          K  slots per index list (max_active_features)
+ *   R  rows of the weight table        out_cols = L1 + n_psqt (row width of the table)
+ * Index lists are int32[B,K], row-major; any entry outside [0,R) (the loader pads with -1,
+ * data_loader/cpp/training_data_loader.cpp:516-519) contributes nothing.
+ *
+ * Summation order of the fp32 paths (what "deterministic" and "bit-exact" refer to):
+ *   forward        s = +0; s += W[idx[k]] for k ascending over the valid slots; result = s + bias
+ *   weight grad    (deterministic entry points) per perspective and table row one chain starting at
+ *                  +0 over the slots naming that row in ascending (position, slot) order; then
+ *                  white chain + black chain.  This is the order of torch's CPU embedding_bag
+ *                  backward, i.e. of the reference's CPU path.
+ *   bias grad      (deterministic entry points) positions are cut into tiles of nnueft_bias_tile();
+ *                  per column a chain over a tile's positions, then a chain over the tile sums.
+ *   The atomic entry points add in an unspecified order.
+ */
+#ifndef NNUEFT_H
+#define NNUEFT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NNUEFT_VERSION 1
+
+#define NNUEFT_E_ARG (-1)         /* null pointer, non-positive or inconsistent dimension, odd L1 */
+#define NNUEFT_E_WORKSPACE (-2)   /* workspace missing, misaligned (256 B) or smaller than nnueft_det_workspace_bytes() */
+#define NNUEFT_E_UNSUPPORTED (-3) /* a dimension beyond what the kernels index (see each entry point) */
+
+int nnueft_version(void);
+const char* nnueft_error_string(int code);
+
+/* Positions per tile of the deterministic bias-gradient order. */
+int nnueft_bias_tile(void);
+
+/*
+ * out[b,:] = (sum_k W[idx[b,k],:]) + bias.
+ * Replaces the `sparse_input_linear_forward` CuPy kernel launched from
+ * model/modules/feature_transformer/sparse_linear_functions.py:85-99
+ * (kernel: sparse_linear_kernel.py:114-157); same result as _torch_sparse_linear, :16-50.
+ * idx int32[B,K]; W f32[R,out_cols] row-major contiguous; bias f32[out_cols]; out f32[B,out_cols].
+ */
+int nnueft_sparse_fwd(const int32_t* idx, const float* W, const float* bias, float* out,
+                      int B, int K, int R, int out_cols, void* stream);
+
+/*
+ * gW[idx[b,k],:] += gout[b,:] and gbias += gout[b,:] with floating-point atomics.
+ * gW f32[R,out_cols] and gbias f32[out_cols] must be zero (or hold a value to accumulate onto).
+ * Replaces `sparse_input_linear_backward`, sparse_linear_functions.py:118-134
+ * (kernel: sparse_linear_kernel.py:237-288).
+ */
+int nnueft_sparse_bwd_atomic(const int32_t* idx, const float* gout, float* gW, float* gbias,
+                             int B, int K, int R, int out_cols, void* stream);
+
+/*
+ * Bytes of scratch the deterministic backward entry points need (256-B aligned device memory,
+ * contents irrelevant on entry, garbage on exit).  n_persp = 1 for nnueft_sparse_bwd_det,
+ * 2 for nnueft_double_bwd_det.  Returns 0 for invalid dimensions.
+ */
+size_t nnueft_det_workspace_bytes(int B, int K, int R, int out_cols, int n_persp);
+
+/*
+ * Same gradient as nnueft_sparse_bwd_atomic in the fixed order stated at the top: a stable
+ * counting sort of the (row, position) pairs followed by a segmented reduction.  Every element
+ * of gW and gbias is written exactly once, so neither needs to be cleared.
+ * No counterpart in the reference (its GPU backward is atomic only); the order is that of the
+ * reference's CPU path (torch embedding_bag backward, sparse_linear_functions.py:43-50).
+ */
+int nnueft_sparse_bwd_det(const int32_t* idx, const float* gout, float* gW, float* gbias,
+                          int B, int K, int R, int out_cols,
+                          void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Both perspectives in one pass, then the side-to-move mix, clamp and pairwise product:
+ *   w = sum W[widx] + bias, b = sum W[bidx] + bias              (first L1 columns)
+ *   x_w = us*w + them*b,  x_b = us*b + them*w
+ *   l0[:, :h] = clamp(x_w[:h]) * clamp(x_w[h:]),  l0[:, h:] = clamp(x_b[:h]) * clamp(x_b[h:]),  h = L1/2
+ *   wpsqt = sum W[widx, L1+psqt_idx] + bias[L1+psqt_idx],  bpsqt likewise
+ * Replaces `fused_double_ft_forward`, fused_ft_functions.py:51-75 (kernel: fused_ft_kernel.py:27-117);
+ * same result as the torch composition double_ft_functions.py:62-80.
+ * us, them f32[B]; widx, bidx int32[B,K]; psqt_idx int64[B]; W f32[R,L1+n_psqt]; bias f32[L1+n_psqt];
+ * l0 f32[B,L1]; wpsqt, bpsqt f32[B]; saved f32[B,4,L1/2].
+ * `saved` receives (x_w[:h], x_w[h:], x_b[:h], x_b[h:]) BEFORE the clamp (the reference stores the
+ * clamped values, fused_ft_kernel.py:95-99); the backward needs them to reproduce torch's clamp
+ * gradient at the boundaries.  L1 must be even.
+ */
+int nnueft_double_fwd(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+                      const int64_t* psqt_idx, const float* W, const float* bias, float max_act,
+                      float* l0, float* wpsqt, float* bpsqt, float* saved,
+                      int B, int K, int R, int L1, int n_psqt, void* stream);
+
+/*
+ * Gradient of nnueft_double_fwd with respect to W and bias, floating-point atomics.
+ * gW f32[R,L1+n_psqt] and gbias f32[L1+n_psqt] must be zero on entry.
+ * Replaces `fused_double_ft_backward`, fused_ft_functions.py:94-120 (kernel: fused_ft_kernel.py:147-272).
+ */
+int nnueft_double_bwd_atomic(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+                             const int64_t* psqt_idx, float max_act,
+                             const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt,
+                             const float* saved, float* gW, float* gbias,
+                             int B, int K, int R, int L1, int n_psqt, void* stream);
+
+/*
+ * Same gradient in the fixed order stated at the top; gW and gbias are fully written.
+ * No counterpart in the reference's GPU code; the order is that of autograd through the
+ * reference's CPU composition (double_ft_functions.py:62-80).
+ */
+int nnueft_double_bwd_det(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+                          const int64_t* psqt_idx, float max_act,
+                          const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt,
+                          const float* saved, float* gW, float* gbias,
+                          int B, int K, int R, int L1, int n_psqt,
+                          void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Quantized feature transformer as the engine evaluates an exported net (no code in the
+ * reference; spec docs/nnue.md:1014-1069 and :2097-2134, constants model/quantize.py:58-73,
+ * tensors produced by QuantizationManager.quantize_feature_transformer_*, model/quantize.py:175-204):
+ *   acc_p[c] = b16[c] + sum_k W16[idx_p[k], c]                      int16, wrapping
+ *   c_p[c]   = min(max(acc_p[c], 0), clip_max)
+ *   out[b, o*h + j] = (c_P(o)[j] * c_P(o)[j+h]) >> shift            o = 0 side to move, 1 the other
+ *   psqt_out[b] = (sum psqt32[idx_P(0), bucket] - sum psqt32[idx_P(1), bucket]) / 2     (C division)
+ * stm u8[B]: 0 white to move, 1 black; W16 int16[R,L1]; b16 int16[L1]; psqt32 int32[R,n_psqt];
+ * psqt_idx int64[B]; out_u8 u8[B,L1]; psqt_out int32[B].  clip_max*clip_max >> shift must fit 8 bits.
+ */
+int nnueft_ft_int16_fwd(const int32_t* widx, const int32_t* bidx, const uint8_t* stm,
+                        const int16_t* W16, const int16_t* b16, const int32_t* psqt32,
+                        const int64_t* psqt_idx, uint8_t* out_u8, int32_t* psqt_out,
+                        int B, int K, int R, int L1, int n_psqt, int clip_max, int shift, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NNUEFT_H */

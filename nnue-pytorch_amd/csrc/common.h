@@ -1,0 +1,84 @@
+// Shared device helpers for the feature-transformer kernels (gfx950, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "nnueft.h"
+
+#define NNUEFT_WAVE 64
+// Positions per tile of the deterministic bias-gradient order (part of the ABI contract).
+#define NNUEFT_BIAS_TILE 32
+
+typedef unsigned long long u64;
+
+// A lane's slice of a row: VW consecutive floats, moved with one 4- or 16-byte access.
+template <int VW>
+struct vecf {
+    float v[VW];
+};
+
+template <int VW>
+__device__ __forceinline__ vecf<VW> ldv(const float* p);
+template <>
+__device__ __forceinline__ vecf<4> ldv<4>(const float* p) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    vecf<4> r;
+    r.v[0] = t.x; r.v[1] = t.y; r.v[2] = t.z; r.v[3] = t.w;
+    return r;
+}
+template <>
+__device__ __forceinline__ vecf<1> ldv<1>(const float* p) {
+    vecf<1> r;
+    r.v[0] = *p;
+    return r;
+}
+
+template <int VW>
+__device__ __forceinline__ void stv(float* p, const vecf<VW>& x);
+template <>
+__device__ __forceinline__ void stv<4>(float* p, const vecf<4>& x) {
+    *reinterpret_cast<float4*>(p) = make_float4(x.v[0], x.v[1], x.v[2], x.v[3]);
+}
+template <>
+__device__ __forceinline__ void stv<1>(float* p, const vecf<1>& x) {
+    *p = x.v[0];
+}
+
+template <int VW>
+__device__ __forceinline__ vecf<VW> vzero() {
+    vecf<VW> r;
+#pragma unroll
+    for (int i = 0; i < VW; ++i) r.v[i] = 0.0f;
+    return r;
+}
+
+template <int VW>
+__device__ __forceinline__ void vadd(vecf<VW>& a, const vecf<VW>& b) {
+#pragma unroll
+    for (int i = 0; i < VW; ++i) a.v[i] = a.v[i] + b.v[i];
+}
+
+__device__ __forceinline__ float clamp_act(float x, float hi) { return x < 0.0f ? 0.0f : (x > hi ? hi : x); }
+
+// Lowest set bit of a wave mask, removed from the mask.  The mask comes from __ballot, so the
+// result is wave-uniform and can drive scalar control flow and v_readlane.
+__device__ __forceinline__ int pop_lane(u64& mask) {
+    const int k = __ffsll((long long)mask) - 1;
+    mask &= mask - 1;
+    return k;
+}
+
+__device__ __forceinline__ int bcast_i(int v, int lane) { return __builtin_amdgcn_readlane(v, lane); }
+__device__ __forceinline__ float bcast_f(float v, int lane) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+static inline bool aligned256(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 255u) == 0; }
+
+#define NNUEFT_LAUNCH_CHECK()                         \
+    do {                                              \
+        hipError_t e__ = hipGetLastError();           \
+        if (e__ != hipSuccess) return (int)e__;       \
+    } while (0)

@@ -1,0 +1,209 @@
+// Forward gather-sum kernels.
+//
+// Work decomposition: one wave (= one workgroup of 64 lanes) per (position, column slice).  A lane
+// owns NQ vectors of VW floats per half-row, 64 lanes apart, so every load instruction of the wave
+// reads 64*VW*4 contiguous bytes of a gathered row (1 KiB with VW = 4).  The index list of the
+// position sits one slot per lane; the valid slots are walked through a ballot mask, so padding
+// costs nothing and no LDS is needed.
+#include "gather.h"
+
+namespace {
+
+constexpr int kUnroll = 4;
+
+// out[b, :] = (sum_k W[idx[b,k], :]) + bias
+template <int VW, int NQ>
+__global__ __launch_bounds__(64) void k_sparse_fwd(const int32_t* __restrict__ idx, const float* __restrict__ W,
+                                                   const float* __restrict__ bias, float* __restrict__ out,
+                                                   int K, int R, int out_cols, int nslices) {
+    const int lane = threadIdx.x;
+    const int b = blockIdx.x / nslices;
+    const int s = blockIdx.x - b * nslices;
+    const int nv = out_cols / VW;
+
+    int col[NQ];
+    bool act[NQ];
+#pragma unroll
+    for (int m = 0; m < NQ; ++m) {
+        const int q = (s * NQ + m) * 64 + lane;
+        act[m] = q < nv;
+        col[m] = act[m] ? q * VW : 0;
+    }
+    vecf<VW> acc[NQ];
+#pragma unroll
+    for (int m = 0; m < NQ; ++m) acc[m] = vzero<VW>();
+
+    const int32_t* ix = idx + (size_t)b * K;
+    for (int k0 = 0; k0 < K; k0 += 64) {
+        const int my = (k0 + lane < K) ? ix[k0 + lane] : -1;
+        const u64 mask = __ballot(my >= 0 && my < R);
+        chain_rows<VW, NQ, kUnroll>(acc, W, (size_t)out_cols, col, my, mask);
+    }
+    float* o = out + (size_t)b * out_cols;
+#pragma unroll
+    for (int m = 0; m < NQ; ++m) {
+        if (act[m]) {
+            vadd<VW>(acc[m], ldv<VW>(bias + col[m]));
+            stv<VW>(o + col[m], acc[m]);
+        }
+    }
+}
+
+// Both perspectives of one position, mix, clamp, pairwise product.
+template <int VW, int NQ>
+__global__ __launch_bounds__(64) void k_double_fwd(const float* __restrict__ us, const float* __restrict__ them,
+                                                   const int32_t* __restrict__ widx,
+                                                   const int32_t* __restrict__ bidx,
+                                                   const int64_t* __restrict__ psqt_idx,
+                                                   const float* __restrict__ W, const float* __restrict__ bias,
+                                                   float max_act, float* __restrict__ l0,
+                                                   float* __restrict__ wpsqt, float* __restrict__ bpsqt,
+                                                   float* __restrict__ saved, int K, int R, int L1, int n_psqt,
+                                                   int nslices) {
+    const int lane = threadIdx.x;
+    const int b = blockIdx.x / nslices;
+    const int s = blockIdx.x - b * nslices;
+    const int h = L1 >> 1;
+    const int hv = h / VW;
+    const size_t out_cols = (size_t)L1 + n_psqt;
+
+    // col[2m] is the lane's m-th vector in the first half, col[2m+1] its partner h columns on.
+    int col[2 * NQ];
+    bool act[NQ];
+#pragma unroll
+    for (int m = 0; m < NQ; ++m) {
+        const int q = (s * NQ + m) * 64 + lane;
+        act[m] = q < hv;
+        col[2 * m] = act[m] ? q * VW : 0;
+        col[2 * m + 1] = col[2 * m] + h;
+    }
+
+    const int64_t pi = psqt_idx[b];
+    const bool do_psqt = (s == 0) && pi >= 0 && pi < n_psqt;
+
+    vecf<VW> acc[2][2 * NQ];
+    float ps[2] = {0.0f, 0.0f};
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+#pragma unroll
+        for (int j = 0; j < 2 * NQ; ++j) acc[p][j] = vzero<VW>();
+        const int32_t* ix = (p ? bidx : widx) + (size_t)b * K;
+        for (int k0 = 0; k0 < K; k0 += 64) {
+            const int my = (k0 + lane < K) ? ix[k0 + lane] : -1;
+            const bool ok = my >= 0 && my < R;
+            const u64 mask = __ballot(ok);
+            float myps = 0.0f;
+            if (do_psqt && ok) myps = W[(size_t)my * out_cols + L1 + pi];
+            chain_rows<VW, 2 * NQ, kUnroll>(acc[p], W, out_cols, col, my, mask);
+            if (do_psqt) {
+                u64 m2 = mask;
+                while (m2) ps[p] = ps[p] + bcast_f(myps, pop_lane(m2));
+            }
+        }
+    }
+
+    const float u = us[b], t = them[b];
+    float* sv = saved + (size_t)b * 2 * L1;
+    float* o = l0 + (size_t)b * L1;
+#pragma unroll
+    for (int m = 0; m < NQ; ++m) {
+        if (!act[m]) continue;
+        const int c = col[2 * m];
+        const vecf<VW> bias0 = ldv<VW>(bias + c), bias1 = ldv<VW>(bias + c + h);
+        vecf<VW> xw0, xw1, xb0, xb1, o0, o1;
+#pragma unroll
+        for (int i = 0; i < VW; ++i) {
+            const float w0 = acc[0][2 * m].v[i] + bias0.v[i];
+            const float w1 = acc[0][2 * m + 1].v[i] + bias1.v[i];
+            const float b0 = acc[1][2 * m].v[i] + bias0.v[i];
+            const float b1 = acc[1][2 * m + 1].v[i] + bias1.v[i];
+            xw0.v[i] = u * w0 + t * b0;
+            xw1.v[i] = u * w1 + t * b1;
+            xb0.v[i] = u * b0 + t * w0;
+            xb1.v[i] = u * b1 + t * w1;
+            o0.v[i] = clamp_act(xw0.v[i], max_act) * clamp_act(xw1.v[i], max_act);
+            o1.v[i] = clamp_act(xb0.v[i], max_act) * clamp_act(xb1.v[i], max_act);
+        }
+        stv<VW>(sv + 0 * h + c, xw0);
+        stv<VW>(sv + 1 * h + c, xw1);
+        stv<VW>(sv + 2 * h + c, xb0);
+        stv<VW>(sv + 3 * h + c, xb1);
+        stv<VW>(o + c, o0);
+        stv<VW>(o + h + c, o1);
+    }
+    if (s == 0 && lane == 0) {
+        const float pb = do_psqt ? bias[L1 + pi] : 0.0f;
+        wpsqt[b] = ps[0] + pb;
+        bpsqt[b] = ps[1] + pb;
+    }
+}
+
+template <int VW, int NQ>
+int launch_sparse_fwd(const int32_t* idx, const float* W, const float* bias, float* out, int B, int K, int R,
+                      int out_cols, hipStream_t st) {
+    const int nv = out_cols / VW;
+    const int nslices = (nv + 64 * NQ - 1) / (64 * NQ);
+    const long long grid = (long long)B * nslices;
+    if (grid > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
+    hipLaunchKernelGGL((k_sparse_fwd<VW, NQ>), dim3((unsigned)grid), dim3(64), 0, st, idx, W, bias, out, K, R,
+                       out_cols, nslices);
+    NNUEFT_LAUNCH_CHECK();
+    return 0;
+}
+
+template <int VW, int NQ>
+int launch_double_fwd(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+                      const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,
+                      float* wpsqt, float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt,
+                      hipStream_t st) {
+    const int hv = (L1 / 2) / VW;
+    const int nslices = hv > 0 ? (hv + 64 * NQ - 1) / (64 * NQ) : 1;
+    const long long grid = (long long)B * nslices;
+    if (grid > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
+    hipLaunchKernelGGL((k_double_fwd<VW, NQ>), dim3((unsigned)grid), dim3(64), 0, st, us, them, widx, bidx,
+                       psqt_idx, W, bias, max_act, l0, wpsqt, bpsqt, saved, K, R, L1, n_psqt, nslices);
+    NNUEFT_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // namespace
+
+extern "C" int nnueft_sparse_fwd(const int32_t* idx, const float* W, const float* bias, float* out, int B, int K,
+                                 int R, int out_cols, void* stream) {
+    if (B < 0 || K <= 0 || R <= 0 || out_cols <= 0) return NNUEFT_E_ARG;
+    if (B == 0) return 0;
+    if (!idx || !W || !bias || !out) return NNUEFT_E_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const bool vec = (out_cols % 4 == 0) && aligned16(W) && aligned16(bias) && aligned16(out);
+    if (vec) {
+        if (out_cols / 4 > 64) return launch_sparse_fwd<4, 2>(idx, W, bias, out, B, K, R, out_cols, st);
+        return launch_sparse_fwd<4, 1>(idx, W, bias, out, B, K, R, out_cols, st);
+    }
+    if (out_cols > 64) return launch_sparse_fwd<1, 2>(idx, W, bias, out, B, K, R, out_cols, st);
+    return launch_sparse_fwd<1, 1>(idx, W, bias, out, B, K, R, out_cols, st);
+}
+
+extern "C" int nnueft_double_fwd(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+                                 const int64_t* psqt_idx, const float* W, const float* bias, float max_act,
+                                 float* l0, float* wpsqt, float* bpsqt, float* saved, int B, int K, int R,
+                                 int L1, int n_psqt, void* stream) {
+    if (B < 0 || K <= 0 || R <= 0 || L1 <= 0 || (L1 & 1) || n_psqt < 0) return NNUEFT_E_ARG;
+    if (B == 0) return 0;
+    if (!us || !them || !widx || !bidx || !psqt_idx || !W || !bias || !l0 || !wpsqt || !bpsqt || !saved)
+        return NNUEFT_E_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const bool vec = (L1 % 8 == 0) && ((L1 + n_psqt) % 4 == 0) && aligned16(W) && aligned16(bias) &&
+                     aligned16(l0) && aligned16(saved);
+    if (vec) {
+        if (L1 / 8 > 64)
+            return launch_double_fwd<4, 2>(us, them, widx, bidx, psqt_idx, W, bias, max_act, l0, wpsqt, bpsqt,
+                                           saved, B, K, R, L1, n_psqt, st);
+        return launch_double_fwd<4, 1>(us, them, widx, bidx, psqt_idx, W, bias, max_act, l0, wpsqt, bpsqt, saved,
+                                       B, K, R, L1, n_psqt, st);
+    }
+    if (L1 / 2 > 64)
+        return launch_double_fwd<1, 2>(us, them, widx, bidx, psqt_idx, W, bias, max_act, l0, wpsqt, bpsqt, saved,
+                                       B, K, R, L1, n_psqt, st);
+    return launch_double_fwd<1, 1>(us, them, widx, bidx, psqt_idx, W, bias, max_act, l0, wpsqt, bpsqt, saved, B,
+                                   K, R, L1, n_psqt, st);
+}

@@ -1,0 +1,67 @@
+"""ctypes binding of libnnueft.so (declarations in include/nnueft.h).
+
+The library is built in-tree by nnueft._build.build() (hipcc, gfx950).  Loading never falls back
+to another implementation: if the shared object is missing or does not export a symbol,
+`load()` raises, and `available()` is False.
+"""
+import ctypes
+import os
+from ctypes import c_float, c_int, c_size_t, c_void_p
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libnnueft.so")
+
+# name -> (restype, argtypes); mirrors include/nnueft.h one to one
+PROTOTYPES = {
+    "nnueft_version": (c_int, []),
+    "nnueft_error_string": (ctypes.c_char_p, [c_int]),
+    "nnueft_bias_tile": (c_int, []),
+    "nnueft_sparse_fwd": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_void_p]),
+    "nnueft_sparse_bwd_atomic": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_void_p]),
+    "nnueft_det_workspace_bytes": (c_size_t, [c_int] * 5),
+    "nnueft_sparse_bwd_det": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
+    "nnueft_double_fwd": (c_int, [c_void_p] * 7 + [c_float] + [c_void_p] * 4 + [c_int] * 5 + [c_void_p]),
+    "nnueft_double_bwd_atomic": (c_int, [c_void_p] * 5 + [c_float] + [c_void_p] * 6 + [c_int] * 5 + [c_void_p]),
+    "nnueft_double_bwd_det": (
+        c_int,
+        [c_void_p] * 5 + [c_float] + [c_void_p] * 6 + [c_int] * 5 + [c_void_p, c_size_t, c_void_p],
+    ),
+    "nnueft_ft_int16_fwd": (c_int, [c_void_p] * 9 + [c_int] * 7 + [c_void_p]),
+}
+
+_lib = None
+_load_error = None
+
+
+def load():
+    """Return the loaded library, raising if it cannot be loaded."""
+    global _lib, _load_error
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        _load_error = RuntimeError(
+            f"{LIB_PATH} not found: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+            "(or nnueft._build.build()); there is no fallback implementation"
+        )
+        raise _load_error
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in PROTOTYPES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def available() -> bool:
+    try:
+        load()
+        return True
+    except (OSError, RuntimeError, AttributeError):
+        return False
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().nnueft_error_string(rc).decode()
+        raise RuntimeError(f"{what} failed with code {rc}: {msg}")

@@ -1,0 +1,147 @@
+"""Fused two-perspective feature transformer as an autograd function.
+
+Same name, argument order, outputs and assertions as the reference's
+model/modules/feature_transformer/fused_ft_functions.py:18-122; the two CuPy kernels it launches
+are replaced by nnueft_double_fwd / nnueft_double_bwd_{atomic,det} of libnnueft.so.
+
+Differences that a caller can observe:
+  * the activation tensor kept for the backward holds the mixed values before the clamp (the
+    reference keeps them after it, fused_ft_kernel.py:95-99), so the clamp passes gradient at
+    exactly 0 and exactly max like torch.clamp does in the reference's CPU path;
+  * NNUEFT_BACKWARD=deterministic (or set_backward_mode) selects a backward whose result does
+    not depend on scheduling.
+"""
+import torch
+from torch import autograd
+
+from . import _native
+from . import sparse_linear_functions as _slf
+from .sparse_linear_functions import _stream_ptr, _workspace
+
+_HAS_CUPY_KERNELS = _native.available()
+
+# Positions a wave of the atomic backward walks before it flushes its bias partial sums
+# (fused_ft_kernel.py:127 has the same constant for the reference's kernel).
+BACKWARD_TILE_SIZE = 4
+
+
+@torch.compiler.disable(recursive=False)
+def _launch_double_fwd(us, them, white_indices, black_indices, psqt_indices, weight, bias, max_ft_activation,
+                       l1_size, l0_, wpsqt, bpsqt, saved):
+    lib = _native.load()
+    B, K = white_indices.shape
+    R, out_cols = weight.shape
+    rc = lib.nnueft_double_fwd(
+        us.data_ptr(), them.data_ptr(), white_indices.data_ptr(), black_indices.data_ptr(),
+        psqt_indices.data_ptr(), weight.data_ptr(), bias.data_ptr(), float(max_ft_activation),
+        l0_.data_ptr(), wpsqt.data_ptr(), bpsqt.data_ptr(), saved.data_ptr(),
+        B, K, R, l1_size, out_cols - l1_size, _stream_ptr(weight.device),
+    )
+    _native.check(rc, "nnueft_double_fwd")
+
+
+@torch.compiler.disable(recursive=False)
+def _launch_double_bwd(us, them, white_indices, black_indices, psqt_indices, max_ft_activation, grad_l0,
+                       grad_wpsqt, grad_bpsqt, saved, num_rows, l1_size, output_size, mode):
+    lib = _native.load()
+    B, K = white_indices.shape
+    device = us.device
+    n_psqt = output_size - l1_size
+    head = (
+        us.data_ptr(), them.data_ptr(), white_indices.data_ptr(), black_indices.data_ptr(),
+        psqt_indices.data_ptr(), float(max_ft_activation),
+        grad_l0.data_ptr(), grad_wpsqt.data_ptr(), grad_bpsqt.data_ptr(), saved.data_ptr(),
+    )
+    if mode == "deterministic":
+        grad_weight = torch.empty(num_rows, output_size, dtype=torch.float32, device=device)
+        grad_bias = torch.empty(output_size, dtype=torch.float32, device=device)
+        if B == 0:
+            return grad_weight.zero_(), grad_bias.zero_()
+        nbytes = lib.nnueft_det_workspace_bytes(B, K, num_rows, output_size, 2)
+        ws = _workspace(nbytes, device)
+        rc = lib.nnueft_double_bwd_det(
+            *head, grad_weight.data_ptr(), grad_bias.data_ptr(), B, K, num_rows, l1_size, n_psqt,
+            ws.data_ptr(), nbytes, _stream_ptr(device),
+        )
+        _native.check(rc, "nnueft_double_bwd_det")
+    else:
+        grad_weight = torch.zeros(num_rows, output_size, dtype=torch.float32, device=device)
+        grad_bias = torch.zeros(output_size, dtype=torch.float32, device=device)
+        rc = lib.nnueft_double_bwd_atomic(
+            *head, grad_weight.data_ptr(), grad_bias.data_ptr(), B, K, num_rows, l1_size, n_psqt,
+            _stream_ptr(device),
+        )
+        _native.check(rc, "nnueft_double_bwd_atomic")
+    return grad_weight, grad_bias
+
+
+class FusedDoubleFtFunction(autograd.Function):
+    @staticmethod
+    def forward(ctx, us, them, white_indices, black_indices, psqt_indices, weight, bias, max_ft_activation, l1_size):
+        ctx.max_ft_activation = float(max_ft_activation)
+        ctx.l1_size = int(l1_size)
+        ctx.backward_mode = _slf.get_backward_mode()
+
+        assert l1_size % 2 == 0
+
+        assert us.is_cuda and them.is_cuda
+        assert white_indices.is_cuda and black_indices.is_cuda and psqt_indices.is_cuda
+        assert weight.is_cuda and bias.is_cuda
+        assert (
+            us.device == them.device == white_indices.device == black_indices.device
+            == psqt_indices.device == weight.device == bias.device
+        )
+
+        assert us.dtype == torch.float32 and them.dtype == torch.float32
+        assert white_indices.dtype == torch.int32 and black_indices.dtype == torch.int32
+        assert psqt_indices.dtype == torch.int64
+        assert weight.dtype == torch.float32 and bias.dtype == torch.float32
+
+        assert white_indices.ndim == 2 and black_indices.ndim == 2
+        assert psqt_indices.ndim == 1
+        assert len(weight.shape) == 2
+        assert len(bias.shape) == 1
+        assert weight.shape[1] == bias.shape[0]
+        assert white_indices.shape == black_indices.shape
+        assert white_indices.shape[0] == psqt_indices.shape[0]
+        assert us.numel() == white_indices.shape[0] and them.numel() == white_indices.shape[0]
+        assert 0 < l1_size <= weight.shape[1]
+
+        assert us.is_contiguous() and them.is_contiguous()
+        assert white_indices.is_contiguous() and black_indices.is_contiguous() and psqt_indices.is_contiguous()
+        assert weight.is_contiguous() and bias.is_contiguous()
+
+        batch_size = white_indices.shape[0]
+        l1_half = l1_size // 2
+        device = us.device
+
+        l0_ = torch.empty(batch_size, l1_size, dtype=torch.float32, device=device)
+        wpsqt = torch.empty(batch_size, 1, dtype=torch.float32, device=device)
+        bpsqt = torch.empty(batch_size, 1, dtype=torch.float32, device=device)
+        preclamp = torch.empty(batch_size, 4, l1_half, dtype=torch.float32, device=device)
+
+        with torch.cuda.device(device):
+            _launch_double_fwd(
+                us, them, white_indices, black_indices, psqt_indices, weight, bias,
+                max_ft_activation, int(l1_size), l0_, wpsqt, bpsqt, preclamp,
+            )
+
+        ctx.save_for_backward(us, them, white_indices, black_indices, psqt_indices, weight, bias, preclamp)
+        return l0_, wpsqt, bpsqt
+
+    @staticmethod
+    def backward(ctx, grad_l0, grad_wpsqt, grad_bpsqt):
+        us, them, white_indices, black_indices, psqt_indices, weight, bias, preclamp = ctx.saved_tensors
+
+        grad_l0 = grad_l0.contiguous()
+        grad_wpsqt = grad_wpsqt.contiguous()
+        grad_bpsqt = grad_bpsqt.contiguous()
+
+        with torch.cuda.device(us.device):
+            grad_weight, grad_bias = _launch_double_bwd(
+                us, them, white_indices, black_indices, psqt_indices, ctx.max_ft_activation,
+                grad_l0, grad_wpsqt, grad_bpsqt, preclamp,
+                weight.shape[0], ctx.l1_size, bias.shape[0], ctx.backward_mode,
+            )
+
+        return None, None, None, None, None, grad_weight, grad_bias, None, None

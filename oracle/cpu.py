@@ -1,0 +1,130 @@
+"""numpy front end of libnnueft_oracle.so (see nnueft_oracle.c for what each function follows).
+
+TEST INFRASTRUCTURE: the checker, never the thing measured or shipped.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libnnueft_oracle.so")
+_lib = None
+
+
+def build(force: bool = False) -> str:
+    """Compile the C restatement (and, where the reference checkout exists, _ref)."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s", "all"])
+    return _LIB_PATH
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+    return _lib
+
+
+def _p(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _c(a, dtype):
+    a = np.ascontiguousarray(a, dtype=dtype)
+    return a
+
+
+def bias_tile() -> int:
+    return int(lib().nnueft_oracle_bias_tile())
+
+
+def sparse_fwd(idx, W, bias):
+    idx, W, bias = _c(idx, np.int32), _c(W, np.float32), _c(bias, np.float32)
+    B, K = idx.shape
+    R, oc = W.shape
+    out = np.empty((B, oc), np.float32)
+    rc = lib().nnueft_oracle_sparse_fwd(_p(idx), _p(W), _p(bias), _p(out), B, K, R, oc)
+    assert rc == 0
+    return out
+
+
+def sparse_bwd(idx, gout, R):
+    idx, gout = _c(idx, np.int32), _c(gout, np.float32)
+    B, K = idx.shape
+    oc = gout.shape[1]
+    gW = np.empty((R, oc), np.float32)
+    gb = np.empty((oc,), np.float32)
+    rc = lib().nnueft_oracle_sparse_bwd(_p(idx), _p(gout), _p(gW), _p(gb), B, K, R, oc)
+    assert rc == 0
+    return gW, gb
+
+
+def double_fwd(us, them, widx, bidx, psqt_idx, W, bias, max_act, L1):
+    us, them = _c(us, np.float32).reshape(-1), _c(them, np.float32).reshape(-1)
+    widx, bidx = _c(widx, np.int32), _c(bidx, np.int32)
+    psqt_idx = _c(psqt_idx, np.int64)
+    W, bias = _c(W, np.float32), _c(bias, np.float32)
+    B, K = widx.shape
+    R, oc = W.shape
+    n_psqt = oc - L1
+    l0 = np.empty((B, L1), np.float32)
+    wp = np.empty((B, 1), np.float32)
+    bp = np.empty((B, 1), np.float32)
+    saved = np.empty((B, 4, L1 // 2), np.float32)
+    rc = lib().nnueft_oracle_double_fwd(_p(us), _p(them), _p(widx), _p(bidx), _p(psqt_idx), _p(W), _p(bias),
+                                        ctypes.c_float(max_act), _p(l0), _p(wp), _p(bp), _p(saved),
+                                        B, K, R, L1, n_psqt)
+    assert rc == 0
+    return l0, wp, bp, saved
+
+
+def double_bwd_rows(us, them, psqt_idx, max_act, grad_l0, grad_wpsqt, grad_bpsqt, saved, n_psqt):
+    us, them = _c(us, np.float32).reshape(-1), _c(them, np.float32).reshape(-1)
+    psqt_idx = _c(psqt_idx, np.int64)
+    grad_l0 = _c(grad_l0, np.float32)
+    gwp, gbp = _c(grad_wpsqt, np.float32).reshape(-1), _c(grad_bpsqt, np.float32).reshape(-1)
+    saved = _c(saved, np.float32)
+    B, L1 = grad_l0.shape
+    G = np.empty((2, B, L1 + n_psqt), np.float32)
+    rc = lib().nnueft_oracle_double_bwd_rows(_p(us), _p(them), _p(psqt_idx), ctypes.c_float(max_act),
+                                             _p(grad_l0), _p(gwp), _p(gbp), _p(saved), _p(G), B, L1, n_psqt)
+    assert rc == 0
+    return G
+
+
+def double_bwd(us, them, widx, bidx, psqt_idx, max_act, grad_l0, grad_wpsqt, grad_bpsqt, saved, R, n_psqt):
+    us, them = _c(us, np.float32).reshape(-1), _c(them, np.float32).reshape(-1)
+    widx, bidx = _c(widx, np.int32), _c(bidx, np.int32)
+    psqt_idx = _c(psqt_idx, np.int64)
+    grad_l0 = _c(grad_l0, np.float32)
+    gwp, gbp = _c(grad_wpsqt, np.float32).reshape(-1), _c(grad_bpsqt, np.float32).reshape(-1)
+    saved = _c(saved, np.float32)
+    B, K = widx.shape
+    L1 = grad_l0.shape[1]
+    oc = L1 + n_psqt
+    gW = np.empty((R, oc), np.float32)
+    gb = np.empty((oc,), np.float32)
+    rc = lib().nnueft_oracle_double_bwd(_p(us), _p(them), _p(widx), _p(bidx), _p(psqt_idx),
+                                        ctypes.c_float(max_act), _p(grad_l0), _p(gwp), _p(gbp), _p(saved),
+                                        _p(gW), _p(gb), B, K, R, L1, n_psqt)
+    assert rc == 0
+    return gW, gb
+
+
+def ft_int16_fwd(widx, bidx, stm, W16, b16, psqt32, psqt_idx, clip_max=255, shift=9):
+    widx, bidx = _c(widx, np.int32), _c(bidx, np.int32)
+    stm = _c(stm, np.uint8)
+    W16, b16, psqt32 = _c(W16, np.int16), _c(b16, np.int16), _c(psqt32, np.int32)
+    psqt_idx = _c(psqt_idx, np.int64)
+    B, K = widx.shape
+    R, L1 = W16.shape
+    n_psqt = psqt32.shape[1]
+    out = np.empty((B, L1), np.uint8)
+    ps = np.empty((B,), np.int32)
+    rc = lib().nnueft_oracle_ft_int16_fwd(_p(widx), _p(bidx), _p(stm), _p(W16), _p(b16), _p(psqt32), _p(psqt_idx),
+                                          _p(out), _p(ps), B, K, R, L1, n_psqt, int(clip_max), int(shift))
+    assert rc == 0
+    return out, ps

@@ -1,0 +1,309 @@
+/*
+ * CPU restatement of the nnue-pytorch sparse feature transformer.
+ *
+ * THIS FILE IS TEST INFRASTRUCTURE.  It is the checker the HIP kernels are
+ * compared against and the "port" CPU baseline timed next to them; nothing in
+ * the shipped library links, loads or calls it.
+ *
+ * What each function follows in the reference (paths relative to the
+ * reference checkout):
+ *
+ *   nnueft_oracle_sparse_fwd      model/modules/feature_transformer/sparse_linear_functions.py:16-50
+ *                                 (_torch_sparse_linear: embedding_bag(sum) over the index list with
+ *                                 negative slots masked, then "+ bias")
+ *   nnueft_oracle_sparse_bwd      autograd of the same function; same maths as
+ *                                 sparse_linear_kernel.py:237-288 (gW[idx,:] += g, gb += g)
+ *   nnueft_oracle_double_fwd      double_ft_functions.py:62-80 (the torch composition) ==
+ *                                 fused_ft_kernel.py:27-117 (the fused kernel)
+ *   nnueft_oracle_double_bwd      autograd of double_ft_functions.py:62-80 ==
+ *                                 fused_ft_kernel.py:147-272, except that the clamp mask is torch's
+ *                                 (gradient passes where 0 <= x <= max, x taken before the clamp)
+ *   nnueft_oracle_ft_int16_fwd    no code in the reference (the accumulate runs in the engine);
+ *                                 spec docs/nnue.md:1014-1069 (int16 accumulate) and :2097-2134
+ *                                 (pairwise product, shift), constants model/quantize.py:58-73
+ *
+ * Summation order (this is what "bit-exact" means for the fp32 paths):
+ *   forward   s = +0; s += W[idx_k] for k ascending over the valid slots; out = s + bias.
+ *             torch's CPU embedding_bag produces exactly this (checked in the tests).
+ *   weight    per perspective, one chain per table row starting at +0 and adding the
+ *   gradient  upstream row of every slot that names the table row, slots visited in ascending
+ *             (position, slot) order; the two perspectives' chains are then added
+ *             (white + black).  torch's CPU embedding_bag backward followed by autograd's
+ *             accumulation of the two uses of `weight` produces exactly this.
+ *   bias      positions are cut into tiles of NNUEFT_ORACLE_BIAS_TILE; per column a chain
+ *   gradient  over the positions of a tile (starting at +0, ascending), then a chain over the
+ *             tile sums (starting at +0, ascending).  This order is this build's own; torch
+ *             reduces in a different, unspecified order, so torch agrees to rounding only.
+ *
+ * Indices outside [0, R) (negative padding included) contribute nothing.
+ *
+ * Build:  gcc -O2 -fopenmp -ffp-contract=off -shared -fPIC nnueft_oracle.c -o libnnueft_oracle.so
+ * -ffp-contract=off matters: a*b+c must round twice, like the separate torch ops it restates.
+ */
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define NNUEFT_ORACLE_BIAS_TILE 32
+#define COLBLK 64
+
+int nnueft_oracle_bias_tile(void) { return NNUEFT_ORACLE_BIAS_TILE; }
+
+static inline int valid(int32_t r, int R) { return r >= 0 && r < R; }
+
+/* out[b,:] = (sum_k W[idx[b,k],:]) + bias */
+int nnueft_oracle_sparse_fwd(const int32_t* idx, const float* W, const float* bias, float* out,
+                             int B, int K, int R, int out_cols)
+{
+#pragma omp parallel for schedule(static)
+    for (int b = 0; b < B; ++b) {
+        float* o = out + (size_t)b * out_cols;
+        for (int c = 0; c < out_cols; ++c) o[c] = 0.0f;
+        for (int k = 0; k < K; ++k) {
+            int32_t r = idx[(size_t)b * K + k];
+            if (!valid(r, R)) continue;
+            const float* w = W + (size_t)r * out_cols;
+            for (int c = 0; c < out_cols; ++c) o[c] = o[c] + w[c];
+        }
+        for (int c = 0; c < out_cols; ++c) o[c] = o[c] + bias[c];
+    }
+    return 0;
+}
+
+/* One perspective's chains: acc[r, c0:c1] += G[b, c0:c1] for slots in ascending (b,k). */
+static void scatter_chain(const int32_t* idx, const float* G, size_t g_stride, float* acc,
+                          int B, int K, int R, int out_cols, int c0, int c1)
+{
+    for (int b = 0; b < B; ++b) {
+        const float* g = G + (size_t)b * g_stride;
+        for (int k = 0; k < K; ++k) {
+            int32_t r = idx[(size_t)b * K + k];
+            if (!valid(r, R)) continue;
+            float* a = acc + (size_t)r * out_cols;
+            for (int c = c0; c < c1; ++c) a[c] = a[c] + g[c];
+        }
+    }
+}
+
+/* Tiled column sum: gbias[c] = chain over tiles of (chain over the tile's positions of v[b,c]). */
+static void bias_tiled(const float* V1, const float* V2, size_t stride, float* gbias, int B, int out_cols)
+{
+#pragma omp parallel for schedule(static)
+    for (int c = 0; c < out_cols; ++c) {
+        float total = 0.0f;
+        for (int t0 = 0; t0 < B; t0 += NNUEFT_ORACLE_BIAS_TILE) {
+            int t1 = t0 + NNUEFT_ORACLE_BIAS_TILE < B ? t0 + NNUEFT_ORACLE_BIAS_TILE : B;
+            float part = 0.0f;
+            for (int b = t0; b < t1; ++b) {
+                float v = V1[(size_t)b * stride + c];
+                if (V2) v = v + V2[(size_t)b * stride + c];
+                part = part + v;
+            }
+            total = total + part;
+        }
+        gbias[c] = total;
+    }
+}
+
+/* gW[r,:] = chain over slots naming r of gout[b,:]; gbias = tiled column sum of gout. */
+int nnueft_oracle_sparse_bwd(const int32_t* idx, const float* gout, float* gW, float* gbias,
+                             int B, int K, int R, int out_cols)
+{
+    memset(gW, 0, (size_t)R * out_cols * sizeof(float));
+    int nblk = (out_cols + COLBLK - 1) / COLBLK;
+#pragma omp parallel for schedule(dynamic)
+    for (int j = 0; j < nblk; ++j) {
+        int c0 = j * COLBLK, c1 = c0 + COLBLK < out_cols ? c0 + COLBLK : out_cols;
+        scatter_chain(idx, gout, (size_t)out_cols, gW, B, K, R, out_cols, c0, c1);
+    }
+    bias_tiled(gout, NULL, (size_t)out_cols, gbias, B, out_cols);
+    return 0;
+}
+
+static inline float clampf(float x, float lo, float hi) { return x < lo ? lo : (x > hi ? hi : x); }
+
+/*
+ * Both perspectives, side-to-move mix, clamp, pairwise product.
+ * saved[b,0..3,:] holds the mixed values BEFORE the clamp, in the order
+ * (x_w[:h], x_w[h:], x_b[:h], x_b[h:]), h = L1/2.
+ */
+int nnueft_oracle_double_fwd(const float* us, const float* them,
+                             const int32_t* widx, const int32_t* bidx, const int64_t* psqt_idx,
+                             const float* W, const float* bias, float max_act,
+                             float* l0, float* wpsqt, float* bpsqt, float* saved,
+                             int B, int K, int R, int L1, int n_psqt)
+{
+    const int out_cols = L1 + n_psqt;
+    const int h = L1 / 2;
+    if (L1 % 2) return -1;
+#pragma omp parallel
+    {
+        float* acc = (float*)malloc(sizeof(float) * 2 * (size_t)L1);
+#pragma omp for schedule(static)
+        for (int b = 0; b < B; ++b) {
+            const int64_t pi = psqt_idx[b];
+            const int psqt_ok = pi >= 0 && pi < n_psqt;
+            float ps[2] = {0.0f, 0.0f};
+            for (int p = 0; p < 2; ++p) {
+                const int32_t* ix = (p == 0 ? widx : bidx) + (size_t)b * K;
+                float* a = acc + (size_t)p * L1;
+                for (int c = 0; c < L1; ++c) a[c] = 0.0f;
+                for (int k = 0; k < K; ++k) {
+                    int32_t r = ix[k];
+                    if (!valid(r, R)) continue;
+                    const float* w = W + (size_t)r * out_cols;
+                    for (int c = 0; c < L1; ++c) a[c] = a[c] + w[c];
+                    if (psqt_ok) ps[p] = ps[p] + w[L1 + pi];
+                }
+                for (int c = 0; c < L1; ++c) a[c] = a[c] + bias[c];
+                if (psqt_ok) ps[p] = ps[p] + bias[L1 + pi];
+            }
+            wpsqt[b] = ps[0];
+            bpsqt[b] = ps[1];
+            const float u = us[b], t = them[b];
+            const float* aw = acc;
+            const float* ab = acc + L1;
+            float* sv = saved + (size_t)b * 4 * h;
+            float* o = l0 + (size_t)b * L1;
+            for (int i = 0; i < h; ++i) {
+                float xw0 = u * aw[i] + t * ab[i];
+                float xw1 = u * aw[i + h] + t * ab[i + h];
+                float xb0 = u * ab[i] + t * aw[i];
+                float xb1 = u * ab[i + h] + t * aw[i + h];
+                sv[0 * h + i] = xw0;
+                sv[1 * h + i] = xw1;
+                sv[2 * h + i] = xb0;
+                sv[3 * h + i] = xb1;
+                o[i] = clampf(xw0, 0.0f, max_act) * clampf(xw1, 0.0f, max_act);
+                o[h + i] = clampf(xb0, 0.0f, max_act) * clampf(xb1, 0.0f, max_act);
+            }
+        }
+        free(acc);
+    }
+    return 0;
+}
+
+/*
+ * Per-position upstream rows of the two sparse-linear outputs:
+ * G[p, b, 0:L1] per the product/clamp/mix chain rule, G[p, b, L1+j] = grad_psqt_p[b] if j == psqt_idx[b] else 0.
+ * Layout [2, B, out_cols].
+ */
+int nnueft_oracle_double_bwd_rows(const float* us, const float* them, const int64_t* psqt_idx, float max_act,
+                                  const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt,
+                                  const float* saved, float* G, int B, int L1, int n_psqt)
+{
+    const int out_cols = L1 + n_psqt;
+    const int h = L1 / 2;
+    if (L1 % 2) return -1;
+#pragma omp parallel for schedule(static)
+    for (int b = 0; b < B; ++b) {
+        const float u = us[b], t = them[b];
+        const float* sv = saved + (size_t)b * 4 * h;
+        const float* g = grad_l0 + (size_t)b * L1;
+        float* gw = G + (size_t)b * out_cols;
+        float* gb = G + ((size_t)B + b) * out_cols;
+        for (int i = 0; i < h; ++i) {
+            float xw0 = sv[i], xw1 = sv[h + i], xb0 = sv[2 * h + i], xb1 = sv[3 * h + i];
+            float cw0 = clampf(xw0, 0.0f, max_act), cw1 = clampf(xw1, 0.0f, max_act);
+            float cb0 = clampf(xb0, 0.0f, max_act), cb1 = clampf(xb1, 0.0f, max_act);
+            float dw0 = (xw0 >= 0.0f && xw0 <= max_act) ? g[i] * cw1 : 0.0f;
+            float dw1 = (xw1 >= 0.0f && xw1 <= max_act) ? g[i] * cw0 : 0.0f;
+            float db0 = (xb0 >= 0.0f && xb0 <= max_act) ? g[h + i] * cb1 : 0.0f;
+            float db1 = (xb1 >= 0.0f && xb1 <= max_act) ? g[h + i] * cb0 : 0.0f;
+            gw[i] = u * dw0 + t * db0;
+            gw[h + i] = u * dw1 + t * db1;
+            gb[i] = t * dw0 + u * db0;
+            gb[h + i] = t * dw1 + u * db1;
+        }
+        const int64_t pi = psqt_idx[b];
+        for (int j = 0; j < n_psqt; ++j) {
+            gw[L1 + j] = (j == pi) ? grad_wpsqt[b] : 0.0f;
+            gb[L1 + j] = (j == pi) ? grad_bpsqt[b] : 0.0f;
+        }
+    }
+    return 0;
+}
+
+/* gW = (white chains) + (black chains); gbias = tiled column sum of (G_w + G_b). */
+int nnueft_oracle_double_bwd(const float* us, const float* them,
+                             const int32_t* widx, const int32_t* bidx, const int64_t* psqt_idx,
+                             float max_act,
+                             const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt,
+                             const float* saved, float* gW, float* gbias,
+                             int B, int K, int R, int L1, int n_psqt)
+{
+    const int out_cols = L1 + n_psqt;
+    float* G = (float*)malloc(sizeof(float) * 2 * (size_t)B * out_cols);
+    float* accb = (float*)calloc((size_t)R * out_cols, sizeof(float));
+    if (!G || !accb) { free(G); free(accb); return -2; }
+    int rc = nnueft_oracle_double_bwd_rows(us, them, psqt_idx, max_act, grad_l0, grad_wpsqt, grad_bpsqt,
+                                           saved, G, B, L1, n_psqt);
+    if (rc) { free(G); free(accb); return rc; }
+    memset(gW, 0, (size_t)R * out_cols * sizeof(float));
+    int nblk = (out_cols + COLBLK - 1) / COLBLK;
+#pragma omp parallel for schedule(dynamic)
+    for (int j = 0; j < nblk; ++j) {
+        int c0 = j * COLBLK, c1 = c0 + COLBLK < out_cols ? c0 + COLBLK : out_cols;
+        scatter_chain(widx, G, (size_t)out_cols, gW, B, K, R, out_cols, c0, c1);
+        scatter_chain(bidx, G + (size_t)B * out_cols, (size_t)out_cols, accb, B, K, R, out_cols, c0, c1);
+        for (int r = 0; r < R; ++r)
+            for (int c = c0; c < c1; ++c)
+                gW[(size_t)r * out_cols + c] = gW[(size_t)r * out_cols + c] + accb[(size_t)r * out_cols + c];
+    }
+    bias_tiled(G, G + (size_t)B * out_cols, (size_t)out_cols, gbias, B, out_cols);
+    free(G);
+    free(accb);
+    return 0;
+}
+
+/*
+ * Quantized feature transformer, as the engine evaluates an exported net.
+ *   acc_p[c]  = b16[c] + sum_k W16[idx_p[k], c]          int16, wrapping
+ *   c_p[c]    = min(max(acc_p[c], 0), clip_max)
+ *   out[b, o*h + j] = (c_{P(o)}[j] * c_{P(o)}[j + h]) >> shift     o = 0: side to move, 1: the other side
+ *   psqt_out[b] = (sum_k psqt32[idx_{P(0)}[k], bucket] - sum_k psqt32[idx_{P(1)}[k], bucket]) / 2   (C division)
+ * stm[b] = 0 when white is to move (P(0) = white), 1 when black is.
+ */
+int nnueft_oracle_ft_int16_fwd(const int32_t* widx, const int32_t* bidx, const uint8_t* stm,
+                               const int16_t* W16, const int16_t* b16, const int32_t* psqt32,
+                               const int64_t* psqt_idx, uint8_t* out_u8, int32_t* psqt_out,
+                               int B, int K, int R, int L1, int n_psqt, int clip_max, int shift)
+{
+    const int h = L1 / 2;
+    if (L1 % 2) return -1;
+#pragma omp parallel
+    {
+        int16_t* acc = (int16_t*)malloc(sizeof(int16_t) * 2 * (size_t)L1);
+#pragma omp for schedule(static)
+        for (int b = 0; b < B; ++b) {
+            const int64_t pi = psqt_idx[b];
+            const int psqt_ok = pi >= 0 && pi < n_psqt;
+            int32_t ps[2] = {0, 0};
+            for (int p = 0; p < 2; ++p) {
+                const int32_t* ix = (p == 0 ? widx : bidx) + (size_t)b * K;
+                int16_t* a = acc + (size_t)p * L1;
+                for (int c = 0; c < L1; ++c) a[c] = b16[c];
+                for (int k = 0; k < K; ++k) {
+                    int32_t r = ix[k];
+                    if (!valid(r, R)) continue;
+                    const int16_t* w = W16 + (size_t)r * L1;
+                    for (int c = 0; c < L1; ++c) a[c] = (int16_t)(uint16_t)((uint16_t)a[c] + (uint16_t)w[c]);
+                    if (psqt_ok) ps[p] = (int32_t)((uint32_t)ps[p] + (uint32_t)psqt32[(size_t)r * n_psqt + pi]);
+                }
+            }
+            const int first = stm[b] ? 1 : 0;
+            for (int o = 0; o < 2; ++o) {
+                const int16_t* a = acc + (size_t)(o == 0 ? first : 1 - first) * L1;
+                uint8_t* dst = out_u8 + (size_t)b * L1 + (size_t)o * h;
+                for (int j = 0; j < h; ++j) {
+                    int32_t c0 = a[j] < 0 ? 0 : (a[j] > clip_max ? clip_max : a[j]);
+                    int32_t c1 = a[j + h] < 0 ? 0 : (a[j + h] > clip_max ? clip_max : a[j + h]);
+                    dst[j] = (uint8_t)((c0 * c1) >> shift);
+                }
+            }
+            psqt_out[b] = (ps[first] - ps[1 - first]) / 2;
+        }
+        free(acc);
+    }
+    return 0;
+}

@@ -1,0 +1,221 @@
+"""HIP kernels (through the C ABI of libnnueft.so) against the CPU oracle on the same seeded inputs.
+
+Bars: forward 1e-5 relative, atomic backward 1e-4 relative, deterministic backward and the int16
+path bit-exact.  (The forward and the deterministic weight gradient are in fact compared for
+equality too: their summation order is the oracle's.)
+"""
+import numpy as np
+import pytest
+import torch
+
+from _cases import double_case, sparse_case
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev():
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    return torch.device("cuda:0")
+
+
+def _t(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(_dev())
+
+
+def _rel_err(a, b):
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
+
+
+def _native():
+    from nnueft import _native
+
+    return _native, _native.load()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+SPARSE_SHAPES = [
+    # B, out_cols, R, K
+    (16, 128, 10, 32),      # reference tests/test_feature_transformer.py:36-40 (duplicates)
+    (8, 64, 10, 8),         # its padding case, :83-89
+    (5, 40, 100, 32),       # l1=32 + 8 psqt
+    (33, 1032, 2000, 32),   # L1=1024 row width
+    (7, 3080, 500, 32),     # L1=3072 row width
+    (9, 37, 50, 70),        # odd width (scalar path), K > 64
+    (64, 272, 24576, 32),   # bench_feature_transformer.py:22-25 width, full table height
+]
+
+
+@pytest.mark.parametrize("B,out_cols,R,K", SPARSE_SHAPES)
+def test_sparse_forward(oracle_cpu, B, out_cols, R, K):
+    c = sparse_case(100 + B, B, out_cols, R, K, allow_holes=True)
+    nat, lib = _native()
+    idx, W, bias = _t(c["idx"]), _t(c["W"]), _t(c["bias"])
+    out = torch.empty(B, out_cols, device=_dev())
+    nat.check(lib.nnueft_sparse_fwd(idx.data_ptr(), W.data_ptr(), bias.data_ptr(), out.data_ptr(), B, K, R,
+                                    out_cols, _stream()), "sparse_fwd")
+    ref = oracle_cpu.sparse_fwd(c["idx"], c["W"], c["bias"])
+    got = out.cpu().numpy()
+    assert _rel_err(got, ref) <= 1e-5
+    assert np.array_equal(got, ref), "forward follows the oracle's summation order, so it is bit-exact"
+
+
+@pytest.mark.parametrize("B,out_cols,R,K", SPARSE_SHAPES)
+def test_sparse_backward_atomic(oracle_cpu, B, out_cols, R, K):
+    c = sparse_case(200 + B, B, out_cols, R, K, allow_holes=True)
+    nat, lib = _native()
+    idx, g = _t(c["idx"]), _t(c["g"])
+    gW = torch.zeros(R, out_cols, device=_dev())
+    gb = torch.zeros(out_cols, device=_dev())
+    nat.check(lib.nnueft_sparse_bwd_atomic(idx.data_ptr(), g.data_ptr(), gW.data_ptr(), gb.data_ptr(), B, K, R,
+                                           out_cols, _stream()), "sparse_bwd_atomic")
+    rW, rb = oracle_cpu.sparse_bwd(c["idx"], c["g"], R)
+    assert _rel_err(gW.cpu().numpy(), rW) <= 1e-4
+    assert _rel_err(gb.cpu().numpy(), rb) <= 1e-4
+
+
+@pytest.mark.parametrize("B,out_cols,R,K", SPARSE_SHAPES)
+def test_sparse_backward_deterministic(oracle_cpu, B, out_cols, R, K):
+    c = sparse_case(300 + B, B, out_cols, R, K, allow_holes=True)
+    nat, lib = _native()
+    idx, g = _t(c["idx"]), _t(c["g"])
+    nbytes = lib.nnueft_det_workspace_bytes(B, K, R, out_cols, 1)
+    assert nbytes > 0
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=_dev())
+    # poison the outputs: every element must be written
+    gW = torch.full((R, out_cols), float("nan"), device=_dev())
+    gb = torch.full((out_cols,), float("nan"), device=_dev())
+    nat.check(lib.nnueft_sparse_bwd_det(idx.data_ptr(), g.data_ptr(), gW.data_ptr(), gb.data_ptr(), B, K, R,
+                                        out_cols, ws.data_ptr(), nbytes, _stream()), "sparse_bwd_det")
+    rW, rb = oracle_cpu.sparse_bwd(c["idx"], c["g"], R)
+    assert np.array_equal(gW.cpu().numpy(), rW)
+    assert np.array_equal(gb.cpu().numpy(), rb)
+
+
+DOUBLE_SHAPES = [
+    # B, L1, R, K, kwargs
+    (4, 32, 100, 32, {}),                      # reference tests/test_fused_double_ft.py:19-26
+    (4, 2048, 100, 32, {}),                    # its second parametrisation
+    (19, 264, 3000, 32, dict(binary_side=True)),   # bench_feature_transformer.py width
+    (70, 128, 24576, 32, dict(halfka=True, weight_scale=0.05, max_act=255 / 256)),
+    (40, 1024, 24576, 32, dict(halfka=True, weight_scale=0.05, max_act=255 / 256)),
+    (24, 3072, 24576, 32, dict(halfka=True, weight_scale=0.05, max_act=255 / 256)),
+    (6, 6, 20, 5, dict(n_psqt=3)),             # h = 3: scalar path
+    (6, 50, 20, 80, dict(n_psqt=8, allow_holes=True)),   # K > 64, holes inside the lists
+    (130, 64, 30, 32, dict(n_psqt=0)),         # no psqt columns, more than one sort chunk
+]
+
+
+def _run_double_fwd(c):
+    nat, lib = _native()
+    B, K, R, L1, n_psqt = c["widx"].shape[0], c["K"], c["R"], c["L1"], c["n_psqt"]
+    d = {k: _t(c[k]) for k in ("us", "them", "widx", "bidx", "psqt_idx", "W", "bias")}
+    l0 = torch.empty(B, L1, device=_dev())
+    wp = torch.empty(B, 1, device=_dev())
+    bp = torch.empty(B, 1, device=_dev())
+    saved = torch.empty(B, 4, L1 // 2, device=_dev())
+    nat.check(lib.nnueft_double_fwd(d["us"].data_ptr(), d["them"].data_ptr(), d["widx"].data_ptr(),
+                                    d["bidx"].data_ptr(), d["psqt_idx"].data_ptr(), d["W"].data_ptr(),
+                                    d["bias"].data_ptr(), c["max_act"], l0.data_ptr(), wp.data_ptr(), bp.data_ptr(),
+                                    saved.data_ptr(), B, K, R, L1, n_psqt, _stream()), "double_fwd")
+    return d, l0, wp, bp, saved
+
+
+@pytest.mark.parametrize("B,L1,R,K,kw", DOUBLE_SHAPES)
+def test_double_forward(oracle_cpu, B, L1, R, K, kw):
+    c = double_case(400 + B, B, L1, R, K, **kw)
+    _, l0, wp, bp, saved = _run_double_fwd(c)
+    r_l0, r_wp, r_bp, r_saved = oracle_cpu.double_fwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"],
+                                                      c["W"], c["bias"], c["max_act"], L1)
+    for got, ref in ((l0, r_l0), (wp, r_wp), (bp, r_bp), (saved, r_saved)):
+        got = got.cpu().numpy()
+        assert _rel_err(got, ref) <= 1e-5
+        assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("mode", ["atomic", "deterministic"])
+@pytest.mark.parametrize("B,L1,R,K,kw", DOUBLE_SHAPES)
+def test_double_backward(oracle_cpu, B, L1, R, K, kw, mode):
+    c = double_case(500 + B, B, L1, R, K, **kw)
+    nat, lib = _native()
+    n_psqt = c["n_psqt"]
+    out_cols = L1 + n_psqt
+    d, l0, wp, bp, saved = _run_double_fwd(c)
+    g_l0, g_wp, g_bp = _t(c["g_l0"]), _t(c["g_wp"]), _t(c["g_bp"])
+    head = (d["us"].data_ptr(), d["them"].data_ptr(), d["widx"].data_ptr(), d["bidx"].data_ptr(),
+            d["psqt_idx"].data_ptr(), c["max_act"], g_l0.data_ptr(), g_wp.data_ptr(), g_bp.data_ptr(),
+            saved.data_ptr())
+    if mode == "atomic":
+        gW = torch.zeros(R, out_cols, device=_dev())
+        gb = torch.zeros(out_cols, device=_dev())
+        nat.check(lib.nnueft_double_bwd_atomic(*head, gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt, _stream()),
+                  "double_bwd_atomic")
+    else:
+        nbytes = lib.nnueft_det_workspace_bytes(B, K, R, out_cols, 2)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=_dev())
+        gW = torch.full((R, out_cols), float("nan"), device=_dev())
+        gb = torch.full((out_cols,), float("nan"), device=_dev())
+        nat.check(lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt, ws.data_ptr(),
+                                            nbytes, _stream()), "double_bwd_det")
+    rW, rb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["max_act"],
+                                   c["g_l0"], c["g_wp"], c["g_bp"], saved.cpu().numpy(), R, n_psqt)
+    gW, gb = gW.cpu().numpy(), gb.cpu().numpy()
+    if mode == "atomic":
+        assert _rel_err(gW, rW) <= 1e-4
+        assert _rel_err(gb, rb) <= 1e-4
+    else:
+        assert np.array_equal(gW, rW)
+        assert np.array_equal(gb, rb)
+
+
+def test_deterministic_backward_repeats_bitwise():
+    """Two runs of the deterministic backward give the same bits (the atomic one need not)."""
+    c = double_case(77, 300, 256, 600, 32, binary_side=True)
+    nat, lib = _native()
+    B, K, R, L1, n_psqt = 300, 32, 600, 256, 8
+    d, l0, wp, bp, saved = _run_double_fwd(c)
+    g_l0, g_wp, g_bp = _t(c["g_l0"]), _t(c["g_wp"]), _t(c["g_bp"])
+    nbytes = lib.nnueft_det_workspace_bytes(B, K, R, L1 + n_psqt, 2)
+    outs = []
+    for fill in (0.0, 123.0):
+        ws = torch.full((nbytes,), int(fill) % 251, dtype=torch.uint8, device=_dev())
+        gW = torch.empty(R, L1 + n_psqt, device=_dev())
+        gb = torch.empty(L1 + n_psqt, device=_dev())
+        nat.check(lib.nnueft_double_bwd_det(d["us"].data_ptr(), d["them"].data_ptr(), d["widx"].data_ptr(),
+                                            d["bidx"].data_ptr(), d["psqt_idx"].data_ptr(), c["max_act"],
+                                            g_l0.data_ptr(), g_wp.data_ptr(), g_bp.data_ptr(), saved.data_ptr(),
+                                            gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt, ws.data_ptr(), nbytes,
+                                            _stream()), "double_bwd_det")
+        outs.append((gW.cpu().numpy().copy(), gb.cpu().numpy().copy()))
+    assert np.array_equal(outs[0][0], outs[1][0])
+    assert np.array_equal(outs[0][1], outs[1][1])
+
+
+INT16_SHAPES = [(5, 32, 50, 32), (33, 1024, 22528, 32), (17, 3072, 22528, 32), (9, 38, 40, 70)]
+
+
+@pytest.mark.parametrize("B,L1,R,K", INT16_SHAPES)
+@pytest.mark.parametrize("clip_max,shift", [(255, 9), (127, 7)])
+def test_int16_forward(oracle_cpu, B, L1, R, K, clip_max, shift):
+    rng = np.random.default_rng(600 + B)
+    from _cases import random_lists
+
+    widx = random_lists(rng, B, K, R, allow_holes=True)
+    bidx = random_lists(rng, B, K, R, allow_holes=True)
+    stm = rng.integers(0, 2, size=B).astype(np.uint8)
+    # large enough that some accumulators wrap around int16
+    W16 = rng.integers(-3000, 3000, size=(R, L1)).astype(np.int16)
+    W16[:, : L1 // 3] = rng.integers(-40, 60, size=(R, L1 // 3)).astype(np.int16)
+    b16 = rng.integers(-200, 400, size=L1).astype(np.int16)
+    psqt32 = rng.integers(-100000, 100000, size=(R, 8)).astype(np.int32)
+    psqt_idx = rng.integers(0, 8, size=B).astype(np.int64)
+    from nnueft.quantized import ft_int16_forward
+
+    out, ps = ft_int16_forward(_t(widx), _t(bidx), _t(stm), _t(W16), _t(b16), _t(psqt32), _t(psqt_idx), clip_max, shift)
+    r_out, r_ps = oracle_cpu.ft_int16_fwd(widx, bidx, stm, W16, b16, psqt32, psqt_idx, clip_max, shift)
+    assert np.array_equal(out.cpu().numpy(), r_out)
+    assert np.array_equal(ps.cpu().numpy(), r_ps)
