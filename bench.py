@@ -1,0 +1,271 @@
+#!/usr/bin/env python3
+"""Feature-transformer forward+backward throughput on one MI355X.
+
+A step is one pass of the hot path over one synthetic batch: the fused two-perspective forward
+(nnueft_double_fwd) and the backward into a dense weight gradient, through the same autograd
+function the trainer calls.  Inputs are resident in HBM before the timed region.
+
+Prints ONE JSON line: positions/s for the workload BASELINE.json's metric is quoted on (L1=3072,
+B=16384, HalfKAv2_hm lists, 24576-row table), the roofline of the forward kernel from HIP event
+timings, and the reference's CPU path (torch embedding_bag composition) timed on the host cores
+on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "nnue-pytorch_amd"))
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+WORKLOADS = {
+    # name: (L1, B)
+    "ft_fwd_bwd_L1_3072_B16384": (3072, 16384),
+    "ft_fwd_bwd_L1_1024_B8192": (1024, 8192),
+    "ft_fwd_bwd_L1_128_B16384": (128, 16384),
+}
+R_ROWS = 24576
+N_PSQT = 8
+K_SLOTS = 32
+
+
+def algorithmic_bytes(L1, B, sum_a, mode):
+    """Logical bytes of one step, no reuse between positions assumed (a = active rows of both lists)."""
+    oc = L1 + N_PSQT
+    fwd = sum_a * oc * 4 + B * (2 * K_SLOTS * 4 + 16 + L1 * 4 + 2 * L1 * 4 + 8)
+    if mode == "atomic":
+        bwd = sum_a * oc * 8 + B * (L1 * 4 + 2 * L1 * 4 + 2 * K_SLOTS * 4 + 24) + R_ROWS * oc * 4
+    else:
+        # read grad_l0 + saved, write the two upstream rows, gather them once per slot, one 8-byte
+        # key/value pass for the counting sort, every table row written once
+        bwd = B * (3 * L1 * 4 + 2 * oc * 4) + sum_a * oc * 4 + sum_a * 8 + R_ROWS * oc * 4
+    return fwd, bwd
+
+
+def make_inputs(L1, B, seed, device):
+    import numpy as np
+    import torch
+    from nnueft import halfka_v2_hm as hk
+
+    us, them, white, black, pc = hk.synthetic_batch(B, seed)
+    rng = np.random.default_rng(seed)
+    oc = L1 + N_PSQT
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    W = (torch.randn(R_ROWS, oc, generator=g) * 0.01)
+    bias = torch.zeros(oc)
+    t = {
+        "us": torch.from_numpy(us), "them": torch.from_numpy(them),
+        "white": torch.from_numpy(white), "black": torch.from_numpy(black),
+        "psqt_idx": torch.from_numpy((pc - 1) // 4),
+        "W": W, "bias": bias,
+        "g_l0": torch.randn(B, L1, generator=g), "g_wp": torch.randn(B, 1, generator=g),
+        "g_bp": torch.randn(B, 1, generator=g),
+    }
+    sum_a = int((white >= 0).sum() + (black >= 0).sum())
+    del rng
+    if device is not None:
+        t = {k: v.to(device) for k, v in t.items()}
+    return t, sum_a
+
+
+def cpu_baseline(L1, B_full, seed, budget_s=20.0):
+    """The reference's CPU path (oracle.ref_torch) on a sample of the workload's positions."""
+    import torch
+    from oracle import ref_torch
+
+    cores = len(os.sched_getaffinity(0))
+    cores = min(cores, 16) if os.environ.get("GRAFT_REPO_ROOT") else cores
+    torch.set_num_threads(cores)
+    B = min(B_full, 4096)
+    t, _ = make_inputs(L1, B_full, seed, None)
+    sl = slice(0, B)
+    W = t["W"].clone().requires_grad_()
+    bias = t["bias"].clone().requires_grad_()
+
+    def step():
+        W.grad = None
+        bias.grad = None
+        out = ref_torch.double_feature_transform(t["us"][sl], t["them"][sl], t["white"][sl], t["black"][sl],
+                                                 t["psqt_idx"][sl], W, bias, 255.0 / 256.0, L1)
+        torch.autograd.backward(list(out), [t["g_l0"][sl], t["g_wp"][sl], t["g_bp"][sl]])
+
+    step()  # warm-up
+    n, t0 = 0, time.perf_counter()
+    while True:
+        step()
+        n += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or n >= 8:
+            break
+    return {
+        "value": B * n / el, "unit": "positions/s", "cores": cores, "kind": "port",
+        "sample": f"first {B} positions of the {B_full}-position batch, same 24576x{L1 + N_PSQT} table, "
+                  f"{n} fwd+bwd steps of the torch embedding_bag composition (autograd backward), 1 warm-up",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="ft_fwd_bwd_L1_3072_B16384", choices=sorted(WORKLOADS))
+    ap.add_argument("--backward", default="deterministic", choices=["deterministic", "atomic"],
+                    help="backward mode the headline value is measured with (the other one is reported beside it)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", default="", help="time only this part (fwd, det, atomic): for profiling runs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import nnueft
+    from nnueft import _native
+    from nnueft.double_ft_functions import double_feature_transform
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    lib = _native.load()  # raises if libnnueft.so is missing: there is no fallback
+    dev = torch.device("cuda:0")
+    L1, B = WORKLOADS[args.workload]
+    seed = 1234 + 3
+    t, sum_a = make_inputs(L1, B, seed, dev)
+    W = t["W"].requires_grad_()
+    bias = t["bias"].requires_grad_()
+    max_act = 255.0 / 256.0
+
+    def step(mode):
+        nnueft.set_backward_mode(mode)
+        W.grad = None
+        bias.grad = None
+        out = double_feature_transform(t["us"], t["them"], t["white"], t["black"], t["psqt_idx"], W, bias,
+                                       max_act, L1, "fused")
+        torch.autograd.backward(list(out), [t["g_l0"], t["g_wp"], t["g_bp"]])
+
+    def time_steps(fn, steps, warmup):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        return wall / steps * 1e3, e0.elapsed_time(e1) / steps
+
+    results = {}
+    modes = [args.backward] + [m for m in ("deterministic", "atomic") if m != args.backward]
+    if args.only in ("det", "atomic"):
+        modes = ["deterministic" if args.only == "det" else "atomic"]
+    if args.only != "fwd":
+        for mode in modes:
+            ms_wall, ms_ev = time_steps(lambda: step(mode), args.steps, args.warmup)
+            results[mode] = ms_wall
+
+    # the forward kernel alone (one launch per call), HIP events on the launch stream
+    B_, K_ = t["white"].shape
+    l0 = torch.empty(B, L1, device=dev)
+    wp = torch.empty(B, 1, device=dev)
+    bp = torch.empty(B, 1, device=dev)
+    saved = torch.empty(B, 4, L1 // 2, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    Wd, bd = W.detach(), bias.detach()
+
+    def fwd_only():
+        rc = lib.nnueft_double_fwd(t["us"].data_ptr(), t["them"].data_ptr(), t["white"].data_ptr(),
+                                   t["black"].data_ptr(), t["psqt_idx"].data_ptr(), Wd.data_ptr(), bd.data_ptr(),
+                                   max_act, l0.data_ptr(), wp.data_ptr(), bp.data_ptr(), saved.data_ptr(),
+                                   B, K_, R_ROWS, L1, N_PSQT, stream)
+        assert rc == 0
+
+    _, fwd_ms = time_steps(fwd_only, max(args.steps, 10), args.warmup)
+
+    # the backward entry points alone
+    bwd_ms = {}
+    if args.only != "fwd":
+        g_l0, g_wp, g_bp = t["g_l0"], t["g_wp"], t["g_bp"]
+        oc = L1 + N_PSQT
+        nbytes = lib.nnueft_det_workspace_bytes(B, K_, R_ROWS, oc, 2)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        gW = torch.empty(R_ROWS, oc, device=dev)
+        gb = torch.empty(oc, device=dev)
+        head = (t["us"].data_ptr(), t["them"].data_ptr(), t["white"].data_ptr(), t["black"].data_ptr(),
+                t["psqt_idx"].data_ptr(), max_act, g_l0.data_ptr(), g_wp.data_ptr(), g_bp.data_ptr(), saved.data_ptr())
+
+        def bwd_det():
+            rc = lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT,
+                                           ws.data_ptr(), nbytes, stream)
+            assert rc == 0
+
+        def bwd_atomic():
+            gW.zero_()
+            gb.zero_()
+            rc = lib.nnueft_double_bwd_atomic(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT, stream)
+            assert rc == 0
+
+        for name, fn in (("deterministic", bwd_det), ("atomic", bwd_atomic)):
+            if name in modes:
+                _, bwd_ms[name] = time_steps(fn, max(args.steps, 10), args.warmup)
+
+    fwd_bytes, _ = algorithmic_bytes(L1, B, sum_a, "atomic")
+    fwd_gbs = fwd_bytes / (fwd_ms * 1e-3) / 1e9
+    head_mode = modes[0]
+    ms_step = results.get(head_mode, float("nan"))
+    out = {
+        "metric": "FT fwd+bwd positions/sec at L1=3072,B=16384; achieved GB/s vs HBM peak"
+        if args.workload == "ft_fwd_bwd_L1_3072_B16384" else f"FT fwd+bwd positions/sec ({args.workload})",
+        "value": B / (ms_step * 1e-3) if ms_step == ms_step else None,
+        "unit": "positions/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": args.workload, "L1": L1, "batch": B, "table_rows": R_ROWS, "psqt_columns": N_PSQT,
+            "slots": K_SLOTS, "active_rows_per_position": sum_a / B, "backward": head_mode,
+            "index_scheme": "HalfKAv2_hm, seeded random positions",
+        },
+        "roofline": {
+            "kernel": "k_double_fwd (nnueft_double_fwd)",
+            "bound": "hbm", "achieved": fwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": fwd_gbs / HBM_PEAK_GBS, "traffic": None,
+            "algorithmic_bytes_per_launch": fwd_bytes, "avg_launch_ms": fwd_ms,
+        },
+    }
+    step_stats = {}
+    for mode in modes:
+        if mode not in results:
+            continue
+        fb, bb = algorithmic_bytes(L1, B, sum_a, mode)
+        ms = results[mode]
+        step_stats[mode] = {
+            "ms_per_step": ms, "positions_per_s": B / (ms * 1e-3),
+            "algorithmic_GBs": (fb + bb) / (ms * 1e-3) / 1e9,
+            "frac_of_hbm_peak": (fb + bb) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "backward_entry_ms": bwd_ms.get(mode),
+            "backward_algorithmic_GBs": bb / (bwd_ms[mode] * 1e-3) / 1e9 if mode in bwd_ms else None,
+        }
+    out["step"] = step_stats
+    if not args.no_cpu_baseline and not args.only:
+        out["cpu_baseline"] = cpu_baseline(L1, B, seed)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

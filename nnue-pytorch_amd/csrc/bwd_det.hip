@@ -271,17 +271,29 @@ __global__ __launch_bounds__(256) void k_fill(const int32_t* __restrict__ widx, 
     const int lane = threadIdx.x;
     const uint32_t id0 = (uint32_t)p * (uint32_t)B + (uint32_t)pos0;
     constexpr int PF = 8;
-    for (int k0 = 0; k0 < K; k0 += 64) {
-        const bool in_k = k0 + lane < K;
+    if (K <= 64) {
+        // one slot group per position: fetch the indices of PF positions ahead of their atomics
+        const bool in_k = lane < K;
         for (int i0 = 0; i0 < npos; i0 += PF) {
             int r[PF];
 #pragma unroll
-            for (int u = 0; u < PF; ++u) r[u] = (in_k && i0 + u < npos) ? ix[(size_t)(i0 + u) * K + k0 + lane] - r0 : -1;
+            for (int u = 0; u < PF; ++u) r[u] = (in_k && i0 + u < npos) ? ix[(size_t)(i0 + u) * K + lane] - r0 : -1;
 #pragma unroll
             for (int u = 0; u < PF; ++u) {
                 if (r[u] >= 0 && r[u] < nr) {
                     const uint32_t slot = atomicAdd(&lds_u32[r[u]], 1u);
                     list[slot] = id0 + (uint32_t)(i0 + u);
+                }
+            }
+        }
+    } else {
+        // all slot groups of a position before the next position
+        for (int i = 0; i < npos; ++i) {
+            for (int k0 = 0; k0 < K; k0 += 64) {
+                const int r = (k0 + lane < K) ? ix[(size_t)i * K + k0 + lane] - r0 : -1;
+                if (r >= 0 && r < nr) {
+                    const uint32_t slot = atomicAdd(&lds_u32[r], 1u);
+                    list[slot] = id0 + (uint32_t)i;
                 }
             }
         }
