@@ -117,7 +117,9 @@ def main():
     ap.add_argument("--backward", default="deterministic", choices=["deterministic", "atomic"],
                     help="backward mode the headline value is measured with (the other one is reported beside it)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", default="", help="time only this part (fwd, det, atomic): for profiling runs")
+    ap.add_argument("--only", default="", choices=["", "fwd", "det", "atomic", "copy"],
+                    help="run only this part (for profiling runs); 'copy' launches a plain elementwise kernel "
+                         "reading and writing 1 GiB each, the yardstick the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -133,6 +135,16 @@ def main():
         sys.exit(2)
     lib = _native.load()  # raises if libnnueft.so is missing: there is no fallback
     dev = torch.device("cuda:0")
+    if args.only == "copy":
+        n = (1 << 30) // 4
+        src = torch.ones(n, device=dev)
+        dst = torch.empty(n, device=dev)
+        for _ in range(args.warmup + args.steps):
+            torch.add(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "torch.add(src, 1.0, out=dst)", "read_bytes": n * 4, "write_bytes": n * 4,
+                          "launches": args.warmup + args.steps}))
+        return
     L1, B = WORKLOADS[args.workload]
     seed = 1234 + 3
     t, sum_a = make_inputs(L1, B, seed, dev)

@@ -139,13 +139,23 @@ __global__ __launch_bounds__(256) void k_tile_colsum(const float* __restrict__ g
     partial[(size_t)tile * out_cols + c] = part;
 }
 
-// gbias[c] = chain over the tiles of partial[tile, c]
-__global__ __launch_bounds__(256) void k_bias_final(const float* __restrict__ partial, float* __restrict__ gbias,
-                                                    int ntiles, int out_cols) {
-    const int c = blockIdx.x * 256 + threadIdx.x;
+// gbias[c] = chain over the tiles of partial[tile, c].  The adds are one dependent chain; the loads
+// are not, so they are issued a batch ahead.
+__global__ __launch_bounds__(64) void k_bias_final(const float* __restrict__ partial, float* __restrict__ gbias,
+                                                   int ntiles, int out_cols) {
+    const int c = blockIdx.x * 64 + threadIdx.x;
     if (c >= out_cols) return;
+    constexpr int PF = 32;
     float total = 0.0f;
-    for (int t = 0; t < ntiles; ++t) total = total + partial[(size_t)t * out_cols + c];
+    int t = 0;
+    for (; t + PF <= ntiles; t += PF) {
+        float v[PF];
+#pragma unroll
+        for (int u = 0; u < PF; ++u) v[u] = partial[(size_t)(t + u) * out_cols + c];
+#pragma unroll
+        for (int u = 0; u < PF; ++u) total = total + v[u];
+    }
+    for (; t < ntiles; ++t) total = total + partial[(size_t)t * out_cols + c];
     gbias[c] = total;
 }
 
@@ -186,12 +196,25 @@ __global__ __launch_bounds__(256) void k_chunk_hist(const int32_t* __restrict__ 
 }
 
 // Per table row: chunk counts -> exclusive offsets; total and white share.
-__global__ __launch_bounds__(256) void k_col_scan(uint32_t* __restrict__ cnt, uint32_t* __restrict__ wcount,
-                                                  uint32_t* __restrict__ seg_off, int R, int cpp, int nchunks) {
-    const int r = blockIdx.x * 256 + threadIdx.x;
+__global__ __launch_bounds__(64) void k_col_scan(uint32_t* __restrict__ cnt, uint32_t* __restrict__ wcount,
+                                                 uint32_t* __restrict__ seg_off, int R, int cpp, int nchunks) {
+    const int r = blockIdx.x * 64 + threadIdx.x;
     if (r >= R) return;
+    constexpr int PF = 16;
     uint32_t run = 0, white = 0;
-    for (int c = 0; c < nchunks; ++c) {
+    int c = 0;
+    for (; c + PF <= nchunks; c += PF) {
+        uint32_t t[PF];
+#pragma unroll
+        for (int u = 0; u < PF; ++u) t[u] = cnt[(size_t)(c + u) * R + r];
+#pragma unroll
+        for (int u = 0; u < PF; ++u) {
+            if (c + u == cpp) white = run;
+            cnt[(size_t)(c + u) * R + r] = run;
+            run += t[u];
+        }
+    }
+    for (; c < nchunks; ++c) {
         if (c == cpp) white = run;
         const uint32_t t = cnt[(size_t)c * R + r];
         cnt[(size_t)c * R + r] = run;
@@ -207,30 +230,27 @@ __global__ __launch_bounds__(256) void k_col_scan(uint32_t* __restrict__ cnt, ui
 // so the longest chains start first.
 constexpr int kScanThreads = 1024;
 constexpr int kLenBins = 1024;
+constexpr int kScanPer = 32;   // rows a thread keeps in registers per pass
 __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict__ seg_off,
                                                            uint32_t* __restrict__ row_order, int R) {
     __shared__ uint32_t sums[kScanThreads];
     __shared__ uint32_t bins[kLenBins];
+    __shared__ uint32_t carry_s;
     const int tid = threadIdx.x;
-    const int per = (R + kScanThreads - 1) / kScanThreads;
-    const int r0 = min(tid * per, R), r1 = min(r0 + per, R);
     if (tid < kLenBins) bins[tid] = 0;
-    uint32_t local = 0;
-    for (int r = r0; r < r1; ++r) local += seg_off[r];
-    sums[tid] = local;
+    if (tid == 0) carry_s = 0;
     __syncthreads();
-    for (int r = r0; r < r1; ++r) atomicAdd(&bins[min(seg_off[r], (uint32_t)(kLenBins - 1))], 1u);
-    // inclusive scan of sums (Hillis-Steele)
-    for (int d = 1; d < kScanThreads; d <<= 1) {
-        const uint32_t add = tid >= d ? sums[tid - d] : 0;
-        __syncthreads();
-        sums[tid] += add;
-        __syncthreads();
+    // pass A: length histogram (for the longest-first order)
+    for (int rb = tid; rb < R; rb += kScanThreads * 8) {
+        uint32_t len[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) len[u] = (rb + u * kScanThreads < R) ? seg_off[rb + u * kScanThreads] : 0;
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (rb + u * kScanThreads < R) atomicAdd(&bins[min(len[u], (uint32_t)(kLenBins - 1))], 1u);
     }
-    uint32_t run = sums[tid] - local;
-    const uint32_t grand = sums[kScanThreads - 1];
     __syncthreads();
-    // bins -> start of each length class, longest class first
+    // bins -> first slot of each length class, longest class first
     if (tid < kLenBins) sums[tid] = bins[kLenBins - 1 - tid];
     __syncthreads();
     for (int d = 1; d < kLenBins; d <<= 1) {
@@ -242,22 +262,49 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
     }
     if (tid < kLenBins) bins[kLenBins - 1 - tid] = sums[tid] - bins[kLenBins - 1 - tid];
     __syncthreads();
-    for (int r = r0; r < r1; ++r) {
-        const uint32_t len = seg_off[r];
-        const uint32_t slot = atomicAdd(&bins[min(len, (uint32_t)(kLenBins - 1))], 1u);
-        row_order[slot] = (uint32_t)r;
-        seg_off[r] = run;
-        run += len;
+    // pass B: exclusive scan of the lengths, kScanThreads * kScanPer rows at a time
+    for (int base = 0; base < R; base += kScanThreads * kScanPer) {
+        const int r0 = base + tid * kScanPer;
+        uint32_t len[kScanPer];
+        uint32_t local = 0;
+#pragma unroll
+        for (int u = 0; u < kScanPer; ++u) {
+            len[u] = (r0 + u < R) ? seg_off[r0 + u] : 0;
+            local += len[u];
+        }
+        sums[tid] = local;
+        __syncthreads();
+        for (int d = 1; d < kScanThreads; d <<= 1) {
+            const uint32_t add = tid >= d ? sums[tid - d] : 0;
+            __syncthreads();
+            sums[tid] += add;
+            __syncthreads();
+        }
+        uint32_t run = carry_s + sums[tid] - local;
+        const uint32_t block_total = sums[kScanThreads - 1];
+#pragma unroll
+        for (int u = 0; u < kScanPer; ++u) {
+            if (r0 + u < R) {
+                const uint32_t slot = atomicAdd(&bins[min(len[u], (uint32_t)(kLenBins - 1))], 1u);
+                row_order[slot] = (uint32_t)(r0 + u);
+                seg_off[r0 + u] = run;
+                run += len[u];
+            }
+        }
+        __syncthreads();
+        if (tid == 0) carry_s += block_total;
+        __syncthreads();
     }
-    if (tid == 0) seg_off[R] = grand;
+    if (tid == 0) seg_off[R] = carry_s;
 }
 
 // Every slot of the chunk writes its position id.  Ranks inside the chunk are handed out position
 // by position (one LDS atomic per position and slot group), so a row's list is in position order.
+// LDS: `range` cursors, then (when they fit) the chunk's index lists staged by all four waves.
 __global__ __launch_bounds__(256) void k_fill(const int32_t* __restrict__ widx, const int32_t* __restrict__ bidx,
                                               const uint32_t* __restrict__ cnt,
                                               const uint32_t* __restrict__ seg_off, uint32_t* __restrict__ list,
-                                              int B, int K, int R, int cpp, int range) {
+                                              int B, int K, int R, int cpp, int range, int stage) {
     extern __shared__ uint32_t lds_u32[];
     const int c = blockIdx.x;
     const int r0 = blockIdx.y * range;
@@ -265,36 +312,39 @@ __global__ __launch_bounds__(256) void k_fill(const int32_t* __restrict__ widx, 
     int pos0, npos, p;
     const int32_t* ix = chunk_indices(widx, bidx, c, cpp, B, K, &pos0, &npos, &p);
     const uint32_t* coff = cnt + (size_t)c * R + r0;
-    for (int j = threadIdx.x; j < nr; j += 256) lds_u32[j] = seg_off[r0 + j] + coff[j];
+    {
+        // cursors = segment offset + offset of this chunk inside the segment; loads batched 8 deep
+        constexpr int PF = 8;
+        for (int j0 = threadIdx.x; j0 < nr; j0 += 256 * PF) {
+            uint32_t a[PF], b[PF];
+#pragma unroll
+            for (int u = 0; u < PF; ++u) {
+                const int j = j0 + u * 256;
+                a[u] = j < nr ? seg_off[r0 + j] : 0;
+                b[u] = j < nr ? coff[j] : 0;
+            }
+#pragma unroll
+            for (int u = 0; u < PF; ++u) {
+                const int j = j0 + u * 256;
+                if (j < nr) lds_u32[j] = a[u] + b[u];
+            }
+        }
+    }
+    int32_t* staged = reinterpret_cast<int32_t*>(lds_u32 + range);
+    if (stage)
+        for (int i = threadIdx.x; i < npos * K; i += 256) staged[i] = ix[i];
     __syncthreads();
     if (threadIdx.x >= 64) return;
     const int lane = threadIdx.x;
     const uint32_t id0 = (uint32_t)p * (uint32_t)B + (uint32_t)pos0;
-    constexpr int PF = 8;
-    if (K <= 64) {
-        // one slot group per position: fetch the indices of PF positions ahead of their atomics
-        const bool in_k = lane < K;
-        for (int i0 = 0; i0 < npos; i0 += PF) {
-            int r[PF];
-#pragma unroll
-            for (int u = 0; u < PF; ++u) r[u] = (in_k && i0 + u < npos) ? ix[(size_t)(i0 + u) * K + lane] - r0 : -1;
-#pragma unroll
-            for (int u = 0; u < PF; ++u) {
-                if (r[u] >= 0 && r[u] < nr) {
-                    const uint32_t slot = atomicAdd(&lds_u32[r[u]], 1u);
-                    list[slot] = id0 + (uint32_t)(i0 + u);
-                }
-            }
-        }
-    } else {
-        // all slot groups of a position before the next position
-        for (int i = 0; i < npos; ++i) {
-            for (int k0 = 0; k0 < K; k0 += 64) {
-                const int r = (k0 + lane < K) ? ix[(size_t)i * K + k0 + lane] - r0 : -1;
-                if (r >= 0 && r < nr) {
-                    const uint32_t slot = atomicAdd(&lds_u32[r], 1u);
-                    list[slot] = id0 + (uint32_t)i;
-                }
+    // all slot groups of a position before the next position
+    for (int i = 0; i < npos; ++i) {
+        for (int k0 = 0; k0 < K; k0 += 64) {
+            int r = -1;
+            if (k0 + lane < K) r = (stage ? staged[i * K + k0 + lane] : ix[(size_t)i * K + k0 + lane]) - r0;
+            if (r >= 0 && r < nr) {
+                const uint32_t slot = atomicAdd(&lds_u32[r], 1u);
+                list[slot] = id0 + (uint32_t)i;
             }
         }
     }
@@ -351,14 +401,25 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
     }
 }
 
-int lds_range(int R) {
+// Table rows per sort pass and whether the chunk's index lists are staged in LDS by k_fill.
+bool lds_plan(int R, int K, int* range_out, int* stage_out, size_t* hist_bytes, size_t* fill_bytes) {
     int dev = 0, max_lds = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return 0;
-    if (hipDeviceGetAttribute(&max_lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess) return 0;
-    int range = max_lds / (int)sizeof(uint32_t);
+    if (hipGetDevice(&dev) != hipSuccess) return false;
+    if (hipDeviceGetAttribute(&max_lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess) return false;
+    if (max_lds < 16 * 1024) return false;
+    const size_t stage_bytes = (size_t)kChunk * K * sizeof(int32_t);
+    const int stage = stage_bytes <= (size_t)max_lds / 4;
+    const size_t avail = (size_t)max_lds - (stage ? stage_bytes : 0);
+    int range = (int)(avail / sizeof(uint32_t));
     range = min(range, 32768);
     range = min(range, (R + 255) / 256 * 256);
-    return range;
+    range = range / 256 * 256;
+    if (range <= 0) return false;
+    *range_out = range;
+    *stage_out = stage;
+    *hist_bytes = (size_t)range * sizeof(uint32_t);
+    *fill_bytes = *hist_bytes + (stage ? stage_bytes : 0);
+    return true;
 }
 
 // Common tail of the two deterministic entry points.
@@ -371,27 +432,27 @@ int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, fl
     uint32_t* list = (uint32_t*)(ws + L.list);
     float* partial = (float*)(ws + L.partial);
 
-    const int range = lds_range(R);
-    if (range <= 0) return NNUEFT_E_UNSUPPORTED;
+    int range = 0, stage = 0;
+    size_t hist_bytes = 0, fill_bytes = 0;
+    if (!lds_plan(R, K, &range, &stage, &hist_bytes, &fill_bytes)) return NNUEFT_E_UNSUPPORTED;
     const int nranges = (R + range - 1) / range;
-    const size_t lds_bytes = (size_t)range * sizeof(uint32_t);
-    if (lds_bytes > 48 * 1024) {
+    if (fill_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void*)k_chunk_hist, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)lds_bytes);
+                                           (int)hist_bytes);
         if (e != hipSuccess) return (int)e;
-        e = hipFuncSetAttribute((const void*)k_fill, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        e = hipFuncSetAttribute((const void*)k_fill, hipFuncAttributeMaxDynamicSharedMemorySize, (int)fill_bytes);
         if (e != hipSuccess) return (int)e;
     }
-    hipLaunchKernelGGL(k_chunk_hist, dim3(L.nchunks, nranges), dim3(256), lds_bytes, st, widx, bidx, cnt, B, K, R,
+    hipLaunchKernelGGL(k_chunk_hist, dim3(L.nchunks, nranges), dim3(256), hist_bytes, st, widx, bidx, cnt, B, K, R,
                        L.cpp, range);
     NNUEFT_LAUNCH_CHECK();
-    hipLaunchKernelGGL(k_col_scan, dim3((R + 255) / 256), dim3(256), 0, st, cnt, wcount, seg_off, R, L.cpp,
+    hipLaunchKernelGGL(k_col_scan, dim3((R + 63) / 64), dim3(64), 0, st, cnt, wcount, seg_off, R, L.cpp,
                        L.nchunks);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_row_scan, dim3(1), dim3(kScanThreads), 0, st, seg_off, row_order, R);
     NNUEFT_LAUNCH_CHECK();
-    hipLaunchKernelGGL(k_fill, dim3(L.nchunks, nranges), dim3(256), lds_bytes, st, widx, bidx, cnt, seg_off, list,
-                       B, K, R, L.cpp, range);
+    hipLaunchKernelGGL(k_fill, dim3(L.nchunks, nranges), dim3(256), fill_bytes, st, widx, bidx, cnt, seg_off, list,
+                       B, K, R, L.cpp, range, stage);
     NNUEFT_LAUNCH_CHECK();
 
     const bool vec = (out_cols % 4 == 0) && aligned16(G) && aligned16(gW);
@@ -399,7 +460,9 @@ int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, fl
     const int nv = out_cols / VWr;
     const int NQ = nv > 64 ? 2 : 1;
     const int nslices = (nv + 64 * NQ - 1) / (64 * NQ);
-    const int slice_v = (nv + nslices - 1) / nslices;
+    // equal slices, rounded up to whole 128-byte lines so no two waves share a cache line of a row
+    const int line_v = 128 / (VWr * (int)sizeof(float));
+    const int slice_v = ((nv + nslices - 1) / nslices + line_v - 1) / line_v * line_v;
     const long long grid = (long long)R * nslices;
     if (grid > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
     const int two = n_persp == 2;
@@ -413,7 +476,7 @@ int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, fl
 #undef SEG_LAUNCH
     NNUEFT_LAUNCH_CHECK();
 
-    hipLaunchKernelGGL(k_bias_final, dim3((out_cols + 255) / 256), dim3(256), 0, st, partial, gbias, L.ntiles,
+    hipLaunchKernelGGL(k_bias_final, dim3((out_cols + 63) / 64), dim3(64), 0, st, partial, gbias, L.ntiles,
                        out_cols);
     NNUEFT_LAUNCH_CHECK();
     return 0;

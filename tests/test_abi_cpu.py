@@ -1,0 +1,59 @@
+"""The C-ABI library loads and exports what include/nnueft.h declares (no GPU, no compute calls)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from nnueft import _native
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "nnueft.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(nnueft_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    syms = declared_symbols()
+    for name in ("nnueft_sparse_fwd", "nnueft_sparse_bwd_atomic", "nnueft_sparse_bwd_det", "nnueft_double_fwd",
+                 "nnueft_double_bwd_atomic", "nnueft_double_bwd_det", "nnueft_det_workspace_bytes",
+                 "nnueft_ft_int16_fwd", "nnueft_version", "nnueft_error_string", "nnueft_bias_tile"):
+        assert name in syms
+
+
+def test_library_exports_every_declared_symbol():
+    assert os.path.exists(_native.LIB_PATH), "libnnueft.so is not built (python -c 'import __graft_entry__ as g; g.build()')"
+    lib = ctypes.CDLL(_native.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(lib, name), f"{name} is declared in nnueft.h but not exported"
+
+
+def test_binding_covers_every_declared_symbol():
+    assert sorted(_native.PROTOTYPES) == declared_symbols()
+    assert _native.available()
+
+
+def test_host_only_entry_points():
+    lib = _native.load()
+    assert lib.nnueft_version() == 1
+    assert lib.nnueft_bias_tile() == 32
+    assert lib.nnueft_error_string(0) == b"success"
+    for code in (-1, -2, -3):
+        assert lib.nnueft_error_string(code).startswith(b"nnueft:")
+    # workspace size: monotone, 256-byte granular, zero for nonsense
+    a = lib.nnueft_det_workspace_bytes(16384, 32, 24576, 3080, 2)
+    b = lib.nnueft_det_workspace_bytes(16384, 32, 24576, 3080, 1)
+    assert a > b > 0 and a % 256 == 0 and b % 256 == 0
+    assert a >= 2 * 16384 * 3080 * 4          # holds the two upstream rows of every position
+    assert lib.nnueft_det_workspace_bytes(0, 32, 10, 8, 1) == 0
+    assert lib.nnueft_det_workspace_bytes(4, 32, 10, 8, 3) == 0
+
+
+def test_check_raises_with_the_library_message():
+    with pytest.raises(RuntimeError, match="invalid argument"):
+        _native.check(-1, "unit test")
+    _native.check(0, "unit test")

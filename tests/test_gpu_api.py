@@ -1,0 +1,293 @@
+"""The Python mirror of the reference interface on the GPU: the reference's own tests restated
+(same shapes, seeds and tolerances), the BASELINE configurations at full size against the oracle,
+edge cases (empty batch, one hot row, non-default stream) and the error paths of the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+import nnueft
+from _cases import double_case, random_lists, sparse_case
+from nnueft import _native
+from nnueft import halfka_v2_hm as hk
+from nnueft.double_ft_functions import double_feature_transform
+from nnueft.sparse_linear_functions import SparseLinearFunction
+from oracle import ref_torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(autouse=True)
+def _restore_mode():
+    old = nnueft.get_backward_mode()
+    yield
+    nnueft.set_backward_mode(old)
+
+
+def _emulate(indices, weight, bias):
+    # tests/test_feature_transformer.py:14-32
+    dense = torch.zeros(indices.shape[0], weight.shape[0], dtype=torch.float32)
+    for i in range(indices.shape[0]):
+        for j in range(indices.shape[1]):
+            if indices[i, j] >= 0:
+                dense[i, indices[i, j]] += 1.0
+    return torch.mm(dense, weight) + bias
+
+
+@pytest.mark.parametrize("mode", ["atomic", "deterministic"])
+def test_reference_sparse_linear_test_on_gpu(mode):
+    # tests/test_feature_transformer.py:35-78 with device = cuda
+    nnueft.set_backward_mode(mode)
+    torch.manual_seed(0)
+    weight0 = torch.rand(10, 128, requires_grad=True)
+    bias0 = torch.rand(128, requires_grad=True)
+    torch.manual_seed(0)
+    weight1 = torch.rand(10, 128, requires_grad=True)
+    bias1 = torch.rand(128, requires_grad=True)
+    indices0 = (torch.rand(16, 32) * 10).to(dtype=torch.int32)
+    indices1 = (torch.rand(16, 32) * 10).to(dtype=torch.int32)
+    out00 = _emulate(indices0, weight0, bias0)
+    out01 = _emulate(indices1, weight0, bias0)
+    out10 = SparseLinearFunction.apply(indices0.to(DEV), weight1.to(DEV), bias1.to(DEV))
+    out11 = SparseLinearFunction.apply(indices1.to(DEV), weight1.to(DEV), bias1.to(DEV))
+    assert torch.max(torch.abs(out00 - out10.cpu())) < 1e-4
+    assert torch.max(torch.abs(out01 - out11.cpu())) < 1e-4
+    (out00 - out01).sum().backward()
+    (out10 - out11).sum().backward()
+    assert torch.max(torch.abs(weight0.grad - weight1.grad)) < 1e-4
+    assert torch.max(torch.abs(bias0.grad - bias1.grad)) < 1e-4
+
+
+def test_reference_padding_test_on_gpu():
+    # tests/test_feature_transformer.py:81-110
+    torch.manual_seed(42)
+    weight = torch.rand(10, 64, device=DEV)
+    bias = torch.rand(64, device=DEV)
+    active = (torch.rand(8, 5) * 10).to(dtype=torch.int32, device=DEV)
+    padded = torch.cat([active, torch.full((8, 3), -1, dtype=torch.int32, device=DEV)], dim=1)
+    a = SparseLinearFunction.apply(active, weight, bias)
+    b = SparseLinearFunction.apply(padded, weight, bias)
+    assert torch.max(torch.abs(a - b)) < 1e-4
+    assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("mode", ["atomic", "deterministic"])
+@pytest.mark.parametrize("l1", [32, 2048])
+def test_reference_fused_vs_torch_test(l1, mode):
+    # tests/test_fused_double_ft.py:19-107
+    nnueft.set_backward_mode(mode)
+    torch.manual_seed(0)
+    torch.cuda.manual_seed_all(0)
+    batch_size, max_active, num_inputs, num_psqt = 4, 32, 100, 8
+    output_size = l1 + num_psqt
+    us = torch.randn(batch_size, 1, device=DEV)
+    them = torch.randn(batch_size, 1, device=DEV)
+    white = torch.randint(0, num_inputs, (batch_size, max_active), dtype=torch.int32, device=DEV)
+    white[:, -2:] = -1
+    black = torch.randint(0, num_inputs, (batch_size, max_active), dtype=torch.int32, device=DEV)
+    black[:, -2:] = -1
+    psqt = torch.randint(0, num_psqt, (batch_size,), dtype=torch.int64, device=DEV)
+    weight = torch.randn(num_inputs, output_size, device=DEV, requires_grad=True)
+    bias = torch.randn(output_size, device=DEV, requires_grad=True)
+
+    l0_f, wp_f, bp_f = double_feature_transform(us, them, white, black, psqt, weight, bias, 127.0, l1, "fused")
+    (l0_f.sum() + wp_f.sum() + bp_f.sum()).backward()
+    gw_f, gb_f = weight.grad.clone(), bias.grad.clone()
+    weight.grad.zero_()
+    bias.grad.zero_()
+    l0_t, wp_t, bp_t = double_feature_transform(us, them, white, black, psqt, weight, bias, 127.0, l1, "torch")
+    (l0_t.sum() + wp_t.sum() + bp_t.sum()).backward()
+    torch.testing.assert_close(l0_f, l0_t, atol=1e-5, rtol=1e-4)
+    torch.testing.assert_close(wp_f, wp_t, atol=1e-5, rtol=1e-4)
+    torch.testing.assert_close(bp_f, bp_t, atol=1e-5, rtol=1e-4)
+    torch.testing.assert_close(gw_f, weight.grad, atol=1e-4, rtol=1e-3)
+    torch.testing.assert_close(gb_f, bias.grad, atol=1e-4, rtol=1e-3)
+    # the "sparse" backend (two sparse-linear launches + torch ops) agrees as well
+    weight.grad.zero_()
+    bias.grad.zero_()
+    l0_s, wp_s, bp_s = double_feature_transform(us, them, white, black, psqt, weight, bias, 127.0, l1, "sparse")
+    (l0_s.sum() + wp_s.sum() + bp_s.sum()).backward()
+    torch.testing.assert_close(l0_s, l0_t, atol=1e-5, rtol=1e-4)
+    torch.testing.assert_close(weight.grad, gw_f, atol=1e-4, rtol=1e-3)
+
+
+def test_deterministic_backward_bits_equal_the_reference_cpu_path():
+    """GPU deterministic mode vs torch CPU autograd of the reference composition, equality of bits
+    (32768 slots per list: torch's CPU backward then accumulates in ascending position order)."""
+    nnueft.set_backward_mode("deterministic")
+    c = double_case(31, 1024, 128, hk.NUM_INPUTS, halfka=True, max_act=255 / 256, weight_scale=0.05)
+    cpu = {k: torch.from_numpy(c[k]) for k in ("us", "them", "widx", "bidx", "psqt_idx", "W", "bias")}
+    Wc = cpu["W"].clone().requires_grad_()
+    bc = cpu["bias"].clone().requires_grad_()
+    out_c = ref_torch.double_feature_transform(cpu["us"], cpu["them"], cpu["widx"], cpu["bidx"], cpu["psqt_idx"],
+                                               Wc, bc, c["max_act"], 128)
+    grads = [torch.from_numpy(c[k]) for k in ("g_l0", "g_wp", "g_bp")]
+    torch.autograd.backward(list(out_c), grads)
+    Wg = cpu["W"].to(DEV).requires_grad_()
+    bg = cpu["bias"].to(DEV).requires_grad_()
+    out_g = double_feature_transform(cpu["us"].to(DEV), cpu["them"].to(DEV), cpu["widx"].to(DEV), cpu["bidx"].to(DEV),
+                                     cpu["psqt_idx"].to(DEV), Wg, bg, c["max_act"], 128, "fused")
+    torch.autograd.backward(list(out_g), [g.to(DEV) for g in grads])
+    for a, b in zip(out_g, out_c):
+        assert torch.equal(a.cpu(), b)
+    assert torch.equal(Wg.grad.cpu(), Wc.grad)
+    torch.testing.assert_close(bg.grad.cpu(), bc.grad, atol=1e-4, rtol=1e-4)
+
+
+FULL = [(1024, 8192), (128, 16384), (3072, 16384)]   # BASELINE.json configs 1-3
+
+
+@pytest.mark.parametrize("L1,B", FULL)
+def test_baseline_configs_full_size_against_oracle(oracle_cpu, L1, B):
+    """fwd bit-exact, deterministic backward bit-exact, atomic backward 1e-4 relative, at full size."""
+    n_psqt, R = 8, hk.NUM_INPUTS
+    us, them, white, black, pc = hk.synthetic_batch(B, 1234 + L1)
+    psqt_idx = (pc - 1) // 4
+    g = torch.Generator().manual_seed(L1)
+    Wn = (torch.randn(R, L1 + n_psqt, generator=g) * 0.01).numpy()
+    bn = np.zeros(L1 + n_psqt, np.float32)
+    grads = [torch.randn(B, L1, generator=g).numpy(), torch.randn(B, 1, generator=g).numpy(),
+             torch.randn(B, 1, generator=g).numpy()]
+    max_act = 255.0 / 256.0
+    r_l0, r_wp, r_bp, r_saved = oracle_cpu.double_fwd(us, them, white, black, psqt_idx, Wn, bn, max_act, L1)
+    r_gW, r_gb = oracle_cpu.double_bwd(us, them, white, black, psqt_idx, max_act, grads[0], grads[1], grads[2],
+                                       r_saved, R, n_psqt)
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    args = [t(us), t(them), t(white), t(black), t(psqt_idx)]
+    det = None
+    for mode in ("deterministic", "atomic", "deterministic"):
+        nnueft.set_backward_mode(mode)
+        W = t(Wn).requires_grad_()
+        bias = t(bn).requires_grad_()
+        out = double_feature_transform(*args, W, bias, max_act, L1, "fused")
+        torch.autograd.backward(list(out), [t(x) for x in grads])
+        assert np.array_equal(out[0].detach().cpu().numpy(), r_l0)
+        assert np.array_equal(out[1].detach().cpu().numpy(), r_wp)
+        assert np.array_equal(out[2].detach().cpu().numpy(), r_bp)
+        gW, gb = W.grad.cpu().numpy(), bias.grad.cpu().numpy()
+        if mode == "deterministic":
+            assert np.array_equal(gW, r_gW)
+            assert np.array_equal(gb, r_gb)
+            if det is not None:          # run to run
+                assert np.array_equal(gW, det[0]) and np.array_equal(gb, det[1])
+            det = (gW, gb)
+        else:
+            assert np.abs(gW - r_gW).max() <= 1e-4 * np.abs(r_gW).max()
+            assert np.abs(gb - r_gb).max() <= 1e-4 * np.abs(r_gb).max()
+        del W, bias, out
+
+
+def test_int16_full_size_against_oracle(oracle_cpu):
+    """BASELINE.json config 5: L1=3072, B=65536, exported numbering (22528 rows), quantized weights."""
+    from nnueft import quantized
+
+    L1, B, R = 3072, 65536, hk.NUM_INPUTS_EXPORT
+    us, them, white, black, pc = hk.synthetic_batch(B, 1239, fold_kings=True)
+    g = torch.Generator().manual_seed(5)
+    W = torch.randn(R, L1 + 8, generator=g) * 0.02
+    W[:, L1:] = torch.randn(R, 8, generator=g) * 0.5
+    bias = torch.randn(L1 + 8, generator=g) * 0.1
+    w16, b16, p32 = quantized.quantize_feature_transformer(W, bias, L1)
+    stm = (1 - us[:, 0]).astype(np.uint8)
+    psqt_idx = (pc - 1) // 4
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    out, ps = quantized.ft_int16_forward(t(white), t(black), t(stm), w16.to(DEV), b16.to(DEV), p32.to(DEV), t(psqt_idx))
+    r_out, r_ps = oracle_cpu.ft_int16_fwd(white, black, stm, w16.numpy(), b16.numpy(), p32.numpy(), psqt_idx)
+    assert np.array_equal(out.cpu().numpy(), r_out)
+    assert np.array_equal(ps.cpu().numpy(), r_ps)
+    assert 0 < r_out.max() <= 127 and (r_out > 0).mean() > 0.05
+
+
+@pytest.mark.parametrize("mode", ["atomic", "deterministic"])
+def test_every_slot_names_the_same_row(oracle_cpu, mode):
+    """Worst case for both backward modes: one table row receives all B*K contributions."""
+    nnueft.set_backward_mode(mode)
+    B, K, R, oc = 2048, 32, 3, 136
+    idx = np.full((B, K), 1, np.int32)
+    c = sparse_case(5, B, oc, R, K)
+    W = torch.from_numpy(c["W"]).to(DEV).requires_grad_()
+    bias = torch.from_numpy(c["bias"]).to(DEV).requires_grad_()
+    out = SparseLinearFunction.apply(torch.from_numpy(idx).to(DEV), W, bias)
+    out.backward(torch.from_numpy(c["g"]).to(DEV))
+    assert np.array_equal(out.detach().cpu().numpy(), oracle_cpu.sparse_fwd(idx, c["W"], c["bias"]))
+    rW, rb = oracle_cpu.sparse_bwd(idx, c["g"], R)
+    if mode == "deterministic":
+        assert np.array_equal(W.grad.cpu().numpy(), rW) and np.array_equal(bias.grad.cpu().numpy(), rb)
+    else:
+        assert np.abs(W.grad.cpu().numpy() - rW).max() <= 1e-4 * np.abs(rW).max()
+        assert np.abs(bias.grad.cpu().numpy() - rb).max() <= 1e-4 * np.abs(rb).max()
+    assert not W.grad[0].any() and not W.grad[2].any()
+
+
+@pytest.mark.parametrize("mode", ["atomic", "deterministic"])
+def test_empty_batch_and_all_padding(mode):
+    nnueft.set_backward_mode(mode)
+    W = torch.randn(20, 40, device=DEV, requires_grad=True)
+    bias = torch.randn(40, device=DEV, requires_grad=True)
+    empty = torch.empty(0, 32, dtype=torch.int32, device=DEV)
+    out = SparseLinearFunction.apply(empty, W, bias)
+    assert out.shape == (0, 40)
+    out.sum().backward()
+    assert not W.grad.any() and not bias.grad.any()
+    W.grad = None
+    bias.grad = None
+    pad = torch.full((5, 32), -1, dtype=torch.int32, device=DEV)
+    out = SparseLinearFunction.apply(pad, W, bias)
+    assert torch.equal(out, bias.detach().expand(5, 40))
+    out.backward(torch.ones_like(out))
+    assert not W.grad.any()
+    assert torch.equal(bias.grad, torch.full((40,), 5.0, device=DEV))
+
+
+def test_non_default_stream(oracle_cpu):
+    c = double_case(41, 300, 256, 500, binary_side=True)
+    t = {k: torch.from_numpy(c[k]).to(DEV) for k in ("us", "them", "widx", "bidx", "psqt_idx", "W", "bias")}
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    nnueft.set_backward_mode("deterministic")
+    with torch.cuda.stream(s):
+        W = t["W"].clone().requires_grad_()
+        bias = t["bias"].clone().requires_grad_()
+        out = double_feature_transform(t["us"], t["them"], t["widx"], t["bidx"], t["psqt_idx"], W, bias,
+                                       c["max_act"], 256, "fused")
+        torch.autograd.backward(list(out), [torch.from_numpy(c[k]).to(DEV) for k in ("g_l0", "g_wp", "g_bp")])
+    s.synchronize()
+    r = oracle_cpu.double_fwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["W"], c["bias"], c["max_act"], 256)
+    assert np.array_equal(out[0].detach().cpu().numpy(), r[0])
+    rW, rb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["max_act"], c["g_l0"],
+                                   c["g_wp"], c["g_bp"], r[3], 500, 8)
+    assert np.array_equal(W.grad.cpu().numpy(), rW) and np.array_equal(bias.grad.cpu().numpy(), rb)
+
+
+def test_abi_rejects_bad_arguments():
+    lib = _native.load()
+    x = torch.zeros(64, device=DEV)
+    p = x.data_ptr()
+    st = torch.cuda.current_stream().cuda_stream
+    assert lib.nnueft_sparse_fwd(p, p, p, p, 4, 0, 10, 8, st) == -1                 # K = 0
+    assert lib.nnueft_sparse_fwd(0, p, p, p, 4, 8, 10, 8, st) == -1                 # null pointer
+    assert lib.nnueft_double_fwd(p, p, p, p, p, p, p, 1.0, p, p, p, p, 4, 8, 10, 7, 1, st) == -1    # odd L1
+    assert lib.nnueft_sparse_bwd_det(p, p, p, p, 4, 8, 10, 8, p, 16, st) == -2      # workspace too small
+    assert lib.nnueft_sparse_bwd_det(p, p, p, p, 4, 8, 10, 8, 0, 1 << 20, st) == -2  # workspace missing
+    assert lib.nnueft_sparse_bwd_det(p, p, p, p, 4, 8, 10, 8, p + 4, 1 << 20, st) == -2  # misaligned
+    assert lib.nnueft_ft_int16_fwd(p, p, p, p, p, p, p, p, p, 4, 8, 10, 8, 8, 70000, 9, st) == -1   # clip_max
+    with pytest.raises(RuntimeError, match="invalid argument"):
+        _native.check(-1, "x")
+    torch.cuda.synchronize()
+
+
+def test_python_preconditions_assert_like_the_reference():
+    W = torch.randn(20, 40, device=DEV)
+    bias = torch.randn(40, device=DEV)
+    idx64 = torch.zeros(4, 8, dtype=torch.int64, device=DEV)
+    with pytest.raises(AssertionError):
+        SparseLinearFunction.apply(idx64, W, bias)                       # sparse_linear_functions.py:59
+    idx = torch.zeros(4, 8, dtype=torch.int32, device=DEV)
+    with pytest.raises(AssertionError):
+        SparseLinearFunction.apply(idx, W.t().contiguous().t(), bias)    # not contiguous, :75
+    us = torch.ones(4, 1, device=DEV)
+    psqt = torch.zeros(4, dtype=torch.int64, device=DEV)
+    with pytest.raises(AssertionError):
+        double_feature_transform(us, us, idx, idx, psqt.int(), W, bias, 1.0, 32, "fused")   # fused_ft_functions.py:33
+    with pytest.raises(AssertionError):
+        double_feature_transform(us, us, idx, idx, psqt, W, bias, 1.0, 31, "fused")         # odd l1_size, :23
