@@ -192,7 +192,9 @@ def main():
     l0 = torch.empty(B, L1, device=dev)
     wp = torch.empty(B, 1, device=dev)
     bp = torch.empty(B, 1, device=dev)
-    saved = torch.empty(B, 4, L1 // 2, device=dev)
+    saved = torch.empty(2, B, L1, device=dev)
+    fwd_ws_bytes = lib.nnueft_fwd_workspace_bytes(B, K_SLOTS, R_ROWS, L1, N_PSQT)
+    fwd_ws = torch.empty(fwd_ws_bytes, dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
     Wd, bd = W.detach(), bias.detach()
 
@@ -200,7 +202,7 @@ def main():
         rc = lib.nnueft_double_fwd(t["us"].data_ptr(), t["them"].data_ptr(), t["white"].data_ptr(),
                                    t["black"].data_ptr(), t["psqt_idx"].data_ptr(), Wd.data_ptr(), bd.data_ptr(),
                                    max_act, l0.data_ptr(), wp.data_ptr(), bp.data_ptr(), saved.data_ptr(),
-                                   B, K_, R_ROWS, L1, N_PSQT, stream)
+                                   B, K_, R_ROWS, L1, N_PSQT, fwd_ws.data_ptr(), fwd_ws_bytes, stream)
         assert rc == 0
 
     _, fwd_ms = time_steps(fwd_only, max(args.steps, 10), args.warmup)
@@ -215,7 +217,8 @@ def main():
         gW = torch.empty(R_ROWS, oc, device=dev)
         gb = torch.empty(oc, device=dev)
         head = (t["us"].data_ptr(), t["them"].data_ptr(), t["white"].data_ptr(), t["black"].data_ptr(),
-                t["psqt_idx"].data_ptr(), max_act, g_l0.data_ptr(), g_wp.data_ptr(), g_bp.data_ptr(), saved.data_ptr())
+                t["psqt_idx"].data_ptr(), bd.data_ptr(), max_act, g_l0.data_ptr(), g_wp.data_ptr(), g_bp.data_ptr(),
+                saved.data_ptr())
 
         def bwd_det():
             rc = lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT,

@@ -85,7 +85,13 @@ int nnueft_sparse_bwd_det(const int32_t* idx, const float* gout, float* gW, floa
                           void* workspace, size_t workspace_bytes, void* stream);
 
 /*
- * Both perspectives in one pass, then the side-to-move mix, clamp and pairwise product:
+ * Bytes of scratch nnueft_double_fwd can use (256-B aligned device memory, contents irrelevant on
+ * entry and on exit).  Returns 0 for invalid dimensions.
+ */
+size_t nnueft_fwd_workspace_bytes(int B, int K, int R, int L1, int n_psqt);
+
+/*
+ * Both perspectives, then the side-to-move mix, clamp and pairwise product:
  *   w = sum W[widx] + bias, b = sum W[bidx] + bias              (first L1 columns)
  *   x_w = us*w + them*b,  x_b = us*b + them*w
  *   l0[:, :h] = clamp(x_w[:h]) * clamp(x_w[h:]),  l0[:, h:] = clamp(x_b[:h]) * clamp(x_b[h:]),  h = L1/2
@@ -93,23 +99,30 @@ int nnueft_sparse_bwd_det(const int32_t* idx, const float* gout, float* gW, floa
  * Replaces `fused_double_ft_forward`, fused_ft_functions.py:51-75 (kernel: fused_ft_kernel.py:27-117);
  * same result as the torch composition double_ft_functions.py:62-80.
  * us, them f32[B]; widx, bidx int32[B,K]; psqt_idx int64[B]; W f32[R,L1+n_psqt]; bias f32[L1+n_psqt];
- * l0 f32[B,L1]; wpsqt, bpsqt f32[B]; saved f32[B,4,L1/2].
- * `saved` receives (x_w[:h], x_w[h:], x_b[:h], x_b[h:]) BEFORE the clamp (the reference stores the
- * clamped values, fused_ft_kernel.py:95-99); the backward needs them to reproduce torch's clamp
- * gradient at the boundaries.  L1 must be even.
+ * l0 f32[B,L1]; wpsqt, bpsqt f32[B]; saved f32[2,B,L1].
+ * `saved` receives the two perspectives' row sums before the bias (saved[0] white, saved[1] black);
+ * the backward recomputes the mixed values from them with the forward's own operations.  (The
+ * reference stores the clamped mixed values instead, fused_ft_kernel.py:95-99, and thereby loses
+ * torch's clamp gradient at exactly 0 and exactly max.)  L1 must be even.
+ * workspace: NULL, or nnueft_fwd_workspace_bytes() bytes.  With a workspace (and 16-byte aligned rows:
+ * L1 % 8 == 0, (L1+n_psqt) % 4 == 0) the gather is blocked for the per-XCD L2 caches: positions are
+ * grouped by the 768-row table block their lists name and each XCD works through its share one
+ * column slice at a time.  Results are bit-identical with and without the workspace.
  */
 int nnueft_double_fwd(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                       const int64_t* psqt_idx, const float* W, const float* bias, float max_act,
                       float* l0, float* wpsqt, float* bpsqt, float* saved,
-                      int B, int K, int R, int L1, int n_psqt, void* stream);
+                      int B, int K, int R, int L1, int n_psqt,
+                      void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Gradient of nnueft_double_fwd with respect to W and bias, floating-point atomics.
- * gW f32[R,L1+n_psqt] and gbias f32[L1+n_psqt] must be zero on entry.
+ * `saved` is the forward's; `bias` the forward's bias.  gW f32[R,L1+n_psqt] and gbias f32[L1+n_psqt]
+ * must be zero on entry.
  * Replaces `fused_double_ft_backward`, fused_ft_functions.py:94-120 (kernel: fused_ft_kernel.py:147-272).
  */
 int nnueft_double_bwd_atomic(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
-                             const int64_t* psqt_idx, float max_act,
+                             const int64_t* psqt_idx, const float* bias, float max_act,
                              const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt,
                              const float* saved, float* gW, float* gbias,
                              int B, int K, int R, int L1, int n_psqt, void* stream);
@@ -120,7 +133,7 @@ int nnueft_double_bwd_atomic(const float* us, const float* them, const int32_t* 
  * reference's CPU composition (double_ft_functions.py:62-80).
  */
 int nnueft_double_bwd_det(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
-                          const int64_t* psqt_idx, float max_act,
+                          const int64_t* psqt_idx, const float* bias, float max_act,
                           const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt,
                           const float* saved, float* gW, float* gbias,
                           int B, int K, int R, int L1, int n_psqt,

@@ -59,8 +59,8 @@ __global__ __launch_bounds__(64) void k_sparse_bwd_atomic(const int32_t* __restr
 template <int NC>
 __global__ __launch_bounds__(64) void k_double_bwd_atomic(
     const float* __restrict__ us, const float* __restrict__ them, const int32_t* __restrict__ widx,
-    const int32_t* __restrict__ bidx, const int64_t* __restrict__ psqt_idx, float max_act,
-    const float* __restrict__ grad_l0, const float* __restrict__ grad_wpsqt, const float* __restrict__ grad_bpsqt,
+    const int32_t* __restrict__ bidx, const int64_t* __restrict__ psqt_idx, const float* __restrict__ bias,
+    float max_act, const float* __restrict__ grad_l0, const float* __restrict__ grad_wpsqt, const float* __restrict__ grad_bpsqt,
     const float* __restrict__ saved, float* __restrict__ gW, float* __restrict__ gbias, int B, int K, int R,
     int L1, int n_psqt, int nslices) {
     const int lane = threadIdx.x;
@@ -81,7 +81,8 @@ __global__ __launch_bounds__(64) void k_double_bwd_atomic(
     const int b1 = min((tile + 1) * kTile, B);
     for (int b = tile * kTile; b < b1; ++b) {
         const float u = us[b], t = them[b];
-        const float* sv = saved + (size_t)b * 2 * L1;
+        const float* sw = saved + (size_t)b * L1;
+        const float* sb = saved + ((size_t)B + b) * L1;
         const float* gl = grad_l0 + (size_t)b * L1;
         float g[2][2][NC];  // [perspective][half][m]
 #pragma unroll
@@ -89,18 +90,9 @@ __global__ __launch_bounds__(64) void k_double_bwd_atomic(
             float gw0 = 0.0f, gw1 = 0.0f, gb0 = 0.0f, gb1 = 0.0f;
             if (act[m]) {
                 const int c = col[m];
-                const float xw0 = sv[c], xw1 = sv[h + c], xb0 = sv[2 * h + c], xb1 = sv[3 * h + c];
-                const float g0 = gl[c], g1 = gl[h + c];
-                const float cw0 = clamp_act(xw0, max_act), cw1 = clamp_act(xw1, max_act);
-                const float cb0 = clamp_act(xb0, max_act), cb1 = clamp_act(xb1, max_act);
-                const float dw0 = (xw0 >= 0.0f && xw0 <= max_act) ? g0 * cw1 : 0.0f;
-                const float dw1 = (xw1 >= 0.0f && xw1 <= max_act) ? g0 * cw0 : 0.0f;
-                const float db0 = (xb0 >= 0.0f && xb0 <= max_act) ? g1 * cb1 : 0.0f;
-                const float db1 = (xb1 >= 0.0f && xb1 <= max_act) ? g1 * cb0 : 0.0f;
-                gw0 = u * dw0 + t * db0;
-                gw1 = u * dw1 + t * db1;
-                gb0 = t * dw0 + u * db0;
-                gb1 = t * dw1 + u * db1;
+                float xw0, xw1, xb0, xb1;
+                mix4(u, t, sw[c], sw[h + c], sb[c], sb[h + c], bias[c], bias[h + c], xw0, xw1, xb0, xb1);
+                grad4(u, t, xw0, xw1, xb0, xb1, gl[c], gl[h + c], max_act, gw0, gw1, gb0, gb1);
             }
             g[0][0][m] = gw0;
             g[0][1][m] = gw1;
@@ -165,14 +157,14 @@ extern "C" int nnueft_sparse_bwd_atomic(const int32_t* idx, const float* gout, f
 }
 
 extern "C" int nnueft_double_bwd_atomic(const float* us, const float* them, const int32_t* widx,
-                                        const int32_t* bidx, const int64_t* psqt_idx, float max_act,
-                                        const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt,
+                                        const int32_t* bidx, const int64_t* psqt_idx, const float* bias,
+                                        float max_act, const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt,
                                         const float* saved, float* gW, float* gbias, int B, int K, int R, int L1,
                                         int n_psqt, void* stream) {
     if (B < 0 || K <= 0 || R <= 0 || L1 <= 0 || (L1 & 1) || n_psqt < 0) return NNUEFT_E_ARG;
     if (B == 0) return 0;
-    if (!us || !them || !widx || !bidx || !psqt_idx || !grad_l0 || !grad_wpsqt || !grad_bpsqt || !saved || !gW ||
-        !gbias)
+    if (!us || !them || !widx || !bidx || !psqt_idx || !bias || !grad_l0 || !grad_wpsqt || !grad_bpsqt || !saved ||
+        !gW || !gbias)
         return NNUEFT_E_ARG;
     hipStream_t st = (hipStream_t)stream;
     const int ntiles = (B + kTile - 1) / kTile;
@@ -180,12 +172,12 @@ extern "C" int nnueft_double_bwd_atomic(const float* us, const float* them, cons
     if (h > 128) {
         const int nslices = (h + 255) / 256;
         hipLaunchKernelGGL(k_double_bwd_atomic<4>, dim3(ntiles * nslices), dim3(64), 0, st, us, them, widx, bidx,
-                           psqt_idx, max_act, grad_l0, grad_wpsqt, grad_bpsqt, saved, gW, gbias, B, K, R, L1, n_psqt,
+                           psqt_idx, bias, max_act, grad_l0, grad_wpsqt, grad_bpsqt, saved, gW, gbias, B, K, R, L1, n_psqt,
                            nslices);
     } else {
         const int nslices = (h + 63) / 64;
         hipLaunchKernelGGL(k_double_bwd_atomic<1>, dim3(ntiles * nslices), dim3(64), 0, st, us, them, widx, bidx,
-                           psqt_idx, max_act, grad_l0, grad_wpsqt, grad_bpsqt, saved, gW, gbias, B, K, R, L1, n_psqt,
+                           psqt_idx, bias, max_act, grad_l0, grad_wpsqt, grad_bpsqt, saved, gW, gbias, B, K, R, L1, n_psqt,
                            nslices);
     }
     NNUEFT_LAUNCH_CHECK();

@@ -6,11 +6,14 @@
 //   k_tile_colsum   sparse only: bias partial sums of gout
 //   k_chunk_hist    per chunk of positions, how often each table row is named     cnt[chunk,row]
 //   k_col_scan      exclusive scan of cnt over the chunks; per-row totals and white-perspective share
-//   k_row_scan      exclusive scan of the totals -> segment offsets; rows ordered longest first
+//   k_row_scan      exclusive scan of the totals -> segment offsets; work split for the reduction
 //   k_fill          every slot writes its position id to its place: segment offset + chunk offset
 //                   + rank inside the chunk, ranks taken position by position so the list of a
 //                   row ends up in ascending (perspective, position) order
-//   k_seg_reduce    one wave per (row, column slice): white chain, black chain, sum, store
+//   k_seg_reduce    persistent waves, one task = (table row, column slice): white chain, black
+//                   chain, sum, store.  Rows are dealt to the 8 XCDs in contiguous ranges of equal
+//                   work and walked one column slice at a time, so the upstream rows a XCD gathers
+//                   (those of the positions of one king bucket, one slice wide) stay in its L2
 //   k_bias_final    chain over the tile partial sums
 #include "gather.h"
 
@@ -18,9 +21,18 @@ namespace {
 
 constexpr int kChunk = 128;        // positions per sort chunk
 constexpr int kRowsUnroll = 8;     // rows in flight per lane group in the segmented reduction
+constexpr int kXcd = 8;            // XCDs of the device; workgroup id % kXcd is the XCD a workgroup lands on
+constexpr int kWavesPerXcd = 512;  // persistent waves per XCD in the segmented reduction
+constexpr int kLongRow = 256;      // table rows named by at least this many slots are reduced first
+
+// Work split of the segmented reduction, written by k_row_scan (uint32 words).
+constexpr int kSchedCtr = 0;       // kXcd task counters, 32 words (128 bytes) apart
+constexpr int kSchedNLong = kXcd * 32;
+constexpr int kSchedRowLo = kSchedNLong + 1;   // kXcd + 1 range bounds
+constexpr int kSchedWords = kSchedRowLo + kXcd + 1;
 
 struct DetLayout {
-    size_t G, partial, cnt, wcount, seg_off, row_order, list, end;
+    size_t G, partial, cnt, wcount, seg_off, long_rows, sched, list, end;
     int cpp;     // chunks per perspective
     int nchunks; // n_persp * cpp
     int ntiles;  // bias tiles
@@ -44,8 +56,10 @@ bool det_layout(int B, int K, int R, int out_cols, int n_persp, DetLayout* L) {
     off += up256((size_t)R * sizeof(uint32_t));
     L->seg_off = off;
     off += up256(((size_t)R + 1) * sizeof(uint32_t));
-    L->row_order = off;
+    L->long_rows = off;
     off += up256((size_t)R * sizeof(uint32_t));
+    L->sched = off;
+    off += up256((size_t)kSchedWords * sizeof(uint32_t));
     L->list = off;
     off += up256((size_t)n_persp * B * K * sizeof(uint32_t));
     L->end = off;
@@ -58,7 +72,8 @@ bool det_layout(int B, int K, int R, int out_cols, int n_persp, DetLayout* L) {
 // walks the tile's positions in order, which is the order of the bias chain.
 template <int VW>
 __global__ __launch_bounds__(64) void k_bwd_rows(const float* __restrict__ us, const float* __restrict__ them,
-                                                 const int64_t* __restrict__ psqt_idx, float max_act,
+                                                 const int64_t* __restrict__ psqt_idx,
+                                                 const float* __restrict__ bias, float max_act,
                                                  const float* __restrict__ grad_l0,
                                                  const float* __restrict__ grad_wpsqt,
                                                  const float* __restrict__ grad_bpsqt,
@@ -79,26 +94,21 @@ __global__ __launch_bounds__(64) void k_bwd_rows(const float* __restrict__ us, c
     if (q < hv) {
         const int c = q * VW;
         vecf<VW> part0 = vzero<VW>(), part1 = vzero<VW>();
+        const vecf<VW> bias0 = ldv<VW>(bias + c), bias1 = ldv<VW>(bias + h + c);
         for (int b = b0; b < b1; ++b) {
             const float u = us[b], t = them[b];
-            const float* sv = saved + (size_t)b * 2 * L1;
-            const vecf<VW> xw0 = ldv<VW>(sv + c), xw1 = ldv<VW>(sv + h + c);
-            const vecf<VW> xb0 = ldv<VW>(sv + 2 * h + c), xb1 = ldv<VW>(sv + 3 * h + c);
+            const float* sw = saved + (size_t)b * L1;
+            const float* sb = saved + ((size_t)B + b) * L1;
+            const vecf<VW> sw0 = ldv<VW>(sw + c), sw1 = ldv<VW>(sw + h + c);
+            const vecf<VW> sb0 = ldv<VW>(sb + c), sb1 = ldv<VW>(sb + h + c);
             const vecf<VW> g0 = ldv<VW>(grad_l0 + (size_t)b * L1 + c);
             const vecf<VW> g1 = ldv<VW>(grad_l0 + (size_t)b * L1 + h + c);
             vecf<VW> gw0, gw1, gb0, gb1;
 #pragma unroll
             for (int i = 0; i < VW; ++i) {
-                const float cw0 = clamp_act(xw0.v[i], max_act), cw1 = clamp_act(xw1.v[i], max_act);
-                const float cb0 = clamp_act(xb0.v[i], max_act), cb1 = clamp_act(xb1.v[i], max_act);
-                const float dw0 = (xw0.v[i] >= 0.0f && xw0.v[i] <= max_act) ? g0.v[i] * cw1 : 0.0f;
-                const float dw1 = (xw1.v[i] >= 0.0f && xw1.v[i] <= max_act) ? g0.v[i] * cw0 : 0.0f;
-                const float db0 = (xb0.v[i] >= 0.0f && xb0.v[i] <= max_act) ? g1.v[i] * cb1 : 0.0f;
-                const float db1 = (xb1.v[i] >= 0.0f && xb1.v[i] <= max_act) ? g1.v[i] * cb0 : 0.0f;
-                gw0.v[i] = u * dw0 + t * db0;
-                gw1.v[i] = u * dw1 + t * db1;
-                gb0.v[i] = t * dw0 + u * db0;
-                gb1.v[i] = t * dw1 + u * db1;
+                float xw0, xw1, xb0, xb1;
+                mix4(u, t, sw0.v[i], sw1.v[i], sb0.v[i], sb1.v[i], bias0.v[i], bias1.v[i], xw0, xw1, xb0, xb1);
+                grad4(u, t, xw0, xw1, xb0, xb1, g0.v[i], g1.v[i], max_act, gw0.v[i], gw1.v[i], gb0.v[i], gb1.v[i]);
                 part0.v[i] = part0.v[i] + (gw0.v[i] + gb0.v[i]);
                 part1.v[i] = part1.v[i] + (gw1.v[i] + gb1.v[i]);
             }
@@ -225,44 +235,25 @@ __global__ __launch_bounds__(64) void k_col_scan(uint32_t* __restrict__ cnt, uin
     seg_off[r] = run;
 }
 
-// Single workgroup: seg_off (holding per-row totals) -> exclusive offsets, seg_off[R] = grand total;
-// row_order = table rows by descending list length (length clipped to kLenBins-1 for the ordering),
-// so the longest chains start first.
+// Single workgroup: seg_off (holding per-row totals) -> exclusive offsets, seg_off[R] = grand total.
+// Also the work split of the segmented reduction: the rows named by >= kLongRow slots (their chains
+// are long and start first), and kXcd contiguous row ranges of equal weight (slots + 1 per row).
 constexpr int kScanThreads = 1024;
-constexpr int kLenBins = 1024;
 constexpr int kScanPer = 32;   // rows a thread keeps in registers per pass
 __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict__ seg_off,
-                                                           uint32_t* __restrict__ row_order, int R) {
-    __shared__ uint32_t sums[kScanThreads];
-    __shared__ uint32_t bins[kLenBins];
-    __shared__ uint32_t carry_s;
+                                                           uint32_t* __restrict__ long_rows,
+                                                           uint32_t* __restrict__ sched, int R) {
+    __shared__ uint32_t wave_tot[kScanThreads / 64];
+    __shared__ uint32_t carry_s, n_long_s;
+    __shared__ uint32_t lo_s[kXcd + 1];
     const int tid = threadIdx.x;
-    if (tid < kLenBins) bins[tid] = 0;
-    if (tid == 0) carry_s = 0;
-    __syncthreads();
-    // pass A: length histogram (for the longest-first order)
-    for (int rb = tid; rb < R; rb += kScanThreads * 8) {
-        uint32_t len[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) len[u] = (rb + u * kScanThreads < R) ? seg_off[rb + u * kScanThreads] : 0;
-#pragma unroll
-        for (int u = 0; u < 8; ++u)
-            if (rb + u * kScanThreads < R) atomicAdd(&bins[min(len[u], (uint32_t)(kLenBins - 1))], 1u);
+    if (tid == 0) {
+        carry_s = 0;
+        n_long_s = 0;
     }
+    if (tid <= kXcd) lo_s[tid] = (uint32_t)R;
+    if (tid < kXcd) sched[kSchedCtr + tid * 32] = 0;
     __syncthreads();
-    // bins -> first slot of each length class, longest class first
-    if (tid < kLenBins) sums[tid] = bins[kLenBins - 1 - tid];
-    __syncthreads();
-    for (int d = 1; d < kLenBins; d <<= 1) {
-        uint32_t add = 0;
-        if (tid < kLenBins && tid >= d) add = sums[tid - d];
-        __syncthreads();
-        if (tid < kLenBins) sums[tid] += add;
-        __syncthreads();
-    }
-    if (tid < kLenBins) bins[kLenBins - 1 - tid] = sums[tid] - bins[kLenBins - 1 - tid];
-    __syncthreads();
-    // pass B: exclusive scan of the lengths, kScanThreads * kScanPer rows at a time
     for (int base = 0; base < R; base += kScanThreads * kScanPer) {
         const int r0 = base + tid * kScanPer;
         uint32_t len[kScanPer];
@@ -272,30 +263,57 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
             len[u] = (r0 + u < R) ? seg_off[r0 + u] : 0;
             local += len[u];
         }
-        sums[tid] = local;
-        __syncthreads();
-        for (int d = 1; d < kScanThreads; d <<= 1) {
-            const uint32_t add = tid >= d ? sums[tid - d] : 0;
-            __syncthreads();
-            sums[tid] += add;
-            __syncthreads();
+        uint32_t incl = local;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const uint32_t v = __shfl_up(incl, off);
+            if ((tid & 63) >= off) incl += v;
         }
-        uint32_t run = carry_s + sums[tid] - local;
-        const uint32_t block_total = sums[kScanThreads - 1];
+        if ((tid & 63) == 63) wave_tot[tid >> 6] = incl;
+        __syncthreads();
+        uint32_t before = carry_s;
+        for (int w = 0; w < (tid >> 6); ++w) before += wave_tot[w];
+        uint32_t run = before + incl - local;
 #pragma unroll
         for (int u = 0; u < kScanPer; ++u) {
             if (r0 + u < R) {
-                const uint32_t slot = atomicAdd(&bins[min(len[u], (uint32_t)(kLenBins - 1))], 1u);
-                row_order[slot] = (uint32_t)(r0 + u);
+                if (len[u] >= (uint32_t)kLongRow) long_rows[atomicAdd(&n_long_s, 1u)] = (uint32_t)(r0 + u);
                 seg_off[r0 + u] = run;
                 run += len[u];
             }
         }
         __syncthreads();
-        if (tid == 0) carry_s += block_total;
+        if (tid == kScanThreads - 1) carry_s = run;
         __syncthreads();
     }
-    if (tid == 0) seg_off[R] = carry_s;
+    const uint32_t total = carry_s;
+    if (tid == 0) {
+        seg_off[R] = total;
+        sched[kSchedNLong] = n_long_s;
+    }
+    __syncthreads();   // seg_off now holds exclusive offsets (written by this workgroup)
+    // XCD of a row = floor(kXcd * (slots before it + rows before it) / (all slots + all rows))
+    const unsigned long long denom = (unsigned long long)total + (unsigned long long)R;
+    for (int rb = tid; rb < R; rb += kScanThreads * 8) {
+        uint32_t off[8], prev[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int r = rb + u * kScanThreads;
+            off[u] = r < R ? seg_off[r] : 0;
+            prev[u] = (r < R && r > 0) ? seg_off[r - 1] : 0;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int r = rb + u * kScanThreads;
+            if (r < R) {
+                const int x = (int)(((unsigned long long)off[u] + r) * kXcd / denom);
+                const int xp = r > 0 ? (int)(((unsigned long long)prev[u] + (r - 1)) * kXcd / denom) : -1;
+                for (int k = xp + 1; k <= x; ++k) lo_s[k] = (uint32_t)r;
+            }
+        }
+    }
+    __syncthreads();
+    if (tid <= kXcd) sched[kSchedRowLo + tid] = lo_s[tid];
 }
 
 // Every slot of the chunk writes its position id.  Ranks inside the chunk are handed out position
@@ -351,22 +369,13 @@ __global__ __launch_bounds__(256) void k_fill(const int32_t* __restrict__ widx, 
 }
 
 // ---------------------------------------------------------------------------------------------
-// Segmented reduction.  One wave per (table row, column slice); rows are taken longest first.
-// list[seg_off[r] .. +wcount[r]) are the white-perspective rows of G, the rest of the segment the
-// black ones.  gW[r] = white chain (+ black chain when two perspectives).
+// Segmented reduction.  list[seg_off[r] .. +wcount[r]) are the white-perspective rows of G naming
+// table row r, the rest of the segment the black ones.  gW[r] = white chain (+ black chain).
 template <int VW, int NQ>
-__global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, const uint32_t* __restrict__ list,
-                                                   const uint32_t* __restrict__ seg_off,
-                                                   const uint32_t* __restrict__ wcount,
-                                                   const uint32_t* __restrict__ row_order,
-                                                   float* __restrict__ gW, int out_cols, int nslices,
-                                                   int slice_v, int two_persp) {
-    const int lane = threadIdx.x;
-    const int ro = blockIdx.x / nslices;
-    const int s = blockIdx.x - ro * nslices;
-    const int r = (int)row_order[ro];
+__device__ __forceinline__ void seg_reduce_task(const float* __restrict__ G, const uint32_t* __restrict__ list,
+                                                uint32_t beg, uint32_t mid, uint32_t end, float* __restrict__ dst,
+                                                int s, int lane, int out_cols, int slice_v, int two_persp) {
     const int nv = out_cols / VW;
-
     int col[NQ];
     bool act[NQ];
 #pragma unroll
@@ -376,9 +385,6 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
         act[m] = w < slice_v && q < nv;
         col[m] = act[m] ? q * VW : 0;
     }
-    const uint32_t beg = seg_off[r], end = seg_off[r + 1];
-    const uint32_t mid = beg + wcount[r];
-
     vecf<VW> acc[2][NQ];
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
@@ -392,12 +398,59 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
             chain_rows<VW, NQ, kRowsUnroll>(acc[p], G, (size_t)out_cols, col, my, mask);
         }
     }
-    float* dst = gW + (size_t)r * out_cols;
 #pragma unroll
     for (int m = 0; m < NQ; ++m) {
         if (!act[m]) continue;
         if (two_persp) vadd<VW>(acc[0][m], acc[1][m]);
         stv<VW>(dst + col[m], acc[0][m]);
+    }
+}
+
+__device__ __forceinline__ uint32_t next_task(uint32_t* ctr, int lane) {
+    uint32_t t = 0;
+    if (lane == 0) t = atomicAdd(ctr, 1u);
+    return (uint32_t)__builtin_amdgcn_readfirstlane((int)t);
+}
+
+// Persistent waves.  Each XCD has its own task counter; a wave takes the next task of its XCD until
+// none is left (the counter only grows, so every wave leaves the loop).  Task order per XCD: the
+// long rows dealt to it (all slices of a row together), then its row range, slice by slice.
+template <int VW, int NQ>
+__global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, const uint32_t* __restrict__ list,
+                                                   const uint32_t* __restrict__ seg_off,
+                                                   const uint32_t* __restrict__ wcount,
+                                                   const uint32_t* __restrict__ long_rows,
+                                                   uint32_t* __restrict__ sched, float* __restrict__ gW,
+                                                   int out_cols, int nslices, int slice_v, int two_persp) {
+    const int lane = threadIdx.x;
+    const int xcd = blockIdx.x % kXcd;
+    const uint32_t n_long = sched[kSchedNLong];
+    const uint32_t my_long = n_long > (uint32_t)xcd ? (n_long - xcd + kXcd - 1) / kXcd : 0;
+    const uint32_t lo = sched[kSchedRowLo + xcd], hi = sched[kSchedRowLo + xcd + 1];
+    const uint32_t nreg = hi - lo;
+    const uint32_t long_tasks = my_long * (uint32_t)nslices;
+    const uint32_t ntasks = long_tasks + nreg * (uint32_t)nslices;
+    uint32_t* ctr = sched + kSchedCtr + xcd * 32;
+
+    uint32_t next = next_task(ctr, lane);
+    while (next < ntasks) {
+        const uint32_t t = next;
+        next = next_task(ctr, lane);   // in flight while this task runs
+        uint32_t r;
+        int s;
+        if (t < long_tasks) {
+            const uint32_t i = t / (uint32_t)nslices;
+            s = (int)(t - i * (uint32_t)nslices);
+            r = long_rows[xcd + i * kXcd];
+        } else {
+            const uint32_t u = t - long_tasks;
+            s = (int)(u / nreg);
+            r = lo + (u - (uint32_t)s * nreg);
+        }
+        const uint32_t beg = seg_off[r], end = seg_off[r + 1];
+        if (t >= long_tasks && end - beg >= (uint32_t)kLongRow) continue;   // done in the long phase
+        seg_reduce_task<VW, NQ>(G, list, beg, beg + wcount[r], end, gW + (size_t)r * out_cols, s, lane, out_cols,
+                                slice_v, two_persp);
     }
 }
 
@@ -428,7 +481,8 @@ int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, fl
     uint32_t* cnt = (uint32_t*)(ws + L.cnt);
     uint32_t* wcount = (uint32_t*)(ws + L.wcount);
     uint32_t* seg_off = (uint32_t*)(ws + L.seg_off);
-    uint32_t* row_order = (uint32_t*)(ws + L.row_order);
+    uint32_t* long_rows = (uint32_t*)(ws + L.long_rows);
+    uint32_t* sched = (uint32_t*)(ws + L.sched);
     uint32_t* list = (uint32_t*)(ws + L.list);
     float* partial = (float*)(ws + L.partial);
 
@@ -449,7 +503,7 @@ int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, fl
     hipLaunchKernelGGL(k_col_scan, dim3((R + 63) / 64), dim3(64), 0, st, cnt, wcount, seg_off, R, L.cpp,
                        L.nchunks);
     NNUEFT_LAUNCH_CHECK();
-    hipLaunchKernelGGL(k_row_scan, dim3(1), dim3(kScanThreads), 0, st, seg_off, row_order, R);
+    hipLaunchKernelGGL(k_row_scan, dim3(1), dim3(kScanThreads), 0, st, seg_off, long_rows, sched, R);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_fill, dim3(L.nchunks, nranges), dim3(256), fill_bytes, st, widx, bidx, cnt, seg_off, list,
                        B, K, R, L.cpp, range, stage);
@@ -463,12 +517,11 @@ int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, fl
     // equal slices, rounded up to whole 128-byte lines so no two waves share a cache line of a row
     const int line_v = 128 / (VWr * (int)sizeof(float));
     const int slice_v = ((nv + nslices - 1) / nslices + line_v - 1) / line_v * line_v;
-    const long long grid = (long long)R * nslices;
-    if (grid > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
+    if ((long long)R * nslices > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
     const int two = n_persp == 2;
-#define SEG_LAUNCH(VW_, NQ_)                                                                                    \
-    hipLaunchKernelGGL((k_seg_reduce<VW_, NQ_>), dim3((unsigned)grid), dim3(64), 0, st, G, list, seg_off, wcount, \
-                       row_order, gW, out_cols, nslices, slice_v, two)
+#define SEG_LAUNCH(VW_, NQ_)                                                                                      \
+    hipLaunchKernelGGL((k_seg_reduce<VW_, NQ_>), dim3(kXcd * kWavesPerXcd), dim3(64), 0, st, G, list, seg_off,      \
+                       wcount, long_rows, sched, gW, out_cols, nslices, slice_v, two)
     if (vec && NQ == 2) SEG_LAUNCH(4, 2);
     else if (vec) SEG_LAUNCH(4, 1);
     else if (NQ == 2) SEG_LAUNCH(1, 2);
@@ -507,13 +560,14 @@ extern "C" int nnueft_sparse_bwd_det(const int32_t* idx, const float* gout, floa
 }
 
 extern "C" int nnueft_double_bwd_det(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
-                                     const int64_t* psqt_idx, float max_act, const float* grad_l0,
+                                     const int64_t* psqt_idx, const float* bias, float max_act,
+                                     const float* grad_l0,
                                      const float* grad_wpsqt, const float* grad_bpsqt, const float* saved,
                                      float* gW, float* gbias, int B, int K, int R, int L1, int n_psqt,
                                      void* workspace, size_t workspace_bytes, void* stream) {
     if (B <= 0 || K <= 0 || R <= 0 || L1 <= 0 || (L1 & 1) || n_psqt < 0) return NNUEFT_E_ARG;
-    if (!us || !them || !widx || !bidx || !psqt_idx || !grad_l0 || !grad_wpsqt || !grad_bpsqt || !saved || !gW ||
-        !gbias)
+    if (!us || !them || !widx || !bidx || !psqt_idx || !bias || !grad_l0 || !grad_wpsqt || !grad_bpsqt || !saved ||
+        !gW || !gbias)
         return NNUEFT_E_ARG;
     if ((long long)B * K > 0x3fffffffLL || (long long)B > 0x3fffffffLL) return NNUEFT_E_UNSUPPORTED;
     const int out_cols = L1 + n_psqt;
@@ -523,14 +577,14 @@ extern "C" int nnueft_double_bwd_det(const float* us, const float* them, const i
     hipStream_t st = (hipStream_t)stream;
     char* ws = (char*)workspace;
     float* G = (float*)(ws + L.G);
-    const bool vec = (L1 % 8 == 0) && (out_cols % 4 == 0) && aligned16(grad_l0) && aligned16(saved);
+    const bool vec = (L1 % 8 == 0) && (out_cols % 4 == 0) && aligned16(grad_l0) && aligned16(saved) && aligned16(bias);
     const int hv = (L1 / 2) / (vec ? 4 : 1);
     const dim3 grid(L.ntiles, max(1, (hv + 63) / 64));
     if (vec)
-        hipLaunchKernelGGL(k_bwd_rows<4>, grid, dim3(64), 0, st, us, them, psqt_idx, max_act, grad_l0, grad_wpsqt,
+        hipLaunchKernelGGL(k_bwd_rows<4>, grid, dim3(64), 0, st, us, them, psqt_idx, bias, max_act, grad_l0, grad_wpsqt,
                            grad_bpsqt, saved, G, (float*)(ws + L.partial), B, L1, n_psqt);
     else
-        hipLaunchKernelGGL(k_bwd_rows<1>, grid, dim3(64), 0, st, us, them, psqt_idx, max_act, grad_l0, grad_wpsqt,
+        hipLaunchKernelGGL(k_bwd_rows<1>, grid, dim3(64), 0, st, us, them, psqt_idx, bias, max_act, grad_l0, grad_wpsqt,
                            grad_bpsqt, saved, G, (float*)(ws + L.partial), B, L1, n_psqt);
     NNUEFT_LAUNCH_CHECK();
     return det_sort_reduce(widx, bidx, G, gW, gbias, B, K, R, out_cols, 2, ws, L, st);

@@ -61,6 +61,34 @@ __device__ __forceinline__ void vadd(vecf<VW>& a, const vecf<VW>& b) {
 
 __device__ __forceinline__ float clamp_act(float x, float hi) { return x < 0.0f ? 0.0f : (x > hi ? hi : x); }
 
+// The four mixed pre-clamp values of a column pair (i, i + L1/2) from the two perspectives' row sums
+// (sw*, sb*: white / black sums of the two columns; b0, b1: bias of the two columns).  Forward and
+// backward both go through this function, so the backward sees exactly the forward's values.
+__device__ __forceinline__ void mix4(float u, float t, float sw0, float sw1, float sb0, float sb1, float b0,
+                                     float b1, float& xw0, float& xw1, float& xb0, float& xb1) {
+    const float w0 = sw0 + b0, w1 = sw1 + b1;
+    const float k0 = sb0 + b0, k1 = sb1 + b1;
+    xw0 = u * w0 + t * k0;
+    xw1 = u * w1 + t * k1;
+    xb0 = u * k0 + t * w0;
+    xb1 = u * k1 + t * w1;
+}
+
+// The four upstream values of that column pair for the two perspectives' sparse-linear outputs.
+__device__ __forceinline__ void grad4(float u, float t, float xw0, float xw1, float xb0, float xb1, float g0,
+                                      float g1, float max_act, float& gw0, float& gw1, float& gb0, float& gb1) {
+    const float cw0 = clamp_act(xw0, max_act), cw1 = clamp_act(xw1, max_act);
+    const float cb0 = clamp_act(xb0, max_act), cb1 = clamp_act(xb1, max_act);
+    const float dw0 = (xw0 >= 0.0f && xw0 <= max_act) ? g0 * cw1 : 0.0f;
+    const float dw1 = (xw1 >= 0.0f && xw1 <= max_act) ? g0 * cw0 : 0.0f;
+    const float db0 = (xb0 >= 0.0f && xb0 <= max_act) ? g1 * cb1 : 0.0f;
+    const float db1 = (xb1 >= 0.0f && xb1 <= max_act) ? g1 * cb0 : 0.0f;
+    gw0 = u * dw0 + t * db0;
+    gw1 = u * dw1 + t * db1;
+    gb0 = t * dw0 + u * db0;
+    gb1 = t * dw1 + u * db1;
+}
+
 // Lowest set bit of a wave mask, removed from the mask.  The mask comes from __ballot, so the
 // result is wave-uniform and can drive scalar control flow and v_readlane.
 __device__ __forceinline__ int pop_lane(u64& mask) {

@@ -7,6 +7,14 @@
 // costs nothing and no LDS is needed.
 #include "gather.h"
 
+namespace nnueft_blocked {
+size_t fwd_workspace(int B);
+int double_fwd_blocked(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+                       const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,
+                       float* wpsqt, float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt, void* ws,
+                       hipStream_t st);
+}  // namespace nnueft_blocked
+
 namespace {
 
 constexpr int kUnroll = 4;
@@ -58,11 +66,13 @@ __global__ __launch_bounds__(64) void k_double_fwd(const float* __restrict__ us,
                                                    const float* __restrict__ W, const float* __restrict__ bias,
                                                    float max_act, float* __restrict__ l0,
                                                    float* __restrict__ wpsqt, float* __restrict__ bpsqt,
-                                                   float* __restrict__ saved, int K, int R, int L1, int n_psqt,
-                                                   int nslices) {
+                                                   float* __restrict__ saved, int B, int K, int R, int L1,
+                                                   int n_psqt, int nslices) {
     const int lane = threadIdx.x;
-    const int b = blockIdx.x / nslices;
-    const int s = blockIdx.x - b * nslices;
+    // slice-major task order: at any time the whole GPU gathers the same 1/nslices of the table's
+    // columns, which keeps the live part of the table inside the memory-side cache
+    const int s = blockIdx.x / B;
+    const int b = blockIdx.x - s * B;
     const int h = L1 >> 1;
     const int hv = h / VW;
     const size_t out_cols = (size_t)L1 + n_psqt;
@@ -103,31 +113,27 @@ __global__ __launch_bounds__(64) void k_double_fwd(const float* __restrict__ us,
     }
 
     const float u = us[b], t = them[b];
-    float* sv = saved + (size_t)b * 2 * L1;
+    float* sw = saved + (size_t)b * L1;
+    float* sb = saved + ((size_t)B + b) * L1;
     float* o = l0 + (size_t)b * L1;
 #pragma unroll
     for (int m = 0; m < NQ; ++m) {
         if (!act[m]) continue;
         const int c = col[2 * m];
         const vecf<VW> bias0 = ldv<VW>(bias + c), bias1 = ldv<VW>(bias + c + h);
-        vecf<VW> xw0, xw1, xb0, xb1, o0, o1;
+        vecf<VW> o0, o1;
 #pragma unroll
         for (int i = 0; i < VW; ++i) {
-            const float w0 = acc[0][2 * m].v[i] + bias0.v[i];
-            const float w1 = acc[0][2 * m + 1].v[i] + bias1.v[i];
-            const float b0 = acc[1][2 * m].v[i] + bias0.v[i];
-            const float b1 = acc[1][2 * m + 1].v[i] + bias1.v[i];
-            xw0.v[i] = u * w0 + t * b0;
-            xw1.v[i] = u * w1 + t * b1;
-            xb0.v[i] = u * b0 + t * w0;
-            xb1.v[i] = u * b1 + t * w1;
-            o0.v[i] = clamp_act(xw0.v[i], max_act) * clamp_act(xw1.v[i], max_act);
-            o1.v[i] = clamp_act(xb0.v[i], max_act) * clamp_act(xb1.v[i], max_act);
+            float xw0, xw1, xb0, xb1;
+            mix4(u, t, acc[0][2 * m].v[i], acc[0][2 * m + 1].v[i], acc[1][2 * m].v[i], acc[1][2 * m + 1].v[i],
+                 bias0.v[i], bias1.v[i], xw0, xw1, xb0, xb1);
+            o0.v[i] = clamp_act(xw0, max_act) * clamp_act(xw1, max_act);
+            o1.v[i] = clamp_act(xb0, max_act) * clamp_act(xb1, max_act);
         }
-        stv<VW>(sv + 0 * h + c, xw0);
-        stv<VW>(sv + 1 * h + c, xw1);
-        stv<VW>(sv + 2 * h + c, xb0);
-        stv<VW>(sv + 3 * h + c, xb1);
+        stv<VW>(sw + c, acc[0][2 * m]);
+        stv<VW>(sw + h + c, acc[0][2 * m + 1]);
+        stv<VW>(sb + c, acc[1][2 * m]);
+        stv<VW>(sb + h + c, acc[1][2 * m + 1]);
         stv<VW>(o + c, o0);
         stv<VW>(o + h + c, o1);
     }
@@ -161,7 +167,7 @@ int launch_double_fwd(const float* us, const float* them, const int32_t* widx, c
     const long long grid = (long long)B * nslices;
     if (grid > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
     hipLaunchKernelGGL((k_double_fwd<VW, NQ>), dim3((unsigned)grid), dim3(64), 0, st, us, them, widx, bidx,
-                       psqt_idx, W, bias, max_act, l0, wpsqt, bpsqt, saved, K, R, L1, n_psqt, nslices);
+                       psqt_idx, W, bias, max_act, l0, wpsqt, bpsqt, saved, B, K, R, L1, n_psqt, nslices);
     NNUEFT_LAUNCH_CHECK();
     return 0;
 }
@@ -183,10 +189,15 @@ extern "C" int nnueft_sparse_fwd(const int32_t* idx, const float* W, const float
     return launch_sparse_fwd<1, 1>(idx, W, bias, out, B, K, R, out_cols, st);
 }
 
+extern "C" size_t nnueft_fwd_workspace_bytes(int B, int K, int R, int L1, int n_psqt) {
+    if (B <= 0 || K <= 0 || R <= 0 || L1 <= 0 || n_psqt < 0) return 0;
+    return nnueft_blocked::fwd_workspace(B);
+}
+
 extern "C" int nnueft_double_fwd(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                                  const int64_t* psqt_idx, const float* W, const float* bias, float max_act,
                                  float* l0, float* wpsqt, float* bpsqt, float* saved, int B, int K, int R,
-                                 int L1, int n_psqt, void* stream) {
+                                 int L1, int n_psqt, void* workspace, size_t workspace_bytes, void* stream) {
     if (B < 0 || K <= 0 || R <= 0 || L1 <= 0 || (L1 & 1) || n_psqt < 0) return NNUEFT_E_ARG;
     if (B == 0) return 0;
     if (!us || !them || !widx || !bidx || !psqt_idx || !W || !bias || !l0 || !wpsqt || !bpsqt || !saved)
@@ -194,6 +205,13 @@ extern "C" int nnueft_double_fwd(const float* us, const float* them, const int32
     hipStream_t st = (hipStream_t)stream;
     const bool vec = (L1 % 8 == 0) && ((L1 + n_psqt) % 4 == 0) && aligned16(W) && aligned16(bias) &&
                      aligned16(l0) && aligned16(saved);
+    if (workspace) {
+        if (!aligned256(workspace) || workspace_bytes < nnueft_blocked::fwd_workspace(B)) return NNUEFT_E_WORKSPACE;
+        // the L2-blocked path needs 16-byte rows; other shapes take the plain kernel below
+        if (vec && (long long)B <= 0x3fffffffLL)
+            return nnueft_blocked::double_fwd_blocked(us, them, widx, bidx, psqt_idx, W, bias, max_act, l0, wpsqt,
+                                                      bpsqt, saved, B, K, R, L1, n_psqt, workspace, st);
+    }
     if (vec) {
         if (L1 / 8 > 64)
             return launch_double_fwd<4, 2>(us, them, widx, bidx, psqt_idx, W, bias, max_act, l0, wpsqt, bpsqt,

@@ -1,0 +1,248 @@
+// Forward, L2-blocked variant (used when the caller passes a workspace).
+//
+// The lists of one perspective of one position name rows of a single 768-row block of the table
+// (one king bucket).  Sorting the (position, perspective) pairs of a batch by that block and
+// giving each XCD a contiguous part of the sorted order, walked one column slice at a time, keeps
+// the rows a XCD is gathering (768 rows x one slice = 0.75-1.5 MB) inside its own 4 MB L2, so the
+// gather runs at L2 speed and the table crosses the fabric about once instead of ~24 times.
+//
+//   k_pair_order   counting sort of the 2B pairs by table block of their first valid index
+//   k_acc_blocked  wave per (pair, column slice): chain from +0 over the list, result to saved[2, B, L1]
+//   k_mix          per position: + bias, side-to-move mix, clamp, product, psqt chains; writes l0
+//
+// Workgroups are handed to the 8 XCDs round-robin by workgroup id, so id % 8 selects the XCD.
+#include "gather.h"
+
+namespace nnueft_blocked {
+
+constexpr int kXcd = 8;
+constexpr int kOrderThreads = 1024;
+constexpr int kMaxBins = 2048;
+
+__device__ __forceinline__ const int32_t* pair_list(const int32_t* __restrict__ widx,
+                                                    const int32_t* __restrict__ bidx, int pair, int B, int K) {
+    const int p = pair >= B;
+    return (p ? bidx : widx) + (size_t)(pair - p * B) * K;
+}
+
+// Table block of a list given its first slot (already loaded); scans on only when that slot is padding.
+__device__ __forceinline__ int pair_key(const int32_t* __restrict__ ix, int first, int K, int R, int block_rows,
+                                        int nbins) {
+    if (first >= 0 && first < R) return first / block_rows;
+    for (int k = 1; k < K; ++k) {
+        const int r = ix[k];
+        if (r >= 0 && r < R) return r / block_rows;
+    }
+    return nbins - 1;   // empty list
+}
+
+// order[] = pair ids (p * B + b) grouped by table block.  Single workgroup.
+__global__ __launch_bounds__(kOrderThreads) void k_pair_order(const int32_t* __restrict__ widx,
+                                                              const int32_t* __restrict__ bidx,
+                                                              uint32_t* __restrict__ order, int B, int K, int R,
+                                                              int block_rows, int nbins) {
+    __shared__ uint32_t bins[kMaxBins];
+    __shared__ uint32_t wave_tot[kOrderThreads / 64];
+    const int tid = threadIdx.x;
+    const int npairs = 2 * B;
+    for (int i = tid; i < nbins; i += kOrderThreads) bins[i] = 0;
+    __syncthreads();
+    constexpr int PF = 8;
+    for (int n0 = tid; n0 < npairs; n0 += kOrderThreads * PF) {
+        int first[PF];
+#pragma unroll
+        for (int u = 0; u < PF; ++u) {
+            const int n = n0 + u * kOrderThreads;
+            first[u] = n < npairs ? pair_list(widx, bidx, n, B, K)[0] : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < PF; ++u) {
+            const int n = n0 + u * kOrderThreads;
+            if (n < npairs)
+                atomicAdd(&bins[pair_key(pair_list(widx, bidx, n, B, K), first[u], K, R, block_rows, nbins)], 1u);
+        }
+    }
+    __syncthreads();
+    // exclusive scan of bins (nbins <= kMaxBins = 2 * kOrderThreads): two entries per thread
+    const uint32_t a = (2 * tid < nbins) ? bins[2 * tid] : 0;
+    const uint32_t c = (2 * tid + 1 < nbins) ? bins[2 * tid + 1] : 0;
+    uint32_t incl = a + c;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t v = __shfl_up(incl, off);
+        if ((tid & 63) >= off) incl += v;
+    }
+    if ((tid & 63) == 63) wave_tot[tid >> 6] = incl;
+    __syncthreads();
+    uint32_t base = 0;
+    for (int w = 0; w < (tid >> 6); ++w) base += wave_tot[w];
+    const uint32_t excl = base + incl - (a + c);
+    __syncthreads();
+    if (2 * tid < nbins) bins[2 * tid] = excl;
+    if (2 * tid + 1 < nbins) bins[2 * tid + 1] = excl + a;
+    __syncthreads();
+    for (int n0 = tid; n0 < npairs; n0 += kOrderThreads * PF) {
+        int first[PF];
+#pragma unroll
+        for (int u = 0; u < PF; ++u) {
+            const int n = n0 + u * kOrderThreads;
+            first[u] = n < npairs ? pair_list(widx, bidx, n, B, K)[0] : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < PF; ++u) {
+            const int n = n0 + u * kOrderThreads;
+            if (n < npairs) {
+                const int key = pair_key(pair_list(widx, bidx, n, B, K), first[u], K, R, block_rows, nbins);
+                order[atomicAdd(&bins[key], 1u)] = (uint32_t)n;
+            }
+        }
+    }
+}
+
+// saved[pair, slice] = chain from +0 over the pair's list (pair = perspective * B + position).
+template <int VW, int NQ, int U>
+__global__ __launch_bounds__(64) void k_acc_blocked(const int32_t* __restrict__ widx,
+                                                    const int32_t* __restrict__ bidx,
+                                                    const uint32_t* __restrict__ order,
+                                                    const float* __restrict__ W, float* __restrict__ acc, int B,
+                                                    int K, int R, int L1, int out_cols, int per_xcd) {
+    const int lane = threadIdx.x;
+    const int xcd = blockIdx.x % kXcd;
+    const int j = blockIdx.x / kXcd;
+    const int s = j / per_xcd;
+    const int n = xcd * per_xcd + (j - s * per_xcd);
+    if (n >= 2 * B) return;
+    const int pair = (int)order[n];
+    const int p = pair >= B;
+    const int b = pair - p * B;
+    const int nv = L1 / VW;
+
+    int col[NQ];
+    bool act[NQ];
+#pragma unroll
+    for (int m = 0; m < NQ; ++m) {
+        const int q = (s * NQ + m) * 64 + lane;
+        act[m] = q < nv;
+        col[m] = act[m] ? q * VW : 0;
+    }
+    vecf<VW> a[NQ];
+#pragma unroll
+    for (int m = 0; m < NQ; ++m) a[m] = vzero<VW>();
+    const int32_t* ix = (p ? bidx : widx) + (size_t)b * K;
+    for (int k0 = 0; k0 < K; k0 += 64) {
+        const int my = (k0 + lane < K) ? ix[k0 + lane] : -1;
+        const u64 mask = __ballot(my >= 0 && my < R);
+        chain_rows<VW, NQ, U>(a, W, (size_t)out_cols, col, my, mask);
+    }
+    float* dst = acc + (size_t)pair * L1;
+#pragma unroll
+    for (int m = 0; m < NQ; ++m)
+        if (act[m]) stv<VW>(dst + col[m], a[m]);
+}
+
+// Per position: bias, mix, clamp, product; slice 0 also does the two psqt chains.
+template <int VW>
+__global__ __launch_bounds__(64) void k_mix(const float* __restrict__ us, const float* __restrict__ them,
+                                            const int32_t* __restrict__ widx, const int32_t* __restrict__ bidx,
+                                            const int64_t* __restrict__ psqt_idx, const float* __restrict__ W,
+                                            const float* __restrict__ bias, const float* __restrict__ saved,
+                                            float max_act, float* __restrict__ l0, float* __restrict__ wpsqt,
+                                            float* __restrict__ bpsqt, int B, int K, int R, int L1, int n_psqt) {
+    const int lane = threadIdx.x;
+    const int b = blockIdx.x;
+    const int s = blockIdx.y;
+    const int h = L1 >> 1;
+    const int hv = h / VW;
+    const size_t out_cols = (size_t)L1 + n_psqt;
+    const int q = s * 64 + lane;
+    if (q < hv) {
+        const int c = q * VW;
+        const float u = us[b], t = them[b];
+        const float* sw = saved + (size_t)b * L1;
+        const float* sb = saved + ((size_t)B + b) * L1;
+        const vecf<VW> sw0 = ldv<VW>(sw + c), sw1 = ldv<VW>(sw + h + c);
+        const vecf<VW> sb0 = ldv<VW>(sb + c), sb1 = ldv<VW>(sb + h + c);
+        const vecf<VW> bias0 = ldv<VW>(bias + c), bias1 = ldv<VW>(bias + h + c);
+        vecf<VW> o0, o1;
+#pragma unroll
+        for (int i = 0; i < VW; ++i) {
+            float xw0, xw1, xb0, xb1;
+            mix4(u, t, sw0.v[i], sw1.v[i], sb0.v[i], sb1.v[i], bias0.v[i], bias1.v[i], xw0, xw1, xb0, xb1);
+            o0.v[i] = clamp_act(xw0, max_act) * clamp_act(xw1, max_act);
+            o1.v[i] = clamp_act(xb0, max_act) * clamp_act(xb1, max_act);
+        }
+        float* o = l0 + (size_t)b * L1;
+        stv<VW>(o + c, o0);
+        stv<VW>(o + h + c, o1);
+    }
+    if (s == 0) {
+        const int64_t pi = psqt_idx[b];
+        const bool do_psqt = pi >= 0 && pi < n_psqt;
+        float ps[2] = {0.0f, 0.0f};
+        if (do_psqt) {
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                const int32_t* ix = (p ? bidx : widx) + (size_t)b * K;
+                for (int k0 = 0; k0 < K; k0 += 64) {
+                    const int my = (k0 + lane < K) ? ix[k0 + lane] : -1;
+                    const bool ok = my >= 0 && my < R;
+                    u64 mask = __ballot(ok);
+                    const float myps = ok ? W[(size_t)my * out_cols + L1 + pi] : 0.0f;
+                    while (mask) ps[p] = ps[p] + bcast_f(myps, pop_lane(mask));
+                }
+            }
+        }
+        if (lane == 0) {
+            const float pb = do_psqt ? bias[L1 + pi] : 0.0f;
+            wpsqt[b] = ps[0] + pb;
+            bpsqt[b] = ps[1] + pb;
+        }
+    }
+}
+
+static inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+size_t fwd_workspace(int B) { return B > 0 ? up256((size_t)2 * B * sizeof(uint32_t)) : 0; }
+
+int table_block_rows(int R, int* nbins) {
+    int block_rows = 768;
+    if ((R + block_rows - 1) / block_rows + 1 > kMaxBins) block_rows = (R + kMaxBins - 2) / (kMaxBins - 1);
+    *nbins = (R + block_rows - 1) / block_rows + 1;
+    return block_rows;
+}
+
+int double_fwd_blocked(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+                       const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,
+                       float* wpsqt, float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt,
+                       void* ws, hipStream_t st) {
+    uint32_t* order = (uint32_t*)ws;
+    int nbins = 0;
+    const int block_rows = table_block_rows(R, &nbins);
+    hipLaunchKernelGGL(k_pair_order, dim3(1), dim3(kOrderThreads), 0, st, widx, bidx, order, B, K, R, block_rows,
+                       nbins);
+    NNUEFT_LAUNCH_CHECK();
+    const int out_cols = L1 + n_psqt;
+    const int nv = L1 / 4;
+    const int per_xcd = (2 * B + kXcd - 1) / kXcd;
+    if (nv > 64) {
+        constexpr int NQ = 2;
+        const int nslices = (nv + 64 * NQ - 1) / (64 * NQ);
+        const long long grid = (long long)kXcd * per_xcd * nslices;
+        if (grid > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
+        hipLaunchKernelGGL((k_acc_blocked<4, NQ, 8>), dim3((unsigned)grid), dim3(64), 0, st, widx, bidx, order, W,
+                           saved, B, K, R, L1, out_cols, per_xcd);
+    } else {
+        const long long grid = (long long)kXcd * per_xcd;
+        if (grid > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
+        hipLaunchKernelGGL((k_acc_blocked<4, 1, 8>), dim3((unsigned)grid), dim3(64), 0, st, widx, bidx, order, W,
+                           saved, B, K, R, L1, out_cols, per_xcd);
+    }
+    NNUEFT_LAUNCH_CHECK();
+    const int hv = (L1 / 2) / 4;
+    hipLaunchKernelGGL(k_mix<4>, dim3(B, (hv + 63) / 64), dim3(64), 0, st, us, them, widx, bidx, psqt_idx, W, bias,
+                       saved, max_act, l0, wpsqt, bpsqt, B, K, R, L1, n_psqt);
+    NNUEFT_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // namespace nnueft_blocked

@@ -20,11 +20,15 @@ PROTOTYPES = {
     "nnueft_sparse_bwd_atomic": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_void_p]),
     "nnueft_det_workspace_bytes": (c_size_t, [c_int] * 5),
     "nnueft_sparse_bwd_det": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
-    "nnueft_double_fwd": (c_int, [c_void_p] * 7 + [c_float] + [c_void_p] * 4 + [c_int] * 5 + [c_void_p]),
-    "nnueft_double_bwd_atomic": (c_int, [c_void_p] * 5 + [c_float] + [c_void_p] * 6 + [c_int] * 5 + [c_void_p]),
+    "nnueft_fwd_workspace_bytes": (c_size_t, [c_int] * 5),
+    "nnueft_double_fwd": (
+        c_int,
+        [c_void_p] * 7 + [c_float] + [c_void_p] * 4 + [c_int] * 5 + [c_void_p, c_size_t, c_void_p],
+    ),
+    "nnueft_double_bwd_atomic": (c_int, [c_void_p] * 6 + [c_float] + [c_void_p] * 6 + [c_int] * 5 + [c_void_p]),
     "nnueft_double_bwd_det": (
         c_int,
-        [c_void_p] * 5 + [c_float] + [c_void_p] * 6 + [c_int] * 5 + [c_void_p, c_size_t, c_void_p],
+        [c_void_p] * 6 + [c_float] + [c_void_p] * 6 + [c_int] * 5 + [c_void_p, c_size_t, c_void_p],
     ),
     "nnueft_ft_int16_fwd": (c_int, [c_void_p] * 9 + [c_int] * 7 + [c_void_p]),
 }

@@ -5,9 +5,10 @@ model/modules/feature_transformer/fused_ft_functions.py:18-122; the two CuPy ker
 are replaced by nnueft_double_fwd / nnueft_double_bwd_{atomic,det} of libnnueft.so.
 
 Differences that a caller can observe:
-  * the activation tensor kept for the backward holds the mixed values before the clamp (the
-    reference keeps them after it, fused_ft_kernel.py:95-99), so the clamp passes gradient at
-    exactly 0 and exactly max like torch.clamp does in the reference's CPU path;
+  * the activation tensor kept for the backward holds the two perspectives' row sums (the reference
+    keeps the clamped mixed values, fused_ft_kernel.py:95-99); the backward recomputes the mix from
+    them, so the clamp passes gradient at exactly 0 and exactly max like torch.clamp does in the
+    reference's CPU path;
   * NNUEFT_BACKWARD=deterministic (or set_backward_mode) selects a backward whose result does
     not depend on scheduling.
 """
@@ -31,17 +32,19 @@ def _launch_double_fwd(us, them, white_indices, black_indices, psqt_indices, wei
     lib = _native.load()
     B, K = white_indices.shape
     R, out_cols = weight.shape
+    nbytes = lib.nnueft_fwd_workspace_bytes(B, K, R, l1_size, out_cols - l1_size)
+    ws = _workspace(nbytes, weight.device)
     rc = lib.nnueft_double_fwd(
         us.data_ptr(), them.data_ptr(), white_indices.data_ptr(), black_indices.data_ptr(),
         psqt_indices.data_ptr(), weight.data_ptr(), bias.data_ptr(), float(max_ft_activation),
         l0_.data_ptr(), wpsqt.data_ptr(), bpsqt.data_ptr(), saved.data_ptr(),
-        B, K, R, l1_size, out_cols - l1_size, _stream_ptr(weight.device),
+        B, K, R, l1_size, out_cols - l1_size, ws.data_ptr(), nbytes, _stream_ptr(weight.device),
     )
     _native.check(rc, "nnueft_double_fwd")
 
 
 @torch.compiler.disable(recursive=False)
-def _launch_double_bwd(us, them, white_indices, black_indices, psqt_indices, max_ft_activation, grad_l0,
+def _launch_double_bwd(us, them, white_indices, black_indices, psqt_indices, bias, max_ft_activation, grad_l0,
                        grad_wpsqt, grad_bpsqt, saved, num_rows, l1_size, output_size, mode):
     lib = _native.load()
     B, K = white_indices.shape
@@ -49,7 +52,7 @@ def _launch_double_bwd(us, them, white_indices, black_indices, psqt_indices, max
     n_psqt = output_size - l1_size
     head = (
         us.data_ptr(), them.data_ptr(), white_indices.data_ptr(), black_indices.data_ptr(),
-        psqt_indices.data_ptr(), float(max_ft_activation),
+        psqt_indices.data_ptr(), bias.data_ptr(), float(max_ft_activation),
         grad_l0.data_ptr(), grad_wpsqt.data_ptr(), grad_bpsqt.data_ptr(), saved.data_ptr(),
     )
     if mode == "deterministic":
@@ -112,26 +115,25 @@ class FusedDoubleFtFunction(autograd.Function):
         assert weight.is_contiguous() and bias.is_contiguous()
 
         batch_size = white_indices.shape[0]
-        l1_half = l1_size // 2
         device = us.device
 
         l0_ = torch.empty(batch_size, l1_size, dtype=torch.float32, device=device)
         wpsqt = torch.empty(batch_size, 1, dtype=torch.float32, device=device)
         bpsqt = torch.empty(batch_size, 1, dtype=torch.float32, device=device)
-        preclamp = torch.empty(batch_size, 4, l1_half, dtype=torch.float32, device=device)
+        row_sums = torch.empty(2, batch_size, l1_size, dtype=torch.float32, device=device)
 
         with torch.cuda.device(device):
             _launch_double_fwd(
                 us, them, white_indices, black_indices, psqt_indices, weight, bias,
-                max_ft_activation, int(l1_size), l0_, wpsqt, bpsqt, preclamp,
+                max_ft_activation, int(l1_size), l0_, wpsqt, bpsqt, row_sums,
             )
 
-        ctx.save_for_backward(us, them, white_indices, black_indices, psqt_indices, weight, bias, preclamp)
+        ctx.save_for_backward(us, them, white_indices, black_indices, psqt_indices, weight, bias, row_sums)
         return l0_, wpsqt, bpsqt
 
     @staticmethod
     def backward(ctx, grad_l0, grad_wpsqt, grad_bpsqt):
-        us, them, white_indices, black_indices, psqt_indices, weight, bias, preclamp = ctx.saved_tensors
+        us, them, white_indices, black_indices, psqt_indices, weight, bias, row_sums = ctx.saved_tensors
 
         grad_l0 = grad_l0.contiguous()
         grad_wpsqt = grad_wpsqt.contiguous()
@@ -139,8 +141,8 @@ class FusedDoubleFtFunction(autograd.Function):
 
         with torch.cuda.device(us.device):
             grad_weight, grad_bias = _launch_double_bwd(
-                us, them, white_indices, black_indices, psqt_indices, ctx.max_ft_activation,
-                grad_l0, grad_wpsqt, grad_bpsqt, preclamp,
+                us, them, white_indices, black_indices, psqt_indices, bias, ctx.max_ft_activation,
+                grad_l0, grad_wpsqt, grad_bpsqt, row_sums,
                 weight.shape[0], ctx.l1_size, bias.shape[0], ctx.backward_mode,
             )
 

@@ -73,7 +73,7 @@ def double_fwd(us, them, widx, bidx, psqt_idx, W, bias, max_act, L1):
     l0 = np.empty((B, L1), np.float32)
     wp = np.empty((B, 1), np.float32)
     bp = np.empty((B, 1), np.float32)
-    saved = np.empty((B, 4, L1 // 2), np.float32)
+    saved = np.empty((2, B, L1), np.float32)
     rc = lib().nnueft_oracle_double_fwd(_p(us), _p(them), _p(widx), _p(bidx), _p(psqt_idx), _p(W), _p(bias),
                                         ctypes.c_float(max_act), _p(l0), _p(wp), _p(bp), _p(saved),
                                         B, K, R, L1, n_psqt)
@@ -81,24 +81,26 @@ def double_fwd(us, them, widx, bidx, psqt_idx, W, bias, max_act, L1):
     return l0, wp, bp, saved
 
 
-def double_bwd_rows(us, them, psqt_idx, max_act, grad_l0, grad_wpsqt, grad_bpsqt, saved, n_psqt):
+def double_bwd_rows(us, them, psqt_idx, bias, max_act, grad_l0, grad_wpsqt, grad_bpsqt, saved, n_psqt):
     us, them = _c(us, np.float32).reshape(-1), _c(them, np.float32).reshape(-1)
     psqt_idx = _c(psqt_idx, np.int64)
+    bias = _c(bias, np.float32)
     grad_l0 = _c(grad_l0, np.float32)
     gwp, gbp = _c(grad_wpsqt, np.float32).reshape(-1), _c(grad_bpsqt, np.float32).reshape(-1)
     saved = _c(saved, np.float32)
     B, L1 = grad_l0.shape
     G = np.empty((2, B, L1 + n_psqt), np.float32)
-    rc = lib().nnueft_oracle_double_bwd_rows(_p(us), _p(them), _p(psqt_idx), ctypes.c_float(max_act),
+    rc = lib().nnueft_oracle_double_bwd_rows(_p(us), _p(them), _p(psqt_idx), _p(bias), ctypes.c_float(max_act),
                                              _p(grad_l0), _p(gwp), _p(gbp), _p(saved), _p(G), B, L1, n_psqt)
     assert rc == 0
     return G
 
 
-def double_bwd(us, them, widx, bidx, psqt_idx, max_act, grad_l0, grad_wpsqt, grad_bpsqt, saved, R, n_psqt):
+def double_bwd(us, them, widx, bidx, psqt_idx, bias, max_act, grad_l0, grad_wpsqt, grad_bpsqt, saved, R, n_psqt):
     us, them = _c(us, np.float32).reshape(-1), _c(them, np.float32).reshape(-1)
     widx, bidx = _c(widx, np.int32), _c(bidx, np.int32)
     psqt_idx = _c(psqt_idx, np.int64)
+    bias = _c(bias, np.float32)
     grad_l0 = _c(grad_l0, np.float32)
     gwp, gbp = _c(grad_wpsqt, np.float32).reshape(-1), _c(grad_bpsqt, np.float32).reshape(-1)
     saved = _c(saved, np.float32)
@@ -107,7 +109,7 @@ def double_bwd(us, them, widx, bidx, psqt_idx, max_act, grad_l0, grad_wpsqt, gra
     oc = L1 + n_psqt
     gW = np.empty((R, oc), np.float32)
     gb = np.empty((oc,), np.float32)
-    rc = lib().nnueft_oracle_double_bwd(_p(us), _p(them), _p(widx), _p(bidx), _p(psqt_idx),
+    rc = lib().nnueft_oracle_double_bwd(_p(us), _p(them), _p(widx), _p(bidx), _p(psqt_idx), _p(bias),
                                         ctypes.c_float(max_act), _p(grad_l0), _p(gwp), _p(gbp), _p(saved),
                                         _p(gW), _p(gb), B, K, R, L1, n_psqt)
     assert rc == 0

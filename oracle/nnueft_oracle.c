@@ -17,7 +17,10 @@
  *                                 fused_ft_kernel.py:27-117 (the fused kernel)
  *   nnueft_oracle_double_bwd      autograd of double_ft_functions.py:62-80 ==
  *                                 fused_ft_kernel.py:147-272, except that the clamp mask is torch's
- *                                 (gradient passes where 0 <= x <= max, x taken before the clamp)
+ *                                 (gradient passes where 0 <= x <= max, x taken before the clamp).
+ *                                 The activations kept between forward and backward are the two
+ *                                 perspectives' row sums (before the bias); the mixed values are
+ *                                 recomputed from them with the forward's own operations.
  *   nnueft_oracle_ft_int16_fwd    no code in the reference (the accumulate runs in the engine);
  *                                 spec docs/nnue.md:1014-1069 (int16 accumulate) and :2097-2134
  *                                 (pairwise product, shift), constants model/quantize.py:58-73
@@ -122,10 +125,22 @@ int nnueft_oracle_sparse_bwd(const int32_t* idx, const float* gout, float* gW, f
 
 static inline float clampf(float x, float lo, float hi) { return x < lo ? lo : (x > hi ? hi : x); }
 
+/* The four mixed pre-clamp values of column pair (i, i+h) from the two perspectives' row sums. */
+static inline void mix4(float u, float t, const float* sw, const float* sb, const float* bias, int i, int h,
+                        float* xw0, float* xw1, float* xb0, float* xb1)
+{
+    const float w0 = sw[i] + bias[i], w1 = sw[i + h] + bias[i + h];
+    const float b0 = sb[i] + bias[i], b1 = sb[i + h] + bias[i + h];
+    *xw0 = u * w0 + t * b0;
+    *xw1 = u * w1 + t * b1;
+    *xb0 = u * b0 + t * w0;
+    *xb1 = u * b1 + t * w1;
+}
+
 /*
  * Both perspectives, side-to-move mix, clamp, pairwise product.
- * saved[b,0..3,:] holds the mixed values BEFORE the clamp, in the order
- * (x_w[:h], x_w[h:], x_b[:h], x_b[h:]), h = L1/2.
+ * saved[p, b, 0:L1] receives the row sums of perspective p (0 white, 1 black) BEFORE the bias:
+ * the chain from +0 over the valid slots.  Everything downstream is a function of them.
  */
 int nnueft_oracle_double_fwd(const float* us, const float* them,
                              const int32_t* widx, const int32_t* bidx, const int64_t* psqt_idx,
@@ -136,49 +151,36 @@ int nnueft_oracle_double_fwd(const float* us, const float* them,
     const int out_cols = L1 + n_psqt;
     const int h = L1 / 2;
     if (L1 % 2) return -1;
-#pragma omp parallel
-    {
-        float* acc = (float*)malloc(sizeof(float) * 2 * (size_t)L1);
-#pragma omp for schedule(static)
-        for (int b = 0; b < B; ++b) {
-            const int64_t pi = psqt_idx[b];
-            const int psqt_ok = pi >= 0 && pi < n_psqt;
-            float ps[2] = {0.0f, 0.0f};
-            for (int p = 0; p < 2; ++p) {
-                const int32_t* ix = (p == 0 ? widx : bidx) + (size_t)b * K;
-                float* a = acc + (size_t)p * L1;
-                for (int c = 0; c < L1; ++c) a[c] = 0.0f;
-                for (int k = 0; k < K; ++k) {
-                    int32_t r = ix[k];
-                    if (!valid(r, R)) continue;
-                    const float* w = W + (size_t)r * out_cols;
-                    for (int c = 0; c < L1; ++c) a[c] = a[c] + w[c];
-                    if (psqt_ok) ps[p] = ps[p] + w[L1 + pi];
-                }
-                for (int c = 0; c < L1; ++c) a[c] = a[c] + bias[c];
-                if (psqt_ok) ps[p] = ps[p] + bias[L1 + pi];
+#pragma omp parallel for schedule(static)
+    for (int b = 0; b < B; ++b) {
+        const int64_t pi = psqt_idx[b];
+        const int psqt_ok = pi >= 0 && pi < n_psqt;
+        float ps[2] = {0.0f, 0.0f};
+        for (int p = 0; p < 2; ++p) {
+            const int32_t* ix = (p == 0 ? widx : bidx) + (size_t)b * K;
+            float* a = saved + ((size_t)p * B + b) * L1;
+            for (int c = 0; c < L1; ++c) a[c] = 0.0f;
+            for (int k = 0; k < K; ++k) {
+                int32_t r = ix[k];
+                if (!valid(r, R)) continue;
+                const float* w = W + (size_t)r * out_cols;
+                for (int c = 0; c < L1; ++c) a[c] = a[c] + w[c];
+                if (psqt_ok) ps[p] = ps[p] + w[L1 + pi];
             }
-            wpsqt[b] = ps[0];
-            bpsqt[b] = ps[1];
-            const float u = us[b], t = them[b];
-            const float* aw = acc;
-            const float* ab = acc + L1;
-            float* sv = saved + (size_t)b * 4 * h;
-            float* o = l0 + (size_t)b * L1;
-            for (int i = 0; i < h; ++i) {
-                float xw0 = u * aw[i] + t * ab[i];
-                float xw1 = u * aw[i + h] + t * ab[i + h];
-                float xb0 = u * ab[i] + t * aw[i];
-                float xb1 = u * ab[i + h] + t * aw[i + h];
-                sv[0 * h + i] = xw0;
-                sv[1 * h + i] = xw1;
-                sv[2 * h + i] = xb0;
-                sv[3 * h + i] = xb1;
-                o[i] = clampf(xw0, 0.0f, max_act) * clampf(xw1, 0.0f, max_act);
-                o[h + i] = clampf(xb0, 0.0f, max_act) * clampf(xb1, 0.0f, max_act);
-            }
+            if (psqt_ok) ps[p] = ps[p] + bias[L1 + pi];
         }
-        free(acc);
+        wpsqt[b] = ps[0];
+        bpsqt[b] = ps[1];
+        const float u = us[b], t = them[b];
+        const float* sw = saved + (size_t)b * L1;
+        const float* sb = saved + ((size_t)B + b) * L1;
+        float* o = l0 + (size_t)b * L1;
+        for (int i = 0; i < h; ++i) {
+            float xw0, xw1, xb0, xb1;
+            mix4(u, t, sw, sb, bias, i, h, &xw0, &xw1, &xb0, &xb1);
+            o[i] = clampf(xw0, 0.0f, max_act) * clampf(xw1, 0.0f, max_act);
+            o[h + i] = clampf(xb0, 0.0f, max_act) * clampf(xb1, 0.0f, max_act);
+        }
     }
     return 0;
 }
@@ -188,7 +190,8 @@ int nnueft_oracle_double_fwd(const float* us, const float* them,
  * G[p, b, 0:L1] per the product/clamp/mix chain rule, G[p, b, L1+j] = grad_psqt_p[b] if j == psqt_idx[b] else 0.
  * Layout [2, B, out_cols].
  */
-int nnueft_oracle_double_bwd_rows(const float* us, const float* them, const int64_t* psqt_idx, float max_act,
+int nnueft_oracle_double_bwd_rows(const float* us, const float* them, const int64_t* psqt_idx,
+                                  const float* bias, float max_act,
                                   const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt,
                                   const float* saved, float* G, int B, int L1, int n_psqt)
 {
@@ -198,12 +201,14 @@ int nnueft_oracle_double_bwd_rows(const float* us, const float* them, const int6
 #pragma omp parallel for schedule(static)
     for (int b = 0; b < B; ++b) {
         const float u = us[b], t = them[b];
-        const float* sv = saved + (size_t)b * 4 * h;
+        const float* sw = saved + (size_t)b * L1;
+        const float* sb = saved + ((size_t)B + b) * L1;
         const float* g = grad_l0 + (size_t)b * L1;
         float* gw = G + (size_t)b * out_cols;
         float* gb = G + ((size_t)B + b) * out_cols;
         for (int i = 0; i < h; ++i) {
-            float xw0 = sv[i], xw1 = sv[h + i], xb0 = sv[2 * h + i], xb1 = sv[3 * h + i];
+            float xw0, xw1, xb0, xb1;
+            mix4(u, t, sw, sb, bias, i, h, &xw0, &xw1, &xb0, &xb1);
             float cw0 = clampf(xw0, 0.0f, max_act), cw1 = clampf(xw1, 0.0f, max_act);
             float cb0 = clampf(xb0, 0.0f, max_act), cb1 = clampf(xb1, 0.0f, max_act);
             float dw0 = (xw0 >= 0.0f && xw0 <= max_act) ? g[i] * cw1 : 0.0f;
@@ -227,7 +232,7 @@ int nnueft_oracle_double_bwd_rows(const float* us, const float* them, const int6
 /* gW = (white chains) + (black chains); gbias = tiled column sum of (G_w + G_b). */
 int nnueft_oracle_double_bwd(const float* us, const float* them,
                              const int32_t* widx, const int32_t* bidx, const int64_t* psqt_idx,
-                             float max_act,
+                             const float* bias, float max_act,
                              const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt,
                              const float* saved, float* gW, float* gbias,
                              int B, int K, int R, int L1, int n_psqt)
@@ -236,7 +241,7 @@ int nnueft_oracle_double_bwd(const float* us, const float* them,
     float* G = (float*)malloc(sizeof(float) * 2 * (size_t)B * out_cols);
     float* accb = (float*)calloc((size_t)R * out_cols, sizeof(float));
     if (!G || !accb) { free(G); free(accb); return -2; }
-    int rc = nnueft_oracle_double_bwd_rows(us, them, psqt_idx, max_act, grad_l0, grad_wpsqt, grad_bpsqt,
+    int rc = nnueft_oracle_double_bwd_rows(us, them, psqt_idx, bias, max_act, grad_l0, grad_wpsqt, grad_bpsqt,
                                            saved, G, B, L1, n_psqt);
     if (rc) { free(G); free(accb); return rc; }
     memset(gW, 0, (size_t)R * out_cols * sizeof(float));

@@ -150,7 +150,7 @@ def test_baseline_configs_full_size_against_oracle(oracle_cpu, L1, B):
              torch.randn(B, 1, generator=g).numpy()]
     max_act = 255.0 / 256.0
     r_l0, r_wp, r_bp, r_saved = oracle_cpu.double_fwd(us, them, white, black, psqt_idx, Wn, bn, max_act, L1)
-    r_gW, r_gb = oracle_cpu.double_bwd(us, them, white, black, psqt_idx, max_act, grads[0], grads[1], grads[2],
+    r_gW, r_gb = oracle_cpu.double_bwd(us, them, white, black, psqt_idx, bn, max_act, grads[0], grads[1], grads[2],
                                        r_saved, R, n_psqt)
     t = lambda a: torch.from_numpy(a).to(DEV)
     args = [t(us), t(them), t(white), t(black), t(psqt_idx)]
@@ -254,8 +254,8 @@ def test_non_default_stream(oracle_cpu):
     s.synchronize()
     r = oracle_cpu.double_fwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["W"], c["bias"], c["max_act"], 256)
     assert np.array_equal(out[0].detach().cpu().numpy(), r[0])
-    rW, rb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["max_act"], c["g_l0"],
-                                   c["g_wp"], c["g_bp"], r[3], 500, 8)
+    rW, rb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["bias"], c["max_act"],
+                                   c["g_l0"], c["g_wp"], c["g_bp"], r[3], 500, 8)
     assert np.array_equal(W.grad.cpu().numpy(), rW) and np.array_equal(bias.grad.cpu().numpy(), rb)
 
 
@@ -266,7 +266,8 @@ def test_abi_rejects_bad_arguments():
     st = torch.cuda.current_stream().cuda_stream
     assert lib.nnueft_sparse_fwd(p, p, p, p, 4, 0, 10, 8, st) == -1                 # K = 0
     assert lib.nnueft_sparse_fwd(0, p, p, p, 4, 8, 10, 8, st) == -1                 # null pointer
-    assert lib.nnueft_double_fwd(p, p, p, p, p, p, p, 1.0, p, p, p, p, 4, 8, 10, 7, 1, st) == -1    # odd L1
+    assert lib.nnueft_double_fwd(p, p, p, p, p, p, p, 1.0, p, p, p, p, 4, 8, 10, 7, 1, None, 0, st) == -1    # odd L1
+    assert lib.nnueft_double_fwd(p, p, p, p, p, p, p, 1.0, p, p, p, p, 4, 8, 10, 8, 0, p, 8, st) == -2       # workspace too small
     assert lib.nnueft_sparse_bwd_det(p, p, p, p, 4, 8, 10, 8, p, 16, st) == -2      # workspace too small
     assert lib.nnueft_sparse_bwd_det(p, p, p, p, 4, 8, 10, 8, 0, 1 << 20, st) == -2  # workspace missing
     assert lib.nnueft_sparse_bwd_det(p, p, p, p, 4, 8, 10, 8, p + 4, 1 << 20, st) == -2  # misaligned

@@ -110,25 +110,29 @@ DOUBLE_SHAPES = [
 ]
 
 
-def _run_double_fwd(c):
+def _run_double_fwd(c, with_workspace=True):
     nat, lib = _native()
     B, K, R, L1, n_psqt = c["widx"].shape[0], c["K"], c["R"], c["L1"], c["n_psqt"]
     d = {k: _t(c[k]) for k in ("us", "them", "widx", "bidx", "psqt_idx", "W", "bias")}
-    l0 = torch.empty(B, L1, device=_dev())
-    wp = torch.empty(B, 1, device=_dev())
-    bp = torch.empty(B, 1, device=_dev())
-    saved = torch.empty(B, 4, L1 // 2, device=_dev())
+    l0 = torch.full((B, L1), float("nan"), device=_dev())
+    wp = torch.full((B, 1), float("nan"), device=_dev())
+    bp = torch.full((B, 1), float("nan"), device=_dev())
+    saved = torch.full((2, B, L1), float("nan"), device=_dev())
+    nbytes = lib.nnueft_fwd_workspace_bytes(B, K, R, L1, n_psqt) if with_workspace else 0
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=_dev())
     nat.check(lib.nnueft_double_fwd(d["us"].data_ptr(), d["them"].data_ptr(), d["widx"].data_ptr(),
                                     d["bidx"].data_ptr(), d["psqt_idx"].data_ptr(), d["W"].data_ptr(),
                                     d["bias"].data_ptr(), c["max_act"], l0.data_ptr(), wp.data_ptr(), bp.data_ptr(),
-                                    saved.data_ptr(), B, K, R, L1, n_psqt, _stream()), "double_fwd")
+                                    saved.data_ptr(), B, K, R, L1, n_psqt,
+                                    ws.data_ptr() if with_workspace else None, nbytes, _stream()), "double_fwd")
     return d, l0, wp, bp, saved
 
 
+@pytest.mark.parametrize("with_workspace", [False, True], ids=["plain", "l2blocked"])
 @pytest.mark.parametrize("B,L1,R,K,kw", DOUBLE_SHAPES)
-def test_double_forward(oracle_cpu, B, L1, R, K, kw):
+def test_double_forward(oracle_cpu, B, L1, R, K, kw, with_workspace):
     c = double_case(400 + B, B, L1, R, K, **kw)
-    _, l0, wp, bp, saved = _run_double_fwd(c)
+    _, l0, wp, bp, saved = _run_double_fwd(c, with_workspace)
     r_l0, r_wp, r_bp, r_saved = oracle_cpu.double_fwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"],
                                                       c["W"], c["bias"], c["max_act"], L1)
     for got, ref in ((l0, r_l0), (wp, r_wp), (bp, r_bp), (saved, r_saved)):
@@ -147,8 +151,8 @@ def test_double_backward(oracle_cpu, B, L1, R, K, kw, mode):
     d, l0, wp, bp, saved = _run_double_fwd(c)
     g_l0, g_wp, g_bp = _t(c["g_l0"]), _t(c["g_wp"]), _t(c["g_bp"])
     head = (d["us"].data_ptr(), d["them"].data_ptr(), d["widx"].data_ptr(), d["bidx"].data_ptr(),
-            d["psqt_idx"].data_ptr(), c["max_act"], g_l0.data_ptr(), g_wp.data_ptr(), g_bp.data_ptr(),
-            saved.data_ptr())
+            d["psqt_idx"].data_ptr(), d["bias"].data_ptr(), c["max_act"], g_l0.data_ptr(), g_wp.data_ptr(),
+            g_bp.data_ptr(), saved.data_ptr())
     if mode == "atomic":
         gW = torch.zeros(R, out_cols, device=_dev())
         gb = torch.zeros(out_cols, device=_dev())
@@ -161,7 +165,7 @@ def test_double_backward(oracle_cpu, B, L1, R, K, kw, mode):
         gb = torch.full((out_cols,), float("nan"), device=_dev())
         nat.check(lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt, ws.data_ptr(),
                                             nbytes, _stream()), "double_bwd_det")
-    rW, rb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["max_act"],
+    rW, rb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["bias"], c["max_act"],
                                    c["g_l0"], c["g_wp"], c["g_bp"], saved.cpu().numpy(), R, n_psqt)
     gW, gb = gW.cpu().numpy(), gb.cpu().numpy()
     if mode == "atomic":
@@ -186,7 +190,8 @@ def test_deterministic_backward_repeats_bitwise():
         gW = torch.empty(R, L1 + n_psqt, device=_dev())
         gb = torch.empty(L1 + n_psqt, device=_dev())
         nat.check(lib.nnueft_double_bwd_det(d["us"].data_ptr(), d["them"].data_ptr(), d["widx"].data_ptr(),
-                                            d["bidx"].data_ptr(), d["psqt_idx"].data_ptr(), c["max_act"],
+                                            d["bidx"].data_ptr(), d["psqt_idx"].data_ptr(), d["bias"].data_ptr(),
+                                            c["max_act"],
                                             g_l0.data_ptr(), g_wp.data_ptr(), g_bp.data_ptr(), saved.data_ptr(),
                                             gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt, ws.data_ptr(), nbytes,
                                             _stream()), "double_bwd_det")

@@ -158,11 +158,10 @@ def test_double_forward_bits_equal_torch_cpu_path(oracle_cpu, B, L1, R, kw):
     assert np.array_equal(l0, t_l0.numpy())
     assert np.array_equal(wp, t_wp.numpy())
     assert np.array_equal(bp, t_bp.numpy())
-    # `saved` is the mix before the clamp: clamp and multiply it and l0 must come back
-    h = L1 // 2
-    cl = np.clip(saved, 0.0, np.float32(c["max_act"]))
-    assert np.array_equal(np.concatenate([cl[:, 0] * cl[:, 1], cl[:, 2] * cl[:, 3]], axis=1), l0)
-    assert saved.shape == (B, 4, h)
+    # `saved` holds the two perspectives' row sums before the bias
+    assert saved.shape == (2, B, L1)
+    assert np.array_equal(saved[0] + c["bias"][:L1], oracle_cpu.sparse_fwd(c["widx"], c["W"], c["bias"])[:, :L1])
+    assert np.array_equal(saved[1] + c["bias"][:L1], oracle_cpu.sparse_fwd(c["bidx"], c["W"], c["bias"])[:, :L1])
 
 
 @pytest.mark.parametrize("B,L1,R,kw", DOUBLE + DOUBLE_BIG)
@@ -173,7 +172,7 @@ def test_double_backward_weight_bits_equal_torch_cpu_autograd(oracle_cpu, B, L1,
                             [torch.from_numpy(c["g_l0"]), torch.from_numpy(c["g_wp"]), torch.from_numpy(c["g_bp"])])
     _, _, _, saved = oracle_cpu.double_fwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["W"],
                                            c["bias"], c["max_act"], L1)
-    gW, gb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["max_act"],
+    gW, gb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["bias"], c["max_act"],
                                    c["g_l0"], c["g_wp"], c["g_bp"], saved, R, c["n_psqt"])
     if B * c["K"] >= 32768:
         assert np.array_equal(gW, W.grad.numpy())
@@ -221,15 +220,18 @@ def test_clamp_gradient_passes_at_the_boundaries_like_torch(oracle_cpu):
     # x exactly 0 and exactly max: torch.clamp passes gradient (0 <= x <= max); the reference's
     # fused kernel would zero it (fused_ft_kernel.py:215-218).  The oracle follows torch.
     B, L1, n_psqt, max_act = 1, 4, 0, 1.0
-    saved = np.array([[[0.0, 1.0], [0.5, 0.5], [-0.1, 1.1], [0.5, 0.5]]], np.float32)
+    # with us = 1, them = 0 and a zero bias the mixed values are the row sums themselves:
+    # x_w = (0, 1 | .5, .5) sits on both clamp boundaries, x_b = (-.1, 1.1 | .5, .5) outside them
+    saved = np.array([[[0.0, 1.0, 0.5, 0.5]], [[-0.1, 1.1, 0.5, 0.5]]], np.float32)
     g = np.ones((B, L1), np.float32)
     one, zero = np.ones((B, 1), np.float32), np.zeros((B, 1), np.float32)
-    G = oracle_cpu.double_bwd_rows(one, zero, np.zeros(B, np.int64), max_act, g, zero, zero, saved, n_psqt)
+    G = oracle_cpu.double_bwd_rows(one, zero, np.zeros(B, np.int64), np.zeros(L1, np.float32), max_act, g, zero, zero,
+                                   saved, n_psqt)
     # white rows: d/dx_w0 = g*c_w1 where the mask holds: [0.5, 0.5] (both boundary values pass)
     assert np.array_equal(G[0, 0], np.array([0.5, 0.5, 0.0, 1.0], np.float32))
     # black rows: x_b0 = -0.1 and 1.1 are outside: no gradient; x_b1 inside: g*c_b0 = [0, 1]
     assert np.array_equal(G[1, 0], np.array([0.0, 0.0, 0.0, 1.0], np.float32))
-    x = torch.tensor(saved[0], requires_grad=True)
+    x = torch.tensor(saved[:, 0].reshape(4, 2), requires_grad=True)     # rows: x_w[:h], x_w[h:], x_b[:h], x_b[h:]
     cl = torch.clamp(x, 0.0, max_act)
     torch.cat([cl[0] * cl[1], cl[2] * cl[3]]).backward(torch.ones(4))
     assert np.array_equal(G[0, 0], torch.cat([x.grad[0], x.grad[1]]).numpy())
@@ -241,9 +243,9 @@ def test_double_backward_invariants(oracle_cpu):
     R, L1, n_psqt = 60, 32, 8
     _, _, _, saved = oracle_cpu.double_fwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["W"],
                                            c["bias"], c["max_act"], L1)
-    G = oracle_cpu.double_bwd_rows(c["us"], c["them"], c["psqt_idx"], c["max_act"], c["g_l0"], c["g_wp"], c["g_bp"],
-                                   saved, n_psqt)
-    gW, gb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["max_act"],
+    G = oracle_cpu.double_bwd_rows(c["us"], c["them"], c["psqt_idx"], c["bias"], c["max_act"], c["g_l0"], c["g_wp"],
+                                   c["g_bp"], saved, n_psqt)
+    gW, gb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["bias"], c["max_act"],
                                    c["g_l0"], c["g_wp"], c["g_bp"], saved, R, n_psqt)
     # column sums: sum_r gW[r] = sum_b n_w(b) G_w[b] + n_b(b) G_b[b]
     nw = (c["widx"] >= 0).sum(1).astype(np.float64)
@@ -328,7 +330,10 @@ def test_int16_forward_agrees_with_float_path_when_nothing_rounds(oracle_cpu):
     bf = np.concatenate([b16.astype(np.float32) / 256.0, np.zeros(8, np.float32)])
     us = (1 - stm).astype(np.float32)[:, None]
     l0, _, _, saved = oracle_cpu.double_fwd(us, 1 - us, widx, bidx, psqt_idx, Wf, bf, 255.0 / 256.0, L1)
-    cl = np.clip(saved.astype(np.float64), 0.0, 255.0 / 256.0) * 256.0
-    want = np.concatenate([np.floor(cl[:, 0] * cl[:, 1] / 512.0), np.floor(cl[:, 2] * cl[:, 3] / 512.0)], axis=1)
+    acc = saved.astype(np.float64) + bf[:L1]                      # [2, B, L1]: white, black accumulators
+    mover = np.where(us[None] == 1.0, acc, acc[::-1])               # side to move first
+    cl = np.clip(mover, 0.0, 255.0 / 256.0) * 256.0
+    want = np.concatenate([np.floor(cl[0, :, :h] * cl[0, :, h:] / 512.0),
+                           np.floor(cl[1, :, :h] * cl[1, :, h:] / 512.0)], axis=1)
     assert np.array_equal(out.astype(np.float64), want)
     assert out.max() <= 127
