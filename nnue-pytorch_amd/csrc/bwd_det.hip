@@ -20,9 +20,18 @@
 namespace {
 
 constexpr int kChunk = 128;        // positions per sort chunk
-constexpr int kRowsUnroll = 8;     // rows in flight per lane group in the segmented reduction
+#ifndef NNUEFT_SEG_U
+#define NNUEFT_SEG_U 8
+#endif
+#ifndef NNUEFT_SEG_NQ
+#define NNUEFT_SEG_NQ 3
+#endif
+#ifndef NNUEFT_SEG_WAVES
+#define NNUEFT_SEG_WAVES 512
+#endif
+constexpr int kRowsUnroll = NNUEFT_SEG_U;  // rows in flight per lane group in the segmented reduction
 constexpr int kXcd = 8;            // XCDs of the device; workgroup id % kXcd is the XCD a workgroup lands on
-constexpr int kWavesPerXcd = 512;  // persistent waves per XCD in the segmented reduction
+constexpr int kWavesPerXcd = NNUEFT_SEG_WAVES;  // persistent waves per XCD in the segmented reduction
 constexpr int kLongRow = 256;      // table rows named by at least this many slots are reduced first
 
 // Work split of the segmented reduction, written by k_row_scan (uint32 words).
@@ -235,6 +244,14 @@ __global__ __launch_bounds__(64) void k_col_scan(uint32_t* __restrict__ cnt, uin
     seg_off[r] = run;
 }
 
+// floor(kXcd * w / denom) for w < denom, without a 64-bit division
+__device__ __forceinline__ int xcd_of(unsigned long long w, unsigned long long denom) {
+    int x = 0;
+#pragma unroll
+    for (int k = 1; k < kXcd; ++k) x += (w * kXcd >= (unsigned long long)k * denom) ? 1 : 0;
+    return x;
+}
+
 // Single workgroup: seg_off (holding per-row totals) -> exclusive offsets, seg_off[R] = grand total.
 // Also the work split of the segmented reduction: the rows named by >= kLongRow slots (their chains
 // are long and start first), and kXcd contiguous row ranges of equal weight (slots + 1 per row).
@@ -306,8 +323,8 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
         for (int u = 0; u < 8; ++u) {
             const int r = rb + u * kScanThreads;
             if (r < R) {
-                const int x = (int)(((unsigned long long)off[u] + r) * kXcd / denom);
-                const int xp = r > 0 ? (int)(((unsigned long long)prev[u] + (r - 1)) * kXcd / denom) : -1;
+                const int x = xcd_of((unsigned long long)off[u] + r, denom);
+                const int xp = r > 0 ? xcd_of((unsigned long long)prev[u] + (r - 1), denom) : -1;
                 for (int k = xp + 1; k <= x; ++k) lo_s[k] = (uint32_t)r;
             }
         }
@@ -512,7 +529,7 @@ int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, fl
     const bool vec = (out_cols % 4 == 0) && aligned16(G) && aligned16(gW);
     const int VWr = vec ? 4 : 1;
     const int nv = out_cols / VWr;
-    const int NQ = nv > 64 ? 2 : 1;
+    const int NQ = nv > 64 ? NNUEFT_SEG_NQ : 1;
     const int nslices = (nv + 64 * NQ - 1) / (64 * NQ);
     // equal slices, rounded up to whole 128-byte lines so no two waves share a cache line of a row
     const int line_v = 128 / (VWr * (int)sizeof(float));
@@ -522,9 +539,9 @@ int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, fl
 #define SEG_LAUNCH(VW_, NQ_)                                                                                      \
     hipLaunchKernelGGL((k_seg_reduce<VW_, NQ_>), dim3(kXcd * kWavesPerXcd), dim3(64), 0, st, G, list, seg_off,      \
                        wcount, long_rows, sched, gW, out_cols, nslices, slice_v, two)
-    if (vec && NQ == 2) SEG_LAUNCH(4, 2);
+    if (vec && NQ > 1) SEG_LAUNCH(4, NNUEFT_SEG_NQ);
     else if (vec) SEG_LAUNCH(4, 1);
-    else if (NQ == 2) SEG_LAUNCH(1, 2);
+    else if (NQ > 1) SEG_LAUNCH(1, NNUEFT_SEG_NQ);
     else SEG_LAUNCH(1, 1);
 #undef SEG_LAUNCH
     NNUEFT_LAUNCH_CHECK();

@@ -15,9 +15,16 @@
 
 namespace nnueft_blocked {
 
+// Tunables of the blocked gather (vectors of 4 floats per lane and row; rows fetched per group).
+#ifndef NNUEFT_ACC_NQ
+#define NNUEFT_ACC_NQ 3
+#endif
+#ifndef NNUEFT_ACC_U
+#define NNUEFT_ACC_U 8
+#endif
+
 constexpr int kXcd = 8;
-constexpr int kOrderThreads = 1024;
-constexpr int kMaxBins = 2048;
+constexpr int kMaxBins = 512;   // table blocks the pair sort tells apart (17 x 512 x 4 bytes of LDS)
 
 __device__ __forceinline__ const int32_t* pair_list(const int32_t* __restrict__ widx,
                                                     const int32_t* __restrict__ bidx, int pair, int B, int K) {
@@ -36,67 +43,82 @@ __device__ __forceinline__ int pair_key(const int32_t* __restrict__ ix, int firs
     return nbins - 1;   // empty list
 }
 
-// order[] = pair ids (p * B + b) grouped by table block.  Single workgroup.
-__global__ __launch_bounds__(kOrderThreads) void k_pair_order(const int32_t* __restrict__ widx,
-                                                              const int32_t* __restrict__ bidx,
-                                                              uint32_t* __restrict__ order, int B, int K, int R,
-                                                              int block_rows, int nbins) {
+// Pair sort, three small launches.  order[] = pair ids (p * B + b) grouped by table block; the
+// order inside a block is arbitrary (it only schedules work).
+//   k_pair_hist     one pair per thread: key to keys[], per-workgroup histogram to hist[bin][wg]
+//   k_pair_scan     exclusive scan of hist (flat, bin-major) in place -> first slot of every (bin, wg)
+//   k_pair_scatter  pairs to their slots through LDS cursors
+constexpr int kPairThreads = 256;
+
+__global__ __launch_bounds__(kPairThreads) void k_pair_hist(const int32_t* __restrict__ widx,
+                                                            const int32_t* __restrict__ bidx,
+                                                            uint32_t* __restrict__ keys,
+                                                            uint32_t* __restrict__ hist, int B, int K, int R,
+                                                            int block_rows, int nbins) {
     __shared__ uint32_t bins[kMaxBins];
-    __shared__ uint32_t wave_tot[kOrderThreads / 64];
     const int tid = threadIdx.x;
-    const int npairs = 2 * B;
-    for (int i = tid; i < nbins; i += kOrderThreads) bins[i] = 0;
+    const int n = blockIdx.x * kPairThreads + tid;
+    for (int i = tid; i < nbins; i += kPairThreads) bins[i] = 0;
     __syncthreads();
-    constexpr int PF = 8;
-    for (int n0 = tid; n0 < npairs; n0 += kOrderThreads * PF) {
-        int first[PF];
-#pragma unroll
-        for (int u = 0; u < PF; ++u) {
-            const int n = n0 + u * kOrderThreads;
-            first[u] = n < npairs ? pair_list(widx, bidx, n, B, K)[0] : -1;
-        }
-#pragma unroll
-        for (int u = 0; u < PF; ++u) {
-            const int n = n0 + u * kOrderThreads;
-            if (n < npairs)
-                atomicAdd(&bins[pair_key(pair_list(widx, bidx, n, B, K), first[u], K, R, block_rows, nbins)], 1u);
-        }
+    if (n < 2 * B) {
+        const int32_t* ix = pair_list(widx, bidx, n, B, K);
+        const int key = pair_key(ix, ix[0], K, R, block_rows, nbins);
+        keys[n] = (uint32_t)key;
+        atomicAdd(&bins[key], 1u);
     }
     __syncthreads();
-    // exclusive scan of bins (nbins <= kMaxBins = 2 * kOrderThreads): two entries per thread
-    const uint32_t a = (2 * tid < nbins) ? bins[2 * tid] : 0;
-    const uint32_t c = (2 * tid + 1 < nbins) ? bins[2 * tid + 1] : 0;
-    uint32_t incl = a + c;
+    for (int i = tid; i < nbins; i += kPairThreads) hist[(size_t)i * gridDim.x + blockIdx.x] = bins[i];
+}
+
+// In-place exclusive scan of data[0..n) by one workgroup of 1024 threads.
+__global__ __launch_bounds__(1024) void k_pair_scan(uint32_t* __restrict__ data, int n) {
+    __shared__ uint32_t wave_tot[16];
+    __shared__ uint32_t carry_s;
+    const int tid = threadIdx.x;
+    constexpr int PER = 8;
+    if (tid == 0) carry_s = 0;
+    __syncthreads();
+    for (int base = 0; base < n; base += 1024 * PER) {
+        const int i0 = base + tid * PER;
+        uint32_t v[PER];
+        uint32_t local = 0;
 #pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const uint32_t v = __shfl_up(incl, off);
-        if ((tid & 63) >= off) incl += v;
-    }
-    if ((tid & 63) == 63) wave_tot[tid >> 6] = incl;
-    __syncthreads();
-    uint32_t base = 0;
-    for (int w = 0; w < (tid >> 6); ++w) base += wave_tot[w];
-    const uint32_t excl = base + incl - (a + c);
-    __syncthreads();
-    if (2 * tid < nbins) bins[2 * tid] = excl;
-    if (2 * tid + 1 < nbins) bins[2 * tid + 1] = excl + a;
-    __syncthreads();
-    for (int n0 = tid; n0 < npairs; n0 += kOrderThreads * PF) {
-        int first[PF];
-#pragma unroll
-        for (int u = 0; u < PF; ++u) {
-            const int n = n0 + u * kOrderThreads;
-            first[u] = n < npairs ? pair_list(widx, bidx, n, B, K)[0] : -1;
+        for (int u = 0; u < PER; ++u) {
+            v[u] = (i0 + u < n) ? data[i0 + u] : 0;
+            local += v[u];
         }
+        uint32_t incl = local;
 #pragma unroll
-        for (int u = 0; u < PF; ++u) {
-            const int n = n0 + u * kOrderThreads;
-            if (n < npairs) {
-                const int key = pair_key(pair_list(widx, bidx, n, B, K), first[u], K, R, block_rows, nbins);
-                order[atomicAdd(&bins[key], 1u)] = (uint32_t)n;
-            }
+        for (int off = 1; off < 64; off <<= 1) {
+            const uint32_t t = __shfl_up(incl, off);
+            if ((tid & 63) >= off) incl += t;
         }
+        if ((tid & 63) == 63) wave_tot[tid >> 6] = incl;
+        __syncthreads();
+        uint32_t run = carry_s;
+        for (int w = 0; w < (tid >> 6); ++w) run += wave_tot[w];
+        run += incl - local;
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            if (i0 + u < n) data[i0 + u] = run;
+            run += v[u];
+        }
+        __syncthreads();
+        if (tid == 1023) carry_s = run;
+        __syncthreads();
     }
+}
+
+__global__ __launch_bounds__(kPairThreads) void k_pair_scatter(const uint32_t* __restrict__ keys,
+                                                               const uint32_t* __restrict__ hist,
+                                                               uint32_t* __restrict__ order, int npairs,
+                                                               int nbins) {
+    __shared__ uint32_t cursor[kMaxBins];
+    const int tid = threadIdx.x;
+    const int n = blockIdx.x * kPairThreads + tid;
+    for (int i = tid; i < nbins; i += kPairThreads) cursor[i] = hist[(size_t)i * gridDim.x + blockIdx.x];
+    __syncthreads();
+    if (n < npairs) order[atomicAdd(&cursor[keys[n]], 1u)] = (uint32_t)n;
 }
 
 // saved[pair, slice] = chain from +0 over the pair's list (pair = perspective * B + position).
@@ -202,7 +224,32 @@ __global__ __launch_bounds__(64) void k_mix(const float* __restrict__ us, const 
 
 static inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-size_t fwd_workspace(int B) { return B > 0 ? up256((size_t)2 * B * sizeof(uint32_t)) : 0; }
+int table_block_rows(int R, int* nbins);
+
+struct FwdLayout {
+    size_t order, keys, hist, end;
+    int ngroups, nbins, block_rows;
+};
+
+bool fwd_layout(int B, int R, FwdLayout* L) {
+    if (B <= 0 || R <= 0) return false;
+    L->block_rows = table_block_rows(R, &L->nbins);
+    L->ngroups = (2 * B + kPairThreads - 1) / kPairThreads;
+    size_t off = 0;
+    L->order = off;
+    off += up256((size_t)2 * B * sizeof(uint32_t));
+    L->keys = off;
+    off += up256((size_t)2 * B * sizeof(uint32_t));
+    L->hist = off;
+    off += up256((size_t)L->ngroups * L->nbins * sizeof(uint32_t));
+    L->end = off;
+    return true;
+}
+
+size_t fwd_workspace(int B, int R) {
+    FwdLayout L;
+    return fwd_layout(B, R, &L) ? L.end : 0;
+}
 
 int table_block_rows(int R, int* nbins) {
     int block_rows = 768;
@@ -215,22 +262,30 @@ int double_fwd_blocked(const float* us, const float* them, const int32_t* widx, 
                        const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,
                        float* wpsqt, float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt,
                        void* ws, hipStream_t st) {
-    uint32_t* order = (uint32_t*)ws;
-    int nbins = 0;
-    const int block_rows = table_block_rows(R, &nbins);
-    hipLaunchKernelGGL(k_pair_order, dim3(1), dim3(kOrderThreads), 0, st, widx, bidx, order, B, K, R, block_rows,
-                       nbins);
+    FwdLayout L;
+    if (!fwd_layout(B, R, &L)) return NNUEFT_E_ARG;
+    char* base = (char*)ws;
+    uint32_t* order = (uint32_t*)(base + L.order);
+    uint32_t* keys = (uint32_t*)(base + L.keys);
+    uint32_t* hist = (uint32_t*)(base + L.hist);
+    hipLaunchKernelGGL(k_pair_hist, dim3(L.ngroups), dim3(kPairThreads), 0, st, widx, bidx, keys, hist, B, K, R,
+                       L.block_rows, L.nbins);
+    NNUEFT_LAUNCH_CHECK();
+    hipLaunchKernelGGL(k_pair_scan, dim3(1), dim3(1024), 0, st, hist, L.ngroups * L.nbins);
+    NNUEFT_LAUNCH_CHECK();
+    hipLaunchKernelGGL(k_pair_scatter, dim3(L.ngroups), dim3(kPairThreads), 0, st, keys, hist, order, 2 * B,
+                       L.nbins);
     NNUEFT_LAUNCH_CHECK();
     const int out_cols = L1 + n_psqt;
     const int nv = L1 / 4;
     const int per_xcd = (2 * B + kXcd - 1) / kXcd;
     if (nv > 64) {
-        constexpr int NQ = 2;
+        constexpr int NQ = NNUEFT_ACC_NQ;
         const int nslices = (nv + 64 * NQ - 1) / (64 * NQ);
         const long long grid = (long long)kXcd * per_xcd * nslices;
         if (grid > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
-        hipLaunchKernelGGL((k_acc_blocked<4, NQ, 8>), dim3((unsigned)grid), dim3(64), 0, st, widx, bidx, order, W,
-                           saved, B, K, R, L1, out_cols, per_xcd);
+        hipLaunchKernelGGL((k_acc_blocked<4, NQ, NNUEFT_ACC_U>), dim3((unsigned)grid), dim3(64), 0, st, widx, bidx,
+                           order, W, saved, B, K, R, L1, out_cols, per_xcd);
     } else {
         const long long grid = (long long)kXcd * per_xcd;
         if (grid > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;

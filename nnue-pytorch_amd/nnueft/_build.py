@@ -32,19 +32,21 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found: libnnueft.so cannot be built")
 
 
-def build(verbose: bool = False) -> str:
-    """Compile every kernel source and link the C-ABI library.  Always recompiles."""
+def build(verbose: bool = False, extra_flags=(), lib_path: str = LIB_PATH) -> str:
+    """Compile every kernel source and link the C-ABI library.  Always recompiles.
+
+    extra_flags / lib_path build a variant (e.g. -DNNUEFT_SEG_U=16) next to the default library."""
     hipcc = hipcc_path()
     srcs = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
     if not srcs:
         raise RuntimeError(f"no kernel sources under {CSRC}")
     objs = []
     procs = []
-    objdir = os.path.join(CSRC, "build")
+    objdir = os.path.join(CSRC, "build", os.path.basename(lib_path).replace(".so", ""))
     os.makedirs(objdir, exist_ok=True)
     for src in srcs:
         obj = os.path.join(objdir, os.path.basename(src)[:-4] + ".o")
-        cmd = [hipcc, *HIPCC_FLAGS, "-I", INCLUDE, "-I", CSRC, "-c", src, "-o", obj]
+        cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, "-I", INCLUDE, "-I", CSRC, "-c", src, "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
@@ -56,13 +58,13 @@ def build(verbose: bool = False) -> str:
             raise RuntimeError(f"hipcc failed on {src}:\n{out}")
         if verbose and out.strip():
             print(out, flush=True)
-    tmp = LIB_PATH + ".tmp"
+    tmp = lib_path + ".tmp"
     cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp]
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stdout}")
-    os.replace(tmp, LIB_PATH)
-    return LIB_PATH
+    os.replace(tmp, lib_path)
+    return lib_path
 
 
 if __name__ == "__main__":

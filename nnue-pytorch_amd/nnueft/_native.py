@@ -9,7 +9,8 @@ import os
 from ctypes import c_float, c_int, c_size_t, c_void_p
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG, "libnnueft.so")
+# NNUEFT_LIBRARY points at another build of the same library (kernel tuning)
+LIB_PATH = os.environ.get("NNUEFT_LIBRARY") or os.path.join(_PKG, "libnnueft.so")
 
 # name -> (restype, argtypes); mirrors include/nnueft.h one to one
 PROTOTYPES = {
