@@ -32,7 +32,10 @@ constexpr int kChunk = 128;        // positions per sort chunk
 constexpr int kRowsUnroll = NNUEFT_SEG_U;  // rows in flight per lane group in the segmented reduction
 constexpr int kXcd = 8;            // XCDs of the device; workgroup id % kXcd is the XCD a workgroup lands on
 constexpr int kWavesPerXcd = NNUEFT_SEG_WAVES;  // persistent waves per XCD in the segmented reduction
-constexpr int kLongRow = 256;      // table rows named by at least this many slots are reduced first
+#ifndef NNUEFT_LONG_ROW
+#define NNUEFT_LONG_ROW 256
+#endif
+constexpr int kLongRow = NNUEFT_LONG_ROW;  // table rows named by at least this many slots are reduced first
 
 // Work split of the segmented reduction, written by k_row_scan (uint32 words).
 constexpr int kSchedCtr = 0;       // kXcd task counters, 32 words (128 bytes) apart
@@ -419,7 +422,7 @@ __device__ __forceinline__ void seg_reduce_task(const float* __restrict__ G, con
     for (int m = 0; m < NQ; ++m) {
         if (!act[m]) continue;
         if (two_persp) vadd<VW>(acc[0][m], acc[1][m]);
-        stv<VW>(dst + col[m], acc[0][m]);
+        stv_stream<VW>(dst + col[m], acc[0][m]);
     }
 }
 

@@ -45,6 +45,29 @@ __device__ __forceinline__ void stv<1>(float* p, const vecf<1>& x) {
     *p = x.v[0];
 }
 
+// Streaming store: the line is marked for early eviction, so write-once outputs do not push the
+// rows being gathered out of L2.
+template <int VW>
+__device__ __forceinline__ void stv_stream(float* p, const vecf<VW>& x);
+template <>
+__device__ __forceinline__ void stv_stream<4>(float* p, const vecf<4>& x) {
+#ifdef NNUEFT_NO_NT
+    stv<4>(p, x);
+#else
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    f4 v = {x.v[0], x.v[1], x.v[2], x.v[3]};
+    __builtin_nontemporal_store(v, reinterpret_cast<f4*>(p));
+#endif
+}
+template <>
+__device__ __forceinline__ void stv_stream<1>(float* p, const vecf<1>& x) {
+#ifdef NNUEFT_NO_NT
+    *p = x.v[0];
+#else
+    __builtin_nontemporal_store(x.v[0], p);
+#endif
+}
+
 template <int VW>
 __device__ __forceinline__ vecf<VW> vzero() {
     vecf<VW> r;

@@ -159,7 +159,7 @@ __global__ __launch_bounds__(64) void k_acc_blocked(const int32_t* __restrict__ 
     float* dst = acc + (size_t)pair * L1;
 #pragma unroll
     for (int m = 0; m < NQ; ++m)
-        if (act[m]) stv<VW>(dst + col[m], a[m]);
+        if (act[m]) stv_stream<VW>(dst + col[m], a[m]);
 }
 
 // Per position: bias, mix, clamp, product; slice 0 also does the two psqt chains.
