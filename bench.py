@@ -28,9 +28,10 @@ MEASURED_FWD_TRAFFIC = {"ft_fwd_bwd_L1_3072_B16384": 8.00e9}
 
 WORKLOADS = {
     # name: (L1, B)
-    "ft_fwd_bwd_L1_3072_B16384": (3072, 16384),
-    "ft_fwd_bwd_L1_1024_B8192": (1024, 8192),
-    "ft_fwd_bwd_L1_128_B16384": (128, 16384),
+    "ft_fwd_bwd_L1_3072_B16384": (3072, 16384),     # BASELINE.json config 3: the metric
+    "ft_fwd_bwd_L1_1024_B8192": (1024, 8192),       # config 1
+    "ft_fwd_bwd_L1_128_B16384": (128, 16384),       # config 2
+    "ft_int16_fwd_L1_3072_B65536": (3072, 65536),   # config 5: quantized forward only
 }
 R_ROWS = 24576
 N_PSQT = 8
@@ -112,6 +113,54 @@ def cpu_baseline(L1, B_full, seed, budget_s=20.0):
     }
 
 
+def run_int16(args, lib, dev):
+    """Quantized forward (BASELINE.json config 5): int16 gather-accumulate, clip, product >> 9 -> u8."""
+    import numpy as np
+    import torch
+    from nnueft import halfka_v2_hm as hk
+    from nnueft import quantized
+
+    L1, B = WORKLOADS[args.workload]
+    R = hk.NUM_INPUTS_EXPORT
+    us, them, white, black, pc = hk.synthetic_batch(B, 1239, fold_kings=True)
+    g = torch.Generator().manual_seed(5)
+    W = torch.randn(R, L1 + N_PSQT, generator=g) * 0.02
+    bias = torch.randn(L1 + N_PSQT, generator=g) * 0.1
+    w16, b16, p32 = quantized.quantize_feature_transformer(W, bias, L1)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    stm = t((1 - us[:, 0]).astype(np.uint8))
+    wi, bi, pi = t(white), t(black), t((pc - 1) // 4)
+    w16, b16, p32 = w16.to(dev), b16.to(dev), p32.to(dev)
+    sum_a = int((white >= 0).sum() + (black >= 0).sum())
+
+    def step():
+        quantized.ft_int16_forward(wi, bi, stm, w16, b16, p32, pi)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / args.steps
+    alg = sum_a * L1 * 2 + B * (2 * K_SLOTS * 4 + L1)
+    print(json.dumps({
+        "metric": "quantized FT forward positions/sec (int16 accumulate, L1=3072, B=65536)",
+        "value": B / (ms * 1e-3), "unit": "positions/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int16",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "L1": L1, "batch": B, "table_rows": R,
+                   "active_rows_per_position": sum_a / B},
+        "roofline": {"kernel": "nnueft_ft_int16_fwd", "bound": "hbm", "achieved": alg / (ms * 1e-3) / 1e9,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": None, "algorithmic_bytes_per_launch": alg, "avg_launch_ms": ms},
+        "cpu_baseline": None,
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -139,6 +188,9 @@ def main():
         sys.exit(2)
     lib = _native.load()  # raises if libnnueft.so is missing: there is no fallback
     dev = torch.device("cuda:0")
+    if args.workload.startswith("ft_int16"):
+        run_int16(args, lib, dev)
+        return
     if args.only == "copy":
         n = (1 << 30) // 4
         src = torch.ones(n, device=dev)

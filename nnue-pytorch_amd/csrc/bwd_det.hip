@@ -16,6 +16,7 @@
 //                   (those of the positions of one king bucket, one slice wide) stay in its L2
 //   k_bias_final    chain over the tile partial sums
 #include "gather.h"
+#include "internal.h"
 
 namespace {
 
@@ -30,7 +31,7 @@ constexpr int kChunk = 128;        // positions per sort chunk
 #define NNUEFT_SEG_WAVES 512
 #endif
 constexpr int kRowsUnroll = NNUEFT_SEG_U;  // rows in flight per lane group in the segmented reduction
-constexpr int kXcd = 8;            // XCDs of the device; workgroup id % kXcd is the XCD a workgroup lands on
+using nnueft_blocked::kXcd;
 constexpr int kWavesPerXcd = NNUEFT_SEG_WAVES;  // persistent waves per XCD in the segmented reduction
 #ifndef NNUEFT_LONG_ROW
 #define NNUEFT_LONG_ROW 256
@@ -549,13 +550,40 @@ int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, fl
 #undef SEG_LAUNCH
     NNUEFT_LAUNCH_CHECK();
 
-    hipLaunchKernelGGL(k_bias_final, dim3((out_cols + 63) / 64), dim3(64), 0, st, partial, gbias, L.ntiles,
-                       out_cols);
+    return nnueft_det::launch_bias_final(partial, gbias, B, out_cols, st);
+}
+
+}  // namespace
+
+namespace nnueft_det {
+
+int launch_bwd_rows(const float* us, const float* them, const int64_t* psqt_idx, const float* bias, float max_act,
+                    const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt, const float* saved,
+                    float* G, float* partial, int B, int L1, int n_psqt, hipStream_t st) {
+    const int out_cols = L1 + n_psqt;
+    const int ntiles = (B + NNUEFT_BIAS_TILE - 1) / NNUEFT_BIAS_TILE;
+    const bool vec = (L1 % 8 == 0) && (out_cols % 4 == 0) && aligned16(grad_l0) && aligned16(saved) &&
+                     aligned16(bias) && aligned16(G) && aligned16(partial);
+    const int hv = (L1 / 2) / (vec ? 4 : 1);
+    const dim3 grid(ntiles, max(1, (hv + 63) / 64));
+    if (vec)
+        hipLaunchKernelGGL(k_bwd_rows<4>, grid, dim3(64), 0, st, us, them, psqt_idx, bias, max_act, grad_l0,
+                           grad_wpsqt, grad_bpsqt, saved, G, partial, B, L1, n_psqt);
+    else
+        hipLaunchKernelGGL(k_bwd_rows<1>, grid, dim3(64), 0, st, us, them, psqt_idx, bias, max_act, grad_l0,
+                           grad_wpsqt, grad_bpsqt, saved, G, partial, B, L1, n_psqt);
     NNUEFT_LAUNCH_CHECK();
     return 0;
 }
 
-}  // namespace
+int launch_bias_final(const float* partial, float* gbias, int B, int out_cols, hipStream_t st) {
+    const int ntiles = (B + NNUEFT_BIAS_TILE - 1) / NNUEFT_BIAS_TILE;
+    hipLaunchKernelGGL(k_bias_final, dim3((out_cols + 63) / 64), dim3(64), 0, st, partial, gbias, ntiles, out_cols);
+    NNUEFT_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // namespace nnueft_det
 
 extern "C" size_t nnueft_det_workspace_bytes(int B, int K, int R, int out_cols, int n_persp) {
     DetLayout L;
@@ -597,15 +625,8 @@ extern "C" int nnueft_double_bwd_det(const float* us, const float* them, const i
     hipStream_t st = (hipStream_t)stream;
     char* ws = (char*)workspace;
     float* G = (float*)(ws + L.G);
-    const bool vec = (L1 % 8 == 0) && (out_cols % 4 == 0) && aligned16(grad_l0) && aligned16(saved) && aligned16(bias);
-    const int hv = (L1 / 2) / (vec ? 4 : 1);
-    const dim3 grid(L.ntiles, max(1, (hv + 63) / 64));
-    if (vec)
-        hipLaunchKernelGGL(k_bwd_rows<4>, grid, dim3(64), 0, st, us, them, psqt_idx, bias, max_act, grad_l0, grad_wpsqt,
-                           grad_bpsqt, saved, G, (float*)(ws + L.partial), B, L1, n_psqt);
-    else
-        hipLaunchKernelGGL(k_bwd_rows<1>, grid, dim3(64), 0, st, us, them, psqt_idx, bias, max_act, grad_l0, grad_wpsqt,
-                           grad_bpsqt, saved, G, (float*)(ws + L.partial), B, L1, n_psqt);
-    NNUEFT_LAUNCH_CHECK();
+    const int rc = nnueft_det::launch_bwd_rows(us, them, psqt_idx, bias, max_act, grad_l0, grad_wpsqt, grad_bpsqt,
+                                               saved, G, (float*)(ws + L.partial), B, L1, n_psqt, st);
+    if (rc) return rc;
     return det_sort_reduce(widx, bidx, G, gW, gbias, B, K, R, out_cols, 2, ws, L, st);
 }

@@ -12,6 +12,7 @@
 //
 // Workgroups are handed to the 8 XCDs round-robin by workgroup id, so id % 8 selects the XCD.
 #include "gather.h"
+#include "internal.h"
 
 namespace nnueft_blocked {
 
@@ -23,7 +24,6 @@ namespace nnueft_blocked {
 #define NNUEFT_ACC_U 8
 #endif
 
-constexpr int kXcd = 8;
 constexpr int kMaxBins = 512;   // table blocks the pair sort tells apart (17 x 512 x 4 bytes of LDS)
 
 __device__ __forceinline__ const int32_t* pair_list(const int32_t* __restrict__ widx,
@@ -226,12 +226,12 @@ static inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 int table_block_rows(int R, int* nbins);
 
-struct FwdLayout {
+struct PairSortLayout {
     size_t order, keys, hist, end;
     int ngroups, nbins, block_rows;
 };
 
-bool fwd_layout(int B, int R, FwdLayout* L) {
+bool pair_sort_layout(int B, int R, PairSortLayout* L) {
     if (B <= 0 || R <= 0) return false;
     L->block_rows = table_block_rows(R, &L->nbins);
     L->ngroups = (2 * B + kPairThreads - 1) / kPairThreads;
@@ -246,9 +246,29 @@ bool fwd_layout(int B, int R, FwdLayout* L) {
     return true;
 }
 
-size_t fwd_workspace(int B, int R) {
-    FwdLayout L;
-    return fwd_layout(B, R, &L) ? L.end : 0;
+size_t pair_sort_workspace(int B, int R) {
+    PairSortLayout L;
+    return pair_sort_layout(B, R, &L) ? L.end : 0;
+}
+
+int launch_pair_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, void* ws, hipStream_t st,
+                     const uint32_t** order_out) {
+    PairSortLayout L;
+    if (!pair_sort_layout(B, R, &L)) return NNUEFT_E_ARG;
+    char* base = (char*)ws;
+    uint32_t* order = (uint32_t*)(base + L.order);
+    uint32_t* keys = (uint32_t*)(base + L.keys);
+    uint32_t* hist = (uint32_t*)(base + L.hist);
+    hipLaunchKernelGGL(k_pair_hist, dim3(L.ngroups), dim3(kPairThreads), 0, st, widx, bidx, keys, hist, B, K, R,
+                       L.block_rows, L.nbins);
+    NNUEFT_LAUNCH_CHECK();
+    hipLaunchKernelGGL(k_pair_scan, dim3(1), dim3(1024), 0, st, hist, L.ngroups * L.nbins);
+    NNUEFT_LAUNCH_CHECK();
+    hipLaunchKernelGGL(k_pair_scatter, dim3(L.ngroups), dim3(kPairThreads), 0, st, keys, hist, order, 2 * B,
+                       L.nbins);
+    NNUEFT_LAUNCH_CHECK();
+    *order_out = order;
+    return 0;
 }
 
 int table_block_rows(int R, int* nbins) {
@@ -262,20 +282,9 @@ int double_fwd_blocked(const float* us, const float* them, const int32_t* widx, 
                        const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,
                        float* wpsqt, float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt,
                        void* ws, hipStream_t st) {
-    FwdLayout L;
-    if (!fwd_layout(B, R, &L)) return NNUEFT_E_ARG;
-    char* base = (char*)ws;
-    uint32_t* order = (uint32_t*)(base + L.order);
-    uint32_t* keys = (uint32_t*)(base + L.keys);
-    uint32_t* hist = (uint32_t*)(base + L.hist);
-    hipLaunchKernelGGL(k_pair_hist, dim3(L.ngroups), dim3(kPairThreads), 0, st, widx, bidx, keys, hist, B, K, R,
-                       L.block_rows, L.nbins);
-    NNUEFT_LAUNCH_CHECK();
-    hipLaunchKernelGGL(k_pair_scan, dim3(1), dim3(1024), 0, st, hist, L.ngroups * L.nbins);
-    NNUEFT_LAUNCH_CHECK();
-    hipLaunchKernelGGL(k_pair_scatter, dim3(L.ngroups), dim3(kPairThreads), 0, st, keys, hist, order, 2 * B,
-                       L.nbins);
-    NNUEFT_LAUNCH_CHECK();
+    const uint32_t* order = nullptr;
+    const int rc = launch_pair_sort(widx, bidx, B, K, R, ws, st, &order);
+    if (rc) return rc;
     const int out_cols = L1 + n_psqt;
     const int nv = L1 / 4;
     const int per_xcd = (2 * B + kXcd - 1) / kXcd;

@@ -1,0 +1,33 @@
+// Functions shared between the translation units of libnnueft (not part of the ABI).
+#pragma once
+
+#include "common.h"
+
+namespace nnueft_blocked {
+
+constexpr int kXcd = 8;   // XCDs of the device; workgroup id % kXcd is the XCD a workgroup lands on
+
+// Pair sort: order[] = ids (perspective * B + position) of the 2B index lists of a batch grouped by
+// the 768-row table block they name.  `ws` needs pair_sort_workspace() bytes; returns the order array
+// (inside ws) through *order.
+size_t pair_sort_workspace(int B, int R);
+int launch_pair_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, void* ws, hipStream_t st,
+                     const uint32_t** order);
+
+int double_fwd_blocked(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+                       const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,
+                       float* wpsqt, float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt, void* ws,
+                       hipStream_t st);
+
+}  // namespace nnueft_blocked
+
+namespace nnueft_det {
+
+// Upstream rows G[2, B, L1 + n_psqt] of the two sparse-linear outputs and the bias partial sums
+// partial[ceil(B / NNUEFT_BIAS_TILE), L1 + n_psqt]; then the chain over the partial sums.
+int launch_bwd_rows(const float* us, const float* them, const int64_t* psqt_idx, const float* bias, float max_act,
+                    const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt, const float* saved,
+                    float* G, float* partial, int B, int L1, int n_psqt, hipStream_t st);
+int launch_bias_final(const float* partial, float* gbias, int B, int out_cols, hipStream_t st);
+
+}  // namespace nnueft_det
