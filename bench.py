@@ -32,6 +32,7 @@ WORKLOADS = {
     "ft_fwd_bwd_L1_1024_B8192": (1024, 8192),       # config 1
     "ft_fwd_bwd_L1_128_B16384": (128, 16384),       # config 2
     "ft_int16_fwd_L1_3072_B65536": (3072, 65536),   # config 5: quantized forward only
+    "full_step_L1_3072_B16384": (3072, 16384),      # config 4: FT + layer stacks + loss + optimizer
 }
 R_ROWS = 24576
 N_PSQT = 8
@@ -161,6 +162,53 @@ def run_int16(args, lib, dev):
     }))
 
 
+def run_full_step(args, dev):
+    """BASELINE.json config 4: the L1=3072 model (FT, pairwise clipped ReLU, 8 bucketed layer stacks),
+    WDL-blended sigmoid loss, optimizer step.  The optimizer is torch's fused Adam: the reference's
+    RangerLite is not part of this build."""
+    import torch
+    import nnueft
+    from nnueft import halfka_v2_hm as hk
+    from nnueft import model as M
+
+    L1, B = WORKLOADS[args.workload]
+    nnueft.set_backward_mode(args.backward)
+    torch.manual_seed(0)
+    model = M.NNUEModel("HalfKAv2_hm^", M.ModelConfig(L1=L1, L2=32, L3=32)).to(dev)
+    us, them, white, black, pc = [torch.from_numpy(a).to(dev) for a in hk.synthetic_batch(B, 1238)]
+    g = torch.Generator().manual_seed(1238)
+    score = (torch.randn(B, 1, generator=g) * 400).clamp(-3000, 3000).to(dev)
+    outcome = (torch.randint(0, 3, (B, 1), generator=g).float() / 2).to(dev)
+    opt = torch.optim.Adam(model.parameters(), lr=8.75e-4, fused=True)
+    params = M.LossParams()
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        out = model(us, them, white, black, pc)
+        loss = M.sf_loss(out * model.quantization.nnue2score, score, outcome, params, 0.75)
+        loss.backward()
+        opt.step()
+        return loss
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    print(json.dumps({
+        "metric": "full model training step positions/sec (L1=3072, B=16384)", "value": B / (ms * 1e-3),
+        "unit": "positions/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": args.workload, "L1": L1, "L2": 32, "L3": 32, "batch": B, "backward": args.backward,
+                   "optimizer": "torch.optim.Adam(fused=True)", "lambda": 0.75, "fake_quantization": True,
+                   "final_loss": float(loss)},
+        "roofline": None, "cpu_baseline": None,
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -190,6 +238,9 @@ def main():
     dev = torch.device("cuda:0")
     if args.workload.startswith("ft_int16"):
         run_int16(args, lib, dev)
+        return
+    if args.workload.startswith("full_step"):
+        run_full_step(args, dev)
         return
     if args.only == "copy":
         n = (1 << 30) // 4

@@ -140,6 +140,27 @@ int nnueft_double_bwd_det(const float* us, const float* them, const int32_t* wid
                           void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * merged[r, c] = q(W[r, c] + V[r % vrows, c]): the table the gather reads, from the real weights
+ * W f32[R, cols] and the virtual (factorised) weights V f32[vrows, cols] shared by all table blocks
+ * (V may be NULL).  With fake_quantize != 0, q(x) = round(x * s) / s (round half to even) with
+ * s = scale_ft for the first L1 columns and scale_psqt for the rest; otherwise q is the identity.
+ * One pass in place of HalfKav2Hm.merged_weight (model/modules/features/halfka_v2_hm.py:68-69),
+ * the two fake_quantize_weights calls and the torch.cat of
+ * ComposedFeatureTransformer.merged_weight_and_bias (composed_feature_transformer.py:61-76;
+ * formula model/quantize.py:48-58).  Bit-identical to those torch ops.
+ */
+int nnueft_table_merge(const float* W, const float* V, float* merged, int R, int cols, int L1, int vrows,
+                       float scale_ft, float scale_psqt, int fake_quantize, void* stream);
+
+/*
+ * gV[v, c] = sum_k gW[k * vrows + v, c], k ascending from +0: the gradient of the virtual weights
+ * given the gradient of the merged table (the backward of `virtual_weight.repeat(NUM_BUCKETS, 1)`,
+ * halfka_v2_hm.py:68-69).  The straight-through estimator makes the gradient of the real weights
+ * gW itself.  gW f32[R, cols]; gV f32[vrows, cols], fully written.
+ */
+int nnueft_table_virtual_grad(const float* gW, float* gV, int R, int cols, int vrows, void* stream);
+
+/*
  * Quantized feature transformer as the engine evaluates an exported net (no code in the
  * reference; spec docs/nnue.md:1014-1069 and :2097-2134, constants model/quantize.py:58-73,
  * tensors produced by QuantizationManager.quantize_feature_transformer_*, model/quantize.py:175-204):

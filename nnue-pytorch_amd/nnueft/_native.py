@@ -31,6 +31,8 @@ PROTOTYPES = {
         c_int,
         [c_void_p] * 6 + [c_float] + [c_void_p] * 6 + [c_int] * 5 + [c_void_p, c_size_t, c_void_p],
     ),
+    "nnueft_table_merge": (c_int, [c_void_p] * 3 + [c_int] * 4 + [c_float] * 2 + [c_int, c_void_p]),
+    "nnueft_table_virtual_grad": (c_int, [c_void_p] * 2 + [c_int] * 3 + [c_void_p]),
     "nnueft_ft_int16_fwd": (c_int, [c_void_p] * 9 + [c_int] * 7 + [c_void_p]),
 }
 

@@ -1,0 +1,505 @@
+"""The callers of the feature transformer, restated for the full-model step (BASELINE config 4).
+
+These are the modules that sit directly above the operator in the reference; they are written
+against the same public names so that code using the reference's classes reads the same:
+
+  QuantizationConfig, QuantizationManager   model/quantize.py:58-113 (constants), :36-56 (fake quantization)
+  HalfKav2Hm                                model/modules/features/halfka_v2_hm.py:39-170
+  ComposedFeatureTransformer                model/modules/feature_transformer/composed_feature_transformer.py:12-151
+  StackedLinear, FactorizedStackedLinear    model/modules/stacked_linear.py
+  LayerStacks                               model/modules/layer_stacks.py:11-84
+  NNUEModel                                 model/model.py:9-133
+  sf_loss                                   model/nnue.py:39-70 (calculate_sf_loss; tablebase remap :19-36)
+
+What differs from the reference: on the GPU the table-side work of the feature transformer (real +
+virtual weights, fake quantization of both column groups, concatenation; five or more passes over a
+300 MB table in torch ops) is one HIP kernel, nnueft_table_merge, and the gradient of the virtual
+weights is one more, nnueft_table_virtual_grad.  Values are bit-identical to the torch ops.
+The dense layer stacks stay torch (small GEMMs through hipBLASLt).
+"""
+import math
+from dataclasses import dataclass, field
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from . import _native
+from . import halfka_v2_hm as hk
+from .double_ft_functions import double_feature_transform
+from .sparse_linear_functions import _stream_ptr
+
+FAKE_QUANTIZE_EPS = 1e-5
+
+
+# ------------------------------------------------------------------------------------------ quantization
+
+@dataclass
+class QuantizationConfig:
+    nnue2score: float = 600.0
+    weight_scale_l1: float = 128.0
+    weight_scale_l2: float = 64.0
+    weight_scale_l_out: float = 128
+    weight_scale_out: float = 16.0
+    weight_quantized_max_hidden: float = 127.0
+    ft_quantized_one: float = 256.0
+    ft_quantized_max: float = 255.0
+    hidden_quantized_one: float = 128.0
+    hidden_quantized_max: float = 127.0
+    inference_l0_division_factor: float = 512.0
+    inference_sqr_crelu_division_factor: float = 128.0
+
+
+def _ste(hard: torch.Tensor, value: torch.Tensor) -> torch.Tensor:
+    """Forward value `hard`, gradient of the identity (straight-through estimator)."""
+    return hard.detach() + (value - value.detach())
+
+
+class QuantizationManager:
+    def __init__(self, config: QuantizationConfig):
+        c = self.config = config
+        self.nnue2score = c.nnue2score
+        self.weight_scale_hidden = [c.weight_scale_l1, c.weight_scale_l2, c.weight_scale_l_out]
+        self.weight_scale_out = c.weight_scale_out
+        self.hidden_quantized_one = c.hidden_quantized_one
+        self.ft_quantized_one = c.ft_quantized_one
+        self.max_hidden_weight = [c.weight_quantized_max_hidden / s for s in self.weight_scale_hidden]
+        self.l0_correction_factor = c.ft_quantized_one ** 2 / c.inference_l0_division_factor / c.hidden_quantized_one
+        self.sqr_crelu_correction_factor = c.hidden_quantized_one / c.inference_sqr_crelu_division_factor
+        self.max_ft_activation = c.ft_quantized_max / c.ft_quantized_one
+        self.max_hidden_activation = c.hidden_quantized_max / c.hidden_quantized_one
+        one = c.hidden_quantized_one
+        self.weight_scales_dict = {
+            "ft_weight": c.ft_quantized_one,
+            "ft_bias": c.ft_quantized_one,
+            "ft_psqt_weight": c.nnue2score * c.weight_scale_out,
+            "ls_l1_weight": c.weight_scale_l1,
+            "ls_l1_bias": c.weight_scale_l1 * one,
+            "ls_l2_weight": c.weight_scale_l2,
+            "ls_l2_bias": c.weight_scale_l2 * one,
+            "ls_output_weight": c.weight_scale_l_out,
+            "ls_output_bias": c.weight_scale_l_out * one,
+        }
+
+    def clip_ft_act(self, x):
+        return torch.clamp(x, 0.0, self.max_ft_activation)
+
+    def clip_ls_act(self, x):
+        return torch.clamp(x, 0, self.max_hidden_activation)
+
+    def fake_quantize_weights(self, tensor, key: str):
+        scale = self.weight_scales_dict[key]
+        return _ste(tensor.mul(scale).round().div(scale), tensor)
+
+    def _fake_quantize_acts(self, x):
+        scale = self.config.hidden_quantized_one
+        return _ste(x.mul(scale).add(FAKE_QUANTIZE_EPS).floor().div(scale), x)
+
+    fake_quantize_ft_act = _fake_quantize_acts
+    fake_quantize_ls_act = _fake_quantize_acts
+
+    def fake_quantize_skip_act(self, x):
+        return x
+
+    def fake_quantize_output(self, x):
+        mult = int(self.config.nnue2score * self.config.weight_scale_out)
+        den = int(self.config.hidden_quantized_one * self.config.weight_scale_l_out * 2.0)
+        q = torch.div(torch.round(x * den).to(torch.int64) * mult, den, rounding_mode="trunc")
+        return _ste(q.to(x.dtype) / float(mult), x)
+
+
+# ------------------------------------------------------------------------------------------ feature block
+
+def _export_row_map():
+    """For every row of the 22528-row exported table, the row of the 24576-row training table it comes
+    from: ten piece-type blocks copied, the king block taken from the opposing-king rows except on the
+    bucket's own king square, which comes from the own-king row (halfka_v2_hm.py:104-135)."""
+    inverse_bucket = {int(b): sq for sq, b in enumerate(hk.KING_BUCKETS) if b >= 0}
+    src = torch.empty(hk.NUM_INPUTS_EXPORT, dtype=torch.long)
+    for b in range(hk.NUM_BUCKETS):
+        s0, d0 = b * hk.NUM_PLANES, b * 704
+        src[d0:d0 + 640] = torch.arange(s0, s0 + 640)
+        src[d0 + 640:d0 + 704] = torch.arange(s0 + 704, s0 + 768)
+        ksq = inverse_bucket[b]
+        src[d0 + 640 + ksq] = s0 + 640 + ksq
+    return src
+
+
+class HalfKav2Hm(nn.Module):
+    HASH = 0x7F234CB8
+    FEATURE_NAME = "HalfKAv2_hm^"
+    INPUT_FEATURE_NAME = "HalfKAv2_hm"
+    MAX_ACTIVE_FEATURES = hk.MAX_ACTIVE_FEATURES
+    NUM_PLANES = hk.NUM_PLANES
+    NUM_BUCKETS = hk.NUM_BUCKETS
+    NUM_INPUTS = hk.NUM_INPUTS
+    NUM_INPUTS_VIRTUAL = hk.NUM_PLANES
+    NUM_REAL_FEATURES = hk.NUM_INPUTS_EXPORT
+
+    def __init__(self, num_outputs: int):
+        super().__init__()
+        self.num_outputs = num_outputs
+        self.weight = nn.Parameter(torch.empty(self.NUM_INPUTS, num_outputs))
+        self.virtual_weight = nn.Parameter(torch.zeros(self.NUM_INPUTS_VIRTUAL, num_outputs))
+        sigma = math.sqrt(1 / self.NUM_INPUTS)
+        with torch.no_grad():
+            self.weight.uniform_(-sigma, sigma)
+
+    def merged_weight(self):
+        return self.weight + self.virtual_weight.repeat(self.NUM_BUCKETS, 1)
+
+    @torch.no_grad()
+    def zero_virtual_weights(self):
+        self.virtual_weight.zero_()
+
+    @torch.no_grad()
+    def coalesce(self):
+        self.weight.add_(self.virtual_weight.repeat(self.NUM_BUCKETS, 1))
+        self.zero_virtual_weights()
+
+    @staticmethod
+    def halfka_psqts():
+        """Initial PSQT value of every table row: +value for an own piece, -value for an opposing one."""
+        values = {hk.PAWN: 126, hk.KNIGHT: 781, hk.BISHOP: 825, hk.ROOK: 1276, hk.QUEEN: 2538}
+        out = [0] * hk.NUM_INPUTS
+        for ksq in range(64):
+            for sq in range(64):
+                for pt, val in values.items():
+                    out[hk.feature_index(hk.WHITE, ksq, sq, pt, hk.WHITE)] = val
+                    out[hk.feature_index(hk.WHITE, ksq, sq, pt, hk.BLACK)] = -val
+        return out
+
+    @torch.no_grad()
+    def init_weights(self, num_psqt_buckets: int, nnue2score: float):
+        self.zero_virtual_weights()
+        col = torch.tensor(self.halfka_psqts(), dtype=self.weight.dtype, device=self.weight.device) / nnue2score
+        l1 = self.num_outputs - num_psqt_buckets
+        self.weight[:, l1:] = col[:, None]
+
+    @torch.no_grad()
+    def get_export_weights(self):
+        merged = self.merged_weight()
+        return merged[_export_row_map().to(merged.device)]
+
+    @torch.no_grad()
+    def load_export_weights(self, export_weight):
+        src = _export_row_map().to(export_weight.device)
+        full = export_weight.new_zeros(self.NUM_INPUTS, export_weight.shape[1])
+        full[src] = export_weight
+        self.weight.data.copy_(full)
+        self.zero_virtual_weights()
+
+    def clip_weights(self, quantization):
+        pass
+
+
+def get_feature_cls(name: str):
+    if name in ("HalfKAv2_hm", "HalfKAv2_hm^"):
+        return [HalfKav2Hm]
+    raise ValueError(f"feature set {name} is not part of this build (HalfKAv2_hm only)")
+
+
+# ------------------------------------------------------------------------------------------ FT module
+
+class _TableMerge(torch.autograd.Function):
+    """merged = q(weight + virtual[row % 768]) in one pass; STE gradient: weight gets the incoming
+    gradient itself, virtual its sum over the table blocks."""
+
+    @staticmethod
+    def forward(ctx, weight, virtual, l1_size, scale_ft, scale_psqt, quantize):
+        lib = _native.load()
+        R, cols = weight.shape
+        merged = torch.empty_like(weight)
+        with torch.cuda.device(weight.device):
+            rc = lib.nnueft_table_merge(weight.data_ptr(), virtual.data_ptr(), merged.data_ptr(), R, cols, l1_size,
+                                        virtual.shape[0], float(scale_ft), float(scale_psqt), int(bool(quantize)),
+                                        _stream_ptr(weight.device))
+        _native.check(rc, "nnueft_table_merge")
+        ctx.vrows = virtual.shape[0]
+        return merged
+
+    @staticmethod
+    def backward(ctx, grad):
+        grad = grad.contiguous()
+        lib = _native.load()
+        R, cols = grad.shape
+        gv = torch.empty(ctx.vrows, cols, dtype=grad.dtype, device=grad.device)
+        with torch.cuda.device(grad.device):
+            rc = lib.nnueft_table_virtual_grad(grad.data_ptr(), gv.data_ptr(), R, cols, ctx.vrows,
+                                               _stream_ptr(grad.device))
+        _native.check(rc, "nnueft_table_virtual_grad")
+        return grad, gv, None, None, None, None
+
+
+@torch.compiler.disable(recursive=False)
+def _table_merge(weight, virtual, l1_size, scale_ft, scale_psqt, quantize):
+    return _TableMerge.apply(weight, virtual, l1_size, scale_ft, scale_psqt, quantize)
+
+
+class ComposedFeatureTransformer(nn.Module):
+    def __init__(self, feature_classes, l1_size: int, num_psqt_buckets: int, quantization: QuantizationManager):
+        super().__init__()
+        if l1_size % 2 != 0:
+            raise ValueError(f"l1_size must be even, got {l1_size}.")
+        self.l1_size = l1_size
+        self.num_psqt_buckets = num_psqt_buckets
+        self.num_outputs = l1_size + num_psqt_buckets
+        self.features = nn.ModuleList([cls(self.num_outputs) for cls in feature_classes])
+        self.bias = nn.Parameter(torch.empty(self.num_outputs))
+        self.NUM_INPUTS = sum(f.NUM_INPUTS for f in self.features)
+        self.MAX_ACTIVE_FEATURES = sum(f.MAX_ACTIVE_FEATURES for f in self.features)
+        self.NUM_REAL_FEATURES = sum(f.NUM_REAL_FEATURES for f in self.features)
+        self.FEATURE_NAME = "+".join(f.FEATURE_NAME for f in self.features)
+        self.INPUT_FEATURE_NAME = "+".join(f.INPUT_FEATURE_NAME for f in self.features)
+        h = 0
+        for f in self.features:
+            h = (((h << 1) | (h >> 31)) & 0xFFFFFFFF) ^ f.HASH
+        self.HASH = h
+        self.quantization = quantization
+        sigma = math.sqrt(1 / self.NUM_INPUTS)
+        with torch.no_grad():
+            self.bias.uniform_(-sigma, sigma)
+
+    def merged_weight_and_bias(self, fake_quantize_weights: bool = False):
+        q = self.quantization
+        only = self.features[0] if len(self.features) == 1 else None
+        if only is not None and isinstance(only, HalfKav2Hm) and only.weight.is_cuda and _native.available():
+            merged = _table_merge(only.weight, only.virtual_weight, self.l1_size,
+                                  q.weight_scales_dict["ft_weight"], q.weight_scales_dict["ft_psqt_weight"],
+                                  fake_quantize_weights)
+        else:
+            merged = torch.cat([f.merged_weight() for f in self.features], dim=0)
+            if fake_quantize_weights:
+                merged = torch.cat([q.fake_quantize_weights(merged[:, :self.l1_size], "ft_weight"),
+                                    q.fake_quantize_weights(merged[:, self.l1_size:], "ft_psqt_weight")], dim=1)
+        b = self.bias[:self.l1_size]
+        if fake_quantize_weights:
+            b = q.fake_quantize_weights(b, "ft_bias")
+        bias = torch.cat([b, torch.zeros_like(self.bias[self.l1_size:], dtype=b.dtype)], dim=0)
+        return merged, bias
+
+    @torch.no_grad()
+    def coalesce(self):
+        for f in self.features:
+            f.coalesce()
+
+    @torch.no_grad()
+    def zero_virtual_weights(self):
+        for f in self.features:
+            f.zero_virtual_weights()
+
+    @torch.no_grad()
+    def init_weights(self):
+        for f in self.features:
+            f.init_weights(self.num_psqt_buckets, self.quantization.nnue2score)
+        self.bias[self.l1_size:] = 0.0
+
+    @torch.no_grad()
+    def get_export_weights(self):
+        return torch.cat([f.get_export_weights() for f in self.features], dim=0)
+
+    @torch.no_grad()
+    def load_export_weights(self, export_weight):
+        at = 0
+        for f in self.features:
+            f.load_export_weights(export_weight[at:at + f.NUM_REAL_FEATURES])
+            at += f.NUM_REAL_FEATURES
+
+    def clip_weights(self, quantization):
+        for f in self.features:
+            f.clip_weights(quantization)
+
+    def forward(self, us, them, white_indices, black_indices, psqt_indices, fake_quantize_acts: bool,
+                fake_quantize_weights: bool, backend: str = "auto"):
+        merged, bias = self.merged_weight_and_bias(fake_quantize_weights)
+        l0_, wpsqt, bpsqt = double_feature_transform(us, them, white_indices, black_indices, psqt_indices, merged,
+                                                     bias, self.quantization.max_ft_activation, self.l1_size, backend)
+        if fake_quantize_acts:
+            l0_ = self.quantization.fake_quantize_ft_act(l0_)
+        return l0_ * self.quantization.l0_correction_factor, wpsqt, bpsqt
+
+
+# ------------------------------------------------------------------------------------------ layer stacks
+
+class StackedLinear(nn.Module):
+    """`count` linear layers of the same shape evaluated as one wide layer; each position picks the
+    output block of its bucket."""
+
+    def __init__(self, in_features, out_features, count, quantization=None, layer_key=None):
+        super().__init__()
+        self.in_features, self.out_features, self.count = in_features, out_features, count
+        self.linear = nn.Linear(in_features, out_features * count)
+        self.quantization, self.layer_key = quantization, layer_key
+        with torch.no_grad():   # every bucket starts from the same layer
+            self.linear.weight.copy_(self.linear.weight[:out_features].repeat(count, 1))
+            self.linear.bias.copy_(self.linear.bias[:out_features].repeat(count))
+
+    def _params(self):
+        return self.linear.weight, self.linear.bias
+
+    def forward(self, x, ls_indices, fake_quantize_weights: bool = False):
+        weight, bias = self._params()
+        if fake_quantize_weights:
+            if self.quantization is None or self.layer_key is None:
+                raise RuntimeError("self.quantization and self.layer_key are required to use fake quantize weights.")
+            weight = self.quantization.fake_quantize_weights(weight, f"{self.layer_key}_weight")
+            bias = self.quantization.fake_quantize_weights(bias, f"{self.layer_key}_bias")
+        wide = F.linear(x, weight, bias).reshape(-1, self.out_features)
+        pick = ls_indices.flatten() + torch.arange(0, ls_indices.shape[0] * self.count, self.count, device=x.device)
+        return wide[pick]
+
+    @torch.no_grad()
+    def at_index(self, index: int):
+        layer = nn.Linear(self.in_features, self.out_features)
+        weight, bias = self._params()
+        lo, hi = index * self.out_features, (index + 1) * self.out_features
+        layer.weight.copy_(weight[lo:hi])
+        layer.bias.copy_(bias[lo:hi])
+        return layer
+
+
+class FactorizedStackedLinear(StackedLinear):
+    """StackedLinear plus one layer shared by all buckets (added to each of them)."""
+
+    def __init__(self, in_features, out_features, count, quantization, layer_key):
+        super().__init__(in_features, out_features, count, quantization, layer_key)
+        self.factorized_linear = nn.Linear(in_features, out_features)
+        self.zero_virtual_weights()
+
+    def _params(self):
+        return (self.linear.weight + self.factorized_linear.weight.repeat(self.count, 1),
+                self.linear.bias + self.factorized_linear.bias.repeat(self.count))
+
+    @torch.no_grad()
+    def zero_virtual_weights(self):
+        self.factorized_linear.weight.zero_()
+        self.factorized_linear.bias.zero_()
+
+    @torch.no_grad()
+    def coalesce_weights(self):
+        self.linear.weight.add_(self.factorized_linear.weight.repeat(self.count, 1))
+        self.linear.bias.add_(self.factorized_linear.bias.repeat(self.count))
+        self.zero_virtual_weights()
+
+
+@dataclass
+class ModelConfig:
+    L1: int = 1024
+    L2: int = 32
+    L3: int = 32
+    quantize_config: QuantizationConfig = field(default_factory=QuantizationConfig)
+
+
+class LayerStacks(nn.Module):
+    def __init__(self, count: int, config, quantization: QuantizationManager):
+        super().__init__()
+        self.count, self.L1, self.L2, self.L3 = count, config.L1, config.L2, config.L3
+        self.quantization = quantization
+        self.l1 = FactorizedStackedLinear(self.L1, self.L2, count, quantization, "ls_l1")
+        self.l2 = StackedLinear(self.L2 * 2, self.L3, count, quantization, "ls_l2")
+        self.output = StackedLinear(self.L2 * 2 + self.L3 * 2, 1, count, quantization, "ls_output")
+        with torch.no_grad():
+            self.output.linear.bias.zero_()
+
+    def _sqr_and_linear(self, x, fake_quantize_acts):
+        q = self.quantization
+        sqr = torch.pow(x, 2.0)
+        if fake_quantize_acts:
+            sqr = q.fake_quantize_ls_act(sqr)
+            x = q.fake_quantize_ls_act(x)
+        return q.clip_ls_act(torch.cat([sqr * q.sqr_crelu_correction_factor, x], dim=1))
+
+    def forward(self, x, ls_indices, fake_quantize_acts: bool = True, fake_quantize_weights: bool = True):
+        q = self.quantization
+        l1c = self.l1(x, ls_indices, fake_quantize_weights)
+        skip = l1c[:, -2].view(-1, 1) - l1c[:, -1].view(-1, 1)
+        l1x = self._sqr_and_linear(l1c, fake_quantize_acts)
+        l2x = self._sqr_and_linear(self.l2(l1x, ls_indices, fake_quantize_weights), fake_quantize_acts)
+        out = self.output(torch.cat([l1x, l2x], dim=1), ls_indices, fake_quantize_weights)
+        if fake_quantize_acts:
+            skip = q.fake_quantize_skip_act(skip)
+        out = out + skip
+        if fake_quantize_acts:
+            out = q.fake_quantize_output(out)
+        assert out.shape[1] == 1
+        return out
+
+    @torch.no_grad()
+    def zero_virtual_weights(self):
+        self.l1.zero_virtual_weights()
+
+
+# ------------------------------------------------------------------------------------------ model + loss
+
+class NNUEModel(nn.Module):
+    def __init__(self, feature_name: str, config: ModelConfig, num_psqt_buckets: int = 8, num_ls_buckets: int = 8):
+        super().__init__()
+        self.L1, self.L2, self.L3 = config.L1, config.L2, config.L3
+        self.quantization = QuantizationManager(config.quantize_config)
+        self.num_psqt_buckets, self.num_ls_buckets = num_psqt_buckets, num_ls_buckets
+        self.input = ComposedFeatureTransformer(get_feature_cls(feature_name), self.L1, num_psqt_buckets,
+                                                self.quantization)
+        self.layer_stacks = LayerStacks(num_ls_buckets, config, self.quantization)
+        self.input.init_weights()
+
+    def calculate_buckets(self, piece_count):
+        psqt_indices = (piece_count - 1) // 4
+        return psqt_indices, psqt_indices
+
+    def forward_ft(self, us, them, white_indices, black_indices, psqt_indices, fake_quantize_acts,
+                   fake_quantize_weights):
+        return self.input(us, them, white_indices, black_indices, psqt_indices, fake_quantize_acts,
+                          fake_quantize_weights)
+
+    def forward(self, us, them, white_indices, black_indices, piece_count, fake_quantize_acts: bool = True,
+                fake_quantize_weights: bool = True):
+        psqt_indices, ls_indices = self.calculate_buckets(piece_count)
+        l0_, wpsqt, bpsqt = self.forward_ft(us, them, white_indices, black_indices, psqt_indices,
+                                            fake_quantize_acts, fake_quantize_weights)
+        # the PSQT term is the perspective average with the sign of the side to move
+        return self.layer_stacks(l0_, ls_indices, fake_quantize_acts, fake_quantize_weights) + (wpsqt - bpsqt) * (us - 0.5)
+
+    @torch.no_grad()
+    def zero_virtual_weights(self):
+        self.input.zero_virtual_weights()
+        self.layer_stacks.zero_virtual_weights()
+
+
+@dataclass
+class LossParams:
+    in_offset: float = 270
+    out_offset: float = 270
+    in_scaling: float = 340
+    out_scaling: float = 380
+    pow_exp: float = 2.5
+    qp_asymmetry: float = 0.0
+    w1: float = 0.0
+    w2: float = 0.5
+    tb_remap_base: float = 4000.0
+    tb_remap_scale: float = 4000.0
+    tb_remap_decay: float = 0.85
+
+
+def remap_tablebase_score(score, base: float, scale: float, decay: float):
+    mate_score, max_mate_ply = 32000, 245
+    magnitude = score.abs()
+    plies = (mate_score - magnitude).clamp(min=0)
+    remapped = base + (decay ** plies) * scale
+    return torch.where(magnitude >= mate_score - max_mate_ply, torch.where(score < 0, -remapped, remapped), score)
+
+
+def sf_loss(scorenet, score, outcome, p: LossParams, actual_lambda):
+    """Win-rate-model loss; `scorenet` is the net output times nnue2score (model/nnue.py:39-70)."""
+    score = remap_tablebase_score(score, p.tb_remap_base, p.tb_remap_scale, p.tb_remap_decay)
+
+    def win_rate(x, offset, scaling):
+        return 0.5 * (1.0 + ((x - offset) / scaling).sigmoid() - ((-x - offset) / scaling).sigmoid())
+
+    qf = win_rate(scorenet, p.in_offset, p.in_scaling)
+    pf = win_rate(score, p.out_offset, p.out_scaling)
+    pt = pf * actual_lambda + outcome * (1.0 - actual_lambda)
+    loss = torch.pow(torch.abs(pt - qf), p.pow_exp)
+    if p.qp_asymmetry != 0.0:
+        loss = loss * ((qf > pt) * p.qp_asymmetry + 1)
+    weights = 1 + (2.0 ** p.w1 - 1) * torch.pow((pf - 0.5) ** 2 * pf * (1 - pf), p.w2)
+    return (loss * weights).sum() / weights.sum()

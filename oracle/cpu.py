@@ -130,3 +130,22 @@ def ft_int16_fwd(widx, bidx, stm, W16, b16, psqt32, psqt_idx, clip_max=255, shif
                                           _p(out), _p(ps), B, K, R, L1, n_psqt, int(clip_max), int(shift))
     assert rc == 0
     return out, ps
+
+
+def table_merge(W, V, L1, scale_ft=256.0, scale_psqt=9600.0, fake_quantize=True):
+    W, V = _c(W, np.float32), _c(V, np.float32)
+    R, cols = W.shape
+    out = np.empty_like(W)
+    rc = lib().nnueft_oracle_table_merge(_p(W), _p(V), _p(out), R, cols, int(L1), V.shape[0],
+                                         ctypes.c_float(scale_ft), ctypes.c_float(scale_psqt), int(bool(fake_quantize)))
+    assert rc == 0
+    return out
+
+
+def table_virtual_grad(gW, vrows):
+    gW = _c(gW, np.float32)
+    R, cols = gW.shape
+    gV = np.empty((vrows, cols), np.float32)
+    rc = lib().nnueft_oracle_table_virtual_grad(_p(gW), _p(gV), R, cols, int(vrows))
+    assert rc == 0
+    return gV

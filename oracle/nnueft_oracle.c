@@ -312,3 +312,42 @@ int nnueft_oracle_ft_int16_fwd(const int32_t* widx, const int32_t* bidx, const u
     }
     return 0;
 }
+
+/*
+ * merged = q(W + V[row % vrows]) -- HalfKav2Hm.merged_weight (model/modules/features/halfka_v2_hm.py:68-69)
+ * followed by the weight fake quantization of ComposedFeatureTransformer.merged_weight_and_bias
+ * (composed_feature_transformer.py:61-76): q(x) = round(x * s) / s, half to even (model/quantize.py:48-58),
+ * s = scale_ft for the first L1 columns, scale_psqt for the others.
+ */
+#include <math.h>
+int nnueft_oracle_table_merge(const float* W, const float* V, float* merged, int R, int cols, int L1, int vrows,
+                              float scale_ft, float scale_psqt, int fake_quantize)
+{
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < R; ++r) {
+        for (int c = 0; c < cols; ++c) {
+            float x = W[(size_t)r * cols + c];
+            if (V) x = x + V[(size_t)(r % vrows) * cols + c];
+            if (fake_quantize) {
+                const float s = c < L1 ? scale_ft : scale_psqt;
+                x = nearbyintf(x * s) / s;
+            }
+            merged[(size_t)r * cols + c] = x;
+        }
+    }
+    return 0;
+}
+
+/* gV[v] = chain from +0 over the table blocks k (ascending) of gW[k * vrows + v]. */
+int nnueft_oracle_table_virtual_grad(const float* gW, float* gV, int R, int cols, int vrows)
+{
+#pragma omp parallel for schedule(static)
+    for (int v = 0; v < vrows; ++v) {
+        for (int c = 0; c < cols; ++c) {
+            float acc = 0.0f;
+            for (int r = v; r < R; r += vrows) acc = acc + gW[(size_t)r * cols + c];
+            gV[(size_t)v * cols + c] = acc;
+        }
+    }
+    return 0;
+}

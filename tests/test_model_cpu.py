@@ -1,0 +1,165 @@
+"""The callers of the operator (quantization constants, feature block, FT module, layer stacks, loss)
+on the CPU: closed forms, known answers and round trips."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from nnueft import halfka_v2_hm as hk
+from nnueft import model as M
+
+
+def test_quantization_constants():
+    # literals of model/quantize.py:58-113
+    q = M.QuantizationManager(M.QuantizationConfig())
+    assert q.l0_correction_factor == 1.0                       # 256^2 / 512 / 128
+    assert q.sqr_crelu_correction_factor == 1.0
+    assert q.max_ft_activation == 255 / 256 and q.max_hidden_activation == 127 / 128
+    assert q.weight_scales_dict["ft_weight"] == 256 and q.weight_scales_dict["ft_psqt_weight"] == 9600
+    assert q.weight_scales_dict["ls_l1_bias"] == 128 * 128 and q.weight_scales_dict["ls_l2_weight"] == 64
+    assert q.max_hidden_weight == [127 / 128, 127 / 64, 127 / 128]
+    assert (255 * 255) >> 9 == 127
+
+
+def test_fake_quantization_known_answers():
+    q = M.QuantizationManager(M.QuantizationConfig())
+    x = torch.tensor([0.0, 1 / 512, 3 / 512, 0.30, -0.30, 1.0], requires_grad=True)
+    w = q.fake_quantize_weights(x, "ft_weight")
+    # round half to even on x*256: 0.5 -> 0, 1.5 -> 2, 76.8 -> 77
+    assert w.tolist() == [0.0, 0.0, 2 / 256, 77 / 256, -77 / 256, 1.0]
+    w.sum().backward()
+    assert x.grad.tolist() == [1.0] * 6                        # straight-through
+    a = q.fake_quantize_ft_act(torch.tensor([0.0, 0.999, 0.5, 127.9 / 128]))
+    assert a.tolist() == [0.0, 127 / 128, 0.5, 127 / 128]      # floor(x*128 + 1e-5) / 128
+    o = q.fake_quantize_output(torch.tensor([[0.1234], [-0.1234]]))
+    den, mult = 128 * 128 * 2, 9600
+    want = math.trunc(round(0.1234 * den) * mult / den) / mult
+    assert o[:, 0].tolist() == [float(np.float32(want)), -float(np.float32(want))]
+
+
+def test_export_remap_closed_form_and_round_trip():
+    torch.manual_seed(0)
+    f = M.HalfKav2Hm(4)
+    with torch.no_grad():
+        f.weight.copy_(torch.arange(hk.NUM_INPUTS * 4, dtype=torch.float32).reshape(-1, 4))
+    exp = f.get_export_weights()
+    assert exp.shape == (hk.NUM_INPUTS_EXPORT, 4)
+    inv = {int(b): sq for sq, b in enumerate(hk.KING_BUCKETS) if b >= 0}
+    for b in (0, 7, 31):
+        s0, d0, ksq = b * 768, b * 704, inv[b]
+        assert torch.equal(exp[d0:d0 + 640], f.weight[s0:s0 + 640])
+        for sq in range(64):
+            src = s0 + 640 + sq if sq == ksq else s0 + 704 + sq      # own king only on its own square
+            assert torch.equal(exp[d0 + 640 + sq], f.weight[src])
+    g = M.HalfKav2Hm(4)
+    g.load_export_weights(exp)
+    assert torch.equal(g.get_export_weights(), exp)                 # identity on the exported rows
+    # rows the export drops are zero after the round trip
+    assert not g.weight[640:704][[s for s in range(64) if s != inv[0]]].any()
+    assert not g.weight[704 + inv[0]].any()
+    # virtual weights are folded in
+    with torch.no_grad():
+        f.virtual_weight.fill_(1.0)
+    assert torch.equal(f.get_export_weights(), exp + 1.0)
+
+
+def test_psqt_initial_values():
+    vals = M.HalfKav2Hm.halfka_psqts()
+    assert len(vals) == hk.NUM_INPUTS
+    assert vals[hk.feature_index(hk.WHITE, 4, 12, hk.PAWN, hk.WHITE)] == 126
+    assert vals[hk.feature_index(hk.WHITE, 4, 12, hk.QUEEN, hk.BLACK)] == -2538
+    assert vals[hk.feature_index(hk.WHITE, 4, 4, hk.KING, hk.WHITE)] == 0
+    v = np.array(vals).reshape(32, 12, 64)
+    assert np.array_equal(v[:, 0::2], -v[:, 1::2])                  # own / opposing piece blocks mirror
+    assert set(np.unique(np.abs(v))) == {0, 126, 781, 825, 1276, 2538}
+
+
+def test_composed_ft_cpu_matches_explicit_formula():
+    torch.manual_seed(1)
+    q = M.QuantizationManager(M.QuantizationConfig())
+    ft = M.ComposedFeatureTransformer([M.HalfKav2Hm], 32, 8, q)
+    ft.init_weights()
+    with torch.no_grad():
+        ft.features[0].virtual_weight.normal_(0, 0.01)
+    assert ft.NUM_INPUTS == 24576 and ft.MAX_ACTIVE_FEATURES == 32 and ft.HASH == 0x7F234CB8
+    us, them, white, black, pc = [torch.from_numpy(a) for a in hk.synthetic_batch(16, 3)]
+    psqt = (pc - 1) // 4
+    l0, wp, bp = ft(us, them, white, black, psqt, True, True)
+    f = ft.features[0]
+    merged = f.weight + f.virtual_weight.repeat(32, 1)
+    merged = torch.cat([(merged[:, :32] * 256).round() / 256, (merged[:, 32:] * 9600).round() / 9600], 1)
+    bias = torch.cat([(ft.bias[:32] * 256).round() / 256, torch.zeros(8)])
+    from oracle import ref_torch
+
+    r_l0, r_wp, r_bp = ref_torch.double_feature_transform(us, them, white, black, psqt, merged, bias, 255 / 256, 32)
+    assert torch.equal(l0, torch.floor(r_l0 * 128 + 1e-5) / 128)
+    assert torch.equal(wp, r_wp) and torch.equal(bp, r_bp)
+    (l0.sum() + wp.sum()).backward()
+    assert f.weight.grad is not None and f.virtual_weight.grad is not None and ft.bias.grad is not None
+    # the virtual gradient is the block sum of the real one
+    assert torch.allclose(f.virtual_weight.grad, f.weight.grad.view(32, 768, -1).sum(0), atol=1e-5)
+
+
+def test_stacked_linear_equals_per_bucket_layers():
+    torch.manual_seed(2)
+    q = M.QuantizationManager(M.QuantizationConfig())
+    sl = M.FactorizedStackedLinear(16, 4, 8, q, "ls_l1")
+    with torch.no_grad():
+        sl.linear.weight.normal_()
+        sl.factorized_linear.weight.normal_()
+        sl.factorized_linear.bias.normal_()
+    x = torch.randn(10, 16)
+    idx = torch.randint(0, 8, (10,))
+    out = sl(x, idx)
+    for i in range(10):
+        layer = sl.at_index(int(idx[i]))
+        w = sl.linear.weight[int(idx[i]) * 4:int(idx[i]) * 4 + 4] + sl.factorized_linear.weight
+        assert torch.allclose(layer.weight, w)
+        assert torch.allclose(out[i], layer(x[i]), atol=1e-5)
+
+
+def test_loss_closed_forms():
+    p = M.LossParams()
+    # prediction and target on the same win-rate curve: loss 0
+    same = M.LossParams(in_scaling=380, out_scaling=380)
+    s = torch.tensor([[-300.0], [0.0], [150.0]])
+    assert float(M.sf_loss(s, s, torch.zeros(3, 1), same, 1.0)) == 0.0
+    # one sample, lambda = 0: |outcome - qf|^2.5
+    sc = torch.tensor([[100.0]])
+    qf = 0.5 * (1 + torch.sigmoid((sc - 270) / 340) - torch.sigmoid((-sc - 270) / 340))
+    got = M.sf_loss(sc, torch.tensor([[0.0]]), torch.tensor([[1.0]]), p, 0.0)
+    assert float(got) == pytest.approx(float((1.0 - qf).abs() ** 2.5), rel=1e-6)
+    # antisymmetry of the win-rate model: qf(0) = 0.5
+    assert float(M.sf_loss(torch.zeros(1, 1), torch.zeros(1, 1), torch.full((1, 1), 0.5), p, 0.3)) == 0.0
+    # tablebase scores are remapped, ordinary scores are not
+    r = M.remap_tablebase_score(torch.tensor([100.0, 31990.0, -31990.0]), 4000.0, 4000.0, 0.85)
+    assert r[0] == 100.0 and r[1] == pytest.approx(4000 + 0.85 ** 10 * 4000) and r[2] == -r[1]
+
+
+def test_full_model_forward_backward_cpu():
+    torch.manual_seed(3)
+    model = M.NNUEModel("HalfKAv2_hm^", M.ModelConfig(L1=64, L2=16, L3=32))
+    us, them, white, black, pc = [torch.from_numpy(a) for a in hk.synthetic_batch(32, 4)]
+    out = model(us, them, white, black, pc)
+    assert out.shape == (32, 1) and torch.isfinite(out).all()
+    loss = M.sf_loss(out * 600.0, torch.randn(32, 1) * 400, torch.full((32, 1), 0.5), M.LossParams(), 1.0)
+    loss.backward()
+    for name, prm in model.named_parameters():
+        assert prm.grad is not None and torch.isfinite(prm.grad).all(), name
+    # material only: the PSQT initialisation makes the side with more material score higher
+    assert float(model.input.features[0].weight[:, 64:].detach().abs().max()) == pytest.approx(2538 / 600)
+
+
+def test_oracle_table_functions(oracle_cpu):
+    rng = np.random.default_rng(0)
+    W = rng.standard_normal((48, 12)).astype(np.float32)
+    V = rng.standard_normal((16, 12)).astype(np.float32)
+    m = oracle_cpu.table_merge(W, V, 8)
+    t = torch.from_numpy(W) + torch.from_numpy(V).repeat(3, 1)
+    t = torch.cat([(t[:, :8] * 256).round() / 256, (t[:, 8:] * 9600).round() / 9600], 1)
+    assert np.array_equal(m, t.numpy())
+    assert np.array_equal(oracle_cpu.table_merge(W, V, 8, fake_quantize=False),
+                          (torch.from_numpy(W) + torch.from_numpy(V).repeat(3, 1)).numpy())
+    g = rng.integers(-9, 9, size=(48, 12)).astype(np.float32)
+    assert np.array_equal(oracle_cpu.table_virtual_grad(g, 16), g.reshape(3, 16, 12).sum(0))
