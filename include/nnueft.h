@@ -176,6 +176,30 @@ int nnueft_ft_int16_fwd(const int32_t* widx, const int32_t* bidx, const uint8_t*
                         const int64_t* psqt_idx, uint8_t* out_u8, int32_t* psqt_out,
                         int B, int K, int R, int L1, int n_psqt, int clip_max, int shift, void* stream);
 
+/*
+ * Quantized layer stacks on the output of nnueft_ft_int16_fwd: the integer evaluation of the
+ * bucketed stack of model/modules/layer_stacks.py:33-84 with the tensors of
+ * QuantizationManager.quantize_fc_layer (model/quantize.py:218-236; int8 weights, int32 biases).
+ * No code in the reference (the engine runs it); each step is the integer image of the
+ * fake-quantized float forward, with a1, a2, a3 the int32 accumulators of the three layers:
+ *   a1 = b1 + W1 . x                                     x u8 [L1], 0..127
+ *   y1 = clip([ (a1*a1) >> sqr_shift1, a1 >> lin_shift1 ], 0, act_max)        2*L2 values
+ *   a2 = b2 + W2 . y1 ;  y2 = clip([ (a2*a2) >> sqr_shift2, a2 >> lin_shift2 ], 0, act_max)
+ *   a3 = bo + Wo . [y1, y2]
+ *   out = 2 * (a3 + a1[L2-2] - a1[L2-1]) * out_mult / out_den         (64-bit, C division)
+ * With the default scales (weights x128 / x64 / x128, activations x128): lin_shift1 = 7,
+ * sqr_shift1 = 21, lin_shift2 = 6, sqr_shift2 = 19, act_max = 127, out_mult = 9600, out_den = 32768;
+ * out is then the stack's output at scale 9600 (the scale of nnueft_ft_int16_fwd's psqt_out).
+ * x u8[B,L1]; bucket int64[B] in [0,count); W1 int8[count*L2, L1]; b1 int32[count*L2];
+ * W2 int8[count*L3, 2*L2]; b2 int32[count*L3]; Wo int8[count, 2*L2+2*L3]; bo int32[count]; out int32[B].
+ * Limits: L1 % 4 == 0, L1 <= 4096, 2 <= L2 <= 32, L3 <= 32.
+ */
+int nnueft_stack_int8_fwd(const uint8_t* x, const int64_t* bucket, const int8_t* W1, const int32_t* b1,
+                          const int8_t* W2, const int32_t* b2, const int8_t* Wo, const int32_t* bo,
+                          int32_t* out, int B, int L1, int L2, int L3, int count,
+                          int lin_shift1, int sqr_shift1, int lin_shift2, int sqr_shift2, int act_max,
+                          int out_mult, int out_den, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -70,3 +70,42 @@ def ft_int16_forward(white_indices, black_indices, stm, w16, b16, psqt32, psqt_i
         )
     _native.check(rc, "nnueft_ft_int16_fwd")
     return out, psqt
+
+
+def quantize_layer_stacks(layer_stacks, quantization=None):
+    """LayerStacks (nnueft.model) -> the six integer tensors nnueft_stack_int8_fwd takes: int8 weights and
+    int32 biases at the scales of QuantizationManager.quantize_fc_layer (model/quantize.py:218-236), the
+    factorised first layer folded in.  Raises when a value does not fit."""
+    q = quantization or layer_stacks.quantization
+    d = q.weight_scales_dict
+    w1, b1 = layer_stacks.l1._params()
+    out = []
+    for (w, b), key in (((w1, b1), "ls_l1"), ((layer_stacks.l2.linear.weight, layer_stacks.l2.linear.bias), "ls_l2"),
+                        ((layer_stacks.output.linear.weight, layer_stacks.output.linear.bias), "ls_output")):
+        out.append(_safe_round_to(w.detach() * d[f"{key}_weight"], torch.int8).contiguous())
+        out.append(_safe_round_to(b.detach() * d[f"{key}_bias"], torch.int32).contiguous())
+    return tuple(out)
+
+
+def stack_int8_forward(x_u8, bucket, w1, b1, w2, b2, wo, bo, lin_shift1=7, sqr_shift1=21, lin_shift2=6,
+                       sqr_shift2=19, act_max=127, out_mult=9600, out_den=32768):
+    """int32 [B]: the stack output at scale out_mult (9600 = nnue2score * 16) for u8 inputs [B, L1]."""
+    assert x_u8.is_cuda and x_u8.dtype == torch.uint8 and x_u8.ndim == 2 and x_u8.is_contiguous()
+    assert bucket.dtype == torch.int64 and bucket.shape == (x_u8.shape[0],)
+    for w, b in ((w1, b1), (w2, b2), (wo, bo)):
+        assert w.dtype == torch.int8 and b.dtype == torch.int32 and w.is_contiguous() and b.is_contiguous()
+        assert w.device == x_u8.device and b.device == x_u8.device
+    B, L1 = x_u8.shape
+    count = bo.shape[0]
+    L2, L3 = w1.shape[0] // count, w2.shape[0] // count
+    assert w1.shape == (count * L2, L1) and w2.shape == (count * L3, 2 * L2) and wo.shape == (count, 2 * L2 + 2 * L3)
+    out = torch.empty(B, dtype=torch.int32, device=x_u8.device)
+    lib = _native.load()
+    with torch.cuda.device(x_u8.device):
+        rc = lib.nnueft_stack_int8_fwd(
+            x_u8.data_ptr(), bucket.data_ptr(), w1.data_ptr(), b1.data_ptr(), w2.data_ptr(), b2.data_ptr(),
+            wo.data_ptr(), bo.data_ptr(), out.data_ptr(), B, L1, L2, L3, count, lin_shift1, sqr_shift1, lin_shift2,
+            sqr_shift2, act_max, out_mult, out_den, _stream_ptr(x_u8.device),
+        )
+    _native.check(rc, "nnueft_stack_int8_fwd")
+    return out

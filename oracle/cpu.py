@@ -149,3 +149,22 @@ def table_virtual_grad(gW, vrows):
     rc = lib().nnueft_oracle_table_virtual_grad(_p(gW), _p(gV), R, cols, int(vrows))
     assert rc == 0
     return gV
+
+
+STACK_DEFAULTS = dict(lin1=7, sqr1=21, lin2=6, sqr2=19, act_max=127, out_mult=9600, out_den=32768)
+
+
+def stack_int8_fwd(x, bucket, W1, b1, W2, b2, Wo, bo, L2, L3, count, **kw):
+    k = dict(STACK_DEFAULTS)
+    k.update(kw)
+    x = _c(x, np.uint8)
+    bucket = _c(bucket, np.int64)
+    W1, W2, Wo = _c(W1, np.int8), _c(W2, np.int8), _c(Wo, np.int8)
+    b1, b2, bo = _c(b1, np.int32), _c(b2, np.int32), _c(bo, np.int32)
+    B, L1 = x.shape
+    out = np.empty((B,), np.int32)
+    rc = lib().nnueft_oracle_stack_int8_fwd(_p(x), _p(bucket), _p(W1), _p(b1), _p(W2), _p(b2), _p(Wo), _p(bo), _p(out),
+                                            B, L1, int(L2), int(L3), int(count), k["lin1"], k["sqr1"], k["lin2"],
+                                            k["sqr2"], k["act_max"], k["out_mult"], k["out_den"])
+    assert rc == 0
+    return out

@@ -351,3 +351,52 @@ int nnueft_oracle_table_virtual_grad(const float* gW, float* gV, int R, int cols
     }
     return 0;
 }
+
+/*
+ * Quantized layer stacks: integer image of the fake-quantized forward of
+ * model/modules/layer_stacks.py:33-84 on the tensors of quantize_fc_layer (model/quantize.py:218-236).
+ * No code in the reference.  See include/nnueft.h for the formula.
+ */
+static inline int clip_act(long long v, int act_max) { return (int)(v < 0 ? 0 : (v > act_max ? act_max : v)); }
+
+int nnueft_oracle_stack_int8_fwd(const uint8_t* x, const int64_t* bucket, const int8_t* W1, const int32_t* b1,
+                                 const int8_t* W2, const int32_t* b2, const int8_t* Wo, const int32_t* bo,
+                                 int32_t* out, int B, int L1, int L2, int L3, int count,
+                                 int lin1, int sqr1, int lin2, int sqr2, int act_max, int out_mult, int out_den)
+{
+    if (L2 > 64 || L3 > 64 || L2 < 2) return -1;
+#pragma omp parallel for schedule(static)
+    for (int p = 0; p < B; ++p) {
+        long long bk = bucket[p];
+        if (bk < 0) bk = 0;
+        if (bk >= count) bk = count - 1;
+        int a1[64], y1[128], a2[64], y2[128];
+        for (int o = 0; o < L2; ++o) {
+            int acc = b1[bk * L2 + o];
+            const int8_t* w = W1 + ((size_t)bk * L2 + o) * L1;
+            for (int i = 0; i < L1; ++i) acc += (int)w[i] * (int)x[(size_t)p * L1 + i];
+            a1[o] = acc;
+        }
+        for (int o = 0; o < L2; ++o) {
+            y1[o] = clip_act(((long long)a1[o] * a1[o]) >> sqr1, act_max);
+            y1[L2 + o] = clip_act((long long)(a1[o] >> lin1), act_max);
+        }
+        for (int j = 0; j < L3; ++j) {
+            int acc = b2[bk * L3 + j];
+            const int8_t* w = W2 + ((size_t)bk * L3 + j) * (2 * L2);
+            for (int i = 0; i < 2 * L2; ++i) acc += (int)w[i] * y1[i];
+            a2[j] = acc;
+        }
+        for (int j = 0; j < L3; ++j) {
+            y2[j] = clip_act(((long long)a2[j] * a2[j]) >> sqr2, act_max);
+            y2[L3 + j] = clip_act((long long)(a2[j] >> lin2), act_max);
+        }
+        const int8_t* w = Wo + (size_t)bk * (2 * L2 + 2 * L3);
+        int a3 = bo[bk];
+        for (int i = 0; i < 2 * L2; ++i) a3 += (int)w[i] * y1[i];
+        for (int i = 0; i < 2 * L3; ++i) a3 += (int)w[2 * L2 + i] * y2[i];
+        const long long num = 2ll * ((long long)a3 + a1[L2 - 2] - a1[L2 - 1]) * out_mult;
+        out[p] = (int32_t)(num / out_den);
+    }
+    return 0;
+}
