@@ -22,9 +22,10 @@ sys.path.insert(0, os.path.join(ROOT, "nnue-pytorch_amd"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
-# Bytes that crossed the L2 boundary per forward launch (FETCH_SIZE x2.0 + WRITE_SIZE x1.0, the scale being
-# what the same counters read for a 1 GiB torch.add): profiles/k_double_fwd_L1_3072_B16384_pmc_fetch_write.txt
-MEASURED_FWD_TRAFFIC = {"ft_fwd_bwd_L1_3072_B16384": 8.00e9}
+# Bytes that crossed the L2 boundary per call of nnueft_double_fwd (FETCH_SIZE x2.0 + WRITE_SIZE x1.0 summed over
+# its kernels, the scale being what the same counters read for a 1 GiB torch.add):
+# profiles/nnueft_double_fwd_L1_3072_B16384_pmc.txt
+MEASURED_FWD_TRAFFIC = {"ft_fwd_bwd_L1_3072_B16384": 1.48e9}
 
 WORKLOADS = {
     # name: (L1, B)
@@ -362,7 +363,7 @@ def main():
             "index_scheme": "HalfKAv2_hm, seeded random positions",
         },
         "roofline": {
-            "kernel": "k_double_fwd (nnueft_double_fwd)",
+            "kernel": "nnueft_double_fwd: k_acc_blocked (the gather, ~3/4 of the time) + k_mix + pair sort",
             "bound": "hbm", "achieved": fwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": fwd_gbs / HBM_PEAK_GBS, "traffic": MEASURED_FWD_TRAFFIC.get(args.workload),
             "algorithmic_bytes_per_launch": fwd_bytes, "avg_launch_ms": fwd_ms,
