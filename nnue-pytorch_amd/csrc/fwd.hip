@@ -184,7 +184,7 @@ extern "C" int nnueft_sparse_fwd(const int32_t* idx, const float* W, const float
 
 extern "C" size_t nnueft_fwd_workspace_bytes(int B, int K, int R, int L1, int n_psqt) {
     if (B <= 0 || K <= 0 || R <= 0 || L1 <= 0 || n_psqt < 0) return 0;
-    return nnueft_blocked::pair_sort_workspace(B, R);
+    return nnueft_blocked::pair_sort_workspace(B, R, 0);
 }
 
 extern "C" int nnueft_double_fwd(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
@@ -199,7 +199,7 @@ extern "C" int nnueft_double_fwd(const float* us, const float* them, const int32
     const bool vec = (L1 % 8 == 0) && ((L1 + n_psqt) % 4 == 0) && aligned16(W) && aligned16(bias) &&
                      aligned16(l0) && aligned16(saved);
     if (workspace) {
-        if (!aligned256(workspace) || workspace_bytes < nnueft_blocked::pair_sort_workspace(B, R))
+        if (!aligned256(workspace) || workspace_bytes < nnueft_blocked::pair_sort_workspace(B, R, 0))
             return NNUEFT_E_WORKSPACE;
         // the L2-blocked path needs 16-byte rows; other shapes take the plain kernel below
         if (vec && (long long)B <= 0x3fffffffLL)

@@ -224,16 +224,16 @@ __global__ __launch_bounds__(64) void k_mix(const float* __restrict__ us, const 
 
 static inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-int table_block_rows(int R, int* nbins);
+int table_block_rows(int R, int hint, int* nbins);
 
 struct PairSortLayout {
     size_t order, keys, hist, end;
     int ngroups, nbins, block_rows;
 };
 
-bool pair_sort_layout(int B, int R, PairSortLayout* L) {
+bool pair_sort_layout(int B, int R, int block_rows_hint, PairSortLayout* L) {
     if (B <= 0 || R <= 0) return false;
-    L->block_rows = table_block_rows(R, &L->nbins);
+    L->block_rows = table_block_rows(R, block_rows_hint, &L->nbins);
     L->ngroups = (2 * B + kPairThreads - 1) / kPairThreads;
     size_t off = 0;
     L->order = off;
@@ -246,15 +246,15 @@ bool pair_sort_layout(int B, int R, PairSortLayout* L) {
     return true;
 }
 
-size_t pair_sort_workspace(int B, int R) {
+size_t pair_sort_workspace(int B, int R, int block_rows_hint) {
     PairSortLayout L;
-    return pair_sort_layout(B, R, &L) ? L.end : 0;
+    return pair_sort_layout(B, R, block_rows_hint, &L) ? L.end : 0;
 }
 
-int launch_pair_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, void* ws, hipStream_t st,
-                     const uint32_t** order_out) {
+int launch_pair_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, int block_rows_hint, void* ws,
+                     hipStream_t st, const uint32_t** order_out) {
     PairSortLayout L;
-    if (!pair_sort_layout(B, R, &L)) return NNUEFT_E_ARG;
+    if (!pair_sort_layout(B, R, block_rows_hint, &L)) return NNUEFT_E_ARG;
     char* base = (char*)ws;
     uint32_t* order = (uint32_t*)(base + L.order);
     uint32_t* keys = (uint32_t*)(base + L.keys);
@@ -271,8 +271,10 @@ int launch_pair_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int
     return 0;
 }
 
-int table_block_rows(int R, int* nbins) {
-    int block_rows = 768;
+// Rows per table block the pair sort tells apart: the hint (the caller's knowledge of the table's
+// block structure) or 768, widened when the table would have more than kMaxBins - 1 blocks.
+int table_block_rows(int R, int hint, int* nbins) {
+    int block_rows = hint > 0 ? hint : 768;
     if ((R + block_rows - 1) / block_rows + 1 > kMaxBins) block_rows = (R + kMaxBins - 2) / (kMaxBins - 1);
     *nbins = (R + block_rows - 1) / block_rows + 1;
     return block_rows;
@@ -283,7 +285,7 @@ int double_fwd_blocked(const float* us, const float* them, const int32_t* widx, 
                        float* wpsqt, float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt,
                        void* ws, hipStream_t st) {
     const uint32_t* order = nullptr;
-    const int rc = launch_pair_sort(widx, bidx, B, K, R, ws, st, &order);
+    const int rc = launch_pair_sort(widx, bidx, B, K, R, 0, ws, st, &order);
     if (rc) return rc;
     const int out_cols = L1 + n_psqt;
     const int nv = L1 / 4;

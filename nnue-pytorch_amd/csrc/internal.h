@@ -8,11 +8,11 @@ namespace nnueft_blocked {
 constexpr int kXcd = 8;   // XCDs of the device; workgroup id % kXcd is the XCD a workgroup lands on
 
 // Pair sort: order[] = ids (perspective * B + position) of the 2B index lists of a batch grouped by
-// the 768-row table block they name.  `ws` needs pair_sort_workspace() bytes; returns the order array
+// the table block they name (block_rows_hint rows per block, 0 = 768).  `ws` needs pair_sort_workspace() bytes; returns the order array
 // (inside ws) through *order.
-size_t pair_sort_workspace(int B, int R);
-int launch_pair_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, void* ws, hipStream_t st,
-                     const uint32_t** order);
+size_t pair_sort_workspace(int B, int R, int block_rows_hint);
+int launch_pair_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, int block_rows_hint, void* ws,
+                     hipStream_t st, const uint32_t** order);
 
 int double_fwd_blocked(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                        const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,

@@ -33,7 +33,8 @@ PROTOTYPES = {
     ),
     "nnueft_table_merge": (c_int, [c_void_p] * 3 + [c_int] * 4 + [c_float] * 2 + [c_int, c_void_p]),
     "nnueft_table_virtual_grad": (c_int, [c_void_p] * 2 + [c_int] * 3 + [c_void_p]),
-    "nnueft_ft_int16_fwd": (c_int, [c_void_p] * 9 + [c_int] * 7 + [c_void_p]),
+    "nnueft_int16_workspace_bytes": (c_size_t, [c_int] * 5),
+    "nnueft_ft_int16_fwd": (c_int, [c_void_p] * 9 + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
     "nnueft_stack_int8_fwd": (c_int, [c_void_p] * 9 + [c_int] * 12 + [c_void_p]),
 }
 

@@ -38,10 +38,13 @@ def quantize_feature_transformer(weight: torch.Tensor, bias: torch.Tensor, l1_si
 
 
 def ft_int16_forward(white_indices, black_indices, stm, w16, b16, psqt32, psqt_indices,
-                     clip_max: int = FT_QUANTIZED_MAX, shift: int = L0_SHIFT):
+                     clip_max: int = FT_QUANTIZED_MAX, shift: int = L0_SHIFT, table_block_rows: int = 0,
+                     use_workspace: bool = True):
     """Returns (u8 [B, L1] with the side to move's half first, int32 [B] psqt difference / 2).
 
     stm: uint8 [B], 0 = white to move, 1 = black to move.
+    table_block_rows: rows per king bucket of the table (scheduling hint); 0 picks 704 for the
+    22528-row exported table and 768 otherwise.
     """
     assert white_indices.is_cuda, "the quantized path has a GPU implementation only"
     assert white_indices.dtype == torch.int32 and black_indices.dtype == torch.int32
@@ -62,11 +65,16 @@ def ft_int16_forward(white_indices, black_indices, stm, w16, b16, psqt32, psqt_i
     out = torch.empty(B, L1, dtype=torch.uint8, device=device)
     psqt = torch.empty(B, dtype=torch.int32, device=device)
     lib = _native.load()
+    if table_block_rows == 0 and R == 22528:
+        table_block_rows = 704
+    nbytes = lib.nnueft_int16_workspace_bytes(B, K, R, L1, table_block_rows) if (use_workspace and B > 0) else 0
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
     with torch.cuda.device(device):
         rc = lib.nnueft_ft_int16_fwd(
             white_indices.data_ptr(), black_indices.data_ptr(), stm.data_ptr(), w16.data_ptr(), b16.data_ptr(),
             psqt32.data_ptr(), psqt_indices.data_ptr(), out.data_ptr(), psqt.data_ptr(),
-            B, K, R, L1, psqt32.shape[1], int(clip_max), int(shift), _stream_ptr(device),
+            B, K, R, L1, psqt32.shape[1], int(clip_max), int(shift), int(table_block_rows),
+            ws.data_ptr() if nbytes else None, nbytes, _stream_ptr(device),
         )
     _native.check(rc, "nnueft_ft_int16_fwd")
     return out, psqt

@@ -271,7 +271,7 @@ def test_abi_rejects_bad_arguments():
     assert lib.nnueft_sparse_bwd_det(p, p, p, p, 4, 8, 10, 8, p, 16, st) == -2      # workspace too small
     assert lib.nnueft_sparse_bwd_det(p, p, p, p, 4, 8, 10, 8, 0, 1 << 20, st) == -2  # workspace missing
     assert lib.nnueft_sparse_bwd_det(p, p, p, p, 4, 8, 10, 8, p + 4, 1 << 20, st) == -2  # misaligned
-    assert lib.nnueft_ft_int16_fwd(p, p, p, p, p, p, p, p, p, 4, 8, 10, 8, 8, 70000, 9, st) == -1   # clip_max
+    assert lib.nnueft_ft_int16_fwd(p, p, p, p, p, p, p, p, p, 4, 8, 10, 8, 8, 70000, 9, 0, None, 0, st) == -1   # clip_max
     with pytest.raises(RuntimeError, match="invalid argument"):
         _native.check(-1, "x")
     torch.cuda.synchronize()

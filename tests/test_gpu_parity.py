@@ -203,9 +203,10 @@ def test_deterministic_backward_repeats_bitwise():
 INT16_SHAPES = [(5, 32, 50, 32), (33, 1024, 22528, 32), (17, 3072, 22528, 32), (9, 38, 40, 70)]
 
 
+@pytest.mark.parametrize("use_workspace", [False, True], ids=["plain", "l2blocked"])
 @pytest.mark.parametrize("B,L1,R,K", INT16_SHAPES)
 @pytest.mark.parametrize("clip_max,shift", [(255, 9), (127, 7)])
-def test_int16_forward(oracle_cpu, B, L1, R, K, clip_max, shift):
+def test_int16_forward(oracle_cpu, B, L1, R, K, clip_max, shift, use_workspace):
     rng = np.random.default_rng(600 + B)
     from _cases import random_lists
 
@@ -220,7 +221,8 @@ def test_int16_forward(oracle_cpu, B, L1, R, K, clip_max, shift):
     psqt_idx = rng.integers(0, 8, size=B).astype(np.int64)
     from nnueft.quantized import ft_int16_forward
 
-    out, ps = ft_int16_forward(_t(widx), _t(bidx), _t(stm), _t(W16), _t(b16), _t(psqt32), _t(psqt_idx), clip_max, shift)
+    out, ps = ft_int16_forward(_t(widx), _t(bidx), _t(stm), _t(W16), _t(b16), _t(psqt32), _t(psqt_idx), clip_max, shift,
+                               use_workspace=use_workspace)
     r_out, r_ps = oracle_cpu.ft_int16_fwd(widx, bidx, stm, W16, b16, psqt32, psqt_idx, clip_max, shift)
     assert np.array_equal(out.cpu().numpy(), r_out)
     assert np.array_equal(ps.cpu().numpy(), r_ps)
