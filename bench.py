@@ -135,19 +135,35 @@ def run_int16(args, lib, dev):
     w16, b16, p32 = w16.to(dev), b16.to(dev), p32.to(dev)
     sum_a = int((white >= 0).sum() + (black >= 0).sum())
 
-    def step():
-        quantized.ft_int16_forward(wi, bi, stm, w16, b16, p32, pi)
+    from nnueft import model as M
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(args.steps):
-        step()
-    e1.record()
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / args.steps
+    torch.manual_seed(5)
+    stacks = M.LayerStacks(8, M.ModelConfig(L1=L1, L2=32, L3=32), M.QuantizationManager(M.QuantizationConfig()))
+    with torch.no_grad():
+        stacks.l1.linear.weight.mul_(0.5)
+    stack_q = [x.to(dev) for x in quantized.quantize_layer_stacks(stacks)]
+
+    def step():
+        return quantized.ft_int16_forward(wi, bi, stm, w16, b16, p32, pi)
+
+    def chain():
+        x_u8, psqt = quantized.ft_int16_forward(wi, bi, stm, w16, b16, p32, pi)
+        return quantized.stack_int8_forward(x_u8, pi, *stack_q) + psqt
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    ms = timed(step)
+    ms_chain = timed(chain)
     alg = sum_a * L1 * 2 + B * (2 * K_SLOTS * 4 + L1)
     print(json.dumps({
         "metric": "quantized FT forward positions/sec (int16 accumulate, L1=3072, B=65536)",
@@ -155,7 +171,8 @@ def run_int16(args, lib, dev):
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int16",
         "data": "synthetic",
         "config": {"workload": args.workload, "L1": L1, "batch": B, "table_rows": R,
-                   "active_rows_per_position": sum_a / B},
+                   "active_rows_per_position": sum_a / B,
+                   "with_int8_layer_stacks_ms": ms_chain, "with_int8_layer_stacks_positions_per_s": B / (ms_chain * 1e-3)},
         "roofline": {"kernel": "nnueft_ft_int16_fwd", "bound": "hbm", "achieved": alg / (ms * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "traffic": None, "algorithmic_bytes_per_launch": alg, "avg_launch_ms": ms},
