@@ -91,10 +91,14 @@ __global__ __launch_bounds__(64) void k_bwd_rows(const float* __restrict__ us, c
                                                  const float* __restrict__ grad_wpsqt,
                                                  const float* __restrict__ grad_bpsqt,
                                                  const float* __restrict__ saved, float* __restrict__ G,
-                                                 float* __restrict__ partial, int B, int L1, int n_psqt) {
+                                                 float* __restrict__ partial, int B, int L1, int n_psqt, int group,
+                                                 int ntiles) {
+    // `group` lanes share a tile (64 for wide rows; narrow rows put 64 / group tiles into one wave)
     const int lane = threadIdx.x;
-    const int tile = blockIdx.x;
+    const int tile = blockIdx.x * (64 / group) + lane / group;
+    const int ql = lane % group;
     const int s = blockIdx.y;
+    if (tile >= ntiles) return;
     const int h = L1 >> 1;
     const int hv = h / VW;
     const size_t out_cols = (size_t)L1 + n_psqt;
@@ -103,7 +107,7 @@ __global__ __launch_bounds__(64) void k_bwd_rows(const float* __restrict__ us, c
     float* Gw = G;
     float* Gb = G + (size_t)B * out_cols;
 
-    const int q = s * 64 + lane;
+    const int q = s * group + ql;
     if (q < hv) {
         const int c = q * VW;
         vecf<VW> part0 = vzero<VW>(), part1 = vzero<VW>();
@@ -134,7 +138,7 @@ __global__ __launch_bounds__(64) void k_bwd_rows(const float* __restrict__ us, c
         stv<VW>(partial + (size_t)tile * out_cols + h + c, part1);
     }
     if (s == 0) {
-        for (int j = lane; j < n_psqt; j += 64) {
+        for (int j = ql; j < n_psqt; j += group) {
             float part = 0.0f;
             for (int b = b0; b < b1; ++b) {
                 const bool hit = psqt_idx[b] == (int64_t)j;
@@ -260,10 +264,10 @@ __device__ __forceinline__ int xcd_of(unsigned long long w, unsigned long long d
 // Also the work split of the segmented reduction: the rows named by >= kLongRow slots (their chains
 // are long and start first), and kXcd contiguous row ranges of equal weight (slots + 1 per row).
 constexpr int kScanThreads = 1024;
-constexpr int kScanPer = 32;   // rows a thread keeps in registers per pass
 __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict__ seg_off,
                                                            uint32_t* __restrict__ long_rows,
-                                                           uint32_t* __restrict__ sched, int R) {
+                                                           uint32_t* __restrict__ sched, int R, int cap) {
+    extern __shared__ uint32_t stage[];   // `cap` row lengths, turned into offsets in place
     __shared__ uint32_t wave_tot[kScanThreads / 64];
     __shared__ uint32_t carry_s, n_long_s;
     __shared__ uint32_t lo_s[kXcd + 1];
@@ -275,36 +279,43 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
     if (tid <= kXcd) lo_s[tid] = (uint32_t)R;
     if (tid < kXcd) sched[kSchedCtr + tid * 32] = 0;
     __syncthreads();
-    for (int base = 0; base < R; base += kScanThreads * kScanPer) {
-        const int r0 = base + tid * kScanPer;
-        uint32_t len[kScanPer];
-        uint32_t local = 0;
+    for (int base = 0; base < R; base += cap) {
+        const int n = min(cap, R - base);
+        // coalesced loads, 8 in flight per thread
+        for (int i0 = tid; i0 < n; i0 += kScanThreads * 8) {
+            uint32_t v[8];
 #pragma unroll
-        for (int u = 0; u < kScanPer; ++u) {
-            len[u] = (r0 + u < R) ? seg_off[r0 + u] : 0;
-            local += len[u];
+            for (int u = 0; u < 8; ++u) v[u] = (i0 + u * kScanThreads < n) ? seg_off[base + i0 + u * kScanThreads] : 0;
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (i0 + u * kScanThreads < n) stage[i0 + u * kScanThreads] = v[u];
         }
+        __syncthreads();
+        // a thread scans `per` consecutive rows (odd count: its LDS reads then spread over all banks)
+        const int per = ((n + kScanThreads - 1) / kScanThreads) | 1;
+        const int i_beg = min(tid * per, n), i_end = min(i_beg + per, n);
+        uint32_t local = 0;
+        for (int i = i_beg; i < i_end; ++i) local += stage[i];
         uint32_t incl = local;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
-            const uint32_t v = __shfl_up(incl, off);
-            if ((tid & 63) >= off) incl += v;
+            const uint32_t t = __shfl_up(incl, off);
+            if ((tid & 63) >= off) incl += t;
         }
         if ((tid & 63) == 63) wave_tot[tid >> 6] = incl;
         __syncthreads();
-        uint32_t before = carry_s;
-        for (int w = 0; w < (tid >> 6); ++w) before += wave_tot[w];
-        uint32_t run = before + incl - local;
-#pragma unroll
-        for (int u = 0; u < kScanPer; ++u) {
-            if (r0 + u < R) {
-                if (len[u] >= (uint32_t)kLongRow) long_rows[atomicAdd(&n_long_s, 1u)] = (uint32_t)(r0 + u);
-                seg_off[r0 + u] = run;
-                run += len[u];
-            }
+        uint32_t run = carry_s;
+        for (int w = 0; w < (tid >> 6); ++w) run += wave_tot[w];
+        run += incl - local;
+        for (int i = i_beg; i < i_end; ++i) {
+            const uint32_t len = stage[i];
+            if (len >= (uint32_t)kLongRow) long_rows[atomicAdd(&n_long_s, 1u)] = (uint32_t)(base + i);
+            stage[i] = run;
+            run += len;
         }
         __syncthreads();
         if (tid == kScanThreads - 1) carry_s = run;
+        for (int i = tid; i < n; i += kScanThreads) seg_off[base + i] = stage[i];
         __syncthreads();
     }
     const uint32_t total = carry_s;
@@ -511,6 +522,13 @@ int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, fl
     size_t hist_bytes = 0, fill_bytes = 0;
     if (!lds_plan(R, K, &range, &stage, &hist_bytes, &fill_bytes)) return NNUEFT_E_UNSUPPORTED;
     const int nranges = (R + range - 1) / range;
+    // rows the single-workgroup row scan stages in LDS at a time (`range` fits by construction)
+    const int scan_cap = max(kScanThreads, min(range, (R + kScanThreads - 1) / kScanThreads * kScanThreads));
+    if ((size_t)scan_cap * sizeof(uint32_t) > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void*)k_row_scan, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)(scan_cap * sizeof(uint32_t)));
+        if (e != hipSuccess) return (int)e;
+    }
     if (fill_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void*)k_chunk_hist, hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)hist_bytes);
@@ -524,7 +542,8 @@ int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, fl
     hipLaunchKernelGGL(k_col_scan, dim3((R + 63) / 64), dim3(64), 0, st, cnt, wcount, seg_off, R, L.cpp,
                        L.nchunks);
     NNUEFT_LAUNCH_CHECK();
-    hipLaunchKernelGGL(k_row_scan, dim3(1), dim3(kScanThreads), 0, st, seg_off, long_rows, sched, R);
+    hipLaunchKernelGGL(k_row_scan, dim3(1), dim3(kScanThreads), (size_t)scan_cap * sizeof(uint32_t), st, seg_off,
+                       long_rows, sched, R, scan_cap);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_fill, dim3(L.nchunks, nranges), dim3(256), fill_bytes, st, widx, bidx, cnt, seg_off, list,
                        B, K, R, L.cpp, range, stage);
@@ -565,13 +584,16 @@ int launch_bwd_rows(const float* us, const float* them, const int64_t* psqt_idx,
     const bool vec = (L1 % 8 == 0) && (out_cols % 4 == 0) && aligned16(grad_l0) && aligned16(saved) &&
                      aligned16(bias) && aligned16(G) && aligned16(partial);
     const int hv = (L1 / 2) / (vec ? 4 : 1);
-    const dim3 grid(ntiles, max(1, (hv + 63) / 64));
+    int group = 64;
+    while (group > 8 && group / 2 >= hv) group /= 2;   // lanes per tile: 64, 32, 16 or 8
+    const int tiles_per_wave = 64 / group;
+    const dim3 grid((ntiles + tiles_per_wave - 1) / tiles_per_wave, max(1, (hv + group - 1) / group));
     if (vec)
         hipLaunchKernelGGL(k_bwd_rows<4>, grid, dim3(64), 0, st, us, them, psqt_idx, bias, max_act, grad_l0,
-                           grad_wpsqt, grad_bpsqt, saved, G, partial, B, L1, n_psqt);
+                           grad_wpsqt, grad_bpsqt, saved, G, partial, B, L1, n_psqt, group, ntiles);
     else
         hipLaunchKernelGGL(k_bwd_rows<1>, grid, dim3(64), 0, st, us, them, psqt_idx, bias, max_act, grad_l0,
-                           grad_wpsqt, grad_bpsqt, saved, G, partial, B, L1, n_psqt);
+                           grad_wpsqt, grad_bpsqt, saved, G, partial, B, L1, n_psqt, group, ntiles);
     NNUEFT_LAUNCH_CHECK();
     return 0;
 }
