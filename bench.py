@@ -53,12 +53,12 @@ def algorithmic_bytes(L1, B, sum_a, mode):
     return fwd, bwd
 
 
-def make_inputs(L1, B, seed, device):
+def make_inputs(L1, B, seed, device, castled_kings=0.0):
     import numpy as np
     import torch
     from nnueft import halfka_v2_hm as hk
 
-    us, them, white, black, pc = hk.synthetic_batch(B, seed)
+    us, them, white, black, pc = hk.synthetic_batch(B, seed, castled_kings=castled_kings)
     rng = np.random.default_rng(seed)
     oc = L1 + N_PSQT
     g = torch.Generator(device="cpu").manual_seed(seed)
@@ -236,6 +236,9 @@ def main():
     ap.add_argument("--backward", default="deterministic", choices=["deterministic", "atomic"],
                     help="backward mode the headline value is measured with (the other one is reported beside it)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--castled-kings", type=float, default=0.0,
+                    help="fraction of positions with the kings on g1/g8 (robustness runs: a skewed bucket "
+                         "distribution like real game data); the headline workload uses 0")
     ap.add_argument("--only", default="", choices=["", "fwd", "det", "atomic", "copy"],
                     help="run only this part (for profiling runs); 'copy' launches a plain elementwise kernel "
                          "reading and writing 1 GiB each, the yardstick the FETCH_SIZE/WRITE_SIZE counters are scaled by")
@@ -272,7 +275,7 @@ def main():
         return
     L1, B = WORKLOADS[args.workload]
     seed = 1234 + 3
-    t, sum_a = make_inputs(L1, B, seed, dev)
+    t, sum_a = make_inputs(L1, B, seed, dev, args.castled_kings)
     W = t["W"].requires_grad_()
     bias = t["bias"].requires_grad_()
     max_act = 255.0 / 256.0
@@ -377,7 +380,7 @@ def main():
         "config": {
             "workload": args.workload, "L1": L1, "batch": B, "table_rows": R_ROWS, "psqt_columns": N_PSQT,
             "slots": K_SLOTS, "active_rows_per_position": sum_a / B, "backward": head_mode,
-            "index_scheme": "HalfKAv2_hm, seeded random positions",
+            "index_scheme": "HalfKAv2_hm, seeded random positions", "castled_kings": args.castled_kings,
         },
         "roofline": {
             "kernel": "nnueft_double_fwd: k_acc_blocked (the gather, ~3/4 of the time) + k_mix + pair sort",

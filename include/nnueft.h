@@ -21,6 +21,13 @@
  *                  +0 over the slots naming that row in ascending (position, slot) order; then
  *                  white chain + black chain.  This is the order of torch's CPU embedding_bag
  *                  backward, i.e. of the reference's CPU path.
+ *                  Exception, for speed on batches where a few rows are named by a large part of
+ *                  the positions: a table row named by more than nnueft_row_split() slots of the
+ *                  batch (both perspectives together) is summed window by window.  Window w holds
+ *                  positions [w * nnueft_row_window(B), (w + 1) * nnueft_row_window(B)); per
+ *                  perspective, each window's slots are chained from +0 as above, the window sums
+ *                  are chained from +0 in ascending w, and the two perspectives are added.  Such
+ *                  a row agrees with the CPU path to rounding, not bit for bit.
  *   bias grad      (deterministic entry points) positions are cut into tiles of nnueft_bias_tile();
  *                  per column a chain over a tile's positions, then a chain over the tile sums.
  *   The atomic entry points add in an unspecified order.
@@ -46,6 +53,11 @@ const char* nnueft_error_string(int code);
 
 /* Positions per tile of the deterministic bias-gradient order. */
 int nnueft_bias_tile(void);
+
+/* Deterministic weight-gradient order: rows named by more slots than nnueft_row_split() are summed
+ * in windows of nnueft_row_window(B) positions (see "Summation order" above). */
+int nnueft_row_split(void);
+int nnueft_row_window(int B);
 
 /*
  * out[b,:] = (sum_k W[idx[b,k],:]) + bias.

@@ -4,6 +4,8 @@
 extern "C" int nnueft_version(void) { return NNUEFT_VERSION; }
 
 extern "C" int nnueft_bias_tile(void) { return NNUEFT_BIAS_TILE; }
+extern "C" int nnueft_row_split(void) { return NNUEFT_ROW_SPLIT; }
+extern "C" int nnueft_row_window(int B) { return B > 0 ? nnueft_window_positions(B) : 0; }
 
 extern "C" const char* nnueft_error_string(int code) {
     switch (code) {

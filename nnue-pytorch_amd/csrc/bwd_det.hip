@@ -13,7 +13,13 @@
 //   k_seg_reduce    persistent waves, one task = (table row, column slice): white chain, black
 //                   chain, sum, store.  Rows are dealt to the 8 XCDs in contiguous ranges of equal
 //                   work and walked one column slice at a time, so the upstream rows a XCD gathers
-//                   (those of the positions of one king bucket, one slice wide) stay in its L2
+//                   (those of the positions of one king bucket, one slice wide) stay in its L2.
+//                   A row named by more than NNUEFT_ROW_SPLIT slots (a king bucket that holds a
+//                   large part of the batch has many) is cut at the window boundaries instead: one
+//                   task per (row, perspective, window, slice) writes that window's sum, and a XCD
+//                   takes whole (perspective, window) pairs, so what it gathers is one slice of
+//                   one window's upstream rows
+//   k_split_combine the window sums of a split row: chain over the windows, white + black
 //   k_bias_final    chain over the tile partial sums
 #include "gather.h"
 #include "internal.h"
@@ -37,18 +43,29 @@ constexpr int kWavesPerXcd = NNUEFT_SEG_WAVES;  // persistent waves per XCD in t
 #define NNUEFT_LONG_ROW 256
 #endif
 constexpr int kLongRow = NNUEFT_LONG_ROW;  // table rows named by at least this many slots are reduced first
+static_assert(NNUEFT_ROW_SPLIT >= NNUEFT_LONG_ROW, "split rows are skipped where long rows are");
+#ifndef NNUEFT_RUN_U
+#define NNUEFT_RUN_U 16
+#endif
+constexpr int kRunUnroll = NNUEFT_RUN_U;   // rows in flight per lane in the chain of one window of a split row
+constexpr uint32_t kSplitFlag = 0x80000000u;   // on a row's slot count between k_col_scan and k_row_scan
 
 // Work split of the segmented reduction, written by k_row_scan (uint32 words).
-constexpr int kSchedCtr = 0;       // kXcd task counters, 32 words (128 bytes) apart
-constexpr int kSchedNLong = kXcd * 32;
-constexpr int kSchedRowLo = kSchedNLong + 1;   // kXcd + 1 range bounds
+constexpr int kSchedCtr = 0;       // kXcd * kSchedQueues task counters, 32 words (128 bytes) apart
+constexpr int kSchedQueues = 16;   // room for that many counters per XCD
+constexpr int kSchedNLong = kXcd * kSchedQueues * 32;         // long_rows[0 .. n_long): long rows that are not split
+constexpr int kSchedNSplit = kSchedNLong + 1;  // long_rows[R - n_split .. R), from the back: split rows
+constexpr int kSchedRowLo = kSchedNSplit + 1;  // kXcd + 1 range bounds
 constexpr int kSchedWords = kSchedRowLo + kXcd + 1;
 
 struct DetLayout {
-    size_t G, partial, cnt, wcount, seg_off, long_rows, sched, list, end;
+    size_t G, partial, cnt, wcount, seg_off, long_rows, wpre, sched, list, runs, end;
     int cpp;     // chunks per perspective
     int nchunks; // n_persp * cpp
     int ntiles;  // bias tiles
+    int wch;     // chunks per window of a split row
+    int nwin;    // windows
+    int max_split;   // most rows that can be split
 };
 
 inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -71,10 +88,19 @@ bool det_layout(int B, int K, int R, int out_cols, int n_persp, DetLayout* L) {
     off += up256(((size_t)R + 1) * sizeof(uint32_t));
     L->long_rows = off;
     off += up256((size_t)R * sizeof(uint32_t));
+    L->wpre = off;
+    off += up256((size_t)R * sizeof(uint32_t));
     L->sched = off;
     off += up256((size_t)kSchedWords * sizeof(uint32_t));
     L->list = off;
     off += up256((size_t)n_persp * B * K * sizeof(uint32_t));
+    static_assert(NNUEFT_ROW_WINDOW_MIN % kChunk == 0, "windows are whole sort chunks");
+    const int wpos = nnueft_window_positions(B);
+    L->wch = wpos / kChunk;
+    L->nwin = (B + wpos - 1) / wpos;
+    L->max_split = (int)(((long long)n_persp * B * K) / (NNUEFT_ROW_SPLIT + 1));
+    L->runs = off;
+    off += up256((size_t)L->max_split * n_persp * L->nwin * out_cols * sizeof(float));
     L->end = off;
     return true;
 }
@@ -249,7 +275,7 @@ __global__ __launch_bounds__(64) void k_col_scan(uint32_t* __restrict__ cnt, uin
     }
     if (nchunks == cpp) white = run;
     wcount[r] = white;
-    seg_off[r] = run;
+    seg_off[r] = run > (uint32_t)NNUEFT_ROW_SPLIT ? (run | kSplitFlag) : run;
 }
 
 // floor(kXcd * w / denom) for w < denom, without a 64-bit division
@@ -261,23 +287,33 @@ __device__ __forceinline__ int xcd_of(unsigned long long w, unsigned long long d
 }
 
 // Single workgroup: seg_off (holding per-row totals) -> exclusive offsets, seg_off[R] = grand total.
-// Also the work split of the segmented reduction: the rows named by >= kLongRow slots (their chains
-// are long and start first), and kXcd contiguous row ranges of equal weight (slots + 1 per row).
+// Also the work split of the segmented reduction: the split rows (flagged by k_col_scan), the other
+// rows named by >= kLongRow slots (their chains are long and start first), and kXcd contiguous row
+// ranges of equal weight (kRowWeight per row, plus its slots unless the row is split: those are
+// reduced elsewhere).
+#ifndef NNUEFT_ROW_WEIGHT
+#define NNUEFT_ROW_WEIGHT 8
+#endif
+constexpr uint32_t kRowWeight = NNUEFT_ROW_WEIGHT;   // cost of a task that finds nothing to add, in slots
 constexpr int kScanThreads = 1024;
 __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict__ seg_off,
                                                            uint32_t* __restrict__ long_rows,
+                                                           uint32_t* __restrict__ wpre,
                                                            uint32_t* __restrict__ sched, int R, int cap) {
     extern __shared__ uint32_t stage[];   // `cap` row lengths, turned into offsets in place
-    __shared__ uint32_t wave_tot[kScanThreads / 64];
-    __shared__ uint32_t carry_s, n_long_s;
+    // two running sums: all slots, slots of split rows
+    __shared__ uint32_t wave_tot[2][kScanThreads / 64];
+    __shared__ uint32_t carry_s[2], n_long_s, n_split_s;
     __shared__ uint32_t lo_s[kXcd + 1];
     const int tid = threadIdx.x;
     if (tid == 0) {
-        carry_s = 0;
+        carry_s[0] = 0;
+        carry_s[1] = 0;
         n_long_s = 0;
+        n_split_s = 0;
     }
     if (tid <= kXcd) lo_s[tid] = (uint32_t)R;
-    if (tid < kXcd) sched[kSchedCtr + tid * 32] = 0;
+    if (tid < kXcd * kSchedQueues) sched[kSchedCtr + tid * 32] = 0;
     __syncthreads();
     for (int base = 0; base < R; base += cap) {
         const int n = min(cap, R - base);
@@ -294,52 +330,79 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
         // a thread scans `per` consecutive rows (odd count: its LDS reads then spread over all banks)
         const int per = ((n + kScanThreads - 1) / kScanThreads) | 1;
         const int i_beg = min(tid * per, n), i_end = min(i_beg + per, n);
-        uint32_t local = 0;
-        for (int i = i_beg; i < i_end; ++i) local += stage[i];
-        uint32_t incl = local;
+        uint32_t local[2] = {0, 0};
+        for (int i = i_beg; i < i_end; ++i) {
+            const uint32_t raw = stage[i];
+            local[0] += raw & ~kSplitFlag;
+            local[1] += (raw & kSplitFlag) ? (raw & ~kSplitFlag) : 0u;
+        }
+        uint32_t incl[2] = {local[0], local[1]};
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
-            const uint32_t t = __shfl_up(incl, off);
-            if ((tid & 63) >= off) incl += t;
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+                const uint32_t t = __shfl_up(incl[k], off);
+                if ((tid & 63) >= off) incl[k] += t;
+            }
         }
-        if ((tid & 63) == 63) wave_tot[tid >> 6] = incl;
+        if ((tid & 63) == 63) {
+            wave_tot[0][tid >> 6] = incl[0];
+            wave_tot[1][tid >> 6] = incl[1];
+        }
         __syncthreads();
-        uint32_t run = carry_s;
-        for (int w = 0; w < (tid >> 6); ++w) run += wave_tot[w];
-        run += incl - local;
+        uint32_t run[2];
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            run[k] = carry_s[k] + incl[k] - local[k];
+            for (int w = 0; w < (tid >> 6); ++w) run[k] += wave_tot[k][w];
+        }
         for (int i = i_beg; i < i_end; ++i) {
-            const uint32_t len = stage[i];
-            if (len >= (uint32_t)kLongRow) long_rows[atomicAdd(&n_long_s, 1u)] = (uint32_t)(base + i);
-            stage[i] = run;
-            run += len;
+            const uint32_t raw = stage[i];
+            const uint32_t len = raw & ~kSplitFlag;
+            stage[i] = run[0];
+            wpre[base + i] = run[0] - run[1];   // slots of the rows before this one that are not split
+            // a row is in at most one of the two lists, so they cannot meet inside long_rows[0..R)
+            if (raw & kSplitFlag) {
+                long_rows[R - 1 - (int)atomicAdd(&n_split_s, 1u)] = (uint32_t)(base + i);
+                run[1] += len;
+            } else if (len >= (uint32_t)kLongRow) {
+                long_rows[atomicAdd(&n_long_s, 1u)] = (uint32_t)(base + i);
+            }
+            run[0] += len;
         }
         __syncthreads();
-        if (tid == kScanThreads - 1) carry_s = run;
+        if (tid == kScanThreads - 1) {
+            carry_s[0] = run[0];
+            carry_s[1] = run[1];
+        }
         for (int i = tid; i < n; i += kScanThreads) seg_off[base + i] = stage[i];
         __syncthreads();
     }
-    const uint32_t total = carry_s;
+    const uint32_t total = carry_s[0];
     if (tid == 0) {
         seg_off[R] = total;
         sched[kSchedNLong] = n_long_s;
+        sched[kSchedNSplit] = n_split_s;
     }
-    __syncthreads();   // seg_off now holds exclusive offsets (written by this workgroup)
-    // XCD of a row = floor(kXcd * (slots before it + rows before it) / (all slots + all rows))
-    const unsigned long long denom = (unsigned long long)total + (unsigned long long)R;
+    __syncthreads();   // seg_off and wpre are complete (written by this workgroup)
+    // XCD of a row = floor(kXcd * weight of the rows before it / weight of all rows)
+    const unsigned long long denom =
+        (unsigned long long)(total - carry_s[1]) + (unsigned long long)R * kRowWeight;
     for (int rb = tid; rb < R; rb += kScanThreads * 8) {
         uint32_t off[8], prev[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int r = rb + u * kScanThreads;
-            off[u] = r < R ? seg_off[r] : 0;
-            prev[u] = (r < R && r > 0) ? seg_off[r - 1] : 0;
+            off[u] = r < R ? wpre[r] : 0;
+            prev[u] = (r < R && r > 0) ? wpre[r - 1] : 0;
         }
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int r = rb + u * kScanThreads;
             if (r < R) {
-                const int x = xcd_of((unsigned long long)off[u] + r, denom);
-                const int xp = r > 0 ? xcd_of((unsigned long long)prev[u] + (r - 1), denom) : -1;
+                const int x = xcd_of((unsigned long long)off[u] + (unsigned long long)r * kRowWeight, denom);
+                const int xp =
+                    r > 0 ? xcd_of((unsigned long long)prev[u] + (unsigned long long)(r - 1) * kRowWeight, denom) : -1;
                 for (int k = xp + 1; k <= x; ++k) lo_s[k] = (uint32_t)r;
             }
         }
@@ -403,7 +466,7 @@ __global__ __launch_bounds__(256) void k_fill(const int32_t* __restrict__ widx, 
 // ---------------------------------------------------------------------------------------------
 // Segmented reduction.  list[seg_off[r] .. +wcount[r]) are the white-perspective rows of G naming
 // table row r, the rest of the segment the black ones.  gW[r] = white chain (+ black chain).
-template <int VW, int NQ>
+template <int VW, int NQ, int U>
 __device__ __forceinline__ void seg_reduce_task(const float* __restrict__ G, const uint32_t* __restrict__ list,
                                                 uint32_t beg, uint32_t mid, uint32_t end, float* __restrict__ dst,
                                                 int s, int lane, int out_cols, int slice_v, int two_persp) {
@@ -427,7 +490,7 @@ __device__ __forceinline__ void seg_reduce_task(const float* __restrict__ G, con
             const uint32_t n = min(64u, e_end - e0);
             const int my = lane < (int)n ? (int)list[e0 + lane] : 0;
             const u64 mask = n >= 64 ? ~0ull : ((1ull << n) - 1ull);
-            chain_rows<VW, NQ, kRowsUnroll>(acc[p], G, (size_t)out_cols, col, my, mask);
+            chain_rows<VW, NQ, U>(acc[p], G, (size_t)out_cols, col, my, mask);
         }
     }
 #pragma unroll
@@ -438,51 +501,128 @@ __device__ __forceinline__ void seg_reduce_task(const float* __restrict__ G, con
     }
 }
 
+// Atomics on one address complete one after the other, some tens of nanoseconds each, so a single
+// counter that every task of a XCD goes through bounds the run time of the kernel.  Each XCD
+// therefore has kQueues counters; counter q hands out the tasks q, q + kQueues, q + 2 kQueues, ...
+#ifndef NNUEFT_SEG_QUEUES
+#define NNUEFT_SEG_QUEUES 8
+#endif
+constexpr int kQueues = NNUEFT_SEG_QUEUES;
 __device__ __forceinline__ uint32_t next_task(uint32_t* ctr, int lane) {
     uint32_t t = 0;
     if (lane == 0) t = atomicAdd(ctr, 1u);
     return (uint32_t)__builtin_amdgcn_readfirstlane((int)t);
 }
 
-// Persistent waves.  Each XCD has its own task counter; a wave takes the next task of its XCD until
-// none is left (the counter only grows, so every wave leaves the loop).  Task order per XCD: the
-// long rows dealt to it (all slices of a row together), then its row range, slice by slice.
+// What the reduction needs to know about the windows of split rows.
+struct RunPlan {
+    const uint32_t* cnt;   // [nchunks, R] offset of a chunk inside the row's segment
+    float* runs;           // [split row, perspective, window, out_cols] window sums
+    int R, cpp, nchunks, wch, nwin, n_persp;
+    int nslices, slice_v;  // 64-lane slices
+};
+
+// Persistent waves.  A wave takes tasks from its home queue of its XCD, then from the XCD's other
+// queues, until none is left (a counter only grows, so every wave leaves every loop).  Task order per XCD: the
+// windows of the split rows, (perspective, window) pair after pair of those dealt to it, slice by
+// slice; the long rows dealt to it (all slices of a row together); then its row range, slice by slice.
 template <int VW, int NQ>
 __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, const uint32_t* __restrict__ list,
                                                    const uint32_t* __restrict__ seg_off,
                                                    const uint32_t* __restrict__ wcount,
                                                    const uint32_t* __restrict__ long_rows,
                                                    uint32_t* __restrict__ sched, float* __restrict__ gW,
-                                                   int out_cols, int nslices, int slice_v, int two_persp) {
+                                                   int out_cols, int nslices, int slice_v, int two_persp,
+                                                   RunPlan rp) {
     const int lane = threadIdx.x;
     const int xcd = blockIdx.x % kXcd;
-    const uint32_t n_long = sched[kSchedNLong];
+    const uint32_t n_long = sched[kSchedNLong], n_split = sched[kSchedNSplit];
+    const uint32_t npairs = (uint32_t)(rp.n_persp * rp.nwin);
+    const uint32_t my_pairs = npairs > (uint32_t)xcd ? (npairs - xcd + kXcd - 1) / kXcd : 0;
+    const uint32_t pair_tasks = (uint32_t)rp.nslices * n_split;
+    const uint32_t run_tasks = my_pairs * pair_tasks;
     const uint32_t my_long = n_long > (uint32_t)xcd ? (n_long - xcd + kXcd - 1) / kXcd : 0;
     const uint32_t lo = sched[kSchedRowLo + xcd], hi = sched[kSchedRowLo + xcd + 1];
     const uint32_t nreg = hi - lo;
-    const uint32_t long_tasks = my_long * (uint32_t)nslices;
-    const uint32_t ntasks = long_tasks + nreg * (uint32_t)nslices;
-    uint32_t* ctr = sched + kSchedCtr + xcd * 32;
+    const uint32_t long_end = run_tasks + my_long * (uint32_t)nslices;
+    const uint32_t ntasks = long_end + nreg * (uint32_t)nslices;
+    static_assert(kQueues <= kSchedQueues, "counters per XCD");
+    const int home = (blockIdx.x / kXcd) % kQueues;
 
+  for (int qi = 0; qi < kQueues; ++qi) {
+    const uint32_t q = (uint32_t)((home + qi) % kQueues);
+    uint32_t* ctr = sched + kSchedCtr + (xcd * kSchedQueues + (int)q) * 32;
+    const uint32_t nq = ntasks > q ? (ntasks - q + kQueues - 1) / kQueues : 0;
     uint32_t next = next_task(ctr, lane);
-    while (next < ntasks) {
-        const uint32_t t = next;
+    while (next < nq) {
+        const uint32_t t = q + next * kQueues;
         next = next_task(ctr, lane);   // in flight while this task runs
+        if (t < run_tasks) {
+            const uint32_t pl = t / pair_tasks;
+            const uint32_t rem = t - pl * pair_tasks;
+            const uint32_t s = rem / n_split;
+            const uint32_t j = rem - s * n_split;
+            const uint32_t pair = (uint32_t)xcd + pl * kXcd;
+            const uint32_t p = pair / (uint32_t)rp.nwin, w = pair - p * (uint32_t)rp.nwin;
+            const uint32_t r = long_rows[(uint32_t)rp.R - 1u - j];
+            const uint32_t c0 = p * (uint32_t)rp.cpp + w * (uint32_t)rp.wch;
+            const uint32_t c1 = min(c0 + (uint32_t)rp.wch, (p + 1u) * (uint32_t)rp.cpp);
+            const uint32_t seg = seg_off[r];
+            const uint32_t beg = seg + rp.cnt[(size_t)c0 * rp.R + r];
+            const uint32_t end = c1 == (uint32_t)rp.nchunks ? seg_off[r + 1] : seg + rp.cnt[(size_t)c1 * rp.R + r];
+            float* dst = rp.runs + ((size_t)(j * (uint32_t)rp.n_persp + p) * rp.nwin + w) * out_cols;
+            seg_reduce_task<VW, 1, kRunUnroll>(G, list, beg, end, end, dst, (int)s, lane, out_cols, rp.slice_v, 0);
+            continue;
+        }
         uint32_t r;
         int s;
-        if (t < long_tasks) {
-            const uint32_t i = t / (uint32_t)nslices;
-            s = (int)(t - i * (uint32_t)nslices);
+        if (t < long_end) {
+            const uint32_t u = t - run_tasks;
+            const uint32_t i = u / (uint32_t)nslices;
+            s = (int)(u - i * (uint32_t)nslices);
             r = long_rows[xcd + i * kXcd];
         } else {
-            const uint32_t u = t - long_tasks;
+            const uint32_t u = t - long_end;
             s = (int)(u / nreg);
             r = lo + (u - (uint32_t)s * nreg);
         }
         const uint32_t beg = seg_off[r], end = seg_off[r + 1];
-        if (t >= long_tasks && end - beg >= (uint32_t)kLongRow) continue;   // done in the long phase
-        seg_reduce_task<VW, NQ>(G, list, beg, beg + wcount[r], end, gW + (size_t)r * out_cols, s, lane, out_cols,
-                                slice_v, two_persp);
+        if (t >= long_end && end - beg >= (uint32_t)kLongRow) continue;   // long or split: done elsewhere
+        seg_reduce_task<VW, NQ, kRowsUnroll>(G, list, beg, beg + wcount[r], end, gW + (size_t)r * out_cols, s, lane,
+                                             out_cols, slice_v, two_persp);
+    }
+  }
+}
+
+// gW[r] of a split row = (chain over the windows of its white window sums) + (the same, black).
+// One wave per (split row, 64-lane slice); an empty window's sum is +0, which changes no bit of a
+// chain that started at +0.
+template <int VW>
+__global__ __launch_bounds__(64) void k_split_combine(const uint32_t* __restrict__ long_rows,
+                                                      const uint32_t* __restrict__ sched,
+                                                      float* __restrict__ gW, int out_cols, RunPlan rp) {
+    const int lane = threadIdx.x;
+    const uint32_t n_split = sched[kSchedNSplit];
+    const int q = blockIdx.y * 64 + lane;
+    if (q >= out_cols / VW) return;
+    const int col = q * VW;
+    for (uint32_t j = blockIdx.x; j < n_split; j += gridDim.x) {
+        const uint32_t r = long_rows[(uint32_t)rp.R - 1u - j];
+        vecf<VW> tot = vzero<VW>();
+        for (int p = 0; p < rp.n_persp; ++p) {
+            const float* src = rp.runs + (size_t)(j * (uint32_t)rp.n_persp + p) * rp.nwin * out_cols + col;
+            vecf<VW> v[NNUEFT_ROW_WINDOWS];
+#pragma unroll
+            for (int w = 0; w < NNUEFT_ROW_WINDOWS; ++w)
+                v[w] = w < rp.nwin ? ldv<VW>(src + (size_t)w * out_cols) : vzero<VW>();
+            vecf<VW> acc = vzero<VW>();
+#pragma unroll
+            for (int w = 0; w < NNUEFT_ROW_WINDOWS; ++w)
+                if (w < rp.nwin) vadd<VW>(acc, v[w]);
+            if (p == 0) tot = acc;
+            else vadd<VW>(tot, acc);
+        }
+        stv_stream<VW>(gW + (size_t)r * out_cols + col, tot);
     }
 }
 
@@ -514,6 +654,7 @@ int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, fl
     uint32_t* wcount = (uint32_t*)(ws + L.wcount);
     uint32_t* seg_off = (uint32_t*)(ws + L.seg_off);
     uint32_t* long_rows = (uint32_t*)(ws + L.long_rows);
+    uint32_t* wpre = (uint32_t*)(ws + L.wpre);
     uint32_t* sched = (uint32_t*)(ws + L.sched);
     uint32_t* list = (uint32_t*)(ws + L.list);
     float* partial = (float*)(ws + L.partial);
@@ -543,7 +684,7 @@ int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, fl
                        L.nchunks);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_row_scan, dim3(1), dim3(kScanThreads), (size_t)scan_cap * sizeof(uint32_t), st, seg_off,
-                       long_rows, sched, R, scan_cap);
+                       long_rows, wpre, sched, R, scan_cap);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_fill, dim3(L.nchunks, nranges), dim3(256), fill_bytes, st, widx, bidx, cnt, seg_off, list,
                        B, K, R, L.cpp, range, stage);
@@ -559,15 +700,35 @@ int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, fl
     const int slice_v = ((nv + nslices - 1) / nslices + line_v - 1) / line_v * line_v;
     if ((long long)R * nslices > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
     const int two = n_persp == 2;
+    RunPlan rp;
+    rp.cnt = cnt;
+    rp.runs = (float*)(ws + L.runs);
+    rp.R = R;
+    rp.cpp = L.cpp;
+    rp.nchunks = L.nchunks;
+    rp.wch = L.wch;
+    rp.nwin = L.nwin;
+    rp.n_persp = n_persp;
+    rp.nslices = (nv + 63) / 64;
+    rp.slice_v = ((nv + rp.nslices - 1) / rp.nslices + line_v - 1) / line_v * line_v;
+    if ((long long)L.max_split * rp.nslices * NNUEFT_ROW_WINDOWS > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
 #define SEG_LAUNCH(VW_, NQ_)                                                                                      \
     hipLaunchKernelGGL((k_seg_reduce<VW_, NQ_>), dim3(kXcd * kWavesPerXcd), dim3(64), 0, st, G, list, seg_off,      \
-                       wcount, long_rows, sched, gW, out_cols, nslices, slice_v, two)
+                       wcount, long_rows, sched, gW, out_cols, nslices, slice_v, two, rp)
     if (vec && NQ > 1) SEG_LAUNCH(4, NNUEFT_SEG_NQ);
     else if (vec) SEG_LAUNCH(4, 1);
     else if (NQ > 1) SEG_LAUNCH(1, NNUEFT_SEG_NQ);
     else SEG_LAUNCH(1, 1);
 #undef SEG_LAUNCH
     NNUEFT_LAUNCH_CHECK();
+    if (L.max_split > 0) {
+        const dim3 cgrid((unsigned)min(L.max_split, 1024), (unsigned)rp.nslices);
+        if (vec)
+            hipLaunchKernelGGL(k_split_combine<4>, cgrid, dim3(64), 0, st, long_rows, sched, gW, out_cols, rp);
+        else
+            hipLaunchKernelGGL(k_split_combine<1>, cgrid, dim3(64), 0, st, long_rows, sched, gW, out_cols, rp);
+        NNUEFT_LAUNCH_CHECK();
+    }
 
     return nnueft_det::launch_bias_final(partial, gbias, B, out_cols, st);
 }

@@ -9,6 +9,20 @@
 #define NNUEFT_WAVE 64
 // Positions per tile of the deterministic bias-gradient order (part of the ABI contract).
 #define NNUEFT_BIAS_TILE 32
+// Deterministic weight gradient: a table row named by more slots than NNUEFT_ROW_SPLIT (both
+// perspectives together) is summed window by window, a window being nnueft_window_positions(B)
+// consecutive positions: at most NNUEFT_ROW_WINDOWS windows of at least NNUEFT_ROW_WINDOW_MIN
+// positions, a multiple of 128.
+#define NNUEFT_ROW_SPLIT 512
+#define NNUEFT_ROW_WINDOWS 8
+#define NNUEFT_ROW_WINDOW_MIN 2048
+static inline int nnueft_window_positions(int B) {
+    int nwin = (B + NNUEFT_ROW_WINDOW_MIN - 1) / NNUEFT_ROW_WINDOW_MIN;
+    if (nwin < 1) nwin = 1;
+    if (nwin > NNUEFT_ROW_WINDOWS) nwin = NNUEFT_ROW_WINDOWS;
+    const int w = (B + nwin - 1) / nwin;
+    return (w + 127) / 128 * 128;
+}
 
 typedef unsigned long long u64;
 

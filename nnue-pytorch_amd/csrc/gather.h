@@ -24,8 +24,8 @@ __device__ __forceinline__ void chain_group(vecf<VW> (&acc)[NV], const float* __
 }
 
 // acc[j] += base[row * stride + col[j] ...]  for every lane of `mask` in ascending lane order,
-// where `row` is that lane's `myrow`.  Groups of U rows, then one group each of U/2, U/4, ... 1
-// for the remainder, so a short list still keeps several rows in flight.
+// where `row` is that lane's `myrow`.  Groups of U rows (U <= 64), then one group per set bit of
+// the remaining count, so a short list still keeps several rows in flight.
 template <int VW, int NV, int U>
 __device__ __forceinline__ void chain_rows(vecf<VW> (&acc)[NV], const float* __restrict__ base, size_t stride,
                                            const int (&col)[NV], int myrow, u64 mask) {
@@ -34,16 +34,23 @@ __device__ __forceinline__ void chain_rows(vecf<VW> (&acc)[NV], const float* __r
         chain_group<VW, NV, U>(acc, base, stride, col, myrow, mask);
         cnt -= U;
     }
-    if constexpr (U >= 16) {
+    // what is left is below U: one group per set bit of the count, largest first
+    if constexpr (U > 32) {
+        if (cnt & 32) chain_group<VW, NV, 32>(acc, base, stride, col, myrow, mask);
+    }
+    if constexpr (U > 16) {
+        if (cnt & 16) chain_group<VW, NV, 16>(acc, base, stride, col, myrow, mask);
+    }
+    if constexpr (U > 8) {
         if (cnt & 8) chain_group<VW, NV, 8>(acc, base, stride, col, myrow, mask);
     }
-    if constexpr (U >= 8) {
+    if constexpr (U > 4) {
         if (cnt & 4) chain_group<VW, NV, 4>(acc, base, stride, col, myrow, mask);
     }
-    if constexpr (U >= 4) {
+    if constexpr (U > 2) {
         if (cnt & 2) chain_group<VW, NV, 2>(acc, base, stride, col, myrow, mask);
     }
-    if constexpr (U >= 2) {
+    if constexpr (U > 1) {
         if (cnt & 1) chain_group<VW, NV, 1>(acc, base, stride, col, myrow, mask);
     }
 }

@@ -17,6 +17,8 @@ PROTOTYPES = {
     "nnueft_version": (c_int, []),
     "nnueft_error_string": (ctypes.c_char_p, [c_int]),
     "nnueft_bias_tile": (c_int, []),
+    "nnueft_row_split": (c_int, []),
+    "nnueft_row_window": (c_int, [c_int]),
     "nnueft_sparse_fwd": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_void_p]),
     "nnueft_sparse_bwd_atomic": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_void_p]),
     "nnueft_det_workspace_bytes": (c_size_t, [c_int] * 5),

@@ -85,16 +85,25 @@ def encode_batch(squares, types, colors, fold_kings: bool = False):
     return out[0], out[1], present.sum(1).astype(np.int32)
 
 
-def random_positions(batch_size: int, seed: int, min_other: int = 2, max_other: int = 30):
+def random_positions(batch_size: int, seed: int, min_other: int = 2, max_other: int = 30,
+                     castled_kings: float = 0.0):
     """Seeded synthetic positions: two kings on distinct squares plus U{min_other..max_other} other
     pieces with uniform type (pawn..queen) and colour on distinct non-king squares.
+
+    castled_kings: fraction of positions whose kings stand on g1 / g8 (as in most game positions),
+    which concentrates the batch on one king bucket per perspective; 0 keeps the kings uniform.
 
     Returns (squares, types, colors) int32 [B, 32] with -1 in unused slots; slot 0 is the white
     king, slot 1 the black king.
     """
     rng = np.random.default_rng(seed)
     B = batch_size
-    perm = np.argsort(rng.random((B, 64)), axis=1)[:, :32].astype(np.int32)
+    keys = rng.random((B, 64))
+    if castled_kings > 0.0:
+        fixed = rng.random(B) < castled_kings
+        keys[fixed, 6] = -2.0     # g1 sorts first: white king
+        keys[fixed, 62] = -1.0    # g8 second: black king
+    perm = np.argsort(keys, axis=1)[:, :32].astype(np.int32)
     n_other = rng.integers(min_other, max_other + 1, size=B)
     slot = np.arange(32)[None, :]
     used = slot < (2 + n_other)[:, None]
@@ -110,11 +119,11 @@ def random_positions(batch_size: int, seed: int, min_other: int = 2, max_other: 
     return squares, types, colors
 
 
-def synthetic_batch(batch_size: int, seed: int, fold_kings: bool = False):
+def synthetic_batch(batch_size: int, seed: int, fold_kings: bool = False, castled_kings: float = 0.0):
     """The batch tuple the loader hands the model (data_loader/_native.py:48-96), from seeded
     synthetic positions: us f32 [B,1] ~ Bernoulli(1/2), them = 1 - us, white/black int32 [B,32],
     piece_count int64 [B].  numpy arrays."""
-    squares, types, colors = random_positions(batch_size, seed)
+    squares, types, colors = random_positions(batch_size, seed, castled_kings=castled_kings)
     white, black, pc = encode_batch(squares, types, colors, fold_kings=fold_kings)
     rng = np.random.default_rng(seed + 7919)
     us = rng.integers(0, 2, size=(batch_size, 1)).astype(np.float32)

@@ -41,6 +41,16 @@ def bias_tile() -> int:
     return int(lib().nnueft_oracle_bias_tile())
 
 
+def row_split() -> int:
+    """Most slots that may name a table row before its gradient is summed window by window."""
+    return int(lib().nnueft_oracle_row_split())
+
+
+def row_window(B: int) -> int:
+    """Positions per window of the split rows' order for a batch of B."""
+    return int(lib().nnueft_oracle_row_window(int(B)))
+
+
 def sparse_fwd(idx, W, bias):
     idx, W, bias = _c(idx, np.int32), _c(W, np.float32), _c(bias, np.float32)
     B, K = idx.shape

@@ -33,6 +33,12 @@
  *             (position, slot) order; the two perspectives' chains are then added
  *             (white + black).  torch's CPU embedding_bag backward followed by autograd's
  *             accumulation of the two uses of `weight` produces exactly this.
+ *             Exception (this build's own order): a table row named by more than
+ *             NNUEFT_ORACLE_ROW_SPLIT slots of the batch, both perspectives together, is summed
+ *             window by window: window w = positions [w*W, (w+1)*W), W = nnueft_oracle_row_window(B);
+ *             per perspective each window's slots are chained from +0, the window sums are
+ *             chained from +0 in ascending w, then white + black.  torch agrees with such a row
+ *             to rounding only (exactly when all addends are small integers).
  *   bias      positions are cut into tiles of NNUEFT_ORACLE_BIAS_TILE; per column a chain
  *   gradient  over the positions of a tile (starting at +0, ascending), then a chain over the
  *             tile sums (starting at +0, ascending).  This order is this build's own; torch
@@ -51,6 +57,20 @@
 #define COLBLK 64
 
 int nnueft_oracle_bias_tile(void) { return NNUEFT_ORACLE_BIAS_TILE; }
+
+#define NNUEFT_ORACLE_ROW_SPLIT 512
+int nnueft_oracle_row_split(void) { return NNUEFT_ORACLE_ROW_SPLIT; }
+
+/* Window length: as few windows as hold at least 2048 positions each, at most 8, equal lengths
+ * rounded up to a multiple of 128. */
+int nnueft_oracle_row_window(int B)
+{
+    int nwin = (B + 2047) / 2048;
+    if (nwin < 1) nwin = 1;
+    if (nwin > 8) nwin = 8;
+    int w = (B + nwin - 1) / nwin;
+    return (w + 127) / 128 * 128;
+}
 
 static inline int valid(int32_t r, int R) { return r >= 0 && r < R; }
 
@@ -73,18 +93,58 @@ int nnueft_oracle_sparse_fwd(const int32_t* idx, const float* W, const float* bi
     return 0;
 }
 
-/* One perspective's chains: acc[r, c0:c1] += G[b, c0:c1] for slots in ascending (b,k). */
-static void scatter_chain(const int32_t* idx, const float* G, size_t g_stride, float* acc,
-                          int B, int K, int R, int out_cols, int c0, int c1)
+/* split_id[r] = ordinal of row r among the rows named by more than NNUEFT_ORACLE_ROW_SPLIT slots
+ * of idx_a and idx_b together (idx_b may be NULL), -1 for the others.  Returns how many. */
+static int find_split_rows(const int32_t* idx_a, const int32_t* idx_b, int B, int K, int R, int32_t* split_id)
 {
+    int64_t* count = (int64_t*)calloc((size_t)R, sizeof(int64_t));
+    if (!count) return -1;
+    for (int pass = 0; pass < 2; ++pass) {
+        const int32_t* idx = pass ? idx_b : idx_a;
+        if (!idx) continue;
+        for (size_t i = 0; i < (size_t)B * K; ++i)
+            if (valid(idx[i], R)) count[idx[i]]++;
+    }
+    int n = 0;
+    for (int r = 0; r < R; ++r) split_id[r] = count[r] > NNUEFT_ORACLE_ROW_SPLIT ? n++ : -1;
+    free(count);
+    return n;
+}
+
+/* One perspective's chains, columns [c0,c1): acc[r] += G[b] for slots in ascending (b,k).  A split
+ * row instead collects each window in `cur`, and at every window boundary adds it to the row's
+ * running sum of windows in `tot` (both [nsplit, c1-c0], zeroed here); acc[r] += nothing until
+ * the end, where acc[r] = tot. */
+static void scatter_chain(const int32_t* idx, const float* G, size_t g_stride, float* acc,
+                          int B, int K, int R, int out_cols, int c0, int c1,
+                          const int32_t* split_id, int nsplit, int window, float* cur, float* tot)
+{
+    const int w = c1 - c0;
+    if (nsplit > 0) {
+        memset(cur, 0, sizeof(float) * (size_t)nsplit * w);
+        memset(tot, 0, sizeof(float) * (size_t)nsplit * w);
+    }
     for (int b = 0; b < B; ++b) {
+        if (nsplit > 0 && b > 0 && b % window == 0)
+            for (size_t i = 0; i < (size_t)nsplit * w; ++i) { tot[i] = tot[i] + cur[i]; cur[i] = 0.0f; }
         const float* g = G + (size_t)b * g_stride;
         for (int k = 0; k < K; ++k) {
             int32_t r = idx[(size_t)b * K + k];
             if (!valid(r, R)) continue;
-            float* a = acc + (size_t)r * out_cols;
-            for (int c = c0; c < c1; ++c) a[c] = a[c] + g[c];
+            if (split_id[r] >= 0) {
+                float* a = cur + (size_t)split_id[r] * w;
+                for (int c = c0; c < c1; ++c) a[c - c0] = a[c - c0] + g[c];
+            } else {
+                float* a = acc + (size_t)r * out_cols;
+                for (int c = c0; c < c1; ++c) a[c] = a[c] + g[c];
+            }
         }
+    }
+    if (nsplit > 0) {
+        for (size_t i = 0; i < (size_t)nsplit * w; ++i) tot[i] = tot[i] + cur[i];
+        for (int r = 0; r < R; ++r)
+            if (split_id[r] >= 0)
+                for (int c = c0; c < c1; ++c) acc[(size_t)r * out_cols + c] = tot[(size_t)split_id[r] * w + (c - c0)];
     }
 }
 
@@ -113,12 +173,24 @@ int nnueft_oracle_sparse_bwd(const int32_t* idx, const float* gout, float* gW, f
                              int B, int K, int R, int out_cols)
 {
     memset(gW, 0, (size_t)R * out_cols * sizeof(float));
+    int32_t* split_id = (int32_t*)malloc(sizeof(int32_t) * (size_t)R);
+    if (!split_id) return -2;
+    const int nsplit = find_split_rows(idx, NULL, B, K, R, split_id);
+    if (nsplit < 0) { free(split_id); return -2; }
+    const int window = nnueft_oracle_row_window(B);
     int nblk = (out_cols + COLBLK - 1) / COLBLK;
+    int failed = 0;
 #pragma omp parallel for schedule(dynamic)
     for (int j = 0; j < nblk; ++j) {
         int c0 = j * COLBLK, c1 = c0 + COLBLK < out_cols ? c0 + COLBLK : out_cols;
-        scatter_chain(idx, gout, (size_t)out_cols, gW, B, K, R, out_cols, c0, c1);
+        float* tmp = (float*)malloc(sizeof(float) * 2 * (size_t)(nsplit ? nsplit : 1) * COLBLK);
+        if (!tmp) { failed = 1; continue; }
+        scatter_chain(idx, gout, (size_t)out_cols, gW, B, K, R, out_cols, c0, c1, split_id, nsplit, window, tmp,
+                      tmp + (size_t)(nsplit ? nsplit : 1) * COLBLK);
+        free(tmp);
     }
+    free(split_id);
+    if (failed) return -2;
     bias_tiled(gout, NULL, (size_t)out_cols, gbias, B, out_cols);
     return 0;
 }
@@ -245,12 +317,23 @@ int nnueft_oracle_double_bwd(const float* us, const float* them,
                                            saved, G, B, L1, n_psqt);
     if (rc) { free(G); free(accb); return rc; }
     memset(gW, 0, (size_t)R * out_cols * sizeof(float));
+    int32_t* split_id = (int32_t*)malloc(sizeof(int32_t) * (size_t)R);
+    const int nsplit = split_id ? find_split_rows(widx, bidx, B, K, R, split_id) : -1;
+    if (nsplit < 0) { free(G); free(accb); free(split_id); return -2; }
+    const int window = nnueft_oracle_row_window(B);
     int nblk = (out_cols + COLBLK - 1) / COLBLK;
+    int failed = 0;
 #pragma omp parallel for schedule(dynamic)
     for (int j = 0; j < nblk; ++j) {
         int c0 = j * COLBLK, c1 = c0 + COLBLK < out_cols ? c0 + COLBLK : out_cols;
-        scatter_chain(widx, G, (size_t)out_cols, gW, B, K, R, out_cols, c0, c1);
-        scatter_chain(bidx, G + (size_t)B * out_cols, (size_t)out_cols, accb, B, K, R, out_cols, c0, c1);
+        const size_t half = (size_t)(nsplit ? nsplit : 1) * COLBLK;
+        float* tmp = (float*)malloc(sizeof(float) * 2 * half);
+        if (!tmp) { failed = 1; continue; }
+        scatter_chain(widx, G, (size_t)out_cols, gW, B, K, R, out_cols, c0, c1, split_id, nsplit, window, tmp,
+                      tmp + half);
+        scatter_chain(bidx, G + (size_t)B * out_cols, (size_t)out_cols, accb, B, K, R, out_cols, c0, c1, split_id,
+                      nsplit, window, tmp, tmp + half);
+        free(tmp);
         for (int r = 0; r < R; ++r)
             for (int c = c0; c < c1; ++c)
                 gW[(size_t)r * out_cols + c] = gW[(size_t)r * out_cols + c] + accb[(size_t)r * out_cols + c];
@@ -258,7 +341,8 @@ int nnueft_oracle_double_bwd(const float* us, const float* them,
     bias_tiled(G, G + (size_t)B * out_cols, (size_t)out_cols, gbias, B, out_cols);
     free(G);
     free(accb);
-    return 0;
+    free(split_id);
+    return failed ? -2 : 0;
 }
 
 /*

@@ -41,6 +41,14 @@ def test_host_only_entry_points():
     lib = _native.load()
     assert lib.nnueft_version() == 1
     assert lib.nnueft_bias_tile() == 32
+    # the constants of the deterministic order are the oracle's
+    from oracle import cpu as oracle_cpu
+
+    assert lib.nnueft_bias_tile() == oracle_cpu.bias_tile()
+    assert lib.nnueft_row_split() == oracle_cpu.row_split()
+    for B in (1, 127, 2048, 2049, 5000, 16384, 16385, 65536, 1000003):
+        assert lib.nnueft_row_window(B) == oracle_cpu.row_window(B)
+    assert lib.nnueft_row_window(0) == 0
     assert lib.nnueft_error_string(0) == b"success"
     for code in (-1, -2, -3):
         assert lib.nnueft_error_string(code).startswith(b"nnueft:")

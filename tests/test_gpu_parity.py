@@ -176,6 +176,68 @@ def test_double_backward(oracle_cpu, B, L1, R, K, kw, mode):
         assert np.array_equal(gb, rb)
 
 
+# Batches in which a few table rows are named by a large part of the positions (as in game data,
+# where most kings stand on their castled squares): rows beyond nnueft_row_split() slots are summed
+# window by window, several windows at these sizes.
+def _skewed_double_case(seed, B, L1, castled, fold=0):
+    from nnueft import halfka_v2_hm as hk
+
+    c = double_case(seed, B, L1, hk.NUM_INPUTS, 32, halfka=True, weight_scale=0.05, max_act=255 / 256)
+    us, them, widx, bidx, pc = hk.synthetic_batch(B, seed, castled_kings=castled)
+    if fold:
+        # crowd every king bucket's features onto its first `fold` rows (lists then hold duplicates)
+        for ix in (widx, bidx):
+            v = ix >= 0
+            ix[v] = ix[v] // hk.NUM_PLANES * hk.NUM_PLANES + ix[v] % hk.NUM_PLANES % fold
+    c.update(us=us, them=them, widx=widx, bidx=bidx, psqt_idx=((pc - 1) // 4).astype(np.int64))
+    return c
+
+
+@pytest.mark.parametrize("B,L1,castled,fold", [(4096, 64, 1.0, 0), (6000, 256, 0.6, 96), (16384, 128, 0.5, 200),
+                                                (3000, 1024, 0.9, 40)])
+def test_double_backward_deterministic_with_split_rows(oracle_cpu, B, L1, castled, fold):
+    c = _skewed_double_case(900 + B, B, L1, castled, fold)
+    nat, lib = _native()
+    R, K, n_psqt = c["R"], c["K"], c["n_psqt"]
+    out_cols = L1 + n_psqt
+    counts = np.bincount(np.concatenate([c["widx"][c["widx"] >= 0], c["bidx"][c["bidx"] >= 0]]), minlength=R)
+    assert (counts > lib.nnueft_row_split()).sum() >= (8 if fold else 2) and B > lib.nnueft_row_window(B)
+    d, l0, wp, bp, saved = _run_double_fwd(c)
+    g_l0, g_wp, g_bp = _t(c["g_l0"]), _t(c["g_wp"]), _t(c["g_bp"])
+    nbytes = lib.nnueft_det_workspace_bytes(B, K, R, out_cols, 2)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=_dev())
+    gW = torch.full((R, out_cols), float("nan"), device=_dev())
+    gb = torch.full((out_cols,), float("nan"), device=_dev())
+    nat.check(lib.nnueft_double_bwd_det(d["us"].data_ptr(), d["them"].data_ptr(), d["widx"].data_ptr(),
+                                        d["bidx"].data_ptr(), d["psqt_idx"].data_ptr(), d["bias"].data_ptr(),
+                                        c["max_act"], g_l0.data_ptr(), g_wp.data_ptr(), g_bp.data_ptr(),
+                                        saved.data_ptr(), gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt,
+                                        ws.data_ptr(), nbytes, _stream()), "double_bwd_det")
+    rW, rb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["bias"], c["max_act"],
+                                   c["g_l0"], c["g_wp"], c["g_bp"], saved.cpu().numpy(), R, n_psqt)
+    assert np.array_equal(gW.cpu().numpy(), rW)
+    assert np.array_equal(gb.cpu().numpy(), rb)
+
+
+@pytest.mark.parametrize("B,out_cols,R,K", [(5000, 72, 40, 16), (9000, 37, 300, 8), (20000, 264, 64, 4)])
+def test_sparse_backward_deterministic_with_split_rows(oracle_cpu, B, out_cols, R, K):
+    c = sparse_case(950 + B, B, out_cols, R, K, allow_holes=True)
+    rng = np.random.default_rng(B)
+    c["idx"][rng.random((B, K)) < 0.3] = 3      # one row named by a third of all slots
+    nat, lib = _native()
+    assert B > lib.nnueft_row_window(B)
+    idx, g = _t(c["idx"]), _t(c["g"])
+    nbytes = lib.nnueft_det_workspace_bytes(B, K, R, out_cols, 1)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=_dev())
+    gW = torch.full((R, out_cols), float("nan"), device=_dev())
+    gb = torch.full((out_cols,), float("nan"), device=_dev())
+    nat.check(lib.nnueft_sparse_bwd_det(idx.data_ptr(), g.data_ptr(), gW.data_ptr(), gb.data_ptr(), B, K, R,
+                                        out_cols, ws.data_ptr(), nbytes, _stream()), "sparse_bwd_det")
+    rW, rb = oracle_cpu.sparse_bwd(c["idx"], c["g"], R)
+    assert np.array_equal(gW.cpu().numpy(), rW)
+    assert np.array_equal(gb.cpu().numpy(), rb)
+
+
 def test_deterministic_backward_repeats_bitwise():
     """Two runs of the deterministic backward give the same bits (the atomic one need not)."""
     c = double_case(77, 300, 256, 600, 32, binary_side=True)

@@ -105,6 +105,128 @@ def test_sparse_backward_weight_bits_equal_torch_cpu_autograd(oracle_cpu, B, oc,
     assert not gW[~named].any()
 
 
+# ---------------------------------------------------------------------------------------------
+# Rows named by more than row_split() slots: summed window by window.  The checks below fix that
+# order through sums whose value under each candidate order is known in closed form: in fp32,
+# 2**24 + 1 rounds back to 2**24, so a chain that starts with 2**24 loses every following 1.0,
+# while ones collected in another window first arrive as one exact integer.
+BIG = float(2 ** 24)
+
+
+def test_row_window_lengths(oracle_cpu):
+    assert oracle_cpu.row_split() == 512
+    # one window up to 2048 positions, then as few as hold >= 2048 each, at most 8, multiples of 128
+    assert [oracle_cpu.row_window(B) for B in (1, 100, 2048, 2049, 4096, 8192, 16384, 16385, 65536, 100000)] == \
+        [128, 128, 2048, 1152, 2048, 2048, 2048, 2176, 8192, 12544]
+
+
+def _ones_after_big(B, K, R, row, positions):
+    """Lists in which `row` is named once by each of `positions`; upstream rows 2**24 at position 0, else 1."""
+    idx = np.full((B, K), -1, np.int32)
+    idx[positions, 0] = row
+    g = np.ones((B, 1), np.float32)
+    g[0, 0] = BIG
+    return idx, g
+
+
+def test_sparse_backward_split_row_sums_windows_separately(oracle_cpu):
+    B, K, R = 4096, 2, 5
+    W = oracle_cpu.row_window(B)
+    assert W == 2048
+    # 600 slots > row_split: position 0 (2**24), 299 ones in window 0, 300 ones in window 1
+    pos = np.r_[0:300, W:W + 300]
+    idx, g = _ones_after_big(B, K, R, 3, pos)
+    gW, _ = oracle_cpu.sparse_bwd(idx, g, R)
+    # window 0 chain: 2**24 swallows its 299 ones; window 1: exactly 300; chain over windows: 2**24 + 300
+    assert gW[3, 0] == BIG + 300.0
+    # the same slots, one fewer than the threshold allows splitting: a plain chain, every 1.0 lost
+    pos = np.r_[0:256, W:W + 256]
+    assert len(pos) == oracle_cpu.row_split()
+    idx, g = _ones_after_big(B, K, R, 3, pos)
+    gW, _ = oracle_cpu.sparse_bwd(idx, g, R)
+    assert gW[3, 0] == BIG
+    # one slot more: split
+    pos = np.r_[0:256, W:W + 257 + 1]
+    idx, g = _ones_after_big(B, K, R, 3, pos)
+    gW, _ = oracle_cpu.sparse_bwd(idx, g, R)
+    assert gW[3, 0] == BIG + 258.0
+
+
+def test_sparse_backward_split_row_window_sums_are_chained_in_order(oracle_cpu):
+    B, K, R = 8192, 1, 2
+    W = oracle_cpu.row_window(B)
+    assert W == 2048
+    # windows 0..3 hold 2**24, 200 ones, 200 ones, 200 ones: ((2**24 + 200) + 200) + 200, all exact
+    pos = np.r_[0:1, W:W + 200, 2 * W:2 * W + 200, 3 * W:3 * W + 200]
+    idx, g = _ones_after_big(B, K, R, 1, pos)
+    gW, _ = oracle_cpu.sparse_bwd(idx, g, R)
+    assert gW[1, 0] == BIG + 600.0
+    # a window sum of 1 is lost against 2**24 wherever it comes after it, kept (as part of 201) before
+    g2 = g.copy()
+    g2[0, 0] = 1.0
+    g2[3 * W, 0] = BIG          # the big addend now opens the last window
+    gW, _ = oracle_cpu.sparse_bwd(idx, g2, R)
+    # window sums 1, 200, 200, (2**24 then 199 ones lost) -> 401 + 2**24: odd, ties to even = 2**24 + 400
+    assert gW[1, 0] == BIG + 400.0
+
+
+def test_sparse_backward_split_rows_exact_on_integers_and_others_untouched(oracle_cpu):
+    rng = np.random.default_rng(5)
+    B, K, R, oc = 6000, 8, 40, 24
+    idx = random_lists(rng, B, K, R, allow_holes=True)
+    idx[rng.random((B, K)) < 0.5] = 7            # row 7: ~24000 slots, far beyond the threshold
+    g_int = rng.integers(-8, 8, size=(B, oc)).astype(np.float32)
+    gW, gb = oracle_cpu.sparse_bwd(idx, g_int, R)
+    C = count_matrix(idx, R)
+    assert np.array_equal(gW.astype(np.float64), C.T @ g_int.astype(np.float64))
+    # real-valued upstream rows: the split rows agree with a float64 sum to rounding, and rows
+    # below the threshold keep the plain chain (checked against a chain written out here)
+    g = rng.standard_normal((B, oc)).astype(np.float32)
+    gW, _ = oracle_cpu.sparse_bwd(idx, g, R)
+    ref = C.T @ g.astype(np.float64)
+    assert np.allclose(gW, ref, rtol=1e-4, atol=1e-3)
+    counts = C.sum(0)
+    small = int(np.argmin(np.where(counts > 0, counts, 1 << 30)))
+    assert 0 < counts[small] <= oracle_cpu.row_split()
+    chain = np.zeros(oc, np.float32)
+    for b in range(B):
+        for k in range(K):
+            if idx[b, k] == small:
+                chain = chain + g[b]
+    assert np.array_equal(gW[small], chain)
+
+
+def test_double_backward_split_counts_both_perspectives_together(oracle_cpu):
+    # row 2 is named by 300 white and 302 black slots: neither list alone exceeds row_split, together
+    # they do.  The PSQT column passes grad_wpsqt / grad_bpsqt straight to the table row.
+    B, K, R, L1, n_psqt = 4096, 2, 4, 8, 2
+    W = oracle_cpu.row_window(B)
+    widx = np.full((B, K), -1, np.int32)
+    bidx = np.full((B, K), -1, np.int32)
+    widx[np.r_[0:1, W:W + 299], 0] = 2         # white: 2**24 in window 0, 299 ones in window 1
+    bidx[np.r_[0:1, W:W + 301], 0] = 2         # black: 1 in window 0, 301 ones in window 1
+    us = np.ones((B, 1), np.float32)
+    them = np.zeros((B, 1), np.float32)
+    psqt_idx = np.zeros(B, np.int64)
+    g_wp = np.ones((B, 1), np.float32)
+    g_wp[0, 0] = BIG
+    g_bp = np.ones((B, 1), np.float32)
+    saved = np.zeros((2, B, L1), np.float32)
+    bias = np.zeros(L1 + n_psqt, np.float32)
+    g_l0 = np.zeros((B, L1), np.float32)
+    gW, _ = oracle_cpu.double_bwd(us, them, widx, bidx, psqt_idx, bias, 127.0, g_l0, g_wp, g_bp, saved, R, n_psqt)
+    # split: white = 2**24 + 299 -> odd, ties to even = 2**24 + 300; black = 1 + 301; sum exact
+    assert gW[2, L1] == BIG + 300.0 + 302.0
+    # with one black slot fewer the row has 601 slots, still split; with the lists cut so the row has
+    # 512 slots in all it is not: white plain chain = 2**24 (ones lost), black = plain 212
+    widx[:] = -1
+    bidx[:] = -1
+    widx[np.r_[0:1, W:W + 299], 0] = 2
+    bidx[np.r_[0:1, W:W + 211], 0] = 2
+    gW, _ = oracle_cpu.double_bwd(us, them, widx, bidx, psqt_idx, bias, 127.0, g_l0, g_wp, g_bp, saved, R, n_psqt)
+    assert gW[2, L1] == BIG + 212.0
+
+
 def test_bias_gradient_tile_order_brute_force(oracle_cpu):
     tile = oracle_cpu.bias_tile()
     rng = np.random.default_rng(2)
