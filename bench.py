@@ -53,12 +53,12 @@ def algorithmic_bytes(L1, B, sum_a, mode):
     return fwd, bwd
 
 
-def make_inputs(L1, B, seed, device, castled_kings=0.0):
+def make_inputs(L1, B, seed, device, positions="uniform"):
     import numpy as np
     import torch
     from nnueft import halfka_v2_hm as hk
 
-    us, them, white, black, pc = hk.synthetic_batch(B, seed, castled_kings=castled_kings)
+    us, them, white, black, pc = hk.synthetic_batch(B, seed, game_like=(positions == "game"))
     rng = np.random.default_rng(seed)
     oc = L1 + N_PSQT
     g = torch.Generator(device="cpu").manual_seed(seed)
@@ -236,9 +236,10 @@ def main():
     ap.add_argument("--backward", default="deterministic", choices=["deterministic", "atomic"],
                     help="backward mode the headline value is measured with (the other one is reported beside it)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--castled-kings", type=float, default=0.0,
-                    help="fraction of positions with the kings on g1/g8 (robustness runs: a skewed bucket "
-                         "distribution like real game data); the headline workload uses 0")
+    ap.add_argument("--positions", default="uniform", choices=["uniform", "game"],
+                    help="uniform: kings and pieces uniform over the board (the headline workload); game: piece "
+                         "placement statistics of real game positions, where one or two king buckets hold a large "
+                         "part of the batch (halfka_v2_hm.game_like_positions); a default run times both")
     ap.add_argument("--only", default="", choices=["", "fwd", "det", "atomic", "copy"],
                     help="run only this part (for profiling runs); 'copy' launches a plain elementwise kernel "
                          "reading and writing 1 GiB each, the yardstick the FETCH_SIZE/WRITE_SIZE counters are scaled by")
@@ -275,12 +276,12 @@ def main():
         return
     L1, B = WORKLOADS[args.workload]
     seed = 1234 + 3
-    t, sum_a = make_inputs(L1, B, seed, dev, args.castled_kings)
+    t, sum_a = make_inputs(L1, B, seed, dev, args.positions)
     W = t["W"].requires_grad_()
     bias = t["bias"].requires_grad_()
     max_act = 255.0 / 256.0
 
-    def step(mode):
+    def step(mode, t=t):
         nnueft.set_backward_mode(mode)
         W.grad = None
         bias.grad = None
@@ -380,7 +381,7 @@ def main():
         "config": {
             "workload": args.workload, "L1": L1, "batch": B, "table_rows": R_ROWS, "psqt_columns": N_PSQT,
             "slots": K_SLOTS, "active_rows_per_position": sum_a / B, "backward": head_mode,
-            "index_scheme": "HalfKAv2_hm, seeded random positions", "castled_kings": args.castled_kings,
+            "index_scheme": "HalfKAv2_hm, seeded random positions", "positions": args.positions,
         },
         "roofline": {
             "kernel": "nnueft_double_fwd: k_acc_blocked (the gather, ~3/4 of the time) + k_mix + pair sort",
@@ -403,6 +404,13 @@ def main():
             "backward_algorithmic_GBs": bb / (bwd_ms[mode] * 1e-3) / 1e9 if mode in bwd_ms else None,
         }
     out["step"] = step_stats
+    if not args.only and args.positions == "uniform":
+        # the same step on game-like index lists (not the headline: a robustness figure)
+        tg, sum_g = make_inputs(L1, B, seed, dev, "game")
+        ms_g, _ = time_steps(lambda: step(head_mode, tg), args.steps, args.warmup)
+        out["game_like_positions"] = {"ms_per_step": ms_g, "positions_per_s": B / (ms_g * 1e-3),
+                                      "active_rows_per_position": sum_g / B, "backward": head_mode}
+        del tg
     if not args.no_cpu_baseline and not args.only:
         out["cpu_baseline"] = cpu_baseline(L1, B, seed)
     else:

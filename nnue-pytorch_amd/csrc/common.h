@@ -13,9 +13,15 @@
 // perspectives together) is summed window by window, a window being nnueft_window_positions(B)
 // consecutive positions: at most NNUEFT_ROW_WINDOWS windows of at least NNUEFT_ROW_WINDOW_MIN
 // positions, a multiple of 128.
+#ifndef NNUEFT_ROW_SPLIT
 #define NNUEFT_ROW_SPLIT 512
+#endif
+#ifndef NNUEFT_ROW_WINDOWS
 #define NNUEFT_ROW_WINDOWS 8
+#endif
+#ifndef NNUEFT_ROW_WINDOW_MIN
 #define NNUEFT_ROW_WINDOW_MIN 2048
+#endif
 static inline int nnueft_window_positions(int B) {
     int nwin = (B + NNUEFT_ROW_WINDOW_MIN - 1) / NNUEFT_ROW_WINDOW_MIN;
     if (nwin < 1) nwin = 1;

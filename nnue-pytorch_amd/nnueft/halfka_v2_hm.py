@@ -119,11 +119,69 @@ def random_positions(batch_size: int, seed: int, min_other: int = 2, max_other: 
     return squares, types, colors
 
 
-def synthetic_batch(batch_size: int, seed: int, fold_kings: bool = False, castled_kings: float = 0.0):
+def game_like_positions(batch_size: int, seed: int):
+    """Seeded synthetic positions with the piece placement statistics of real game positions.
+
+    game_like_stats.npz (written by make_game_like_stats.py from the reference's sample data) holds,
+    per piece kind and square, how often it occurs from white's point of view with white's king
+    mirrored onto files e-h: one table for each of white's three most common king buckets, one for
+    the rest.  A position draws its class, the kings from their rows of the class's table, and
+    every other (kind, square) independently with its frequency, one piece per square.  Most
+    kings end up on their castled squares and most pawns near their home ranks, so one or two
+    king buckets hold a large part of a batch and a few hundred table rows half of all slots,
+    which uniform positions (random_positions) do not show.
+
+    Returns (squares, types, colors) like random_positions.
+    """
+    import os
+
+    stats = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "game_like_stats.npz"))
+    freq, share = stats["freq"].astype(np.float64), stats["share"].astype(np.float64)
+    rng = np.random.default_rng(seed)
+    B = batch_size
+    cls = rng.choice(len(share), size=B, p=share / share.sum())
+    squares = np.full((B, 32), -1, np.int32)
+    types = np.full((B, 32), -1, np.int32)
+    colors = np.full((B, 32), -1, np.int32)
+    for c in range(len(share)):
+        rows = np.nonzero(cls == c)[0]
+        n = len(rows)
+        if n == 0:
+            continue
+        pk = freq[c, 10:12] / freq[c, 10:12].sum(1, keepdims=True)
+        wk = rng.choice(64, size=n, p=pk[0])
+        bk = rng.choice(64, size=n, p=pk[1])
+        clash = wk == bk
+        while clash.any():
+            bk[clash] = rng.choice(64, size=int(clash.sum()), p=pk[1])
+            clash = wk == bk
+        # race between the ten other kinds on every square: kind k claims it when u_k < freq_k,
+        # the smallest u_k / freq_k wins
+        ratio = rng.random((n, 10, 64)) / np.maximum(freq[c, :10], 1e-12)[None]
+        kind = ratio.argmin(1)
+        taken = ratio.min(1) < 1.0
+        sq = np.arange(64)[None, :]
+        taken &= (sq != wk[:, None]) & (sq != bk[:, None])
+        taken &= np.cumsum(taken, axis=1) <= 30    # at most 30 others (a surplus is rare)
+        squares[rows, 0], types[rows, 0], colors[rows, 0] = wk, KING, WHITE
+        squares[rows, 1], types[rows, 1], colors[rows, 1] = bk, KING, BLACK
+        slot = 1 + np.cumsum(taken, axis=1)
+        b_i, s_i = np.nonzero(taken)
+        squares[rows[b_i], slot[b_i, s_i]] = s_i
+        types[rows[b_i], slot[b_i, s_i]] = kind[b_i, s_i] // 2
+        colors[rows[b_i], slot[b_i, s_i]] = kind[b_i, s_i] % 2
+    return squares, types, colors
+
+
+def synthetic_batch(batch_size: int, seed: int, fold_kings: bool = False, castled_kings: float = 0.0,
+                    game_like: bool = False):
     """The batch tuple the loader hands the model (data_loader/_native.py:48-96), from seeded
-    synthetic positions: us f32 [B,1] ~ Bernoulli(1/2), them = 1 - us, white/black int32 [B,32],
-    piece_count int64 [B].  numpy arrays."""
-    squares, types, colors = random_positions(batch_size, seed, castled_kings=castled_kings)
+    synthetic positions (random_positions, or game_like_positions when `game_like`): us f32 [B,1]
+    ~ Bernoulli(1/2), them = 1 - us, white/black int32 [B,32], piece_count int64 [B].  numpy arrays."""
+    if game_like:
+        squares, types, colors = game_like_positions(batch_size, seed)
+    else:
+        squares, types, colors = random_positions(batch_size, seed, castled_kings=castled_kings)
     white, black, pc = encode_batch(squares, types, colors, fold_kings=fold_kings)
     rng = np.random.default_rng(seed + 7919)
     us = rng.integers(0, 2, size=(batch_size, 1)).astype(np.float32)

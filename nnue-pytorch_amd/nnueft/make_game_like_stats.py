@@ -1,0 +1,83 @@
+"""Writes game_like_stats.npz: how often each (piece, square) occurs in real game positions.
+
+Source: the positions of the reference's own sample file .pgo/small.binpack, decoded by the
+reference's loader built under oracle/_ref (so this runs only where the reference checkout is
+present).  What is kept are 12 x 64 tables of frequencies seen from white's point of view
+(p_idx = 2 * piece_type + (piece is black), oriented square): one for each of the three most
+common king buckets of white and one for all others, since where the pieces stand depends on
+where the king went.  Nothing of the positions themselves is kept.
+nnueft.halfka_v2_hm.game_like_positions() draws synthetic positions from the tables.
+
+    python nnue-pytorch_amd/nnueft/make_game_like_stats.py /root/reference/.pgo/small.binpack
+"""
+import ctypes
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(HERE, "..", ".."))
+from oracle import loader_ref as lr  # noqa: E402
+
+
+class _Skip(ctypes.Structure):
+    # data_loader/cpp/training_data_loader_structs.h:3-14
+    _fields_ = [("filtered", ctypes.c_bool), ("random_fen_skipping", ctypes.c_int), ("wld_filtered", ctypes.c_bool),
+                ("early_fen_skipping", ctypes.c_int), ("soft_early_fen_skipping", ctypes.c_int),
+                ("simple_eval_skipping", ctypes.c_int), ("param_index", ctypes.c_int)] + \
+               [(n, ctypes.c_double) for n in ("pc_y0 pc_y1 pc_y2 pc_y3 pc_y4 ply_x1 ply_y1 ply_x2 ply_y2 "
+                                               "ply_x3 ply_y3 ply_x4 ply_y4").split()]
+
+
+class _Ddp(ctypes.Structure):
+    _fields_ = [("rank", ctypes.c_int), ("world_size", ctypes.c_int)]
+
+
+def main(path):
+    lib = ctypes.CDLL(lr.LIB_PATH)
+    lib.create_sparse_batch_stream.restype = ctypes.c_void_p
+    lib.create_sparse_batch_stream.argtypes = [ctypes.c_char_p, ctypes.c_int, ctypes.c_int,
+                                               ctypes.POINTER(ctypes.c_char_p), ctypes.c_int, ctypes.c_bool,
+                                               _Skip, _Ddp]
+    lib.fetch_next_sparse_batch.restype = ctypes.POINTER(lr._SparseBatch)
+    lib.fetch_next_sparse_batch.argtypes = [ctypes.c_void_p]
+    lib.destroy_sparse_batch.argtypes = [ctypes.POINTER(lr._SparseBatch)]
+    lib.destroy_sparse_batch_stream.argtypes = [ctypes.c_void_p]
+    files = (ctypes.c_char_p * 1)(path.encode())
+    skip = _Skip()
+    for n in ("pc_y0", "pc_y1", "pc_y2", "pc_y3", "pc_y4", "ply_y1", "ply_y2", "ply_y3", "ply_y4"):
+        setattr(skip, n, 1.0)
+    skip.ply_x1, skip.ply_x2, skip.ply_x3, skip.ply_x4 = 0, 1, 2, 3
+    stream = lib.create_sparse_batch_stream(b"HalfKAv2_hm", 1, 1, files, 8192, False, skip, _Ddp(0, 1))
+    lists = []
+    while True:
+        p = lib.fetch_next_sparse_batch(stream)
+        if not p:
+            break
+        sb = p.contents
+        w = np.ctypeslib.as_array(sb.white, shape=(sb.size, sb.max_active_features))
+        lists.append(w.copy())
+        lib.destroy_sparse_batch(p)
+    lib.destroy_sparse_batch_stream(stream)
+    w = np.concatenate(lists)
+    n_pos = len(w)
+    bucket = w[:, 0] // 768
+    top = np.argsort(np.bincount(bucket, minlength=32))[::-1][:3]
+    cls = np.full(n_pos, 3)
+    for i, b in enumerate(top):
+        cls[bucket == b] = i
+    freq = np.zeros((4, 12, 64), np.float32)
+    share = np.zeros(4, np.float32)
+    for c in range(4):
+        sel = w[cls == c]
+        share[c] = len(sel) / n_pos
+        v = sel[sel >= 0] % 768
+        freq[c] = (np.bincount(v, minlength=768) / max(len(sel), 1)).reshape(12, 64)
+    np.savez_compressed(os.path.join(HERE, "game_like_stats.npz"), freq=freq, share=share, buckets=top.astype(np.int32),
+                        positions=np.int64(n_pos))
+    print("positions", n_pos, "classes", top, share, "pieces per position", freq.sum((1, 2)))
+
+
+if __name__ == "__main__":
+    main(sys.argv[1])

@@ -180,10 +180,11 @@ def test_double_backward(oracle_cpu, B, L1, R, K, kw, mode):
 # where most kings stand on their castled squares): rows beyond nnueft_row_split() slots are summed
 # window by window, several windows at these sizes.
 def _skewed_double_case(seed, B, L1, castled, fold=0):
+    """castled < 0: game-like positions; else that share of the kings on g1 / g8."""
     from nnueft import halfka_v2_hm as hk
 
     c = double_case(seed, B, L1, hk.NUM_INPUTS, 32, halfka=True, weight_scale=0.05, max_act=255 / 256)
-    us, them, widx, bidx, pc = hk.synthetic_batch(B, seed, castled_kings=castled)
+    us, them, widx, bidx, pc = hk.synthetic_batch(B, seed, castled_kings=castled, game_like=castled < 0)
     if fold:
         # crowd every king bucket's features onto its first `fold` rows (lists then hold duplicates)
         for ix in (widx, bidx):
@@ -194,7 +195,7 @@ def _skewed_double_case(seed, B, L1, castled, fold=0):
 
 
 @pytest.mark.parametrize("B,L1,castled,fold", [(4096, 64, 1.0, 0), (6000, 256, 0.6, 96), (16384, 128, 0.5, 200),
-                                                (3000, 1024, 0.9, 40)])
+                                                (3000, 1024, 0.9, 40), (16384, 64, -1, 0), (5000, 3072, -1, 0)])
 def test_double_backward_deterministic_with_split_rows(oracle_cpu, B, L1, castled, fold):
     c = _skewed_double_case(900 + B, B, L1, castled, fold)
     nat, lib = _native()

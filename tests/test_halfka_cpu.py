@@ -133,3 +133,44 @@ def test_synthetic_batch_tuple():
     again = hk.synthetic_batch(512, seed=5)
     assert all(np.array_equal(a, b) for a, b in zip((us, them, white, black, pc), again))
     assert 16.0 < pc.mean() < 20.0     # 2 kings + U{2..30}: mean 18
+
+
+def test_game_like_positions_are_well_formed_and_concentrated():
+    B = 8192
+    squares, types, colors = hk.game_like_positions(B, seed=9)
+    again = hk.game_like_positions(B, seed=9)
+    assert all(np.array_equal(a, b) for a, b in zip((squares, types, colors), again))
+    used = squares >= 0
+    assert ((types >= 0) == used).all() and ((colors >= 0) == used).all()
+    for i in range(0, B, 97):
+        sq = squares[i][used[i]]
+        assert len(set(sq.tolist())) == len(sq)                 # one piece per square
+    assert ((types == hk.KING) & (colors == hk.WHITE)).sum(1).tolist() == [1] * B
+    assert ((types == hk.KING) & (colors == hk.BLACK)).sum(1).tolist() == [1] * B
+    white, black, pc = hk.encode_batch(squares, types, colors)
+    assert pc.min() >= 2 and pc.max() <= 32 and 14.0 < pc.mean() < 20.0
+    # what makes these positions a different workload from the uniform ones: one king bucket holds
+    # more than a fifth of the batch, and the rows named by more than 512 slots hold a third of all slots
+    bucket = np.bincount(white[:, 0] // hk.NUM_PLANES, minlength=hk.NUM_BUCKETS)
+    assert bucket.max() > 0.2 * B
+    rows = np.bincount(np.concatenate([white[white >= 0], black[black >= 0]]), minlength=hk.NUM_INPUTS)
+    assert rows[rows > 512].sum() > rows.sum() / 3
+    us, them, w2, b2, pc2 = hk.synthetic_batch(B, seed=9, game_like=True)
+    assert np.array_equal(w2, white) and np.array_equal(b2, black)
+
+
+@pytest.mark.skipif(not loader_ref.available(), reason="oracle/_ref not built (needs the reference checkout)")
+def test_live_reference_encoder_on_game_like_positions():
+    squares, types, colors = hk.game_like_positions(400, seed=78)
+    keep = []
+    for i in range(400):
+        sq = {int(s): int(t) for s, t in zip(squares[i], types[i]) if s >= 0}
+        kings = [s for s, t in sq.items() if t == hk.KING]
+        far = max(abs(kings[0] % 8 - kings[1] % 8), abs(kings[0] // 8 - kings[1] // 8)) > 1
+        if far and all(not (t == hk.PAWN and s // 8 in (0, 7)) for s, t in sq.items()):
+            keep.append(i)
+    assert len(keep) > 200
+    fens = [hk.to_fen(squares[i], types[i], colors[i], white_to_move=bool(i & 1)) for i in keep]
+    ref = loader_ref.encode_fens(fens)
+    white, black, pc = hk.encode_batch(squares[keep], types[keep], colors[keep])
+    assert np.array_equal(white, ref["white"]) and np.array_equal(black, ref["black"])
