@@ -59,7 +59,7 @@ constexpr int kSchedRowLo = kSchedNSplit + 1;  // kXcd + 1 range bounds
 constexpr int kSchedWords = kSchedRowLo + kXcd + 1;
 
 struct DetLayout {
-    size_t G, partial, cnt, wcount, seg_off, long_rows, wpre, sched, list, runs, end;
+    size_t G, partial, cnt, wcount, seg_off, long_rows, sched, list, runs, end;
     int cpp;     // chunks per perspective
     int nchunks; // n_persp * cpp
     int ntiles;  // bias tiles
@@ -87,8 +87,6 @@ bool det_layout(int B, int K, int R, int out_cols, int n_persp, DetLayout* L) {
     L->seg_off = off;
     off += up256(((size_t)R + 1) * sizeof(uint32_t));
     L->long_rows = off;
-    off += up256((size_t)R * sizeof(uint32_t));
-    L->wpre = off;
     off += up256((size_t)R * sizeof(uint32_t));
     L->sched = off;
     off += up256((size_t)kSchedWords * sizeof(uint32_t));
@@ -298,12 +296,11 @@ constexpr uint32_t kRowWeight = NNUEFT_ROW_WEIGHT;   // cost of a task that find
 constexpr int kScanThreads = 1024;
 __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict__ seg_off,
                                                            uint32_t* __restrict__ long_rows,
-                                                           uint32_t* __restrict__ wpre,
                                                            uint32_t* __restrict__ sched, int R, int cap) {
     extern __shared__ uint32_t stage[];   // `cap` row lengths, turned into offsets in place
     // two running sums: all slots, slots of split rows
     __shared__ uint32_t wave_tot[2][kScanThreads / 64];
-    __shared__ uint32_t carry_s[2], n_long_s, n_split_s;
+    __shared__ uint32_t carry_s[2], total_s[2], n_long_s, n_split_s;
     __shared__ uint32_t lo_s[kXcd + 1];
     const int tid = threadIdx.x;
     if (tid == 0) {
@@ -314,6 +311,32 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
     }
     if (tid <= kXcd) lo_s[tid] = (uint32_t)R;
     if (tid < kXcd * kSchedQueues) sched[kSchedCtr + tid * 32] = 0;
+    // The row ranges need the two totals before the scan reaches the rows.  A table that fits the
+    // staging buffer gets them from the scan's own first step; a larger one is summed here first.
+    const bool one_pass = R <= cap;
+    if (!one_pass) {
+        uint32_t s0 = 0, s1 = 0;
+        for (int i = tid; i < R; i += kScanThreads) {
+            const uint32_t raw = seg_off[i];
+            s0 += raw & ~kSplitFlag;
+            s1 += (raw & kSplitFlag) ? (raw & ~kSplitFlag) : 0u;
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            s0 += __shfl_down(s0, off);
+            s1 += __shfl_down(s1, off);
+        }
+        if ((tid & 63) == 0) {
+            wave_tot[0][tid >> 6] = s0;
+            wave_tot[1][tid >> 6] = s1;
+        }
+        __syncthreads();
+        if (tid < 2) {
+            uint32_t t = 0;
+            for (int w = 0; w < kScanThreads / 64; ++w) t += wave_tot[tid][w];
+            total_s[tid] = t;
+        }
+    }
     __syncthreads();
     for (int base = 0; base < R; base += cap) {
         const int n = min(cap, R - base);
@@ -350,17 +373,31 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
             wave_tot[1][tid >> 6] = incl[1];
         }
         __syncthreads();
-        uint32_t run[2];
+        uint32_t run[2], all[2];
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
             run[k] = carry_s[k] + incl[k] - local[k];
-            for (int w = 0; w < (tid >> 6); ++w) run[k] += wave_tot[k][w];
+            all[k] = 0;
+            for (int w = 0; w < kScanThreads / 64; ++w) {
+                const uint32_t x = wave_tot[k][w];
+                if (w < (tid >> 6)) run[k] += x;
+                all[k] += x;
+            }
+            if (!one_pass) all[k] = total_s[k];
+        }
+        // XCD of a row = floor(kXcd * weight of the rows before it / weight of all rows), weight =
+        // kRowWeight + its slots unless it is split; a range begins where that number goes up
+        const unsigned long long denom = (unsigned long long)(all[0] - all[1]) + (unsigned long long)R * kRowWeight;
+        int x_cur = 0;
+        if (i_beg < i_end) {
+            x_cur = xcd_of((unsigned long long)(run[0] - run[1]) + (unsigned long long)(base + i_beg) * kRowWeight, denom);
+            if (base + i_beg == 0)
+                for (int k = 0; k <= x_cur; ++k) lo_s[k] = 0;
         }
         for (int i = i_beg; i < i_end; ++i) {
             const uint32_t raw = stage[i];
             const uint32_t len = raw & ~kSplitFlag;
             stage[i] = run[0];
-            wpre[base + i] = run[0] - run[1];   // slots of the rows before this one that are not split
             // a row is in at most one of the two lists, so they cannot meet inside long_rows[0..R)
             if (raw & kSplitFlag) {
                 long_rows[R - 1 - (int)atomicAdd(&n_split_s, 1u)] = (uint32_t)(base + i);
@@ -369,6 +406,13 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
                 long_rows[atomicAdd(&n_long_s, 1u)] = (uint32_t)(base + i);
             }
             run[0] += len;
+            const int r_next = base + i + 1;
+            if (r_next < R) {
+                const int x_next =
+                    xcd_of((unsigned long long)(run[0] - run[1]) + (unsigned long long)r_next * kRowWeight, denom);
+                for (int k = x_cur + 1; k <= x_next; ++k) lo_s[k] = (uint32_t)r_next;
+                x_cur = x_next;
+            }
         }
         __syncthreads();
         if (tid == kScanThreads - 1) {
@@ -378,36 +422,11 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
         for (int i = tid; i < n; i += kScanThreads) seg_off[base + i] = stage[i];
         __syncthreads();
     }
-    const uint32_t total = carry_s[0];
     if (tid == 0) {
-        seg_off[R] = total;
+        seg_off[R] = carry_s[0];
         sched[kSchedNLong] = n_long_s;
         sched[kSchedNSplit] = n_split_s;
     }
-    __syncthreads();   // seg_off and wpre are complete (written by this workgroup)
-    // XCD of a row = floor(kXcd * weight of the rows before it / weight of all rows)
-    const unsigned long long denom =
-        (unsigned long long)(total - carry_s[1]) + (unsigned long long)R * kRowWeight;
-    for (int rb = tid; rb < R; rb += kScanThreads * 8) {
-        uint32_t off[8], prev[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int r = rb + u * kScanThreads;
-            off[u] = r < R ? wpre[r] : 0;
-            prev[u] = (r < R && r > 0) ? wpre[r - 1] : 0;
-        }
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int r = rb + u * kScanThreads;
-            if (r < R) {
-                const int x = xcd_of((unsigned long long)off[u] + (unsigned long long)r * kRowWeight, denom);
-                const int xp =
-                    r > 0 ? xcd_of((unsigned long long)prev[u] + (unsigned long long)(r - 1) * kRowWeight, denom) : -1;
-                for (int k = xp + 1; k <= x; ++k) lo_s[k] = (uint32_t)r;
-            }
-        }
-    }
-    __syncthreads();
     if (tid <= kXcd) sched[kSchedRowLo + tid] = lo_s[tid];
 }
 
@@ -654,7 +673,6 @@ int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, fl
     uint32_t* wcount = (uint32_t*)(ws + L.wcount);
     uint32_t* seg_off = (uint32_t*)(ws + L.seg_off);
     uint32_t* long_rows = (uint32_t*)(ws + L.long_rows);
-    uint32_t* wpre = (uint32_t*)(ws + L.wpre);
     uint32_t* sched = (uint32_t*)(ws + L.sched);
     uint32_t* list = (uint32_t*)(ws + L.list);
     float* partial = (float*)(ws + L.partial);
@@ -684,7 +702,7 @@ int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, fl
                        L.nchunks);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_row_scan, dim3(1), dim3(kScanThreads), (size_t)scan_cap * sizeof(uint32_t), st, seg_off,
-                       long_rows, wpre, sched, R, scan_cap);
+                       long_rows, sched, R, scan_cap);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_fill, dim3(L.nchunks, nranges), dim3(256), fill_bytes, st, widx, bidx, cnt, seg_off, list,
                        B, K, R, L.cpp, range, stage);

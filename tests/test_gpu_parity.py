@@ -220,7 +220,9 @@ def test_double_backward_deterministic_with_split_rows(oracle_cpu, B, L1, castle
     assert np.array_equal(gb.cpu().numpy(), rb)
 
 
-@pytest.mark.parametrize("B,out_cols,R,K", [(5000, 72, 40, 16), (9000, 37, 300, 8), (20000, 264, 64, 4)])
+# (the last two tables are taller than the row scan stages at once: several passes, totals summed first)
+@pytest.mark.parametrize("B,out_cols,R,K", [(5000, 72, 40, 16), (9000, 37, 300, 8), (20000, 264, 64, 4),
+                                            (3000, 8, 70001, 8), (2500, 12, 40000, 16)])
 def test_sparse_backward_deterministic_with_split_rows(oracle_cpu, B, out_cols, R, K):
     c = sparse_case(950 + B, B, out_cols, R, K, allow_holes=True)
     rng = np.random.default_rng(B)
