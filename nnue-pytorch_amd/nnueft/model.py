@@ -201,37 +201,46 @@ def get_feature_cls(name: str):
 
 # ------------------------------------------------------------------------------------------ FT module
 
+@torch.compiler.disable(recursive=False)
+def _launch_table_merge(weight, virtual, l1_size, scale_ft, scale_psqt, quantize):
+    lib = _native.load()
+    R, cols = weight.shape
+    merged = torch.empty_like(weight)
+    with torch.cuda.device(weight.device):
+        rc = lib.nnueft_table_merge(weight.data_ptr(), virtual.data_ptr(), merged.data_ptr(), R, cols, l1_size,
+                                    virtual.shape[0], float(scale_ft), float(scale_psqt), int(bool(quantize)),
+                                    _stream_ptr(weight.device))
+    _native.check(rc, "nnueft_table_merge")
+    return merged
+
+
+@torch.compiler.disable(recursive=False)
+def _launch_table_virtual_grad(grad, vrows):
+    lib = _native.load()
+    R, cols = grad.shape
+    gv = torch.empty(vrows, cols, dtype=grad.dtype, device=grad.device)
+    with torch.cuda.device(grad.device):
+        rc = lib.nnueft_table_virtual_grad(grad.data_ptr(), gv.data_ptr(), R, cols, vrows, _stream_ptr(grad.device))
+    _native.check(rc, "nnueft_table_virtual_grad")
+    return gv
+
+
 class _TableMerge(torch.autograd.Function):
     """merged = q(weight + virtual[row % 768]) in one pass; STE gradient: weight gets the incoming
-    gradient itself, virtual its sum over the table blocks."""
+    gradient itself, virtual its sum over the table blocks.  The launches sit in functions dynamo
+    does not trace (it would choke on data_ptr() and the raw stream handle)."""
 
     @staticmethod
     def forward(ctx, weight, virtual, l1_size, scale_ft, scale_psqt, quantize):
-        lib = _native.load()
-        R, cols = weight.shape
-        merged = torch.empty_like(weight)
-        with torch.cuda.device(weight.device):
-            rc = lib.nnueft_table_merge(weight.data_ptr(), virtual.data_ptr(), merged.data_ptr(), R, cols, l1_size,
-                                        virtual.shape[0], float(scale_ft), float(scale_psqt), int(bool(quantize)),
-                                        _stream_ptr(weight.device))
-        _native.check(rc, "nnueft_table_merge")
         ctx.vrows = virtual.shape[0]
-        return merged
+        return _launch_table_merge(weight, virtual, l1_size, scale_ft, scale_psqt, quantize)
 
     @staticmethod
     def backward(ctx, grad):
         grad = grad.contiguous()
-        lib = _native.load()
-        R, cols = grad.shape
-        gv = torch.empty(ctx.vrows, cols, dtype=grad.dtype, device=grad.device)
-        with torch.cuda.device(grad.device):
-            rc = lib.nnueft_table_virtual_grad(grad.data_ptr(), gv.data_ptr(), R, cols, ctx.vrows,
-                                               _stream_ptr(grad.device))
-        _native.check(rc, "nnueft_table_virtual_grad")
-        return grad, gv, None, None, None, None
+        return grad, _launch_table_virtual_grad(grad, ctx.vrows), None, None, None, None
 
 
-@torch.compiler.disable(recursive=False)
 def _table_merge(weight, virtual, l1_size, scale_ft, scale_psqt, quantize):
     return _TableMerge.apply(weight, virtual, l1_size, scale_ft, scale_psqt, quantize)
 

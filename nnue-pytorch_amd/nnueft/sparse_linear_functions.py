@@ -34,7 +34,9 @@ def get_backward_mode() -> str:
     return _BACKWARD_MODE
 
 
+@torch.compiler.disable
 def _stream_ptr(device) -> int:
+    # opaque to dynamo: traced, current_stream() is a torch.Stream proxy without a raw handle
     return torch.cuda.current_stream(device).cuda_stream
 
 

@@ -99,3 +99,33 @@ def test_full_model_trains_on_gpu():
         a = model(us, them, white, black, pc, False, False).cpu()
         b = cpu_model(us.cpu(), them.cpu(), white.cpu(), black.cpu(), pc.cpu(), False, False)
     torch.testing.assert_close(a, b, atol=2e-4, rtol=1e-3)
+
+
+@pytest.mark.parametrize("backend", ["aot_eager", "inductor"])
+def test_model_under_torch_compile_on_gpu(backend):
+    """The reference compiles the model (train.py:296).  The launchers are opaque to dynamo
+    (torch.compiler.disable), so the graph breaks around the HIP kernels and the results are those
+    of the eager module, deterministic backward included."""
+    old = nnueft.get_backward_mode()
+    nnueft.set_backward_mode("deterministic")
+    try:
+        model = _make_model(128, 11).to(DEV)
+        batch = [torch.from_numpy(a).to(DEV) for a in hk.synthetic_batch(512, 12)]
+        out = model(*batch)
+        out.sum().backward()
+        ref = {n: p.grad.clone() for n, p in model.named_parameters()}
+        model.zero_grad()
+        torch._dynamo.reset()
+        cm = torch.compile(model, backend=backend)
+        for _ in range(2):      # second call: the cached graph
+            model.zero_grad()
+            o = cm(*batch)
+            o.sum().backward()
+            torch.testing.assert_close(o, out, atol=1e-5, rtol=1e-5)
+            if backend == "aot_eager":   # same kernels upstream, so the same bits (inductor fuses the layer stacks)
+                assert torch.equal(model.input.features[0].weight.grad, ref["input.features.0.weight"])
+            for n, p in model.named_parameters():
+                torch.testing.assert_close(p.grad, ref[n], atol=1e-4, rtol=1e-4)
+    finally:
+        nnueft.set_backward_mode(old)
+        torch._dynamo.reset()

@@ -163,3 +163,48 @@ def test_oracle_table_functions(oracle_cpu):
                           (torch.from_numpy(W) + torch.from_numpy(V).repeat(3, 1)).numpy())
     g = rng.integers(-9, 9, size=(48, 12)).astype(np.float32)
     assert np.array_equal(oracle_cpu.table_virtual_grad(g, 16), g.reshape(3, 16, 12).sum(0))
+
+
+# The reference trains under torch.compile (train.py:296) and saves whole modules with torch.save;
+# both must keep working with the operators of this build in the graph.
+def _tiny_model_and_batch():
+    from nnueft import halfka_v2_hm as hk
+
+    torch.manual_seed(0)
+    m = M.NNUEModel("HalfKAv2_hm^", M.ModelConfig(L1=64, L2=8, L3=16))
+    batch = [torch.from_numpy(a) for a in hk.synthetic_batch(32, 3)]
+    return m, batch
+
+
+def test_module_survives_torch_save_and_load():
+    import io
+
+    m, batch = _tiny_model_and_batch()
+    out = m(*batch)
+    buf = io.BytesIO()
+    torch.save(m, buf)            # a file this test wrote itself
+    buf.seek(0)
+    m2 = torch.load(buf, weights_only=False)
+    assert torch.equal(m2(*batch), out)
+    buf = io.BytesIO()
+    torch.save(m.state_dict(), buf)
+    buf.seek(0)
+    m3 = M.NNUEModel("HalfKAv2_hm^", M.ModelConfig(L1=64, L2=8, L3=16))
+    m3.load_state_dict(torch.load(buf, weights_only=True))
+    assert torch.equal(m3(*batch), out)
+
+
+@pytest.mark.parametrize("backend", ["eager", "aot_eager"])
+def test_model_under_torch_compile_on_cpu(backend):
+    m, batch = _tiny_model_and_batch()
+    out = m(*batch)
+    out.sum().backward()
+    ref = {n: p.grad.clone() for n, p in m.named_parameters()}
+    m.zero_grad()
+    torch._dynamo.reset()
+    cm = torch.compile(m, backend=backend)
+    o = cm(*batch)
+    o.sum().backward()
+    assert torch.allclose(o, out, atol=1e-6)
+    for n, p in m.named_parameters():
+        assert torch.allclose(p.grad, ref[n], atol=1e-5), n
