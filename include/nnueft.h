@@ -218,6 +218,53 @@ int nnueft_stack_int8_fwd(const uint8_t* x, const int64_t* bucket, const int8_t*
                           int lin_shift1, int sqr_shift1, int lin_shift2, int sqr_shift2, int act_max,
                           int out_mult, int out_den, void* stream);
 
+/*
+ * out[i] = (floor(x[i] * scale + eps) / scale) * post_mul, each operation rounding on its own: the
+ * activation fake quantization of the feature transformer's output (_fake_quantize_acts,
+ * model/quantize.py:36-45, called from composed_feature_transformer.py:143-144) together with the
+ * l0 correction factor that follows it (:149), in one pass over [B, L1] instead of six.  The
+ * straight-through estimator makes the gradient of x the incoming gradient times post_mul.
+ * x, out f32[n]; out may be x.
+ */
+int nnueft_act_fake_quantize(const float* x, float* out, long long n, float scale, float eps, float post_mul,
+                             void* stream);
+
+/*
+ * RangerLite parameter update, one call per parameter tensor (n contiguous f32 elements each of
+ * p, grad and the state tensors).  They replace the reference's CuPy kernels of the same names,
+ * model/optimizers/ranger_lite.py:46-201 (launched from :325-477 and :563-583), element for element:
+ *   vm   = vm * beta2 + (g * g) * one_minus_beta2              (skipped when update_variance == 0:
+ *                                                                the *_phase2 kernels, after
+ *                                                                nnueft_ranger_lite_update_variance)
+ *   den  = sqrt(vm / bias_correction2) + eps
+ *   pnm:  pos = (step odd ? grad_ma : neg_grad_ma), neg = the other one
+ *         pos = pos * beta1_sq + g * one_minus_beta1_sq          (written back to its buffer)
+ *         dir = (pos * one_plus_pnm - neg * pnm_factor) / noise_norm
+ *   adam: grad_ma = grad_ma * beta1 + g * one_minus_beta1 ;  dir = grad_ma
+ *   p    = (wd_factor != 0 ? p * (1 - wd_factor) : p) - lr_div_bc1 * (dir / den)
+ * Every operation rounds on its own, in this order.  wd_factor and update_variance fold the
+ * reference's "full" and "phase2" variants into one entry point each.
+ * lookahead_params: NULL, or the slow weights on a merge step; then, in the same pass,
+ *   p = p * lookahead_alpha + lookahead_params * (1 - lookahead_alpha) ;  lookahead_params = p
+ * which is lookahead_process_step (ranger_lite.py:737-760) without a second sweep over the
+ * tensors.  nnueft_ranger_lite_lookahead_merge is that blend alone.
+ */
+int nnueft_ranger_lite_update_pnm(float* p, const float* grad, float* grad_ma, float* neg_grad_ma,
+                                  float* variance_ma, long long n, float beta2, float one_minus_beta2,
+                                  float bias_correction2, float beta1_sq, float one_minus_beta1_sq,
+                                  float one_plus_pnm, float pnm_factor, float noise_norm, float lr_div_bc1,
+                                  float eps, long long step, float wd_factor, int update_variance,
+                                  float* lookahead_params, float lookahead_alpha, void* stream);
+int nnueft_ranger_lite_update_adam(float* p, const float* grad, float* grad_ma, float* variance_ma,
+                                   long long n, float beta2, float one_minus_beta2, float bias_correction2,
+                                   float beta1, float one_minus_beta1, float lr_div_bc1, float eps,
+                                   float wd_factor, int update_variance, float* lookahead_params,
+                                   float lookahead_alpha, void* stream);
+int nnueft_ranger_lite_update_variance(const float* grad, float* variance_ma, long long n, float beta2,
+                                       float one_minus_beta2, void* stream);
+int nnueft_ranger_lite_lookahead_merge(float* p, float* lookahead_params, long long n, float alpha,
+                                       void* stream);
+
 #ifdef __cplusplus
 }
 #endif

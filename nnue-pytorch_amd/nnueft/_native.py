@@ -6,7 +6,7 @@ to another implementation: if the shared object is missing or does not export a 
 """
 import ctypes
 import os
-from ctypes import c_float, c_int, c_size_t, c_void_p
+from ctypes import c_float, c_int, c_longlong, c_size_t, c_void_p
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
 # NNUEFT_LIBRARY points at another build of the same library (kernel tuning)
@@ -38,6 +38,16 @@ PROTOTYPES = {
     "nnueft_int16_workspace_bytes": (c_size_t, [c_int] * 5),
     "nnueft_ft_int16_fwd": (c_int, [c_void_p] * 9 + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
     "nnueft_stack_int8_fwd": (c_int, [c_void_p] * 9 + [c_int] * 12 + [c_void_p]),
+    "nnueft_act_fake_quantize": (c_int, [c_void_p] * 2 + [c_longlong] + [c_float] * 3 + [c_void_p]),
+    "nnueft_ranger_lite_update_pnm": (
+        c_int,
+        [c_void_p] * 5 + [c_longlong] + [c_float] * 10 + [c_longlong, c_float, c_int, c_void_p, c_float, c_void_p],
+    ),
+    "nnueft_ranger_lite_update_adam": (
+        c_int, [c_void_p] * 4 + [c_longlong] + [c_float] * 7 + [c_float, c_int, c_void_p, c_float, c_void_p],
+    ),
+    "nnueft_ranger_lite_update_variance": (c_int, [c_void_p] * 2 + [c_longlong] + [c_float] * 2 + [c_void_p]),
+    "nnueft_ranger_lite_lookahead_merge": (c_int, [c_void_p] * 2 + [c_longlong, c_float, c_void_p]),
 }
 
 _lib = None

@@ -245,6 +245,31 @@ def _table_merge(weight, virtual, l1_size, scale_ft, scale_psqt, quantize):
     return _TableMerge.apply(weight, virtual, l1_size, scale_ft, scale_psqt, quantize)
 
 
+@torch.compiler.disable(recursive=False)
+def _launch_act_fake_quantize(x, scale, post_mul):
+    lib = _native.load()
+    out = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        rc = lib.nnueft_act_fake_quantize(x.data_ptr(), out.data_ptr(), x.numel(), float(scale),
+                                          float(FAKE_QUANTIZE_EPS), float(post_mul), _stream_ptr(x.device))
+    _native.check(rc, "nnueft_act_fake_quantize")
+    return out
+
+
+class _ActFakeQuantize(torch.autograd.Function):
+    """(floor(x * scale + eps) / scale) * post_mul in one pass; the straight-through estimator leaves
+    the gradient as it comes, times post_mul."""
+
+    @staticmethod
+    def forward(ctx, x, scale, post_mul):
+        ctx.post_mul = float(post_mul)
+        return _launch_act_fake_quantize(x.contiguous(), scale, post_mul)
+
+    @staticmethod
+    def backward(ctx, grad):
+        return (grad if ctx.post_mul == 1.0 else grad * ctx.post_mul), None, None
+
+
 class ComposedFeatureTransformer(nn.Module):
     def __init__(self, feature_classes, l1_size: int, num_psqt_buckets: int, quantization: QuantizationManager):
         super().__init__()
@@ -323,9 +348,15 @@ class ComposedFeatureTransformer(nn.Module):
         merged, bias = self.merged_weight_and_bias(fake_quantize_weights)
         l0_, wpsqt, bpsqt = double_feature_transform(us, them, white_indices, black_indices, psqt_indices, merged,
                                                      bias, self.quantization.max_ft_activation, self.l1_size, backend)
+        q = self.quantization
+        if fake_quantize_acts and l0_.is_cuda and l0_.dtype == torch.float32 and _native.available():
+            # activation grid and correction factor in one pass over [B, L1]
+            return _ActFakeQuantize.apply(l0_, q.hidden_quantized_one, q.l0_correction_factor), wpsqt, bpsqt
         if fake_quantize_acts:
-            l0_ = self.quantization.fake_quantize_ft_act(l0_)
-        return l0_ * self.quantization.l0_correction_factor, wpsqt, bpsqt
+            l0_ = q.fake_quantize_ft_act(l0_)
+        if q.l0_correction_factor != 1.0:     # x * 1.0 is x, and so is its gradient
+            l0_ = l0_ * q.l0_correction_factor
+        return l0_, wpsqt, bpsqt
 
 
 # ------------------------------------------------------------------------------------------ layer stacks
@@ -512,3 +543,21 @@ def sf_loss(scorenet, score, outcome, p: LossParams, actual_lambda):
         loss = loss * ((qf > pt) * p.qp_asymmetry + 1)
     weights = 1 + (2.0 ** p.w1 - 1) * torch.pow((pf - 0.5) ** 2 * pf * (1 - pf), p.w2)
     return (loss * weights).sum() / weights.sum()
+
+
+def optimizer_param_groups(model: "NNUEModel", lr: float = 8.75e-4, ft_weight_decay: float = 0.0,
+                           dense_weight_decay: float = 0.0, factorized_weight_decay: float = 0.0):
+    """The ten parameter groups the reference hands its optimizer (model/nnue.py:120-177): feature
+    transformer weights / biases, then weight and bias of every layer of the stacks, biases never decayed."""
+    def named(module, biases):
+        return [p for n, p in module.named_parameters() if ("bias" in n) == biases and p.requires_grad]
+
+    ls = model.layer_stacks
+    groups = [
+        (named(model.input, False), ft_weight_decay), (named(model.input, True), 0.0),
+        ([ls.l1.factorized_linear.weight], factorized_weight_decay), ([ls.l1.factorized_linear.bias], 0.0),
+        ([ls.l1.linear.weight], dense_weight_decay), ([ls.l1.linear.bias], 0.0),
+        ([ls.l2.linear.weight], dense_weight_decay), ([ls.l2.linear.bias], 0.0),
+        ([ls.output.linear.weight], dense_weight_decay), ([ls.output.linear.bias], 0.0),
+    ]
+    return [{"params": params, "lr": lr, "weight_decay": wd} for params, wd in groups]

@@ -178,3 +178,35 @@ def stack_int8_fwd(x, bucket, W1, b1, W2, b2, Wo, bo, L2, L3, count, **kw):
                                             k["sqr2"], k["act_max"], k["out_mult"], k["out_den"])
     assert rc == 0
     return out
+
+
+def ranger_lite_update(p, grad, grad_ma, neg_grad_ma, variance_ma, lookahead, *, beta2, bias_correction2, beta1,
+                       one_minus_beta1, one_plus_pnm=0.0, pnm_factor=0.0, noise_norm=1.0, lr_div_bc1, eps, step=1,
+                       wd_factor=0.0, update_variance=True, alpha=0.5):
+    """In place on float32 numpy arrays (neg_grad_ma / lookahead may be None).  beta1 / one_minus_beta1 are the
+    squared ones when neg_grad_ma is given, as in the reference's kernels."""
+    f = ctypes.c_float
+    for a in (p, grad, grad_ma, variance_ma) + tuple(x for x in (neg_grad_ma, lookahead) if x is not None):
+        assert a.dtype == np.float32 and a.flags.c_contiguous
+    rc = lib().nnueft_oracle_ranger_lite_update(
+        _p(p), _p(grad), _p(grad_ma), _p(neg_grad_ma) if neg_grad_ma is not None else None, _p(variance_ma),
+        _p(lookahead) if lookahead is not None else None, ctypes.c_longlong(p.size),
+        f(beta2), f(np.float32(1.0 - beta2)), f(bias_correction2), f(beta1), f(one_minus_beta1), f(one_plus_pnm),
+        f(pnm_factor), f(noise_norm), f(lr_div_bc1), f(eps), ctypes.c_longlong(step), f(wd_factor),
+        int(bool(update_variance)), f(alpha))
+    assert rc == 0
+
+
+def ranger_lite_update_variance(grad, variance_ma, beta2):
+    rc = lib().nnueft_oracle_ranger_lite_update_variance(_p(grad), _p(variance_ma), ctypes.c_longlong(grad.size),
+                                                         ctypes.c_float(beta2), ctypes.c_float(np.float32(1.0 - beta2)))
+    assert rc == 0
+
+
+def act_fake_quantize(x, scale=128.0, eps=1e-5, post_mul=1.0):
+    x = _c(x, np.float32)
+    out = np.empty_like(x)
+    rc = lib().nnueft_oracle_act_fake_quantize(_p(x), _p(out), ctypes.c_longlong(x.size), ctypes.c_float(scale),
+                                               ctypes.c_float(eps), ctypes.c_float(post_mul))
+    assert rc == 0
+    return out

@@ -21,6 +21,8 @@
  *                                 The activations kept between forward and backward are the two
  *                                 perspectives' row sums (before the bias); the mixed values are
  *                                 recomputed from them with the forward's own operations.
+ *   nnueft_oracle_ranger_lite_*   model/optimizers/ranger_lite.py:46-201 (fused update kernels),
+ *                                 :737-760 (lookahead merge)
  *   nnueft_oracle_ft_int16_fwd    no code in the reference (the accumulate runs in the engine);
  *                                 spec docs/nnue.md:1014-1069 (int16 accumulate) and :2097-2134
  *                                 (pairwise product, shift), constants model/quantize.py:58-73
@@ -482,5 +484,69 @@ int nnueft_oracle_stack_int8_fwd(const uint8_t* x, const int64_t* bucket, const 
         const long long num = 2ll * ((long long)a3 + a1[L2 - 2] - a1[L2 - 1]) * out_mult;
         out[p] = (int32_t)(num / out_den);
     }
+    return 0;
+}
+
+/*
+ * RangerLite update of one parameter tensor; follows the reference's fused kernels
+ * (model/optimizers/ranger_lite.py:46-201) and, where lookahead is given, lookahead_process_step
+ * (:737-760).  neg_grad_ma NULL: plain first moment (the *_adam kernels; beta1 / one_minus_beta1 are
+ * then beta1 itself), else the positive-negative pair (beta1 = beta1^2).  update_variance 0: the
+ * *_phase2 kernels.  lookahead NULL: no merge.  Every operation rounds on its own.
+ */
+#include <math.h>
+int nnueft_oracle_ranger_lite_update(float* p, const float* grad, float* grad_ma, float* neg_grad_ma,
+                                     float* variance_ma, float* lookahead, long long n,
+                                     float beta2, float one_minus_beta2, float bias_correction2,
+                                     float beta1, float one_minus_beta1, float one_plus_pnm, float pnm_factor,
+                                     float noise_norm, float lr_div_bc1, float eps, long long step, float wd_factor,
+                                     int update_variance, float alpha)
+{
+    const int odd = (int)(step & 1);
+    const float one_minus_alpha = 1.0f - alpha;
+    for (long long i = 0; i < n; ++i) {
+        const float g = grad[i];
+        float vm = variance_ma[i];
+        if (update_variance) {
+            vm = vm * beta2 + (g * g) * one_minus_beta2;
+            variance_ma[i] = vm;
+        }
+        const float denom = sqrtf(vm / bias_correction2) + eps;
+        float dir;
+        if (neg_grad_ma) {
+            float* pos = odd ? grad_ma : neg_grad_ma;
+            const float* neg = odd ? neg_grad_ma : grad_ma;
+            const float np_ = pos[i] * beta1 + g * one_minus_beta1;
+            dir = (np_ * one_plus_pnm - neg[i] * pnm_factor) / noise_norm;
+            pos[i] = np_;
+        } else {
+            const float gm = grad_ma[i] * beta1 + g * one_minus_beta1;
+            grad_ma[i] = gm;
+            dir = gm;
+        }
+        float q = p[i];
+        if (wd_factor != 0.0f) q = q * (1.0f - wd_factor);
+        q = q - lr_div_bc1 * (dir / denom);
+        if (lookahead) {
+            q = q * alpha + lookahead[i] * one_minus_alpha;
+            lookahead[i] = q;
+        }
+        p[i] = q;
+    }
+    return 0;
+}
+
+int nnueft_oracle_ranger_lite_update_variance(const float* grad, float* variance_ma, long long n, float beta2,
+                                              float one_minus_beta2)
+{
+    for (long long i = 0; i < n; ++i) variance_ma[i] = variance_ma[i] * beta2 + (grad[i] * grad[i]) * one_minus_beta2;
+    return 0;
+}
+
+/* out = (floor(x * scale + eps) / scale) * post_mul: _fake_quantize_acts (model/quantize.py:36-45) and the
+ * correction factor applied after it (composed_feature_transformer.py:143-149). */
+int nnueft_oracle_act_fake_quantize(const float* x, float* out, long long n, float scale, float eps, float post_mul)
+{
+    for (long long i = 0; i < n; ++i) out[i] = (floorf(x[i] * scale + eps) / scale) * post_mul;
     return 0;
 }

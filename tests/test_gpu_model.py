@@ -129,3 +129,17 @@ def test_model_under_torch_compile_on_gpu(backend):
     finally:
         nnueft.set_backward_mode(old)
         torch._dynamo.reset()
+
+
+@pytest.mark.parametrize("n,post_mul", [(1, 1.0), (7, 0.5), (4096 * 33 + 3, 1.0), (16384 * 3072 // 8, 1.3)])
+def test_act_fake_quantize_kernel(oracle_cpu, n, post_mul):
+    from nnueft.model import _ActFakeQuantize
+
+    g = torch.Generator().manual_seed(n)
+    x = (torch.rand(n, generator=g) * 1.2 - 0.1).to(DEV).requires_grad_()
+    out = _ActFakeQuantize.apply(x, 128.0, post_mul)
+    ref = oracle_cpu.act_fake_quantize(x.detach().cpu().numpy(), 128.0, M.FAKE_QUANTIZE_EPS, post_mul)
+    assert np.array_equal(out.detach().cpu().numpy(), ref)
+    up = torch.randn(n, generator=g).to(DEV)
+    out.backward(up)
+    assert torch.equal(x.grad, up * post_mul)

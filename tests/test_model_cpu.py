@@ -208,3 +208,19 @@ def test_model_under_torch_compile_on_cpu(backend):
     assert torch.allclose(o, out, atol=1e-6)
     for n, p in m.named_parameters():
         assert torch.allclose(p.grad, ref[n], atol=1e-5), n
+
+
+@pytest.mark.parametrize("post_mul", [1.0, 0.75, 1.3])
+def test_act_fake_quantize_oracle_equals_the_torch_ops(oracle_cpu, post_mul):
+    g = torch.Generator().manual_seed(21)
+    x = torch.cat([torch.rand(5000, generator=g), torch.randn(3000, generator=g) * 3,
+                   torch.arange(0, 129).float() / 128, torch.tensor([0.0, -0.0, 127 / 128, 1.0, 1e-6, -1e-6])])
+    q = M.QuantizationManager(M.QuantizationConfig())
+    ref = q.fake_quantize_ft_act(x) * post_mul           # mul, add, floor, div, then the correction factor
+    got = oracle_cpu.act_fake_quantize(x.numpy(), scale=q.hidden_quantized_one, eps=M.FAKE_QUANTIZE_EPS,
+                                       post_mul=post_mul)
+    assert np.array_equal(got, ref.numpy())
+    # the grid: multiples of 1/128, never above x by more than the epsilon's worth
+    if post_mul == 1.0:
+        assert np.array_equal(got * 128, np.floor(got * 128))
+        assert (got <= x.numpy() + 1e-5 / 128 + 1e-7).all()
