@@ -219,6 +219,30 @@ int nnueft_stack_int8_fwd(const uint8_t* x, const int64_t* bucket, const int8_t*
                           int out_mult, int out_den, void* stream);
 
 /*
+ * Bucketed linear layer: y[b, :] = bias[bucket[b]] + W[bucket[b]] x[b], where W holds `count` blocks
+ * of [out, in] one after the other (the layout of nn.Linear(in, out * count)).  Same values, up to
+ * the order of the floating-point sums, as StackedLinear.forward of the reference
+ * (model/modules/stacked_linear.py:38-66): F.linear over all blocks followed by select_output; the
+ * backward is what autograd derives from that: gx[b] = W[bucket[b]]^T gy[b]; gW and gbias of a
+ * block sum gy[b] (x) x[b] and gy[b] over the positions of that bucket (ascending position order,
+ * so the result does not change from run to run), blocks no position uses get zeros.
+ * x f32[B, in]; bucket int64[B], every entry in [0, count) (a position outside is skipped: its row
+ * of y and gx is left unwritten); W f32[count * out, in]; bias f32[count * out]; y, gy f32[B, out];
+ * gx f32[B, in] or NULL; gW, gbias fully written.  Limits: out <= 32, count <= 64, in % 32 == 0,
+ * x and W 16-byte aligned.  workspace: nnueft_bucket_linear_workspace_bytes(B, count) bytes; the
+ * forward leaves the grouping of the positions in it, and a backward call given that same buffer
+ * untouched (and the same bucket tensor) may say so with workspace_from_fwd = 1 to skip regrouping.
+ * Tolerance against the reference: 1e-5 relative to the largest magnitude of the result.
+ */
+size_t nnueft_bucket_linear_workspace_bytes(int B, int count);
+int nnueft_bucket_linear_fwd(const float* x, const int64_t* bucket, const float* W, const float* bias, float* y,
+                             int B, int in, int out, int count, void* workspace, size_t workspace_bytes,
+                             void* stream);
+int nnueft_bucket_linear_bwd(const float* x, const int64_t* bucket, const float* W, const float* gy, float* gx,
+                             float* gW, float* gbias, int B, int in, int out, int count, void* workspace,
+                             size_t workspace_bytes, int workspace_from_fwd, void* stream);
+
+/*
  * out[i] = (floor(x[i] * scale + eps) / scale) * post_mul, each operation rounding on its own: the
  * activation fake quantization of the feature transformer's output (_fake_quantize_acts,
  * model/quantize.py:36-45, called from composed_feature_transformer.py:143-144) together with the

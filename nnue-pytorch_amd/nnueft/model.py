@@ -361,6 +361,65 @@ class ComposedFeatureTransformer(nn.Module):
 
 # ------------------------------------------------------------------------------------------ layer stacks
 
+@torch.compiler.disable(recursive=False)
+def _launch_bucket_linear_fwd(x, bucket, weight, bias, out_features, count):
+    lib = _native.load()
+    B, n_in = x.shape
+    y = torch.empty(B, out_features, dtype=torch.float32, device=x.device)
+    nbytes = lib.nnueft_bucket_linear_workspace_bytes(B, count)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.nnueft_bucket_linear_fwd(x.data_ptr(), bucket.data_ptr(), weight.data_ptr(), bias.data_ptr(),
+                                          y.data_ptr(), B, n_in, out_features, count, ws.data_ptr(), nbytes,
+                                          _stream_ptr(x.device))
+    _native.check(rc, "nnueft_bucket_linear_fwd")
+    return y, ws
+
+
+@torch.compiler.disable(recursive=False)
+def _launch_bucket_linear_bwd(x, bucket, weight, gy, out_features, count, need_gx, ws):
+    lib = _native.load()
+    B, n_in = x.shape
+    gx = torch.empty_like(x) if need_gx else None
+    gw = torch.empty_like(weight)
+    gb = torch.empty(count * out_features, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        # ws still holds the grouping of the positions the forward call made (a few bytes per position)
+        rc = lib.nnueft_bucket_linear_bwd(x.data_ptr(), bucket.data_ptr(), weight.data_ptr(), gy.data_ptr(),
+                                          gx.data_ptr() if need_gx else None, gw.data_ptr(), gb.data_ptr(), B, n_in,
+                                          out_features, count, ws.data_ptr(), ws.numel(), 1, _stream_ptr(x.device))
+    _native.check(rc, "nnueft_bucket_linear_bwd")
+    return gx, gw, gb
+
+
+class _BucketLinear(torch.autograd.Function):
+    """y[b] = bias[bucket[b]] + weight[bucket[b]] x[b]: every position meets the block of its own
+    bucket only (the wide layer followed by a selection computes the other blocks to drop them)."""
+
+    @staticmethod
+    def forward(ctx, x, bucket, weight, bias, out_features, count):
+        x, weight, bias = x.contiguous(), weight.contiguous(), bias.contiguous()
+        bucket = bucket.flatten().contiguous()
+        y, ws = _launch_bucket_linear_fwd(x, bucket, weight, bias, out_features, count)
+        ctx.save_for_backward(x, bucket, weight, ws)
+        ctx.shape = (out_features, count)
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        x, bucket, weight, ws = ctx.saved_tensors
+        out_features, count = ctx.shape
+        gx, gw, gb = _launch_bucket_linear_bwd(x, bucket, weight, gy.contiguous(), out_features, count,
+                                               ctx.needs_input_grad[0], ws)
+        return gx, None, gw, gb, None, None
+
+
+def _bucket_linear_applies(x, in_features, out_features, count):
+    # worth it where the layer is wide; the small layers behind it stay torch GEMMs
+    return (x.is_cuda and x.dtype == torch.float32 and in_features >= 256 and in_features % 32 == 0
+            and out_features <= 32 and count <= 64 and _native.available())
+
+
 class StackedLinear(nn.Module):
     """`count` linear layers of the same shape evaluated as one wide layer; each position picks the
     output block of its bucket."""
@@ -384,6 +443,8 @@ class StackedLinear(nn.Module):
                 raise RuntimeError("self.quantization and self.layer_key are required to use fake quantize weights.")
             weight = self.quantization.fake_quantize_weights(weight, f"{self.layer_key}_weight")
             bias = self.quantization.fake_quantize_weights(bias, f"{self.layer_key}_bias")
+        if _bucket_linear_applies(x, self.in_features, self.out_features, self.count):
+            return _BucketLinear.apply(x, ls_indices, weight, bias, self.out_features, self.count)
         wide = F.linear(x, weight, bias).reshape(-1, self.out_features)
         pick = ls_indices.flatten() + torch.arange(0, ls_indices.shape[0] * self.count, self.count, device=x.device)
         return wide[pick]

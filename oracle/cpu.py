@@ -210,3 +210,26 @@ def act_fake_quantize(x, scale=128.0, eps=1e-5, post_mul=1.0):
                                                ctypes.c_float(eps), ctypes.c_float(post_mul))
     assert rc == 0
     return out
+
+
+def bucket_linear_fwd(x, bucket, W, bias, out, count):
+    x, W, bias = _c(x, np.float32), _c(W, np.float32), _c(bias, np.float32)
+    bucket = _c(bucket, np.int64)
+    B, n_in = x.shape
+    y = np.zeros((B, out), np.float32)
+    rc = lib().nnueft_oracle_bucket_linear_fwd(_p(x), _p(bucket), _p(W), _p(bias), _p(y), B, n_in, out, count)
+    assert rc == 0
+    return y
+
+
+def bucket_linear_bwd(x, bucket, W, gy, out, count):
+    x, W, gy = _c(x, np.float32), _c(W, np.float32), _c(gy, np.float32)
+    bucket = _c(bucket, np.int64)
+    B, n_in = x.shape
+    gx = np.zeros((B, n_in), np.float32)
+    gW = np.empty((count * out, n_in), np.float32)
+    gb = np.empty((count * out,), np.float32)
+    rc = lib().nnueft_oracle_bucket_linear_bwd(_p(x), _p(bucket), _p(W), _p(gy), _p(gx), _p(gW), _p(gb), B, n_in, out,
+                                               count)
+    assert rc == 0
+    return gx, gW, gb

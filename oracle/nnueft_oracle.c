@@ -550,3 +550,54 @@ int nnueft_oracle_act_fake_quantize(const float* x, float* out, long long n, flo
     for (long long i = 0; i < n; ++i) out[i] = (floorf(x[i] * scale + eps) / scale) * post_mul;
     return 0;
 }
+
+/*
+ * Bucketed linear layer and its gradients: StackedLinear.forward (model/modules/stacked_linear.py:38-66;
+ * F.linear over all blocks, then select_output) and what autograd derives from it, written for the
+ * one block a position selects.  Sums run over ascending input index / ascending position; the
+ * GPU kernels associate differently, so they are compared to a tolerance.
+ */
+int nnueft_oracle_bucket_linear_fwd(const float* x, const int64_t* bucket, const float* W, const float* bias,
+                                    float* y, int B, int in, int out, int count)
+{
+#pragma omp parallel for schedule(static)
+    for (int b = 0; b < B; ++b) {
+        const int64_t k = bucket[b];
+        if (k < 0 || k >= count) continue;
+        for (int o = 0; o < out; ++o) {
+            const float* w = W + ((size_t)k * out + o) * in;
+            double acc = bias[k * out + o];
+            for (int i = 0; i < in; ++i) acc += (double)x[(size_t)b * in + i] * (double)w[i];
+            y[(size_t)b * out + o] = (float)acc;
+        }
+    }
+    return 0;
+}
+
+int nnueft_oracle_bucket_linear_bwd(const float* x, const int64_t* bucket, const float* W, const float* gy,
+                                    float* gx, float* gW, float* gbias, int B, int in, int out, int count)
+{
+    double* aw = (double*)calloc((size_t)count * out * in, sizeof(double));
+    double* ab = (double*)calloc((size_t)count * out, sizeof(double));
+    if (!aw || !ab) { free(aw); free(ab); return -2; }
+    for (int b = 0; b < B; ++b) {
+        const int64_t k = bucket[b];
+        if (k < 0 || k >= count) continue;
+        for (int i = 0; i < in; ++i) {
+            double acc = 0.0;
+            for (int o = 0; o < out; ++o) acc += (double)gy[(size_t)b * out + o] * (double)W[((size_t)k * out + o) * in + i];
+            if (gx) gx[(size_t)b * in + i] = (float)acc;
+        }
+        for (int o = 0; o < out; ++o) {
+            const double g = gy[(size_t)b * out + o];
+            ab[k * out + o] += g;
+            double* row = aw + ((size_t)k * out + o) * in;
+            for (int i = 0; i < in; ++i) row[i] += g * (double)x[(size_t)b * in + i];
+        }
+    }
+    for (size_t i = 0; i < (size_t)count * out * in; ++i) gW[i] = (float)aw[i];
+    for (int i = 0; i < count * out; ++i) gbias[i] = (float)ab[i];
+    free(aw);
+    free(ab);
+    return 0;
+}

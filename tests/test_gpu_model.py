@@ -143,3 +143,75 @@ def test_act_fake_quantize_kernel(oracle_cpu, n, post_mul):
     up = torch.randn(n, generator=g).to(DEV)
     out.backward(up)
     assert torch.equal(x.grad, up * post_mul)
+
+
+@pytest.mark.parametrize("B,n_in,out,count", [(1, 32, 1, 1), (37, 64, 16, 8), (300, 128, 32, 8), (1000, 3072, 32, 8),
+                                              (4097, 1024, 16, 8), (513, 96, 7, 3), (64, 256, 32, 64)])
+def test_bucket_linear_kernels(oracle_cpu, B, n_in, out, count):
+    from nnueft import _native
+
+    lib = _native.load()
+    rng = np.random.default_rng(B + n_in)
+    x = rng.standard_normal((B, n_in)).astype(np.float32)
+    W = (rng.standard_normal((count * out, n_in)) / np.sqrt(n_in)).astype(np.float32)
+    bias = rng.standard_normal(count * out).astype(np.float32)
+    bucket = rng.integers(0, count, size=B).astype(np.int64)
+    if count > 2:
+        bucket[bucket == 1] = 0          # one bucket nobody uses: its gradient blocks must come out zero
+    gy = rng.standard_normal((B, out)).astype(np.float32)
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    dx, dW, db, dk, dgy = t(x), t(W), t(bias), t(bucket), t(gy)
+    nbytes = lib.nnueft_bucket_linear_workspace_bytes(B, count)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    y = torch.full((B, out), float("nan"), device=DEV)
+    _native.check(lib.nnueft_bucket_linear_fwd(dx.data_ptr(), dk.data_ptr(), dW.data_ptr(), db.data_ptr(), y.data_ptr(),
+                                               B, n_in, out, count, ws.data_ptr(), nbytes, stream), "fwd")
+    ref = oracle_cpu.bucket_linear_fwd(x, bucket, W, bias, out, count)
+    tol = lambda r: 1e-5 * max(float(np.abs(r).max()), 1e-30)
+    assert np.abs(y.cpu().numpy() - ref).max() <= tol(ref)
+    gx = torch.full((B, n_in), float("nan"), device=DEV)
+    gW = torch.full((count * out, n_in), float("nan"), device=DEV)
+    gb = torch.full((count * out,), float("nan"), device=DEV)
+    _native.check(lib.nnueft_bucket_linear_bwd(dx.data_ptr(), dk.data_ptr(), dW.data_ptr(), dgy.data_ptr(),
+                                               gx.data_ptr(), gW.data_ptr(), gb.data_ptr(), B, n_in, out, count,
+                                               ws.data_ptr(), nbytes, 1, stream), "bwd")   # grouping left by the forward
+    rx, rW, rb = oracle_cpu.bucket_linear_bwd(x, bucket, W, gy, out, count)
+    assert np.abs(gx.cpu().numpy() - rx).max() <= tol(rx)
+    assert np.abs(gW.cpu().numpy() - rW).max() <= tol(rW)
+    assert np.abs(gb.cpu().numpy() - rb).max() <= tol(rb)
+    if count > 2:
+        assert not gW.cpu().numpy()[out:2 * out].any() and not gb.cpu().numpy()[out:2 * out].any()
+    # twice the same bits
+    gW2 = torch.empty_like(gW)
+    ws.zero_()                                   # regrouped inside this call
+    _native.check(lib.nnueft_bucket_linear_bwd(dx.data_ptr(), dk.data_ptr(), dW.data_ptr(), dgy.data_ptr(), None,
+                                               gW2.data_ptr(), gb.data_ptr(), B, n_in, out, count, ws.data_ptr(),
+                                               nbytes, 0, stream), "bwd")
+    assert torch.equal(gW, gW2)
+
+
+def test_stacked_linear_on_gpu_equals_the_wide_layer():
+    torch.manual_seed(3)
+    q = M.QuantizationManager(M.QuantizationConfig())
+    layer = M.FactorizedStackedLinear(512, 16, 8, q, "ls_l1")
+    with torch.no_grad():
+        layer.factorized_linear.weight.normal_(0, 0.02)
+    gpu = M.FactorizedStackedLinear(512, 16, 8, q, "ls_l1").to(DEV)
+    gpu.load_state_dict(layer.state_dict())
+    x = torch.rand(700, 512)
+    idx = torch.randint(0, 8, (700,))
+    for fq in (False, True):
+        layer.zero_grad()
+        gpu.zero_grad()
+        xc = x.clone().requires_grad_()
+        xg = x.to(DEV).requires_grad_()
+        yc = layer(xc, idx, fq)
+        yg = gpu(xg, idx.to(DEV), fq)
+        torch.testing.assert_close(yg.cpu(), yc, rtol=1e-4, atol=1e-5)
+        up = torch.randn_like(yc)
+        yc.backward(up)
+        yg.backward(up.to(DEV))
+        torch.testing.assert_close(xg.grad.cpu(), xc.grad, rtol=1e-4, atol=1e-5)
+        for (n, a), (_, b) in zip(layer.named_parameters(), gpu.named_parameters()):
+            torch.testing.assert_close(b.grad.cpu(), a.grad, rtol=1e-4, atol=2e-5, msg=n)

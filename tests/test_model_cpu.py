@@ -224,3 +224,25 @@ def test_act_fake_quantize_oracle_equals_the_torch_ops(oracle_cpu, post_mul):
     if post_mul == 1.0:
         assert np.array_equal(got * 128, np.floor(got * 128))
         assert (got <= x.numpy() + 1e-5 / 128 + 1e-7).all()
+
+
+@pytest.mark.parametrize("B,n_in,out,count", [(50, 64, 5, 3), (300, 96, 16, 8), (64, 32, 32, 1)])
+def test_bucket_linear_oracle_equals_wide_layer_and_selection(oracle_cpu, B, n_in, out, count):
+    # the reference's formula (stacked_linear.py:38-66): F.linear over all blocks, reshape, pick one block per position
+    import torch.nn.functional as F
+
+    rng = np.random.default_rng(B)
+    x = rng.standard_normal((B, n_in)).astype(np.float32)
+    W = rng.standard_normal((count * out, n_in)).astype(np.float32)
+    b = rng.standard_normal(count * out).astype(np.float32)
+    k = rng.integers(0, count, size=B)
+    gy = rng.standard_normal((B, out)).astype(np.float32)
+    tx, tW, tb = [torch.from_numpy(a).requires_grad_() for a in (x, W, b)]
+    wide = F.linear(tx, tW, tb).reshape(-1, out)
+    y = wide[torch.from_numpy(k) + torch.arange(0, B * count, count)]
+    y.backward(torch.from_numpy(gy))
+    assert np.allclose(oracle_cpu.bucket_linear_fwd(x, k, W, b, out, count), y.detach().numpy(), rtol=1e-5, atol=1e-5)
+    gx, gW, gb = oracle_cpu.bucket_linear_bwd(x, k, W, gy, out, count)
+    assert np.allclose(gx, tx.grad.numpy(), rtol=1e-5, atol=1e-5)
+    assert np.allclose(gW, tW.grad.numpy(), rtol=1e-5, atol=1e-5)
+    assert np.allclose(gb, tb.grad.numpy(), rtol=1e-5, atol=1e-5)
