@@ -30,11 +30,11 @@ extern "C" int nnueft_act_fake_quantize(const float* x, float* out, long long n,
     hipStream_t st = (hipStream_t)stream;
     if (aligned16(x) && aligned16(out) && n >= 4) {
         const long long wg = (n / 4 + 255) / 256;
-        hipLaunchKernelGGL(k_act_fake_quantize<4>, dim3((unsigned)max(1LL, min(wg, 256LL * 32))), dim3(256), 0, st, x,
+        hipLaunchKernelGGL(k_act_fake_quantize<4>, dim3((unsigned)max(1LL, min(wg, 0x7fffffffLL))), dim3(256), 0, st, x,
                            out, n, scale, eps, post_mul);
     } else {
         const long long wg = (n + 255) / 256;
-        hipLaunchKernelGGL(k_act_fake_quantize<1>, dim3((unsigned)max(1LL, min(wg, 256LL * 32))), dim3(256), 0, st, x,
+        hipLaunchKernelGGL(k_act_fake_quantize<1>, dim3((unsigned)max(1LL, min(wg, 0x7fffffffLL))), dim3(256), 0, st, x,
                            out, n, scale, eps, post_mul);
     }
     NNUEFT_LAUNCH_CHECK();
