@@ -229,18 +229,22 @@ int nnueft_stack_int8_fwd(const uint8_t* x, const int64_t* bucket, const int8_t*
  * x f32[B, in]; bucket int64[B], every entry in [0, count) (a position outside is skipped: its row
  * of y and gx is left unwritten); W f32[count * out, in]; bias f32[count * out]; y, gy f32[B, out];
  * gx f32[B, in] or NULL; gW, gbias fully written.  Limits: out <= 32, count <= 64, in % 32 == 0,
- * x and W 16-byte aligned.  workspace: nnueft_bucket_linear_workspace_bytes(B, count) bytes; the
- * forward leaves the grouping of the positions in it, and a backward call given that same buffer
- * untouched (and the same bucket tensor) may say so with workspace_from_fwd = 1 to skip regrouping.
+ * x and W 16-byte aligned.  workspace: nnueft_bucket_linear_workspace_bytes(B, count) bytes.  A call
+ * first groups the positions by bucket into the workspace; nnueft_bucket_linear_group does only
+ * that, and a call given a workspace that already holds the grouping of the same bucket tensor
+ * (from it or from an earlier call, untouched since) says so with workspace_grouped = 1 and skips it:
+ * the three layers of a stack and their backward passes share one grouping.
  * Tolerance against the reference: 1e-5 relative to the largest magnitude of the result.
  */
 size_t nnueft_bucket_linear_workspace_bytes(int B, int count);
+int nnueft_bucket_linear_group(const int64_t* bucket, int B, int count, void* workspace, size_t workspace_bytes,
+                               void* stream);
 int nnueft_bucket_linear_fwd(const float* x, const int64_t* bucket, const float* W, const float* bias, float* y,
                              int B, int in, int out, int count, void* workspace, size_t workspace_bytes,
-                             void* stream);
+                             int workspace_grouped, void* stream);
 int nnueft_bucket_linear_bwd(const float* x, const int64_t* bucket, const float* W, const float* gy, float* gx,
                              float* gW, float* gbias, int B, int in, int out, int count, void* workspace,
-                             size_t workspace_bytes, int workspace_from_fwd, void* stream);
+                             size_t workspace_bytes, int workspace_grouped, void* stream);
 
 /*
  * out[i] = (floor(x[i] * scale + eps) / scale) * post_mul, each operation rounding on its own: the

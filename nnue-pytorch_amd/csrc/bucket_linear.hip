@@ -337,9 +337,18 @@ extern "C" size_t nnueft_bucket_linear_workspace_bytes(int B, int count) {
     return bucket_layout(B, count, &L) ? L.end : 0;
 }
 
+extern "C" int nnueft_bucket_linear_group(const int64_t* bucket, int B, int count, void* workspace,
+                                          size_t workspace_bytes, void* stream) {
+    if (!bucket) return NNUEFT_E_ARG;
+    BucketLayout L;
+    if (!bucket_layout(B, count, &L)) return NNUEFT_E_ARG;
+    if (!workspace || !aligned256(workspace) || workspace_bytes < L.end) return NNUEFT_E_WORKSPACE;
+    return launch_order(bucket, (char*)workspace, L, B, count, (hipStream_t)stream);
+}
+
 extern "C" int nnueft_bucket_linear_fwd(const float* x, const int64_t* bucket, const float* W, const float* bias,
                                         float* y, int B, int in, int out, int count, void* workspace,
-                                        size_t workspace_bytes, void* stream) {
+                                        size_t workspace_bytes, int workspace_grouped, void* stream) {
     const int bad = check_args(B, in, out, count);
     if (bad) return bad;
     if (!x || !bucket || !W || !bias || !y) return NNUEFT_E_ARG;
@@ -349,8 +358,10 @@ extern "C" int nnueft_bucket_linear_fwd(const float* x, const int64_t* bucket, c
     if (!workspace || !aligned256(workspace) || workspace_bytes < L.end) return NNUEFT_E_WORKSPACE;
     hipStream_t st = (hipStream_t)stream;
     char* ws = (char*)workspace;
-    const int rc = launch_order(bucket, ws, L, B, count, st);
-    if (rc) return rc;
+    if (!workspace_grouped) {
+        const int rc = launch_order(bucket, ws, L, B, count, st);
+        if (rc) return rc;
+    }
     const uint32_t* order = (const uint32_t*)(ws + L.order);
     const uint32_t* ntiles = (const uint32_t*)(ws + L.ntiles);
     const uint32_t* tiles = (const uint32_t*)(ws + L.tiles);
@@ -369,7 +380,7 @@ extern "C" int nnueft_bucket_linear_fwd(const float* x, const int64_t* bucket, c
 
 extern "C" int nnueft_bucket_linear_bwd(const float* x, const int64_t* bucket, const float* W, const float* gy,
                                         float* gx, float* gW, float* gbias, int B, int in, int out, int count,
-                                        void* workspace, size_t workspace_bytes, int workspace_from_fwd,
+                                        void* workspace, size_t workspace_bytes, int workspace_grouped,
                                         void* stream) {
     const int bad = check_args(B, in, out, count);
     if (bad) return bad;
@@ -379,7 +390,7 @@ extern "C" int nnueft_bucket_linear_bwd(const float* x, const int64_t* bucket, c
     if (!workspace || !aligned256(workspace) || workspace_bytes < L.end) return NNUEFT_E_WORKSPACE;
     hipStream_t st = (hipStream_t)stream;
     char* ws = (char*)workspace;
-    if (!workspace_from_fwd) {
+    if (!workspace_grouped) {
         const int rc = launch_order(bucket, ws, L, B, count, st);
         if (rc) return rc;
     }

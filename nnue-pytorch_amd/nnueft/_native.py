@@ -39,7 +39,8 @@ PROTOTYPES = {
     "nnueft_ft_int16_fwd": (c_int, [c_void_p] * 9 + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
     "nnueft_stack_int8_fwd": (c_int, [c_void_p] * 9 + [c_int] * 12 + [c_void_p]),
     "nnueft_bucket_linear_workspace_bytes": (c_size_t, [c_int] * 2),
-    "nnueft_bucket_linear_fwd": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
+    "nnueft_bucket_linear_group": (c_int, [c_void_p] + [c_int] * 2 + [c_void_p, c_size_t, c_void_p]),
+    "nnueft_bucket_linear_fwd": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_void_p, c_size_t, c_int, c_void_p]),
     "nnueft_bucket_linear_bwd": (c_int, [c_void_p] * 7 + [c_int] * 4 + [c_void_p, c_size_t, c_int, c_void_p]),
     "nnueft_act_fake_quantize": (c_int, [c_void_p] * 2 + [c_longlong] + [c_float] * 3 + [c_void_p]),
     "nnueft_ranger_lite_update_pnm": (

@@ -362,18 +362,32 @@ class ComposedFeatureTransformer(nn.Module):
 # ------------------------------------------------------------------------------------------ layer stacks
 
 @torch.compiler.disable(recursive=False)
-def _launch_bucket_linear_fwd(x, bucket, weight, bias, out_features, count):
+def bucket_grouping(bucket, count):
+    """The positions of a batch grouped by bucket, as the bucketed linear kernels read them: an opaque
+    byte tensor to hand to every StackedLinear of the stack (they share `bucket`)."""
+    lib = _native.load()
+    bucket = bucket.flatten().contiguous()
+    B = bucket.shape[0]
+    nbytes = lib.nnueft_bucket_linear_workspace_bytes(B, count)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=bucket.device)
+    with torch.cuda.device(bucket.device):
+        rc = lib.nnueft_bucket_linear_group(bucket.data_ptr(), B, count, ws.data_ptr(), nbytes,
+                                            _stream_ptr(bucket.device))
+    _native.check(rc, "nnueft_bucket_linear_group")
+    return ws
+
+
+@torch.compiler.disable(recursive=False)
+def _launch_bucket_linear_fwd(x, bucket, weight, bias, out_features, count, ws):
     lib = _native.load()
     B, n_in = x.shape
     y = torch.empty(B, out_features, dtype=torch.float32, device=x.device)
-    nbytes = lib.nnueft_bucket_linear_workspace_bytes(B, count)
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
     with torch.cuda.device(x.device):
         rc = lib.nnueft_bucket_linear_fwd(x.data_ptr(), bucket.data_ptr(), weight.data_ptr(), bias.data_ptr(),
-                                          y.data_ptr(), B, n_in, out_features, count, ws.data_ptr(), nbytes,
+                                          y.data_ptr(), B, n_in, out_features, count, ws.data_ptr(), ws.numel(), 1,
                                           _stream_ptr(x.device))
     _native.check(rc, "nnueft_bucket_linear_fwd")
-    return y, ws
+    return y
 
 
 @torch.compiler.disable(recursive=False)
@@ -397,13 +411,13 @@ class _BucketLinear(torch.autograd.Function):
     bucket only (the wide layer followed by a selection computes the other blocks to drop them)."""
 
     @staticmethod
-    def forward(ctx, x, bucket, weight, bias, out_features, count):
+    def forward(ctx, x, bucket, weight, bias, out_features, count, grouping):
         x, weight, bias = x.contiguous(), weight.contiguous(), bias.contiguous()
         bucket = bucket.flatten().contiguous()
-        y, ws = _launch_bucket_linear_fwd(x, bucket, weight, bias, out_features, count)
+        ws = grouping if grouping is not None else bucket_grouping(bucket, count)
         ctx.save_for_backward(x, bucket, weight, ws)
         ctx.shape = (out_features, count)
-        return y
+        return _launch_bucket_linear_fwd(x, bucket, weight, bias, out_features, count, ws)
 
     @staticmethod
     def backward(ctx, gy):
@@ -411,12 +425,12 @@ class _BucketLinear(torch.autograd.Function):
         out_features, count = ctx.shape
         gx, gw, gb = _launch_bucket_linear_bwd(x, bucket, weight, gy.contiguous(), out_features, count,
                                                ctx.needs_input_grad[0], ws)
-        return gx, None, gw, gb, None, None
+        return gx, None, gw, gb, None, None, None
 
 
 def _bucket_linear_applies(x, in_features, out_features, count):
-    # worth it where the layer is wide; the small layers behind it stay torch GEMMs
-    return (x.is_cuda and x.dtype == torch.float32 and in_features >= 256 and in_features % 32 == 0
+    # every layer of the stacks qualifies at the usual sizes (in = 3072, 64, 128)
+    return (x.is_cuda and x.dtype == torch.float32 and in_features >= 32 and in_features % 32 == 0
             and out_features <= 32 and count <= 64 and _native.available())
 
 
@@ -436,7 +450,8 @@ class StackedLinear(nn.Module):
     def _params(self):
         return self.linear.weight, self.linear.bias
 
-    def forward(self, x, ls_indices, fake_quantize_weights: bool = False):
+    def forward(self, x, ls_indices, fake_quantize_weights: bool = False, grouping=None):
+        """grouping: bucket_grouping(ls_indices, count) when several layers share ls_indices (optional)."""
         weight, bias = self._params()
         if fake_quantize_weights:
             if self.quantization is None or self.layer_key is None:
@@ -444,7 +459,7 @@ class StackedLinear(nn.Module):
             weight = self.quantization.fake_quantize_weights(weight, f"{self.layer_key}_weight")
             bias = self.quantization.fake_quantize_weights(bias, f"{self.layer_key}_bias")
         if _bucket_linear_applies(x, self.in_features, self.out_features, self.count):
-            return _BucketLinear.apply(x, ls_indices, weight, bias, self.out_features, self.count)
+            return _BucketLinear.apply(x, ls_indices, weight, bias, self.out_features, self.count, grouping)
         wide = F.linear(x, weight, bias).reshape(-1, self.out_features)
         pick = ls_indices.flatten() + torch.arange(0, ls_indices.shape[0] * self.count, self.count, device=x.device)
         return wide[pick]
@@ -512,11 +527,15 @@ class LayerStacks(nn.Module):
 
     def forward(self, x, ls_indices, fake_quantize_acts: bool = True, fake_quantize_weights: bool = True):
         q = self.quantization
-        l1c = self.l1(x, ls_indices, fake_quantize_weights)
+        # the three layers pick blocks by the same indices: group the positions once
+        grouping = None
+        if _bucket_linear_applies(x, self.l1.in_features, self.l1.out_features, self.count):
+            grouping = bucket_grouping(ls_indices, self.count)
+        l1c = self.l1(x, ls_indices, fake_quantize_weights, grouping)
         skip = l1c[:, -2].view(-1, 1) - l1c[:, -1].view(-1, 1)
         l1x = self._sqr_and_linear(l1c, fake_quantize_acts)
-        l2x = self._sqr_and_linear(self.l2(l1x, ls_indices, fake_quantize_weights), fake_quantize_acts)
-        out = self.output(torch.cat([l1x, l2x], dim=1), ls_indices, fake_quantize_weights)
+        l2x = self._sqr_and_linear(self.l2(l1x, ls_indices, fake_quantize_weights, grouping), fake_quantize_acts)
+        out = self.output(torch.cat([l1x, l2x], dim=1), ls_indices, fake_quantize_weights, grouping)
         if fake_quantize_acts:
             skip = q.fake_quantize_skip_act(skip)
         out = out + skip

@@ -166,7 +166,7 @@ def test_bucket_linear_kernels(oracle_cpu, B, n_in, out, count):
     stream = torch.cuda.current_stream().cuda_stream
     y = torch.full((B, out), float("nan"), device=DEV)
     _native.check(lib.nnueft_bucket_linear_fwd(dx.data_ptr(), dk.data_ptr(), dW.data_ptr(), db.data_ptr(), y.data_ptr(),
-                                               B, n_in, out, count, ws.data_ptr(), nbytes, stream), "fwd")
+                                               B, n_in, out, count, ws.data_ptr(), nbytes, 0, stream), "fwd")
     ref = oracle_cpu.bucket_linear_fwd(x, bucket, W, bias, out, count)
     tol = lambda r: 1e-5 * max(float(np.abs(r).max()), 1e-30)
     assert np.abs(y.cpu().numpy() - ref).max() <= tol(ref)
@@ -175,7 +175,7 @@ def test_bucket_linear_kernels(oracle_cpu, B, n_in, out, count):
     gb = torch.full((count * out,), float("nan"), device=DEV)
     _native.check(lib.nnueft_bucket_linear_bwd(dx.data_ptr(), dk.data_ptr(), dW.data_ptr(), dgy.data_ptr(),
                                                gx.data_ptr(), gW.data_ptr(), gb.data_ptr(), B, n_in, out, count,
-                                               ws.data_ptr(), nbytes, 1, stream), "bwd")   # grouping left by the forward
+                                               ws.data_ptr(), nbytes, 1, stream), "bwd")   # grouping left by the forward call
     rx, rW, rb = oracle_cpu.bucket_linear_bwd(x, bucket, W, gy, out, count)
     assert np.abs(gx.cpu().numpy() - rx).max() <= tol(rx)
     assert np.abs(gW.cpu().numpy() - rW).max() <= tol(rW)
@@ -184,7 +184,13 @@ def test_bucket_linear_kernels(oracle_cpu, B, n_in, out, count):
         assert not gW.cpu().numpy()[out:2 * out].any() and not gb.cpu().numpy()[out:2 * out].any()
     # twice the same bits
     gW2 = torch.empty_like(gW)
-    ws.zero_()                                   # regrouped inside this call
+    ws.zero_()
+    _native.check(lib.nnueft_bucket_linear_group(dk.data_ptr(), B, count, ws.data_ptr(), nbytes, stream), "group")
+    y2 = torch.empty_like(y)
+    _native.check(lib.nnueft_bucket_linear_fwd(dx.data_ptr(), dk.data_ptr(), dW.data_ptr(), db.data_ptr(), y2.data_ptr(),
+                                               B, n_in, out, count, ws.data_ptr(), nbytes, 1, stream), "fwd")
+    assert torch.equal(y, y2)
+    ws.zero_()                                   # regrouped inside the next call
     _native.check(lib.nnueft_bucket_linear_bwd(dx.data_ptr(), dk.data_ptr(), dW.data_ptr(), dgy.data_ptr(), None,
                                                gW2.data_ptr(), gb.data_ptr(), B, n_in, out, count, ws.data_ptr(),
                                                nbytes, 0, stream), "bwd")
