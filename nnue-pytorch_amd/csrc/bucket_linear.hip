@@ -238,6 +238,9 @@ __global__ __launch_bounds__(64) void k_bucket_bwd_x(const float* __restrict__ g
 // order, so the result is the same on every run.  Two positions per MFMA step, lanes 0-31 the even
 // one of the pair; the position numbers of a run arrive in one coalesced load.
 constexpr int kBwdWaves = 8;
+#ifndef NNUEFT_BWDW_PF
+#define NNUEFT_BWDW_PF 32
+#endif
 __global__ __launch_bounds__(kBwdWaves * 64) void k_bucket_bwd_w(const float* __restrict__ x,
                                                                  const float* __restrict__ gy,
                                                                  float* __restrict__ gW, float* __restrict__ gbias,
@@ -255,7 +258,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void k_bucket_bwd_w(const float* __
     float bsum = 0.0f;
     for (uint32_t e0 = beg + 64u * wave; e0 < end; e0 += 64u * kBwdWaves) {
         const uint32_t mine = e0 + lane < end ? order[e0 + lane] : 0xffffffffu;
-        constexpr int PF = 8;
+        constexpr int PF = NNUEFT_BWDW_PF;
 #pragma unroll
         for (int u0 = 0; u0 < 32; u0 += PF) {
             float a[PF], b0[PF], b1[PF];
