@@ -20,7 +20,9 @@ from . import _native
 _HAS_CUPY_KERNELS = _native.available()
 
 # "atomic" (reference semantics, unordered fp32 atomics) or "deterministic" (sort + segmented reduction)
-_BACKWARD_MODE = os.environ.get("NNUEFT_BACKWARD", "atomic")
+# "deterministic": sort + segmented reduction (any result of it is one the reference's unordered atomics
+# could have produced, and on MI355X it is five times faster); "atomic": the reference's scheme
+_BACKWARD_MODE = os.environ.get("NNUEFT_BACKWARD", "deterministic")
 
 
 def set_backward_mode(mode: str) -> None:
