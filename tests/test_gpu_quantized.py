@@ -72,3 +72,34 @@ def test_quantized_chain_tracks_the_float_model(oracle_cpu):
     assert np.array_equal(x_u8.cpu().numpy(), r_x) and np.array_equal(psqt.cpu().numpy(), r_ps)
     r_out = oracle_cpu.stack_int8_fwd(r_x, (pc - 1) // 4, *[s.numpy() for s in stack], 16, 32, 8)
     assert np.array_equal(out.cpu().numpy(), r_out)
+
+
+@pytest.mark.parametrize("compression", ["none", "leb128"])
+def test_net_read_back_from_a_nnue_file_evaluates_the_same(compression):
+    """model -> .nnue bytes -> model: the integer kernels give the same outputs for both."""
+    import io
+
+    from nnueft import serialize as S
+
+    torch.manual_seed(5)
+    L1, B = 128, 300
+    cfg = dict(L1=L1, L2=15, L3=32)
+    model = M.NNUEModel("HalfKAv2_hm^", M.ModelConfig(**cfg))
+    with torch.no_grad():
+        model.input.features[0].virtual_weight.normal_(0, 0.01)
+        model.layer_stacks.l1.factorized_linear.weight.normal_(0, 0.01)
+    buf = bytes(S.NNUEWriter(model, "round trip", compression).buf)
+    back = S.NNUEReader(io.BytesIO(buf), "HalfKAv2_hm^", M.ModelConfig(**cfg)).model
+    us, _, _, _, pc = hk.synthetic_batch(B, 31)
+    _, _, wf, bf, _ = hk.synthetic_batch(B, 31, fold_kings=True)
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    stm, bucket = t((1 - us[:, 0]).astype(np.uint8)), t((pc - 1) // 4)
+    outs = []
+    for m in (model, back):
+        w16, b16, p32 = quantized.quantize_feature_transformer(m.input.get_export_weights().float(),
+                                                               m.input.bias.detach().float(), L1)
+        x_u8, psqt = quantized.ft_int16_forward(t(wf), t(bf), stm, w16.to(DEV), b16.to(DEV), p32.to(DEV), bucket)
+        out = quantized.stack_int8_forward(x_u8, bucket, *[s.to(DEV) for s in quantized.quantize_layer_stacks(m.layer_stacks)])
+        outs.append((x_u8.cpu(), psqt.cpu(), out.cpu()))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
