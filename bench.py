@@ -192,6 +192,7 @@ def run_full_step(args, dev):
 
     L1, B = WORKLOADS[args.workload]
     nnueft.set_backward_mode(args.backward)
+    nnueft.set_sort_placement(args.sort_placement)
     torch.manual_seed(0)
     model = M.NNUEModel("HalfKAv2_hm^", M.ModelConfig(L1=L1, L2=32, L3=32)).to(dev)
     us, them, white, black, pc = [torch.from_numpy(a).to(dev) for a in hk.synthetic_batch(B, 1238)]
@@ -207,10 +208,11 @@ def run_full_step(args, dev):
         opt = torch.optim.Adam(model.parameters(), lr=8.75e-4, fused=True)
         opt_name = "torch.optim.Adam(fused=True)"
     params = M.LossParams()
+    fwd = torch.compile(model, backend=args.compile) if args.compile else model
 
     def step():
         opt.zero_grad(set_to_none=True)
-        out = model(us, them, white, black, pc)
+        out = fwd(us, them, white, black, pc)
         loss = M.sf_loss(out * model.quantization.nnue2score, score, outcome, params, 0.75)
         loss.backward()
         opt.step()
@@ -229,7 +231,7 @@ def run_full_step(args, dev):
         "unit": "positions/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": args.workload, "L1": L1, "L2": 32, "L3": 32, "batch": B, "backward": args.backward,
-                   "optimizer": opt_name, "lambda": 0.75, "fake_quantization": True,
+                   "optimizer": opt_name, "torch_compile": args.compile or None, "lambda": 0.75, "fake_quantization": True,
                    "final_loss": float(loss)},
         "roofline": None, "cpu_baseline": None,
     }))
@@ -246,6 +248,12 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--optimizer", default="rangerlite", choices=["rangerlite", "adam"],
                     help="full_step workload only")
+    ap.add_argument("--compile", default="", choices=["", "inductor", "aot_eager"],
+                    help="full_step workload only: torch.compile the model with this backend, as the reference's "
+                         "train.py does (the kernels of this build stay opaque to it); off by default")
+    ap.add_argument("--sort-placement", default="inline", choices=["inline", "backward", "forward"],
+                    help="where the index sort of the deterministic backward runs (nnueft.set_sort_placement); "
+                         "the default is the library's")
     ap.add_argument("--positions", default="uniform", choices=["uniform", "game"],
                     help="uniform: kings and pieces uniform over the board (the headline workload); game: piece "
                          "placement statistics of real game positions, where one or two king buckets hold a large "
@@ -263,6 +271,7 @@ def main():
     from nnueft import _native
     from nnueft.double_ft_functions import double_feature_transform
 
+    nnueft.set_sort_placement(args.sort_placement)
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
@@ -355,9 +364,13 @@ def main():
                 t["psqt_idx"].data_ptr(), bd.data_ptr(), max_act, g_l0.data_ptr(), g_wp.data_ptr(), g_bp.data_ptr(),
                 saved.data_ptr())
 
+        from nnueft.sparse_linear_functions import _aux_stream_ptr
+
+        aux_stream = _aux_stream_ptr(dev)      # what FusedDoubleFtFunction passes
+
         def bwd_det():
             rc = lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT,
-                                           ws.data_ptr(), nbytes, stream)
+                                           ws.data_ptr(), nbytes, None, stream, aux_stream)
             assert rc == 0
 
         def bwd_atomic():
@@ -369,6 +382,24 @@ def main():
         for name, fn in (("deterministic", bwd_det), ("atomic", bwd_atomic)):
             if name in modes:
                 _, bwd_ms[name] = time_steps(fn, max(args.steps, 10), args.warmup)
+
+        if "deterministic" in modes:
+            # with the lists sorted beforehand, as in the step above (the sort runs beside the forward)
+            sbytes = lib.nnueft_det_sort_bytes(B, K_, R_ROWS, oc, 2)
+            lists = torch.empty(sbytes, dtype=torch.uint8, device=dev)
+
+            def sort_only():
+                rc = lib.nnueft_det_sort(t["white"].data_ptr(), t["black"].data_ptr(), B, K_, R_ROWS, oc, 2,
+                                         lists.data_ptr(), sbytes, stream)
+                assert rc == 0
+
+            def bwd_presorted():
+                rc = lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT,
+                                               ws.data_ptr(), nbytes, lists.data_ptr(), stream, None)
+                assert rc == 0
+
+            _, bwd_ms["sort"] = time_steps(sort_only, max(args.steps, 10), args.warmup)
+            _, bwd_ms["deterministic_presorted"] = time_steps(bwd_presorted, max(args.steps, 10), args.warmup)
 
     fwd_bytes, _ = algorithmic_bytes(L1, B, sum_a, "atomic")
     fwd_gbs = fwd_bytes / (fwd_ms * 1e-3) / 1e9
@@ -392,6 +423,7 @@ def main():
             "workload": args.workload, "L1": L1, "batch": B, "table_rows": R_ROWS, "psqt_columns": N_PSQT,
             "slots": K_SLOTS, "active_rows_per_position": sum_a / B, "backward": head_mode,
             "index_scheme": "HalfKAv2_hm, seeded random positions", "positions": args.positions,
+            "sort_placement": args.sort_placement,
         },
         "roofline": {
             "kernel": "nnueft_double_fwd: k_acc_blocked (the gather, ~3/4 of the time) + k_mix + pair sort",
@@ -413,6 +445,9 @@ def main():
             "backward_entry_ms": bwd_ms.get(mode),
             "backward_algorithmic_GBs": bb / (bwd_ms[mode] * 1e-3) / 1e9 if mode in bwd_ms else None,
         }
+        if mode == "deterministic" and "sort" in bwd_ms:
+            step_stats[mode]["sort_entry_ms"] = bwd_ms["sort"]
+            step_stats[mode]["backward_presorted_entry_ms"] = bwd_ms["deterministic_presorted"]
     out["step"] = step_stats
     if not args.only and args.positions == "uniform":
         # the same step on game-like index lists (not the headline: a robustness figure)

@@ -143,13 +143,36 @@ int nnueft_double_bwd_atomic(const float* us, const float* them, const int32_t* 
  * Same gradient in the fixed order stated at the top; gW and gbias are fully written.
  * No counterpart in the reference's GPU code; the order is that of autograd through the
  * reference's CPU composition (double_ft_functions.py:62-80).
+ * sorted_lists: NULL, or the block nnueft_det_sort wrote for these index lists and sizes (typically
+ * while the forward pass ran: the sort reads nothing but the lists); the call then skips its own
+ * sort.  The block stays valid for further calls.
+ * aux_stream: NULL, or a second stream of the same device.
+ *   With sorted_lists NULL: sorting the index lists and computing the upstream rows are independent;
+ *   given a second stream the call runs the sort there, beside the other work on `stream`, and
+ *   joins the two before the reduction (events, no host wait).
+ *   With sorted_lists given: the stream nnueft_det_sort was enqueued on, if the caller has not
+ *   ordered `stream` after that sort itself; the reduction then waits for all work enqueued on
+ *   aux_stream so far, the upstream rows do not.
+ *   Either way, on return all later work enqueued on `stream` is ordered after the whole call, and
+ *   nothing is left pending on aux_stream that the caller has to wait for.
  */
 int nnueft_double_bwd_det(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                           const int64_t* psqt_idx, const float* bias, float max_act,
                           const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt,
                           const float* saved, float* gW, float* gbias,
                           int B, int K, int R, int L1, int n_psqt,
-                          void* workspace, size_t workspace_bytes, void* stream);
+                          void* workspace, size_t workspace_bytes, void* sorted_lists, void* stream,
+                          void* aux_stream);
+
+/*
+ * The part of the deterministic backward that depends on the index lists only: the stable sort of
+ * the (table row, position) pairs and the work split of the reduction.  sorted_lists: device
+ * memory of nnueft_det_sort_bytes(...) bytes, 256-byte aligned; pass it to nnueft_double_bwd_det
+ * with the same lists and sizes.  n_persp = 2: both lists; 1: widx only (bidx ignored).
+ */
+size_t nnueft_det_sort_bytes(int B, int K, int R, int out_cols, int n_persp);
+int nnueft_det_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, int out_cols, int n_persp,
+                    void* sorted_lists, size_t sorted_bytes, void* stream);
 
 /*
  * merged[r, c] = q(W[r, c] + V[r % vrows, c]): the table the gather reads, from the real weights

@@ -60,6 +60,7 @@ constexpr int kSchedWords = kSchedRowLo + kXcd + 1;
 
 struct DetLayout {
     size_t G, partial, cnt, wcount, seg_off, long_rows, sched, list, runs, end;
+    size_t sort_begin, sort_end;   // cnt .. list: what the sort writes and the reduction reads (one block)
     int cpp;     // chunks per perspective
     int nchunks; // n_persp * cpp
     int ntiles;  // bias tiles
@@ -80,6 +81,7 @@ bool det_layout(int B, int K, int R, int out_cols, int n_persp, DetLayout* L) {
     off += up256(n_persp == 2 ? (size_t)2 * B * out_cols * sizeof(float) : 0);
     L->partial = off;
     off += up256((size_t)L->ntiles * out_cols * sizeof(float));
+    L->sort_begin = off;
     L->cnt = off;
     off += up256((size_t)L->nchunks * R * sizeof(uint32_t));
     L->wcount = off;
@@ -92,6 +94,7 @@ bool det_layout(int B, int K, int R, int out_cols, int n_persp, DetLayout* L) {
     off += up256((size_t)kSchedWords * sizeof(uint32_t));
     L->list = off;
     off += up256((size_t)n_persp * B * K * sizeof(uint32_t));
+    L->sort_end = off;
     static_assert(NNUEFT_ROW_WINDOW_MIN % kChunk == 0, "windows are whole sort chunks");
     const int wpos = nnueft_window_positions(B);
     L->wch = wpos / kChunk;
@@ -193,7 +196,11 @@ __global__ __launch_bounds__(256) void k_tile_colsum(const float* __restrict__ g
 // gbias[c] = chain over the tiles of partial[tile, c].  The adds are one dependent chain; the loads
 // are not, so they are issued a batch ahead.
 __global__ __launch_bounds__(64) void k_bias_final(const float* __restrict__ partial, float* __restrict__ gbias,
-                                                   int ntiles, int out_cols) {
+                                                   int ntiles, int out_cols, uint32_t* __restrict__ sched) {
+    // the last kernel of the backward also rewinds the task counters, so the sorted lists can serve
+    // another reduction (a second backward through the same graph)
+    if (sched && blockIdx.x == 0)
+        for (int i = threadIdx.x; i < kXcd * kSchedQueues; i += 64) sched[kSchedCtr + i * 32] = 0;
     const int c = blockIdx.x * 64 + threadIdx.x;
     if (c >= out_cols) return;
     constexpr int PF = 32;
@@ -666,16 +673,17 @@ bool lds_plan(int R, int K, int* range_out, int* stage_out, size_t* hist_bytes, 
     return true;
 }
 
-// Common tail of the two deterministic entry points.
-int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, float* gW, float* gbias, int B,
-                    int K, int R, int out_cols, int n_persp, char* ws, const DetLayout& L, hipStream_t st) {
+// The sort: everything the reduction needs to know about the index lists (it reads no gradient).
+// `sorted` is the block [L.sort_begin, L.sort_end) of the layout, wherever the caller keeps it.
+int det_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, char* sorted, const DetLayout& L,
+             hipStream_t st) {
+    char* ws = sorted - L.sort_begin;
     uint32_t* cnt = (uint32_t*)(ws + L.cnt);
     uint32_t* wcount = (uint32_t*)(ws + L.wcount);
     uint32_t* seg_off = (uint32_t*)(ws + L.seg_off);
     uint32_t* long_rows = (uint32_t*)(ws + L.long_rows);
     uint32_t* sched = (uint32_t*)(ws + L.sched);
     uint32_t* list = (uint32_t*)(ws + L.list);
-    float* partial = (float*)(ws + L.partial);
 
     int range = 0, stage = 0;
     size_t hist_bytes = 0, fill_bytes = 0;
@@ -707,6 +715,20 @@ int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, fl
     hipLaunchKernelGGL(k_fill, dim3(L.nchunks, nranges), dim3(256), fill_bytes, st, widx, bidx, cnt, seg_off, list,
                        B, K, R, L.cpp, range, stage);
     NNUEFT_LAUNCH_CHECK();
+    return 0;
+}
+
+// The reduction over the sorted lists, and the last step of the bias gradient.
+int det_reduce(const float* G, float* gW, float* gbias, int B, int R, int out_cols, int n_persp, char* ws,
+               char* sorted, const DetLayout& L, hipStream_t st) {
+    char* sw = sorted - L.sort_begin;
+    uint32_t* cnt = (uint32_t*)(sw + L.cnt);
+    uint32_t* wcount = (uint32_t*)(sw + L.wcount);
+    uint32_t* seg_off = (uint32_t*)(sw + L.seg_off);
+    uint32_t* long_rows = (uint32_t*)(sw + L.long_rows);
+    uint32_t* sched = (uint32_t*)(sw + L.sched);
+    uint32_t* list = (uint32_t*)(sw + L.list);
+    float* partial = (float*)(ws + L.partial);
 
     const bool vec = (out_cols % 4 == 0) && aligned16(G) && aligned16(gW);
     const int VWr = vec ? 4 : 1;
@@ -748,7 +770,7 @@ int det_sort_reduce(const int32_t* widx, const int32_t* bidx, const float* G, fl
         NNUEFT_LAUNCH_CHECK();
     }
 
-    return nnueft_det::launch_bias_final(partial, gbias, B, out_cols, st);
+    return nnueft_det::launch_bias_final(partial, gbias, B, out_cols, sched, st);
 }
 
 }  // namespace
@@ -777,9 +799,10 @@ int launch_bwd_rows(const float* us, const float* them, const int64_t* psqt_idx,
     return 0;
 }
 
-int launch_bias_final(const float* partial, float* gbias, int B, int out_cols, hipStream_t st) {
+int launch_bias_final(const float* partial, float* gbias, int B, int out_cols, uint32_t* sched, hipStream_t st) {
     const int ntiles = (B + NNUEFT_BIAS_TILE - 1) / NNUEFT_BIAS_TILE;
-    hipLaunchKernelGGL(k_bias_final, dim3((out_cols + 63) / 64), dim3(64), 0, st, partial, gbias, ntiles, out_cols);
+    hipLaunchKernelGGL(k_bias_final, dim3((out_cols + 63) / 64), dim3(64), 0, st, partial, gbias, ntiles, out_cols,
+                       sched);
     NNUEFT_LAUNCH_CHECK();
     return 0;
 }
@@ -790,6 +813,23 @@ extern "C" size_t nnueft_det_workspace_bytes(int B, int K, int R, int out_cols, 
     DetLayout L;
     if (!det_layout(B, K, R, out_cols, n_persp, &L)) return 0;
     return L.end;
+}
+
+extern "C" size_t nnueft_det_sort_bytes(int B, int K, int R, int out_cols, int n_persp) {
+    DetLayout L;
+    if (!det_layout(B, K, R, out_cols, n_persp, &L)) return 0;
+    return L.sort_end - L.sort_begin;
+}
+
+extern "C" int nnueft_det_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, int out_cols,
+                               int n_persp, void* sorted_lists, size_t sorted_bytes, void* stream) {
+    if (!widx || (n_persp == 2 && !bidx)) return NNUEFT_E_ARG;
+    if ((long long)B * K > 0x3fffffffLL || (long long)B > 0x3fffffffLL) return NNUEFT_E_UNSUPPORTED;
+    DetLayout L;
+    if (!det_layout(B, K, R, out_cols, n_persp, &L)) return NNUEFT_E_ARG;
+    if (!sorted_lists || !aligned256(sorted_lists) || sorted_bytes < L.sort_end - L.sort_begin)
+        return NNUEFT_E_WORKSPACE;
+    return det_sort(widx, n_persp == 2 ? bidx : widx, B, K, R, (char*)sorted_lists, L, (hipStream_t)stream);
 }
 
 extern "C" int nnueft_sparse_bwd_det(const int32_t* idx, const float* gout, float* gW, float* gbias, int B, int K,
@@ -805,7 +845,9 @@ extern "C" int nnueft_sparse_bwd_det(const int32_t* idx, const float* gout, floa
     hipLaunchKernelGGL(k_tile_colsum, dim3(L.ntiles, (out_cols + 255) / 256), dim3(256), 0, st, gout,
                        (float*)(ws + L.partial), B, out_cols);
     NNUEFT_LAUNCH_CHECK();
-    return det_sort_reduce(idx, idx, gout, gW, gbias, B, K, R, out_cols, 1, ws, L, st);
+    const int rc = det_sort(idx, idx, B, K, R, ws + L.sort_begin, L, st);
+    if (rc) return rc;
+    return det_reduce(gout, gW, gbias, B, R, out_cols, 1, ws, ws + L.sort_begin, L, st);
 }
 
 extern "C" int nnueft_double_bwd_det(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
@@ -813,7 +855,8 @@ extern "C" int nnueft_double_bwd_det(const float* us, const float* them, const i
                                      const float* grad_l0,
                                      const float* grad_wpsqt, const float* grad_bpsqt, const float* saved,
                                      float* gW, float* gbias, int B, int K, int R, int L1, int n_psqt,
-                                     void* workspace, size_t workspace_bytes, void* stream) {
+                                     void* workspace, size_t workspace_bytes, void* sorted_lists, void* stream,
+                                     void* aux_stream) {
     if (B <= 0 || K <= 0 || R <= 0 || L1 <= 0 || (L1 & 1) || n_psqt < 0) return NNUEFT_E_ARG;
     if (!us || !them || !widx || !bidx || !psqt_idx || !bias || !grad_l0 || !grad_wpsqt || !grad_bpsqt || !saved ||
         !gW || !gbias)
@@ -826,8 +869,55 @@ extern "C" int nnueft_double_bwd_det(const float* us, const float* them, const i
     hipStream_t st = (hipStream_t)stream;
     char* ws = (char*)workspace;
     float* G = (float*)(ws + L.G);
-    const int rc = nnueft_det::launch_bwd_rows(us, them, psqt_idx, bias, max_act, grad_l0, grad_wpsqt, grad_bpsqt,
-                                               saved, G, (float*)(ws + L.partial), B, L1, n_psqt, st);
+    // The sort reads only the index lists, the upstream rows only the activations: with a second
+    // stream they run side by side and meet before the reduction.
+    hipStream_t aux = (hipStream_t)aux_stream;
+    if (sorted_lists) {
+        // the caller ran nnueft_det_sort on these lists already; if on aux_stream, it may still be
+        // running there: only the reduction has to wait for it, the upstream rows do not
+        if (!aligned256(sorted_lists)) return NNUEFT_E_WORKSPACE;
+        int rc = nnueft_det::launch_bwd_rows(us, them, psqt_idx, bias, max_act, grad_l0, grad_wpsqt, grad_bpsqt,
+                                             saved, G, (float*)(ws + L.partial), B, L1, n_psqt, st);
+        if (rc) return rc;
+        if (aux && aux != st) {
+            hipEvent_t sorted = nullptr;
+            hipError_t e = hipEventCreateWithFlags(&sorted, hipEventDisableTiming);
+            if (e == hipSuccess) e = hipEventRecord(sorted, aux);
+            if (e == hipSuccess) e = hipStreamWaitEvent(st, sorted, 0);
+            if (sorted) (void)hipEventDestroy(sorted);
+            if (e != hipSuccess) return (int)e;
+        }
+        return det_reduce(G, gW, gbias, B, R, out_cols, 2, ws, (char*)sorted_lists, L, st);
+    }
+    hipEvent_t forked = nullptr, sorted = nullptr;
+    if (aux && aux != st) {
+        hipError_t e = hipEventCreateWithFlags(&forked, hipEventDisableTiming);
+        if (e == hipSuccess) e = hipEventCreateWithFlags(&sorted, hipEventDisableTiming);
+        if (e == hipSuccess) e = hipEventRecord(forked, st);
+        if (e == hipSuccess) e = hipStreamWaitEvent(aux, forked, 0);
+        if (e != hipSuccess) {
+            if (forked) (void)hipEventDestroy(forked);
+            if (sorted) (void)hipEventDestroy(sorted);
+            return (int)e;
+        }
+    } else {
+        aux = st;
+    }
+    int rc = det_sort(widx, bidx, B, K, R, ws + L.sort_begin, L, aux);
+    if (rc == 0 && aux != st) {
+        hipError_t e = hipEventRecord(sorted, aux);
+        if (e != hipSuccess) rc = (int)e;
+    }
+    if (rc == 0)
+        rc = nnueft_det::launch_bwd_rows(us, them, psqt_idx, bias, max_act, grad_l0, grad_wpsqt, grad_bpsqt, saved, G,
+                                         (float*)(ws + L.partial), B, L1, n_psqt, st);
+    if (aux != st) {
+        // always rejoin, also after a failed launch: the caller's stream must not run ahead of the other one
+        const hipError_t e = hipStreamWaitEvent(st, sorted, 0);
+        if (rc == 0 && e != hipSuccess) rc = (int)e;
+        (void)hipEventDestroy(forked);
+        (void)hipEventDestroy(sorted);
+    }
     if (rc) return rc;
-    return det_sort_reduce(widx, bidx, G, gW, gbias, B, K, R, out_cols, 2, ws, L, st);
+    return det_reduce(G, gW, gbias, B, R, out_cols, 2, ws, ws + L.sort_begin, L, st);
 }

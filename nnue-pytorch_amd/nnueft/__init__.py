@@ -5,7 +5,8 @@ The public names are those of the reference's model/modules/feature_transformer/
 """
 from .double_ft_functions import double_feature_transform
 from .fused_ft_functions import FusedDoubleFtFunction
-from .sparse_linear_functions import SparseLinearFunction, get_backward_mode, set_backward_mode
+from .sparse_linear_functions import (SparseLinearFunction, get_backward_mode, get_sort_placement,
+                                      set_backward_mode, set_sort_placement)
 
 __all__ = [
     "FusedDoubleFtFunction",
@@ -13,4 +14,6 @@ __all__ = [
     "double_feature_transform",
     "get_backward_mode",
     "set_backward_mode",
+    "get_sort_placement",
+    "set_sort_placement",
 ]

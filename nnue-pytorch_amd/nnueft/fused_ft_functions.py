@@ -17,7 +17,7 @@ from torch import autograd
 
 from . import _native
 from . import sparse_linear_functions as _slf
-from .sparse_linear_functions import _stream_ptr, _workspace
+from .sparse_linear_functions import _aux_stream, _aux_stream_ptr, _stream_ptr, _workspace
 
 _HAS_CUPY_KERNELS = _native.available()
 
@@ -44,8 +44,29 @@ def _launch_double_fwd(us, them, white_indices, black_indices, psqt_indices, wei
 
 
 @torch.compiler.disable(recursive=False)
+def _launch_det_sort(white_indices, black_indices, num_rows, output_size):
+    """The sort of the deterministic backward reads nothing but the index lists, so it starts here, in
+    the forward pass, on a second stream, and is long done when the backward pass wants it.
+    Returns the sorted lists, an opaque byte tensor that is complete once the second stream has run."""
+    lib = _native.load()
+    B, K = white_indices.shape
+    device = white_indices.device
+    nbytes = lib.nnueft_det_sort_bytes(B, K, num_rows, output_size, 2)
+    buf = _workspace(nbytes, device)
+    cur, aux = torch.cuda.current_stream(device), _aux_stream(device)
+    aux.wait_stream(cur)                     # the lists and buf are ordered on the caller's stream
+    rc = lib.nnueft_det_sort(white_indices.data_ptr(), black_indices.data_ptr(), B, K, num_rows, output_size, 2,
+                             buf.data_ptr(), nbytes, aux.cuda_stream)
+    _native.check(rc, "nnueft_det_sort")
+    for t in (buf, white_indices, black_indices):
+        t.record_stream(aux)                 # their memory is not handed out again before the sort has run
+    return buf
+
+
+@torch.compiler.disable(recursive=False)
 def _launch_double_bwd(us, them, white_indices, black_indices, psqt_indices, bias, max_ft_activation, grad_l0,
-                       grad_wpsqt, grad_bpsqt, saved, num_rows, l1_size, output_size, mode):
+                       grad_wpsqt, grad_bpsqt, saved, num_rows, l1_size, output_size, mode, presorted=None,
+                       second_stream=False):
     lib = _native.load()
     B, K = white_indices.shape
     device = us.device
@@ -62,9 +83,13 @@ def _launch_double_bwd(us, them, white_indices, black_indices, psqt_indices, bia
             return grad_weight.zero_(), grad_bias.zero_()
         nbytes = lib.nnueft_det_workspace_bytes(B, K, num_rows, output_size, 2)
         ws = _workspace(nbytes, device)
+        # presorted: the lists sorted during the forward pass on the second stream; the entry point makes
+        # its reduction (not its first kernel) wait for that stream
+        sorted_ptr = presorted.data_ptr() if presorted is not None else None
         rc = lib.nnueft_double_bwd_det(
             *head, grad_weight.data_ptr(), grad_bias.data_ptr(), B, K, num_rows, l1_size, n_psqt,
-            ws.data_ptr(), nbytes, _stream_ptr(device),
+            ws.data_ptr(), nbytes, sorted_ptr, _stream_ptr(device),
+            _aux_stream_ptr(device) if second_stream else None,
         )
         _native.check(rc, "nnueft_double_bwd_det")
     else:
@@ -84,6 +109,7 @@ class FusedDoubleFtFunction(autograd.Function):
         ctx.max_ft_activation = float(max_ft_activation)
         ctx.l1_size = int(l1_size)
         ctx.backward_mode = _slf.get_backward_mode()
+        ctx.sort_placement = _slf.get_sort_placement()
 
         assert l1_size % 2 == 0
 
@@ -123,6 +149,12 @@ class FusedDoubleFtFunction(autograd.Function):
         row_sums = torch.empty(2, batch_size, l1_size, dtype=torch.float32, device=device)
 
         with torch.cuda.device(device):
+            # first, so that it runs beside the forward kernel
+            ctx.presorted = None
+            if (ctx.sort_placement == "forward" and ctx.backward_mode == "deterministic" and batch_size > 0
+                    and (ctx.needs_input_grad[5] or ctx.needs_input_grad[6])):
+                ctx.presorted = _launch_det_sort(white_indices, black_indices, weight.shape[0], weight.shape[1])
+
             _launch_double_fwd(
                 us, them, white_indices, black_indices, psqt_indices, weight, bias,
                 max_ft_activation, int(l1_size), l0_, wpsqt, bpsqt, row_sums,
@@ -143,7 +175,8 @@ class FusedDoubleFtFunction(autograd.Function):
             grad_weight, grad_bias = _launch_double_bwd(
                 us, them, white_indices, black_indices, psqt_indices, bias, ctx.max_ft_activation,
                 grad_l0, grad_wpsqt, grad_bpsqt, row_sums,
-                weight.shape[0], ctx.l1_size, bias.shape[0], ctx.backward_mode,
+                weight.shape[0], ctx.l1_size, bias.shape[0], ctx.backward_mode, ctx.presorted,
+                ctx.sort_placement != "inline",
             )
 
         return None, None, None, None, None, grad_weight, grad_bias, None, None

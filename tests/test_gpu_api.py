@@ -19,9 +19,10 @@ DEV = "cuda:0"
 
 @pytest.fixture(autouse=True)
 def _restore_mode():
-    old = nnueft.get_backward_mode()
+    old, old_sort = nnueft.get_backward_mode(), nnueft.get_sort_placement()
     yield
     nnueft.set_backward_mode(old)
+    nnueft.set_sort_placement(old_sort)
 
 
 def _emulate(indices, weight, bias):
@@ -257,6 +258,46 @@ def test_non_default_stream(oracle_cpu):
     rW, rb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["bias"], c["max_act"],
                                    c["g_l0"], c["g_wp"], c["g_bp"], r[3], 500, 8)
     assert np.array_equal(W.grad.cpu().numpy(), rW) and np.array_equal(bias.grad.cpu().numpy(), rb)
+
+
+@pytest.mark.parametrize("on_stream", [False, True], ids=["default_stream", "side_stream"])
+def test_sort_placements_give_the_same_bits(oracle_cpu, on_stream):
+    """The index sort inline, on a second stream in the backward pass, or started by the forward
+    pass: same outputs and gradients, bit for bit, also when the graph is walked twice."""
+    nnueft.set_backward_mode("deterministic")
+    B, L1 = 5000, 512
+    c = double_case(77, B, L1, hk.NUM_INPUTS, 32, halfka=True, max_act=255 / 256, weight_scale=0.05)
+    us, them, widx, bidx, pc = hk.synthetic_batch(B, 77, game_like=True)     # has rows that are split
+    c.update(us=us, them=them, widx=widx, bidx=bidx, psqt_idx=((pc - 1) // 4).astype(np.int64))
+    t = {k: torch.from_numpy(c[k]).to(DEV) for k in ("us", "them", "widx", "bidx", "psqt_idx", "W", "bias")}
+    grads = [torch.from_numpy(c[k]).to(DEV) for k in ("g_l0", "g_wp", "g_bp")]
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream() if on_stream else torch.cuda.current_stream()
+    got = {}
+    for where in ("inline", "backward", "forward"):
+        nnueft.set_sort_placement(where)
+        with torch.cuda.stream(stream):
+            W = t["W"].clone().requires_grad_()
+            bias = t["bias"].clone().requires_grad_()
+            out = double_feature_transform(t["us"], t["them"], t["widx"], t["bidx"], t["psqt_idx"], W, bias,
+                                           c["max_act"], L1, "fused")
+            torch.autograd.backward(list(out), grads, retain_graph=True)
+            first = (W.grad.clone(), bias.grad.clone())
+            W.grad = bias.grad = None
+            torch.autograd.backward(list(out), grads)
+        stream.synchronize()
+        assert torch.equal(first[0], W.grad) and torch.equal(first[1], bias.grad)
+        got[where] = (out[0].detach(), W.grad, bias.grad)
+    for where in ("backward", "forward"):
+        for a, b in zip(got[where], got["inline"]):
+            assert torch.equal(a, b)
+    r = oracle_cpu.double_fwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["W"], c["bias"],
+                              c["max_act"], L1)
+    rW, rb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["bias"], c["max_act"],
+                                   c["g_l0"], c["g_wp"], c["g_bp"], r[3], hk.NUM_INPUTS, 8)
+    assert np.array_equal(got["inline"][1].cpu().numpy(), rW) and np.array_equal(got["inline"][2].cpu().numpy(), rb)
+    with pytest.raises(ValueError):
+        nnueft.set_sort_placement("elsewhere")
 
 
 def test_abi_rejects_bad_arguments():

@@ -164,7 +164,28 @@ def test_double_backward(oracle_cpu, B, L1, R, K, kw, mode):
         gW = torch.full((R, out_cols), float("nan"), device=_dev())
         gb = torch.full((out_cols,), float("nan"), device=_dev())
         nat.check(lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt, ws.data_ptr(),
-                                            nbytes, _stream()), "double_bwd_det")
+                                            nbytes, None, _stream(), None), "double_bwd_det")
+        # the same with the sort on a second stream
+        gW2 = torch.full((R, out_cols), float("nan"), device=_dev())
+        gb2 = torch.full((out_cols,), float("nan"), device=_dev())
+        aux = torch.cuda.Stream()
+        nat.check(lib.nnueft_double_bwd_det(*head, gW2.data_ptr(), gb2.data_ptr(), B, K, R, L1, n_psqt, ws.data_ptr(),
+                                            nbytes, None, _stream(), aux.cuda_stream), "double_bwd_det")
+        assert torch.equal(gW, gW2) and torch.equal(gb, gb2)
+        # the same with lists sorted beforehand, used twice
+        sbytes = lib.nnueft_det_sort_bytes(B, K, R, out_cols, 2)
+        assert 0 < sbytes < nbytes
+        lists = torch.full((sbytes,), 0x5A, dtype=torch.uint8, device=_dev())
+        nat.check(lib.nnueft_det_sort(d["widx"].data_ptr(), d["bidx"].data_ptr(), B, K, R, out_cols, 2,
+                                      lists.data_ptr(), sbytes, _stream()), "det_sort")
+        for _ in range(2):
+            gW2.fill_(float("nan"))
+            gb2.fill_(float("nan"))
+            ws.fill_(0xC3)
+            nat.check(lib.nnueft_double_bwd_det(*head, gW2.data_ptr(), gb2.data_ptr(), B, K, R, L1, n_psqt,
+                                                ws.data_ptr(), nbytes, lists.data_ptr(), _stream(), None),
+                      "double_bwd_det")
+            assert torch.equal(gW, gW2) and torch.equal(gb, gb2)
     rW, rb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["bias"], c["max_act"],
                                    c["g_l0"], c["g_wp"], c["g_bp"], saved.cpu().numpy(), R, n_psqt)
     gW, gb = gW.cpu().numpy(), gb.cpu().numpy()
@@ -213,11 +234,27 @@ def test_double_backward_deterministic_with_split_rows(oracle_cpu, B, L1, castle
                                         d["bidx"].data_ptr(), d["psqt_idx"].data_ptr(), d["bias"].data_ptr(),
                                         c["max_act"], g_l0.data_ptr(), g_wp.data_ptr(), g_bp.data_ptr(),
                                         saved.data_ptr(), gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt,
-                                        ws.data_ptr(), nbytes, _stream()), "double_bwd_det")
+                                        ws.data_ptr(), nbytes, None, _stream(), torch.cuda.Stream().cuda_stream),
+              "double_bwd_det")
     rW, rb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["bias"], c["max_act"],
                                    c["g_l0"], c["g_wp"], c["g_bp"], saved.cpu().numpy(), R, n_psqt)
     assert np.array_equal(gW.cpu().numpy(), rW)
     assert np.array_equal(gb.cpu().numpy(), rb)
+    # lists sorted beforehand: same bits, also on the second use of the sorted block
+    sbytes = lib.nnueft_det_sort_bytes(B, K, R, out_cols, 2)
+    lists = torch.empty(sbytes, dtype=torch.uint8, device=_dev())
+    nat.check(lib.nnueft_det_sort(d["widx"].data_ptr(), d["bidx"].data_ptr(), B, K, R, out_cols, 2,
+                                  lists.data_ptr(), sbytes, _stream()), "det_sort")
+    for _ in range(2):
+        gW2 = torch.full((R, out_cols), float("nan"), device=_dev())
+        gb2 = torch.full((out_cols,), float("nan"), device=_dev())
+        nat.check(lib.nnueft_double_bwd_det(d["us"].data_ptr(), d["them"].data_ptr(), d["widx"].data_ptr(),
+                                            d["bidx"].data_ptr(), d["psqt_idx"].data_ptr(), d["bias"].data_ptr(),
+                                            c["max_act"], g_l0.data_ptr(), g_wp.data_ptr(), g_bp.data_ptr(),
+                                            saved.data_ptr(), gW2.data_ptr(), gb2.data_ptr(), B, K, R, L1, n_psqt,
+                                            ws.data_ptr(), nbytes, lists.data_ptr(), _stream(), None),
+                  "double_bwd_det")
+        assert torch.equal(gW, gW2) and torch.equal(gb, gb2)
 
 
 # (the last two tables are taller than the row scan stages at once: several passes, totals summed first)
@@ -259,7 +296,7 @@ def test_deterministic_backward_repeats_bitwise():
                                             c["max_act"],
                                             g_l0.data_ptr(), g_wp.data_ptr(), g_bp.data_ptr(), saved.data_ptr(),
                                             gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt, ws.data_ptr(), nbytes,
-                                            _stream()), "double_bwd_det")
+                                            None, _stream(), None), "double_bwd_det")
         outs.append((gW.cpu().numpy().copy(), gb.cpu().numpy().copy()))
     assert np.array_equal(outs[0][0], outs[1][0])
     assert np.array_equal(outs[0][1], outs[1][1])
