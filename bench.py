@@ -237,6 +237,83 @@ def run_full_step(args, dev):
     }))
 
 
+def run_handoff(args, dev):
+    """The step before the path: batches in host memory laid out as the loader leaves them, staged and
+    copied to the GPU by nnueft.batch_handoff, feeding the same forward+backward step.  Reports the cost
+    of the hand-off alone and the step rate with every batch crossing PCIe (the headline rate has its
+    inputs resident)."""
+    import numpy as np
+    import torch
+    import nnueft
+    from nnueft import halfka_v2_hm as hk
+    from nnueft.batch_handoff import DevicePrefetcher, SparseBatch
+    from nnueft.double_ft_functions import double_feature_transform
+
+    L1, B = WORKLOADS[args.workload]
+    nnueft.set_backward_mode(args.backward)
+    rng = np.random.default_rng(5)
+    batches = []
+    for i in range(4):
+        us, them, white, black, pc = hk.synthetic_batch(B, 4000 + i)
+        batches.append(SparseBatch.from_arrays(hk.NUM_INPUTS, us.reshape(B), rng.random(B, dtype=np.float32),
+                                               rng.normal(0, 300, B).astype(np.float32), white, black, pc))
+    words = 3 * B + 2 * B * K_SLOTS + B
+    g = torch.Generator().manual_seed(0)
+    W = (torch.randn(R_ROWS, L1 + N_PSQT, generator=g) * 0.05).to(dev).requires_grad_()
+    bias = torch.randn(L1 + N_PSQT, generator=g).to(dev).requires_grad_()
+    g_l0 = torch.randn(B, L1, generator=g).to(dev)
+    g_p = torch.randn(B, 1, generator=g).to(dev)
+
+    # the hand-off alone, synchronous: host staging + DMA + unpack kernel
+    for _ in range(args.warmup):
+        batches[0].get_tensors(dev)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        batches[i % 4].get_tensors(dev)
+    host_ms = (time.perf_counter() - t0) / args.steps * 1e3
+    torch.cuda.synchronize()
+    sync_ms = (time.perf_counter() - t0) / args.steps * 1e3
+
+    def step(t):
+        us, them, white, black, outcome, score, piece_count = t
+        W.grad = None
+        bias.grad = None
+        out = double_feature_transform(us, them, white, black, (piece_count - 1) // 4, W, bias, 255.0 / 256.0, L1,
+                                       "fused")
+        torch.autograd.backward(list(out), [g_l0, g_p, g_p])
+
+    def rate(source, n):
+        it = iter(source)
+        for _ in range(args.warmup):
+            step(next(it))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            step(next(it))
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n * 1e3
+
+    total = args.steps + args.warmup
+    resident = batches[0].get_tensors(dev)
+    ms_res = rate((resident for _ in range(total)), args.steps)
+    pf = DevicePrefetcher((batches[i % 4] for i in range(total)), dev, depth=4)
+    ms_pf = rate(pf, args.steps)
+    pf.close()
+    ms_inline = rate((batches[i % 4].get_tensors(dev) for i in range(total)), args.steps)
+    print(json.dumps({
+        "metric": "FT fwd+bwd positions/sec with every batch handed over from host memory",
+        "config": {"workload": args.workload, "L1": L1, "batch": B, "backward": args.backward,
+                   "bytes_per_batch": words * 4},
+        "handoff_alone": {"host_ms_per_batch": host_ms, "ms_per_batch_incl_copy": sync_ms,
+                          "GBs": words * 4 / (sync_ms * 1e-3) / 1e9},
+        "step_ms": {"inputs_resident": ms_res, "prefetcher": ms_pf, "handoff_on_the_training_stream": ms_inline},
+        "positions_per_s": {"inputs_resident": B / (ms_res * 1e-3), "prefetcher": B / (ms_pf * 1e-3),
+                            "handoff_on_the_training_stream": B / (ms_inline * 1e-3)},
+        "steps": args.steps, "warmup": args.warmup, "n_gpus": 1, "data": "synthetic",
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -258,7 +335,7 @@ def main():
                     help="uniform: kings and pieces uniform over the board (the headline workload); game: piece "
                          "placement statistics of real game positions, where one or two king buckets hold a large "
                          "part of the batch (halfka_v2_hm.game_like_positions); a default run times both")
-    ap.add_argument("--only", default="", choices=["", "fwd", "det", "atomic", "copy"],
+    ap.add_argument("--only", default="", choices=["", "fwd", "det", "atomic", "copy", "handoff"],
                     help="run only this part (for profiling runs); 'copy' launches a plain elementwise kernel "
                          "reading and writing 1 GiB each, the yardstick the FETCH_SIZE/WRITE_SIZE counters are scaled by")
     args = ap.parse_args()
@@ -292,6 +369,9 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"calibration": "torch.add(src, 1.0, out=dst)", "read_bytes": n * 4, "write_bytes": n * 4,
                           "launches": args.warmup + args.steps}))
+        return
+    if args.only == "handoff":
+        run_handoff(args, dev)
         return
     L1, B = WORKLOADS[args.workload]
     seed = 1234 + 3

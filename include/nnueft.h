@@ -316,6 +316,14 @@ int nnueft_ranger_lite_update_variance(const float* grad, float* variance_ma, lo
 int nnueft_ranger_lite_lookahead_merge(float* p, float* lookahead_params, long long n, float alpha,
                                        void* stream);
 
+/*
+ * Loader hand-off: from the words of a batch already on the device, them[i] = 1 - us[i] and
+ * piece_count[i] = (int64) piece_count32[i], i < B, in one launch.  Replaces the `1.0 - us` and
+ * `.to(dtype=torch.int64)` ops at the end of SparseBatch.get_tensors (data_loader/_native.py:76-86).
+ */
+int nnueft_batch_unpack(const float* us, const int32_t* piece_count32, float* them, int64_t* piece_count,
+                        int B, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

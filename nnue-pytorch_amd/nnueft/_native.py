@@ -45,6 +45,7 @@ PROTOTYPES = {
     "nnueft_bucket_linear_fwd": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_void_p, c_size_t, c_int, c_void_p]),
     "nnueft_bucket_linear_bwd": (c_int, [c_void_p] * 7 + [c_int] * 4 + [c_void_p, c_size_t, c_int, c_void_p]),
     "nnueft_act_fake_quantize": (c_int, [c_void_p] * 2 + [c_longlong] + [c_float] * 3 + [c_void_p]),
+    "nnueft_batch_unpack": (c_int, [c_void_p] * 4 + [c_int, c_void_p]),
     "nnueft_ranger_lite_update_pnm": (
         c_int,
         [c_void_p] * 5 + [c_longlong] + [c_float] * 10 + [c_longlong, c_float, c_int, c_void_p, c_float, c_void_p],
