@@ -317,6 +317,48 @@ int nnueft_ranger_lite_lookahead_merge(float* p, float* lookahead_params, long l
                                        void* stream);
 
 /*
+ * The per-position chains after the bucketed layers, one launch each instead of a dozen or more
+ * elementwise torch ops (every operation still rounds on its own, in the order of those ops).
+ *
+ * nnueft_sqr_crelu_*: y f32[B, 2n] = clamp(cat[fq(x * x) * sqr_factor, fq(x)], 0, max_act) for x f32[B, n],
+ * fq(v) = floor(v * scale + eps) / scale when fake_quantize, else v; skip (NULL or f32[B]) receives
+ * x[:, n-2] - x[:, n-1].  LayerStacks.forward's two `_sqr_crelu`-style blocks and the skip connection
+ * (model/modules/layer_stacks.py:39-70).  Backward: fq is straight-through, the clamp passes the
+ * gradient where 0 <= value <= max_act; gskip (NULL or f32[B]) is added to / subtracted from the
+ * last two columns of gx.
+ */
+int nnueft_sqr_crelu_fwd(const float* x, float* y, float* skip, int B, int n, float scale, float eps,
+                         float sqr_factor, float max_act, int fake_quantize, void* stream);
+int nnueft_sqr_crelu_bwd(const float* x, const float* gy, const float* gskip, float* gx, int B, int n, float scale,
+                         float eps, float sqr_factor, float max_act, int fake_quantize, void* stream);
+
+/*
+ * net[i] = fq_out(lin[i] + skip[i]) + (wpsqt[i] - bpsqt[i]) * (us[i] - 0.5), all f32[B];
+ * fq_out(v) = trunc(round(v * den) * mult / den) / mult in 64-bit integers when fake_quantize
+ * (fake_quantize_output of model/quantize.py; model/modules/layer_stacks.py:76-80, model/model.py:131).  Backward: lin and skip
+ * receive gnet itself; gwpsqt = gnet * (us - 0.5), gbpsqt = -gwpsqt.
+ */
+int nnueft_stack_output_fwd(const float* lin, const float* skip, const float* wpsqt, const float* bpsqt,
+                            const float* us, float* net, int B, long long den, long long mult, int fake_quantize,
+                            void* stream);
+int nnueft_stack_output_bwd(const float* gnet, const float* us, float* gwpsqt, float* gbpsqt, int B, void* stream);
+
+/*
+ * The training loss of model/nnue.py:39-70 (win-rate model, tablebase score remap, lambda blend,
+ * |pt - qf|^pow_exp with optional asymmetry, position weights) for scorenet/score/outcome f32[B].
+ * terms f32[3, B] receives loss_i * w_i, w_i and w_i * dloss_i/dscorenet_i; sums f32[2] the sums of the
+ * first two rows (each thread of one 1024-thread workgroup chains every 1024th element, then a fixed
+ * pairwise tree: the same bits on every run); loss[0] = sums[0] / sums[1].
+ * Backward: grad_scorenet[i] = terms[2, i] * (grad_loss[0] / sums[1]); grad_loss is a device scalar.
+ */
+int nnueft_sf_loss_fwd(const float* scorenet, const float* score, const float* outcome, float* terms, float* sums,
+                       float* loss, int B, float in_offset, float in_scaling, float out_offset, float out_scaling,
+                       float pow_exp, float qp_asymmetry, float w1, float w2, float tb_remap_base,
+                       float tb_remap_scale, float tb_remap_decay, double lambda, void* stream);
+int nnueft_sf_loss_bwd(const float* terms, const float* sums, const float* grad_loss, float* grad_scorenet, int B,
+                       void* stream);
+
+/*
  * Loader hand-off: from the words of a batch already on the device, them[i] = 1 - us[i] and
  * piece_count[i] = (int64) piece_count32[i], i < B, in one launch.  Replaces the `1.0 - us` and
  * `.to(dtype=torch.int64)` ops at the end of SparseBatch.get_tensors (data_loader/_native.py:76-86).

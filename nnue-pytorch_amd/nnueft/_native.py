@@ -6,7 +6,7 @@ to another implementation: if the shared object is missing or does not export a 
 """
 import ctypes
 import os
-from ctypes import c_float, c_int, c_longlong, c_size_t, c_void_p
+from ctypes import c_double, c_float, c_int, c_longlong, c_size_t, c_void_p
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
 # NNUEFT_LIBRARY points at another build of the same library (kernel tuning)
@@ -45,6 +45,12 @@ PROTOTYPES = {
     "nnueft_bucket_linear_fwd": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_void_p, c_size_t, c_int, c_void_p]),
     "nnueft_bucket_linear_bwd": (c_int, [c_void_p] * 7 + [c_int] * 4 + [c_void_p, c_size_t, c_int, c_void_p]),
     "nnueft_act_fake_quantize": (c_int, [c_void_p] * 2 + [c_longlong] + [c_float] * 3 + [c_void_p]),
+    "nnueft_sqr_crelu_fwd": (c_int, [c_void_p] * 3 + [c_int] * 2 + [c_float] * 4 + [c_int, c_void_p]),
+    "nnueft_sqr_crelu_bwd": (c_int, [c_void_p] * 4 + [c_int] * 2 + [c_float] * 4 + [c_int, c_void_p]),
+    "nnueft_stack_output_fwd": (c_int, [c_void_p] * 6 + [c_int, c_longlong, c_longlong, c_int, c_void_p]),
+    "nnueft_stack_output_bwd": (c_int, [c_void_p] * 4 + [c_int, c_void_p]),
+    "nnueft_sf_loss_fwd": (c_int, [c_void_p] * 6 + [c_int] + [c_float] * 11 + [c_double, c_void_p]),
+    "nnueft_sf_loss_bwd": (c_int, [c_void_p] * 4 + [c_int, c_void_p]),
     "nnueft_batch_unpack": (c_int, [c_void_p] * 4 + [c_int, c_void_p]),
     "nnueft_ranger_lite_update_pnm": (
         c_int,

@@ -101,9 +101,14 @@ class QuantizationManager:
     def fake_quantize_skip_act(self, x):
         return x
 
-    def fake_quantize_output(self, x):
+    def output_quantization(self):
+        """(den, mult) of fake_quantize_output."""
         mult = int(self.config.nnue2score * self.config.weight_scale_out)
         den = int(self.config.hidden_quantized_one * self.config.weight_scale_l_out * 2.0)
+        return den, mult
+
+    def fake_quantize_output(self, x):
+        den, mult = self.output_quantization()
         q = torch.div(torch.round(x * den).to(torch.int64) * mult, den, rounding_mode="trunc")
         return _ste(q.to(x.dtype) / float(mult), x)
 
@@ -207,8 +212,9 @@ def _launch_table_merge(weight, virtual, l1_size, scale_ft, scale_psqt, quantize
     R, cols = weight.shape
     merged = torch.empty_like(weight)
     with torch.cuda.device(weight.device):
-        rc = lib.nnueft_table_merge(weight.data_ptr(), virtual.data_ptr(), merged.data_ptr(), R, cols, l1_size,
-                                    virtual.shape[0], float(scale_ft), float(scale_psqt), int(bool(quantize)),
+        rc = lib.nnueft_table_merge(weight.data_ptr(), None if virtual is None else virtual.data_ptr(),
+                                    merged.data_ptr(), R, cols, l1_size, 1 if virtual is None else virtual.shape[0],
+                                    float(scale_ft), float(scale_psqt), int(bool(quantize)),
                                     _stream_ptr(weight.device))
     _native.check(rc, "nnueft_table_merge")
     return merged
@@ -232,13 +238,16 @@ class _TableMerge(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, weight, virtual, l1_size, scale_ft, scale_psqt, quantize):
-        ctx.vrows = virtual.shape[0]
+        ctx.vrows = None if virtual is None else virtual.shape[0]
         return _launch_table_merge(weight, virtual, l1_size, scale_ft, scale_psqt, quantize)
 
     @staticmethod
     def backward(ctx, grad):
         grad = grad.contiguous()
-        return grad, _launch_table_virtual_grad(grad, ctx.vrows), None, None, None, None
+        gv = None
+        if ctx.vrows is not None and ctx.needs_input_grad[1]:
+            gv = _launch_table_virtual_grad(grad, ctx.vrows)
+        return grad, gv, None, None, None, None
 
 
 def _table_merge(weight, virtual, l1_size, scale_ft, scale_psqt, quantize):
@@ -268,6 +277,150 @@ class _ActFakeQuantize(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad):
         return (grad if ctx.post_mul == 1.0 else grad * ctx.post_mul), None, None
+
+
+def _fused_tail_applies(x) -> bool:
+    return x.is_cuda and x.dtype == torch.float32
+
+
+@torch.compiler.disable(recursive=False)
+def _launch_sqr_crelu(x, want_skip, scale, c, m, fq):
+    lib = _native.load()
+    B, n = x.shape
+    y = torch.empty(B, 2 * n, dtype=x.dtype, device=x.device)
+    skip = torch.empty(B, 1, dtype=x.dtype, device=x.device) if want_skip else None
+    if B:
+        with torch.cuda.device(x.device):
+            rc = lib.nnueft_sqr_crelu_fwd(x.data_ptr(), y.data_ptr(), skip.data_ptr() if want_skip else None, B, n,
+                                          float(scale), float(FAKE_QUANTIZE_EPS), float(c), float(m), int(fq),
+                                          _stream_ptr(x.device))
+        _native.check(rc, "nnueft_sqr_crelu_fwd")
+    return y, skip
+
+
+@torch.compiler.disable(recursive=False)
+def _launch_sqr_crelu_bwd(x, gy, gskip, scale, c, m, fq):
+    lib = _native.load()
+    B, n = x.shape
+    gx = torch.empty_like(x)
+    if B:
+        with torch.cuda.device(x.device):
+            rc = lib.nnueft_sqr_crelu_bwd(x.data_ptr(), gy.data_ptr(), None if gskip is None else gskip.data_ptr(),
+                                          gx.data_ptr(), B, n, float(scale), float(FAKE_QUANTIZE_EPS), float(c),
+                                          float(m), int(fq), _stream_ptr(x.device))
+        _native.check(rc, "nnueft_sqr_crelu_bwd")
+    return gx
+
+
+class _SqrCrelu(torch.autograd.Function):
+    """clamp(cat[fq(x^2) * c, fq(x)], 0, m) and, on request, the skip value x[:, -2] - x[:, -1], as one
+    kernel; fq is straight-through."""
+
+    @staticmethod
+    def forward(ctx, x, want_skip, scale, c, m, fq):
+        x = x.contiguous()
+        ctx.save_for_backward(x)
+        ctx.args = (float(scale), float(c), float(m), bool(fq))
+        ctx.want_skip = bool(want_skip)
+        return _launch_sqr_crelu(x, want_skip, scale, c, m, fq)
+
+    @staticmethod
+    def backward(ctx, gy, gskip):
+        (x,) = ctx.saved_tensors
+        if gy is None:
+            gy = torch.zeros(x.shape[0], 2 * x.shape[1], dtype=x.dtype, device=x.device)
+        gskip = gskip.contiguous() if (ctx.want_skip and gskip is not None) else None
+        return _launch_sqr_crelu_bwd(x, gy.contiguous(), gskip, *ctx.args), None, None, None, None, None
+
+
+@torch.compiler.disable(recursive=False)
+def _launch_stack_output(lin, skip, wpsqt, bpsqt, us, den, mult, fq):
+    lib = _native.load()
+    B = lin.shape[0]
+    net = torch.empty_like(lin)
+    if B:
+        with torch.cuda.device(lin.device):
+            rc = lib.nnueft_stack_output_fwd(lin.data_ptr(), skip.data_ptr(), wpsqt.data_ptr(), bpsqt.data_ptr(),
+                                             us.data_ptr(), net.data_ptr(), B, int(den), int(mult), int(fq),
+                                             _stream_ptr(lin.device))
+        _native.check(rc, "nnueft_stack_output_fwd")
+    return net
+
+
+@torch.compiler.disable(recursive=False)
+def _launch_stack_output_bwd(g, us):
+    lib = _native.load()
+    gw, gb = torch.empty_like(g), torch.empty_like(g)
+    if g.shape[0]:
+        with torch.cuda.device(g.device):
+            rc = lib.nnueft_stack_output_bwd(g.data_ptr(), us.data_ptr(), gw.data_ptr(), gb.data_ptr(), g.shape[0],
+                                             _stream_ptr(g.device))
+        _native.check(rc, "nnueft_stack_output_bwd")
+    return gw, gb
+
+
+class _StackOutput(torch.autograd.Function):
+    """fq_out(lin + skip) + (wpsqt - bpsqt) * (us - 0.5) as one kernel; fq_out is straight-through."""
+
+    @staticmethod
+    def forward(ctx, lin, skip, wpsqt, bpsqt, us, den, mult, fq):
+        lin, skip, wpsqt, bpsqt, us = (t.contiguous() for t in (lin, skip, wpsqt, bpsqt, us))
+        ctx.save_for_backward(us)
+        return _launch_stack_output(lin, skip, wpsqt, bpsqt, us, den, mult, fq)
+
+    @staticmethod
+    def backward(ctx, g):
+        (us,) = ctx.saved_tensors
+        g = g.contiguous()
+        gw, gb = _launch_stack_output_bwd(g, us)
+        return g, g, gw, gb, None, None, None, None
+
+
+@torch.compiler.disable(recursive=False)
+def _launch_sf_loss(scorenet, score, outcome, p, actual_lambda):
+    lib = _native.load()
+    B = scorenet.shape[0]
+    terms = torch.empty(3, B, dtype=torch.float32, device=scorenet.device)
+    sums = torch.empty(2, dtype=torch.float32, device=scorenet.device)
+    loss = torch.empty((), dtype=torch.float32, device=scorenet.device)
+    with torch.cuda.device(scorenet.device):
+        rc = lib.nnueft_sf_loss_fwd(scorenet.data_ptr(), score.data_ptr(), outcome.data_ptr(), terms.data_ptr(),
+                                    sums.data_ptr(), loss.data_ptr(), B, p.in_offset, p.in_scaling, p.out_offset,
+                                    p.out_scaling, p.pow_exp, p.qp_asymmetry, p.w1, p.w2, p.tb_remap_base,
+                                    p.tb_remap_scale, p.tb_remap_decay, float(actual_lambda),
+                                    _stream_ptr(scorenet.device))
+    _native.check(rc, "nnueft_sf_loss_fwd")
+    return terms, sums, loss
+
+
+@torch.compiler.disable(recursive=False)
+def _launch_sf_loss_bwd(terms, sums, grad_loss, shape):
+    lib = _native.load()
+    B = terms.shape[1]
+    g = torch.empty(shape, dtype=torch.float32, device=terms.device)
+    with torch.cuda.device(terms.device):
+        rc = lib.nnueft_sf_loss_bwd(terms.data_ptr(), sums.data_ptr(), grad_loss.data_ptr(), g.data_ptr(), B,
+                                    _stream_ptr(terms.device))
+    _native.check(rc, "nnueft_sf_loss_bwd")
+    return g
+
+
+class _SfLoss(torch.autograd.Function):
+    """sf_loss as two launches forward (per-position terms, fixed-order sums) and one backward."""
+
+    @staticmethod
+    def forward(ctx, scorenet, score, outcome, p, actual_lambda):
+        scorenet = scorenet.contiguous()
+        terms, sums, loss = _launch_sf_loss(scorenet, score.contiguous(), outcome.contiguous(), p, actual_lambda)
+        ctx.save_for_backward(terms, sums)
+        ctx.shape = scorenet.shape
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_loss):
+        terms, sums = ctx.saved_tensors
+        grad_loss = grad_loss.contiguous().to(torch.float32)
+        return _launch_sf_loss_bwd(terms, sums, grad_loss, ctx.shape), None, None, None, None
 
 
 class ComposedFeatureTransformer(nn.Module):
@@ -450,14 +603,38 @@ class StackedLinear(nn.Module):
     def _params(self):
         return self.linear.weight, self.linear.bias
 
+    def _shared(self):
+        """(weight, bias) of a layer added to every bucket's block, or (None, None)."""
+        return None, None
+
+    def _params_one_pass(self, fake_quantize_weights: bool):
+        """_params() and the two fake_quantize_weights calls as one kernel per tensor (the table merge:
+        q(W + V[row % rows of V]), straight-through gradient, the shared layer's gradient summed over the
+        buckets); the values are those of the torch ops, bit for bit."""
+        sw, sb = self._shared()
+        weight, bias = self.linear.weight, self.linear.bias
+        if not fake_quantize_weights and sw is None:
+            return weight, bias
+        q = self.quantization
+        ws = q.weight_scales_dict[f"{self.layer_key}_weight"] if fake_quantize_weights else 1.0
+        bs = q.weight_scales_dict[f"{self.layer_key}_bias"] if fake_quantize_weights else 1.0
+        weight = _table_merge(weight, sw, weight.shape[1], ws, ws, fake_quantize_weights)
+        bias = _table_merge(bias.view(-1, 1), None if sb is None else sb.view(-1, 1), 1, bs, bs,
+                            fake_quantize_weights).view(-1)
+        return weight, bias
+
     def forward(self, x, ls_indices, fake_quantize_weights: bool = False, grouping=None):
         """grouping: bucket_grouping(ls_indices, count) when several layers share ls_indices (optional)."""
-        weight, bias = self._params()
-        if fake_quantize_weights:
-            if self.quantization is None or self.layer_key is None:
-                raise RuntimeError("self.quantization and self.layer_key are required to use fake quantize weights.")
-            weight = self.quantization.fake_quantize_weights(weight, f"{self.layer_key}_weight")
-            bias = self.quantization.fake_quantize_weights(bias, f"{self.layer_key}_bias")
+        if fake_quantize_weights and (self.quantization is None or self.layer_key is None):
+            raise RuntimeError("self.quantization and self.layer_key are required to use fake quantize weights.")
+        w = self.linear.weight
+        if w.is_cuda and w.dtype == torch.float32 and w.is_contiguous():
+            weight, bias = self._params_one_pass(fake_quantize_weights)
+        else:
+            weight, bias = self._params()
+            if fake_quantize_weights:
+                weight = self.quantization.fake_quantize_weights(weight, f"{self.layer_key}_weight")
+                bias = self.quantization.fake_quantize_weights(bias, f"{self.layer_key}_bias")
         if _bucket_linear_applies(x, self.in_features, self.out_features, self.count):
             return _BucketLinear.apply(x, ls_indices, weight, bias, self.out_features, self.count, grouping)
         wide = F.linear(x, weight, bias).reshape(-1, self.out_features)
@@ -485,6 +662,9 @@ class FactorizedStackedLinear(StackedLinear):
     def _params(self):
         return (self.linear.weight + self.factorized_linear.weight.repeat(self.count, 1),
                 self.linear.bias + self.factorized_linear.bias.repeat(self.count))
+
+    def _shared(self):
+        return self.factorized_linear.weight, self.factorized_linear.bias
 
     @torch.no_grad()
     def zero_virtual_weights(self):
@@ -525,23 +705,36 @@ class LayerStacks(nn.Module):
             x = q.fake_quantize_ls_act(x)
         return q.clip_ls_act(torch.cat([sqr * q.sqr_crelu_correction_factor, x], dim=1))
 
-    def forward(self, x, ls_indices, fake_quantize_acts: bool = True, fake_quantize_weights: bool = True):
+    def _sqr_crelu(self, x, fake_quantize_acts, want_skip=False):
+        """_sqr_and_linear (and the skip value) as one kernel on the GPU."""
         q = self.quantization
+        if _fused_tail_applies(x):
+            return _SqrCrelu.apply(x, want_skip, q.hidden_quantized_one, q.sqr_crelu_correction_factor,
+                                   q.max_hidden_activation, fake_quantize_acts)
+        skip = x[:, -2].view(-1, 1) - x[:, -1].view(-1, 1) if want_skip else None
+        return self._sqr_and_linear(x, fake_quantize_acts), skip
+
+    def forward_parts(self, x, ls_indices, fake_quantize_acts: bool = True, fake_quantize_weights: bool = True):
+        """(output layer's result, skip value), both [B, 1], before they are added and quantized."""
         # the three layers pick blocks by the same indices: group the positions once
         grouping = None
         if _bucket_linear_applies(x, self.l1.in_features, self.l1.out_features, self.count):
             grouping = bucket_grouping(ls_indices, self.count)
         l1c = self.l1(x, ls_indices, fake_quantize_weights, grouping)
-        skip = l1c[:, -2].view(-1, 1) - l1c[:, -1].view(-1, 1)
-        l1x = self._sqr_and_linear(l1c, fake_quantize_acts)
-        l2x = self._sqr_and_linear(self.l2(l1x, ls_indices, fake_quantize_weights, grouping), fake_quantize_acts)
+        l1x, skip = self._sqr_crelu(l1c, fake_quantize_acts, want_skip=True)
+        l2x, _ = self._sqr_crelu(self.l2(l1x, ls_indices, fake_quantize_weights, grouping), fake_quantize_acts)
         out = self.output(torch.cat([l1x, l2x], dim=1), ls_indices, fake_quantize_weights, grouping)
+        assert out.shape[1] == 1
+        return out, skip
+
+    def forward(self, x, ls_indices, fake_quantize_acts: bool = True, fake_quantize_weights: bool = True):
+        q = self.quantization
+        out, skip = self.forward_parts(x, ls_indices, fake_quantize_acts, fake_quantize_weights)
         if fake_quantize_acts:
             skip = q.fake_quantize_skip_act(skip)
         out = out + skip
         if fake_quantize_acts:
             out = q.fake_quantize_output(out)
-        assert out.shape[1] == 1
         return out
 
     @torch.no_grad()
@@ -577,6 +770,10 @@ class NNUEModel(nn.Module):
         l0_, wpsqt, bpsqt = self.forward_ft(us, them, white_indices, black_indices, psqt_indices,
                                             fake_quantize_acts, fake_quantize_weights)
         # the PSQT term is the perspective average with the sign of the side to move
+        if _fused_tail_applies(l0_):
+            lin, skip = self.layer_stacks.forward_parts(l0_, ls_indices, fake_quantize_acts, fake_quantize_weights)
+            den, mult = self.quantization.output_quantization()
+            return _StackOutput.apply(lin, skip, wpsqt, bpsqt, us, den, mult, fake_quantize_acts)
         return self.layer_stacks(l0_, ls_indices, fake_quantize_acts, fake_quantize_weights) + (wpsqt - bpsqt) * (us - 0.5)
 
     @torch.no_grad()
@@ -610,6 +807,9 @@ def remap_tablebase_score(score, base: float, scale: float, decay: float):
 
 def sf_loss(scorenet, score, outcome, p: LossParams, actual_lambda):
     """Win-rate-model loss; `scorenet` is the net output times nnue2score (model/nnue.py:39-70)."""
+    if _fused_tail_applies(scorenet) and score.dtype == torch.float32 and outcome.dtype == torch.float32 \
+            and scorenet.numel() > 0 and score.shape == scorenet.shape == outcome.shape:
+        return _SfLoss.apply(scorenet, score, outcome, p, actual_lambda)
     score = remap_tablebase_score(score, p.tb_remap_base, p.tb_remap_scale, p.tb_remap_decay)
 
     def win_rate(x, offset, scaling):

@@ -221,3 +221,106 @@ def test_stacked_linear_on_gpu_equals_the_wide_layer():
         torch.testing.assert_close(xg.grad.cpu(), xc.grad, rtol=1e-4, atol=1e-5)
         for (n, a), (_, b) in zip(layer.named_parameters(), gpu.named_parameters()):
             torch.testing.assert_close(b.grad.cpu(), a.grad, rtol=1e-4, atol=2e-5, msg=n)
+    # the one-pass weight preparation gives the bits of the torch ops it replaces
+    for fq in (False, True):
+        w1, b1 = gpu._params_one_pass(fq)
+        w0, b0 = gpu._params()
+        if fq:
+            w0, b0 = q.fake_quantize_weights(w0, "ls_l1_weight"), q.fake_quantize_weights(b0, "ls_l1_bias")
+        assert torch.equal(w1, w0) and torch.equal(b1, b0)
+    plain = M.StackedLinear(64, 32, 8, q, "ls_l2").to(DEV)
+    w1, b1 = plain._params_one_pass(True)
+    assert torch.equal(w1, q.fake_quantize_weights(plain.linear.weight, "ls_l2_weight"))
+    assert torch.equal(b1, q.fake_quantize_weights(plain.linear.bias, "ls_l2_bias"))
+    w1, b1 = plain._params_one_pass(False)
+    assert w1 is plain.linear.weight and b1 is plain.linear.bias
+
+
+def _tail_inputs(B, n, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(B, n, generator=g) * 0.7
+    # values on and next to the quantization grid and the clamp bounds
+    edge = torch.tensor([0.0, 1.0, -1.0, 1.0 / 127, 126.5 / 127, 127.0 / 127, 2.0, -0.0039])[: B * n]
+    x.view(-1)[: edge.numel()] = edge
+    return x
+
+
+@pytest.mark.parametrize("B,n", [(1, 2), (33, 16), (4097, 32)])
+@pytest.mark.parametrize("fq", [True, False])
+def test_sqr_crelu_kernel_equals_the_torch_ops(B, n, fq):
+    """One kernel against the chain of torch ops it replaces (LayerStacks._sqr_and_linear on the CPU,
+    autograd for the gradient): same bits forward; the gradient to one rounding."""
+    q = M.QuantizationManager(M.QuantizationConfig())
+    ls = M.LayerStacks(8, M.ModelConfig(L1=64, L2=n, L3=32), q)
+    x = _tail_inputs(B, n, 5 + B)
+    xc = x.clone().requires_grad_()
+    yc, sc = ls._sqr_crelu(xc, fq, want_skip=True)
+    xg = x.to(DEV).requires_grad_()
+    yg, sg = ls._sqr_crelu(xg, fq, want_skip=True)
+    assert torch.equal(yg.cpu(), yc) and torch.equal(sg.cpu(), sc)
+    g = torch.Generator().manual_seed(9)
+    gy, gs = torch.randn(B, 2 * n, generator=g), torch.randn(B, 1, generator=g)
+    torch.autograd.backward([yc, sc], [gy, gs])
+    torch.autograd.backward([yg, sg], [gy.to(DEV), gs.to(DEV)])
+    torch.testing.assert_close(xg.grad.cpu(), xc.grad, rtol=1e-6, atol=1e-7)
+    # without the skip value
+    xg2 = x.to(DEV).requires_grad_()
+    y2, none = ls._sqr_crelu(xg2, fq)
+    assert none is None and torch.equal(y2, yg)
+    y2.backward(gy.to(DEV))
+    xc2 = x.clone().requires_grad_()
+    ls._sqr_and_linear(xc2, fq).backward(gy)
+    torch.testing.assert_close(xg2.grad.cpu(), xc2.grad, rtol=1e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("fq", [True, False])
+def test_stack_output_kernel_equals_the_torch_ops(fq):
+    q = M.QuantizationManager(M.QuantizationConfig())
+    B = 5000
+    g = torch.Generator().manual_seed(4)
+    lin, skip = torch.randn(B, 1, generator=g) * 0.5, torch.randn(B, 1, generator=g) * 0.2
+    wp, bp = torch.randn(B, 1, generator=g) * 0.3, torch.randn(B, 1, generator=g) * 0.3
+    us = torch.randint(0, 2, (B, 1), generator=g).float()
+    cpu = [t.clone().requires_grad_() for t in (lin, skip, wp, bp)]
+    v = cpu[0] + cpu[1]
+    if fq:
+        v = q.fake_quantize_output(v)
+    want = v + (cpu[2] - cpu[3]) * (us - 0.5)
+    gpu = [t.to(DEV).requires_grad_() for t in (lin, skip, wp, bp)]
+    den, mult = q.output_quantization()
+    got = M._StackOutput.apply(*gpu, us.to(DEV), den, mult, fq)
+    assert torch.equal(got.cpu(), want)
+    up = torch.randn(B, 1, generator=g)
+    want.backward(up)
+    got.backward(up.to(DEV))
+    for a, b in zip(gpu, cpu):
+        assert torch.equal(a.grad.cpu(), b.grad)
+
+
+@pytest.mark.parametrize("params,lam", [(M.LossParams(), 0.75), (M.LossParams(qp_asymmetry=0.3, w1=1.0), 1.0),
+                                         (M.LossParams(pow_exp=2.0, w1=0.5, w2=0.25), 0.3)])
+@pytest.mark.parametrize("B", [1, 1000, 16384])
+def test_sf_loss_kernels_against_the_torch_formula(params, lam, B):
+    """The fused loss against sf_loss written in torch ops, evaluated in float64 on the CPU with autograd
+    for the gradient.  Tolerance: 1e-5 relative for the loss; for the gradient 1e-4 of the largest entry,
+    2e-3 with position weights (w1 != 0): they depend on 1 - pf, which float32 holds to about 1e-2
+    relative for a tablebase score, whoever evaluates it."""
+    g = torch.Generator().manual_seed(B)
+    net = (torch.randn(B, 1, generator=g) * 400)
+    score = (torch.randn(B, 1, generator=g) * 600).clamp(-3000, 3000)
+    score.view(-1)[: min(B, 4)] = torch.tensor([31990.0, -31800.0, 31755.0, -32000.0])[: min(B, 4)]   # tablebase scores
+    outcome = torch.randint(0, 3, (B, 1), generator=g).float() / 2
+    x64 = net.double().requires_grad_()
+    want = M.sf_loss(x64, score.double(), outcome.double(), params, lam)
+    want.backward()
+    xg = net.to(DEV).requires_grad_()
+    got = M.sf_loss(xg, score.to(DEV), outcome.to(DEV), params, lam)
+    assert got.shape == () and got.dtype == torch.float32
+    got.backward()
+    assert abs(got.item() - want.item()) <= 1e-5 * abs(want.item())
+    scale = x64.grad.abs().max().item()
+    tol = 2e-3 if params.w1 != 0.0 else 1e-4
+    assert (xg.grad.cpu().double() - x64.grad).abs().max().item() <= tol * scale
+    # twice the same bits
+    again = M.sf_loss(net.to(DEV), score.to(DEV), outcome.to(DEV), params, lam)
+    assert torch.equal(again, got.detach())
