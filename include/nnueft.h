@@ -128,6 +128,23 @@ int nnueft_double_fwd(const float* us, const float* them, const int32_t* widx, c
                       void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * nnueft_double_fwd whose l0 already carries the activation grid its caller applies next:
+ *   l0 = (floor(l0 * act_scale + act_eps) / act_scale) * act_post_mul,
+ * i.e. `fake_quantize_ft_act(l0_) * l0_correction_factor` of ComposedFeatureTransformer.forward
+ * (composed_feature_transformer.py:143-149) inside the kernel that produces l0, instead of one more
+ * pass over [B, L1].  Every operation rounds on its own: the same bits as the separate pass
+ * (nnueft_act_fake_quantize).  `saved`, wpsqt and bpsqt are those of nnueft_double_fwd, so the
+ * backward entry points serve both (the grid is straight-through; the caller scales grad_l0 by
+ * act_post_mul).
+ */
+int nnueft_double_fwd_act(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+                          const int64_t* psqt_idx, const float* W, const float* bias, float max_act,
+                          float* l0, float* wpsqt, float* bpsqt, float* saved,
+                          int B, int K, int R, int L1, int n_psqt,
+                          void* workspace, size_t workspace_bytes,
+                          float act_scale, float act_eps, float act_post_mul, void* stream);
+
+/*
  * Gradient of nnueft_double_fwd with respect to W and bias, floating-point atomics.
  * `saved` is the forward's; `bias` the forward's bias.  gW f32[R,L1+n_psqt] and gbias f32[L1+n_psqt]
  * must be zero on entry.

@@ -45,28 +45,64 @@ bool bucket_layout(int B, int count, BucketLayout* L) {
 
 // Single workgroup.  order[] = the positions of bucket 0 ascending, then bucket 1, ...; positions
 // whose bucket is outside [0, count) are left out.  tiles[2t] = first index into order, tiles[2t+1]
-// = bucket << 8 | positions in the tile.  Two sweeps over the positions, 1024 at a time: count per
-// (wave, bucket) with ballots, then place with the same ballots.
+// = bucket << 8 | positions in the tile.
+// The kernel is one workgroup, so every latency it waits for is run time: a thread keeps the buckets
+// of kOrderAhead positions in registers (loads issued together), counts with ballots, and the
+// workgroup synchronises three times per block of kOrderThreads * kOrderAhead positions, not per step.
+//   counts   per (step, wave, bucket) to LDS, ranks inside the ballot kept in registers
+//   prefix   wave w turns the counts of buckets w, w + NW, ... into places, in (step, wave) order
+//   place    order[place of (step, wave, bucket) + rank] = position
+// The lanes of the wave that hold the same bucket as this one (valid lanes only): one ballot per bit
+// of the bucket number instead of one per bucket.
+__device__ __forceinline__ u64 same_bucket(int c, bool valid, int nbits) {
+    u64 m = __ballot(valid);
+    for (int j = 0; j < nbits; ++j) {
+        const bool bit = (c >> j) & 1;
+        const u64 bj = __ballot(valid && bit);
+        m &= bit ? bj : ~bj;
+    }
+    return m;
+}
+
+template <int kOrderAhead>
 __global__ __launch_bounds__(kOrderThreads) void k_bucket_order(const int64_t* __restrict__ bucket,
                                                                 uint32_t* __restrict__ order,
                                                                 uint32_t* __restrict__ bucket_off,
                                                                 uint32_t* __restrict__ ntiles,
                                                                 uint32_t* __restrict__ tiles, int B, int count) {
     constexpr int NW = kOrderThreads / 64;
+    constexpr int NS = kOrderAhead * NW;             // (step, wave) pairs of a block, in position order
+    extern __shared__ uint32_t cnt_s[];              // [count][NS]
     __shared__ uint32_t total_s[kMaxCount];          // positions per bucket
     __shared__ uint32_t cursor_s[kMaxCount];         // next free place of each bucket
-    __shared__ uint32_t wave_cnt[NW][kMaxCount];     // this sweep step: positions per (wave, bucket)
     __shared__ uint32_t tile_base_s[kMaxCount + 1];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (tid < kMaxCount) total_s[tid] = 0;
     __syncthreads();
-    // sweep 1: totals
-    for (int b0 = 0; b0 < B; b0 += kOrderThreads) {
-        const int b = b0 + tid;
-        const int c = b < B ? (int)bucket[b] : -1;
-        for (int k = 0; k < count; ++k) {
-            const u64 m = __ballot(c == k);
-            if (lane == 0 && m) atomicAdd(&total_s[k], (uint32_t)__popcll(m));
+    // totals.  The first block's buckets stay in registers for the
+    // second pass (a batch of up to kOrderThreads * kOrderAhead positions is read from memory once).
+    constexpr int NB = kOrderThreads * kOrderAhead;
+    const int nbits = count > 1 ? 32 - __clz(count - 1) : 0;
+    const u64 lt = (1ull << lane) - 1ull;
+    int first[kOrderAhead];
+#pragma unroll
+    for (int u = 0; u < kOrderAhead; ++u) {
+        const int b = u * kOrderThreads + tid;
+        first[u] = b < B ? (int)bucket[b] : -1;
+    }
+    for (int b0 = 0; b0 < B; b0 += NB) {
+        int cs[kOrderAhead];
+#pragma unroll
+        for (int u = 0; u < kOrderAhead; ++u) {
+            const int b = b0 + u * kOrderThreads + tid;
+            cs[u] = b0 == 0 ? first[u] : (b < B ? (int)bucket[b] : -1);
+        }
+#pragma unroll
+        for (int u = 0; u < kOrderAhead; ++u) {
+            if (b0 + u * kOrderThreads >= B) break;
+            const bool valid = cs[u] >= 0 && cs[u] < count;
+            const u64 m = same_bucket(cs[u], valid, nbits);
+            if (valid && (m & lt) == 0) atomicAdd(&total_s[cs[u]], (uint32_t)__popcll(m));   // first of its group
         }
     }
     __syncthreads();
@@ -91,28 +127,53 @@ __global__ __launch_bounds__(kOrderThreads) void k_bucket_order(const int64_t* _
             tiles[2 * (tile_base_s[k] + t) + 1] = ((uint32_t)k << 8) | min((uint32_t)kTile, total_s[k] - t * kTile);
         }
     }
-    __syncthreads();
-    // sweep 2: places, ascending position inside a bucket
-    for (int b0 = 0; b0 < B; b0 += kOrderThreads) {
-        const int b = b0 + tid;
-        const int c = b < B ? (int)bucket[b] : -1;
-        uint32_t rank = 0;
-        for (int k = 0; k < count; ++k) {
-            const u64 m = __ballot(c == k);
-            if (lane == 0) wave_cnt[wave][k] = (uint32_t)__popcll(m);
-            if (c == k) rank = (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
+    // places, ascending position inside a bucket
+    for (int b0 = 0; b0 < B; b0 += NB) {
+        int cs[kOrderAhead];
+        uint32_t rank[kOrderAhead];
+#pragma unroll
+        for (int u = 0; u < kOrderAhead; ++u) {
+            const int b = b0 + u * kOrderThreads + tid;
+            cs[u] = b0 == 0 ? first[u] : (b < B ? (int)bucket[b] : -1);
+        }
+        for (int i = tid; i < count * NS; i += kOrderThreads) cnt_s[i] = 0;
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < kOrderAhead; ++u) {
+            const bool valid = cs[u] >= 0 && cs[u] < count;
+            const u64 m = same_bucket(cs[u], valid, nbits);
+            rank[u] = (uint32_t)__popcll(m & lt);
+            if (valid && rank[u] == 0) cnt_s[cs[u] * NS + u * NW + wave] = (uint32_t)__popcll(m);
         }
         __syncthreads();
-        if (c >= 0 && c < count) {
-            uint32_t before = 0;
-            for (int w = 0; w < wave; ++w) before += wave_cnt[w][c];
-            order[cursor_s[c] + before + rank] = (uint32_t)b;
+        for (int k = wave; k < count; k += NW) {
+            constexpr int PER = NS / 64;
+            uint32_t v[PER], sum = 0;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) {
+                v[i] = cnt_s[k * NS + lane * PER + i];
+                sum += v[i];
+            }
+            uint32_t incl = sum;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const uint32_t t = __shfl_up(incl, off);
+                if (lane >= off) incl += t;
+            }
+            uint32_t run = cursor_s[k] + incl - sum;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) {
+                cnt_s[k * NS + lane * PER + i] = run;
+                run += v[i];
+            }
+            if (lane == 63) cursor_s[k] = run;
         }
         __syncthreads();
-        if (tid < count) {
-            uint32_t add = 0;
-            for (int w = 0; w < NW; ++w) add += wave_cnt[w][tid];
-            cursor_s[tid] += add;
+#pragma unroll
+        for (int u = 0; u < kOrderAhead; ++u) {
+            const int c = cs[u];
+            if (c >= 0 && c < count)
+                order[cnt_s[c * NS + u * NW + wave] + rank[u]] = (uint32_t)(b0 + u * kOrderThreads + tid);
         }
         __syncthreads();
     }
@@ -326,9 +387,18 @@ int check_args(int B, int in, int out, int count) {
 }
 
 int launch_order(const int64_t* bucket, char* ws, const BucketLayout& L, int B, int count, hipStream_t st) {
-    hipLaunchKernelGGL(k_bucket_order, dim3(1), dim3(kOrderThreads), 0, st, bucket, (uint32_t*)(ws + L.order),
-                       (uint32_t*)(ws + L.bucket_off), (uint32_t*)(ws + L.ntiles), (uint32_t*)(ws + L.tiles), B,
-                       count);
+    // counts of a block in LDS: count x steps x waves words, at most 32 KB
+    if (count <= 32) {
+        const size_t lds = (size_t)count * 16 * (kOrderThreads / 64) * sizeof(uint32_t);
+        hipLaunchKernelGGL(k_bucket_order<16>, dim3(1), dim3(kOrderThreads), lds, st, bucket,
+                           (uint32_t*)(ws + L.order), (uint32_t*)(ws + L.bucket_off), (uint32_t*)(ws + L.ntiles),
+                           (uint32_t*)(ws + L.tiles), B, count);
+    } else {
+        const size_t lds = (size_t)count * 4 * (kOrderThreads / 64) * sizeof(uint32_t);
+        hipLaunchKernelGGL(k_bucket_order<4>, dim3(1), dim3(kOrderThreads), lds, st, bucket,
+                           (uint32_t*)(ws + L.order), (uint32_t*)(ws + L.bucket_off), (uint32_t*)(ws + L.ntiles),
+                           (uint32_t*)(ws + L.tiles), B, count);
+    }
     NNUEFT_LAUNCH_CHECK();
     return 0;
 }

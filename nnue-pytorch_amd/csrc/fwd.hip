@@ -187,10 +187,15 @@ extern "C" size_t nnueft_fwd_workspace_bytes(int B, int K, int R, int L1, int n_
     return nnueft_blocked::pair_sort_workspace(B, R, 0);
 }
 
-extern "C" int nnueft_double_fwd(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
-                                 const int64_t* psqt_idx, const float* W, const float* bias, float max_act,
-                                 float* l0, float* wpsqt, float* bpsqt, float* saved, int B, int K, int R,
-                                 int L1, int n_psqt, void* workspace, size_t workspace_bytes, void* stream) {
+extern "C" int nnueft_act_fake_quantize(const float* x, float* out, long long n, float scale, float eps,
+                                        float post_mul, void* stream);
+
+namespace {
+
+int double_fwd(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+               const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0, float* wpsqt,
+               float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt, void* workspace,
+               size_t workspace_bytes, void* stream, ActGrid act) {
     if (B < 0 || K <= 0 || R <= 0 || L1 <= 0 || (L1 & 1) || n_psqt < 0) return NNUEFT_E_ARG;
     if (B == 0) return 0;
     if (!us || !them || !widx || !bidx || !psqt_idx || !W || !bias || !l0 || !wpsqt || !bpsqt || !saved)
@@ -204,7 +209,15 @@ extern "C" int nnueft_double_fwd(const float* us, const float* them, const int32
         // the L2-blocked path needs 16-byte rows; other shapes take the plain kernel below
         if (vec && (long long)B <= 0x3fffffffLL)
             return nnueft_blocked::double_fwd_blocked(us, them, widx, bidx, psqt_idx, W, bias, max_act, l0, wpsqt,
-                                                      bpsqt, saved, B, K, R, L1, n_psqt, workspace, st);
+                                                      bpsqt, saved, B, K, R, L1, n_psqt, workspace, st, act);
+    }
+    if (act.on) {
+        // the plain kernels know nothing of the grid: run them, then the grid in place
+        ActGrid off{};
+        const int rc = double_fwd(us, them, widx, bidx, psqt_idx, W, bias, max_act, l0, wpsqt, bpsqt, saved, B, K, R,
+                                  L1, n_psqt, nullptr, 0, stream, off);
+        if (rc) return rc;
+        return nnueft_act_fake_quantize(l0, l0, (long long)B * L1, act.scale, act.eps, act.post_mul, stream);
     }
     if (vec) {
         if (L1 / 8 > 64)
@@ -218,4 +231,26 @@ extern "C" int nnueft_double_fwd(const float* us, const float* them, const int32
                                        B, K, R, L1, n_psqt, st);
     return launch_double_fwd<1, 1>(us, them, widx, bidx, psqt_idx, W, bias, max_act, l0, wpsqt, bpsqt, saved, B,
                                    K, R, L1, n_psqt, st);
+}
+
+}  // namespace
+
+extern "C" int nnueft_double_fwd(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+                                 const int64_t* psqt_idx, const float* W, const float* bias, float max_act,
+                                 float* l0, float* wpsqt, float* bpsqt, float* saved, int B, int K, int R,
+                                 int L1, int n_psqt, void* workspace, size_t workspace_bytes, void* stream) {
+    ActGrid off{};
+    return double_fwd(us, them, widx, bidx, psqt_idx, W, bias, max_act, l0, wpsqt, bpsqt, saved, B, K, R, L1, n_psqt,
+                      workspace, workspace_bytes, stream, off);
+}
+
+extern "C" int nnueft_double_fwd_act(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+                                     const int64_t* psqt_idx, const float* W, const float* bias, float max_act,
+                                     float* l0, float* wpsqt, float* bpsqt, float* saved, int B, int K, int R,
+                                     int L1, int n_psqt, void* workspace, size_t workspace_bytes, float act_scale,
+                                     float act_eps, float act_post_mul, void* stream) {
+    if (!(act_scale > 0.0f)) return NNUEFT_E_ARG;
+    ActGrid act{act_scale, act_eps, act_post_mul, 1};
+    return double_fwd(us, them, widx, bidx, psqt_idx, W, bias, max_act, l0, wpsqt, bpsqt, saved, B, K, R, L1, n_psqt,
+                      workspace, workspace_bytes, stream, act);
 }

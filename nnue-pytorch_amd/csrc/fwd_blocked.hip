@@ -169,7 +169,8 @@ __global__ __launch_bounds__(64) void k_mix(const float* __restrict__ us, const 
                                             const int64_t* __restrict__ psqt_idx, const float* __restrict__ W,
                                             const float* __restrict__ bias, const float* __restrict__ saved,
                                             float max_act, float* __restrict__ l0, float* __restrict__ wpsqt,
-                                            float* __restrict__ bpsqt, int B, int K, int R, int L1, int n_psqt) {
+                                            float* __restrict__ bpsqt, int B, int K, int R, int L1, int n_psqt,
+                                            ActGrid act) {
     const int lane = threadIdx.x;
     const int b = blockIdx.x;
     const int s = blockIdx.y;
@@ -192,6 +193,10 @@ __global__ __launch_bounds__(64) void k_mix(const float* __restrict__ us, const 
             mix4(u, t, sw0.v[i], sw1.v[i], sb0.v[i], sb1.v[i], bias0.v[i], bias1.v[i], xw0, xw1, xb0, xb1);
             o0.v[i] = clamp_act(xw0, max_act) * clamp_act(xw1, max_act);
             o1.v[i] = clamp_act(xb0, max_act) * clamp_act(xb1, max_act);
+            if (act.on) {   // the activation grid the caller would otherwise apply in a pass of its own
+                o0.v[i] = (floorf(o0.v[i] * act.scale + act.eps) / act.scale) * act.post_mul;
+                o1.v[i] = (floorf(o1.v[i] * act.scale + act.eps) / act.scale) * act.post_mul;
+            }
         }
         float* o = l0 + (size_t)b * L1;
         stv<VW>(o + c, o0);
@@ -283,7 +288,7 @@ int table_block_rows(int R, int hint, int* nbins) {
 int double_fwd_blocked(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                        const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,
                        float* wpsqt, float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt,
-                       void* ws, hipStream_t st) {
+                       void* ws, hipStream_t st, ActGrid act) {
     const uint32_t* order = nullptr;
     const int rc = launch_pair_sort(widx, bidx, B, K, R, 0, ws, st, &order);
     if (rc) return rc;
@@ -306,7 +311,7 @@ int double_fwd_blocked(const float* us, const float* them, const int32_t* widx, 
     NNUEFT_LAUNCH_CHECK();
     const int hv = (L1 / 2) / 4;
     hipLaunchKernelGGL(k_mix<4>, dim3(B, (hv + 63) / 64), dim3(64), 0, st, us, them, widx, bidx, psqt_idx, W, bias,
-                       saved, max_act, l0, wpsqt, bpsqt, B, K, R, L1, n_psqt);
+                       saved, max_act, l0, wpsqt, bpsqt, B, K, R, L1, n_psqt, act);
     NNUEFT_LAUNCH_CHECK();
     return 0;
 }

@@ -3,6 +3,13 @@
 
 #include "common.h"
 
+// The activation grid of the feature transformer's output, (floor(x * scale + eps) / scale) * post_mul,
+// when the forward applies it itself (on == 0: it does not).
+struct ActGrid {
+    float scale, eps, post_mul;
+    int on;
+};
+
 namespace nnueft_blocked {
 
 constexpr int kXcd = 8;   // XCDs of the device; workgroup id % kXcd is the XCD a workgroup lands on
@@ -17,7 +24,7 @@ int launch_pair_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int
 int double_fwd_blocked(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                        const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,
                        float* wpsqt, float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt, void* ws,
-                       hipStream_t st);
+                       hipStream_t st, ActGrid act);
 
 }  // namespace nnueft_blocked
 

@@ -28,19 +28,25 @@ BACKWARD_TILE_SIZE = 4
 
 @torch.compiler.disable(recursive=False)
 def _launch_double_fwd(us, them, white_indices, black_indices, psqt_indices, weight, bias, max_ft_activation,
-                       l1_size, l0_, wpsqt, bpsqt, saved):
+                       l1_size, l0_, wpsqt, bpsqt, saved, act_grid=None):
     lib = _native.load()
     B, K = white_indices.shape
     R, out_cols = weight.shape
     nbytes = lib.nnueft_fwd_workspace_bytes(B, K, R, l1_size, out_cols - l1_size)
     ws = _workspace(nbytes, weight.device)
-    rc = lib.nnueft_double_fwd(
+    head = (
         us.data_ptr(), them.data_ptr(), white_indices.data_ptr(), black_indices.data_ptr(),
         psqt_indices.data_ptr(), weight.data_ptr(), bias.data_ptr(), float(max_ft_activation),
         l0_.data_ptr(), wpsqt.data_ptr(), bpsqt.data_ptr(), saved.data_ptr(),
-        B, K, R, l1_size, out_cols - l1_size, ws.data_ptr(), nbytes, _stream_ptr(weight.device),
+        B, K, R, l1_size, out_cols - l1_size, ws.data_ptr(), nbytes,
     )
-    _native.check(rc, "nnueft_double_fwd")
+    if act_grid is None:
+        rc = lib.nnueft_double_fwd(*head, _stream_ptr(weight.device))
+        _native.check(rc, "nnueft_double_fwd")
+    else:
+        scale, eps, post_mul = act_grid
+        rc = lib.nnueft_double_fwd_act(*head, float(scale), float(eps), float(post_mul), _stream_ptr(weight.device))
+        _native.check(rc, "nnueft_double_fwd_act")
 
 
 @torch.compiler.disable(recursive=False)
@@ -105,7 +111,12 @@ def _launch_double_bwd(us, them, white_indices, black_indices, psqt_indices, bia
 
 class FusedDoubleFtFunction(autograd.Function):
     @staticmethod
-    def forward(ctx, us, them, white_indices, black_indices, psqt_indices, weight, bias, max_ft_activation, l1_size):
+    def forward(ctx, us, them, white_indices, black_indices, psqt_indices, weight, bias, max_ft_activation, l1_size,
+                act_grid=None):
+        """act_grid (not part of the reference's signature): None, or (scale, eps, post_mul): l0 comes out as
+        (floor(l0 * scale + eps) / scale) * post_mul, the activation grid and correction factor that
+        ComposedFeatureTransformer applies next, with a straight-through gradient."""
+        ctx.act_grid = None if act_grid is None else tuple(float(v) for v in act_grid)
         ctx.max_ft_activation = float(max_ft_activation)
         ctx.l1_size = int(l1_size)
         ctx.backward_mode = _slf.get_backward_mode()
@@ -157,7 +168,7 @@ class FusedDoubleFtFunction(autograd.Function):
 
             _launch_double_fwd(
                 us, them, white_indices, black_indices, psqt_indices, weight, bias,
-                max_ft_activation, int(l1_size), l0_, wpsqt, bpsqt, row_sums,
+                max_ft_activation, int(l1_size), l0_, wpsqt, bpsqt, row_sums, ctx.act_grid,
             )
 
         ctx.save_for_backward(us, them, white_indices, black_indices, psqt_indices, weight, bias, row_sums)
@@ -170,6 +181,8 @@ class FusedDoubleFtFunction(autograd.Function):
         grad_l0 = grad_l0.contiguous()
         grad_wpsqt = grad_wpsqt.contiguous()
         grad_bpsqt = grad_bpsqt.contiguous()
+        if ctx.act_grid is not None and ctx.act_grid[2] != 1.0:
+            grad_l0 = grad_l0 * ctx.act_grid[2]
 
         with torch.cuda.device(us.device):
             grad_weight, grad_bias = _launch_double_bwd(
@@ -179,4 +192,4 @@ class FusedDoubleFtFunction(autograd.Function):
                 ctx.sort_placement != "inline",
             )
 
-        return None, None, None, None, None, grad_weight, grad_bias, None, None
+        return None, None, None, None, None, grad_weight, grad_bias, None, None, None

@@ -27,6 +27,7 @@ from torch import nn
 from . import _native
 from . import halfka_v2_hm as hk
 from .double_ft_functions import double_feature_transform
+from .fused_ft_functions import FusedDoubleFtFunction
 from .sparse_linear_functions import _stream_ptr
 
 FAKE_QUANTIZE_EPS = 1e-5
@@ -499,9 +500,15 @@ class ComposedFeatureTransformer(nn.Module):
     def forward(self, us, them, white_indices, black_indices, psqt_indices, fake_quantize_acts: bool,
                 fake_quantize_weights: bool, backend: str = "auto"):
         merged, bias = self.merged_weight_and_bias(fake_quantize_weights)
+        q = self.quantization
+        if (fake_quantize_acts and backend in ("auto", "fused") and merged.is_cuda and _native.available()
+                and all(t.is_cuda for t in (us, them, white_indices, black_indices, psqt_indices, bias))):
+            # the activation grid and the correction factor inside the kernel that writes l0
+            return FusedDoubleFtFunction.apply(
+                us, them, white_indices, black_indices, psqt_indices, merged, bias, q.max_ft_activation,
+                self.l1_size, (q.hidden_quantized_one, FAKE_QUANTIZE_EPS, q.l0_correction_factor))
         l0_, wpsqt, bpsqt = double_feature_transform(us, them, white_indices, black_indices, psqt_indices, merged,
                                                      bias, self.quantization.max_ft_activation, self.l1_size, backend)
-        q = self.quantization
         if fake_quantize_acts and l0_.is_cuda and l0_.dtype == torch.float32 and _native.available():
             # activation grid and correction factor in one pass over [B, L1]
             return _ActFakeQuantize.apply(l0_, q.hidden_quantized_one, q.l0_correction_factor), wpsqt, bpsqt

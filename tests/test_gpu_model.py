@@ -146,7 +146,8 @@ def test_act_fake_quantize_kernel(oracle_cpu, n, post_mul):
 
 
 @pytest.mark.parametrize("B,n_in,out,count", [(1, 32, 1, 1), (37, 64, 16, 8), (300, 128, 32, 8), (1000, 3072, 32, 8),
-                                              (4097, 1024, 16, 8), (513, 96, 7, 3), (64, 256, 32, 64)])
+                                              (4097, 1024, 16, 8), (513, 96, 7, 3), (64, 256, 32, 64),
+                                              (20000, 32, 4, 8), (5000, 32, 2, 40), (16384, 64, 3, 32)])
 def test_bucket_linear_kernels(oracle_cpu, B, n_in, out, count):
     from nnueft import _native
 

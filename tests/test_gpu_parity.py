@@ -130,6 +130,36 @@ def _run_double_fwd(c, with_workspace=True):
 
 @pytest.mark.parametrize("with_workspace", [False, True], ids=["plain", "l2blocked"])
 @pytest.mark.parametrize("B,L1,R,K,kw", DOUBLE_SHAPES)
+def test_double_forward_with_activation_grid(oracle_cpu, B, L1, R, K, kw, with_workspace):
+    """nnueft_double_fwd_act = nnueft_double_fwd followed by the activation grid, bit for bit (the grid
+    against the oracle's act_fake_quantize)."""
+    c = double_case(450 + B, B, L1, R, K, **kw)
+    nat, lib = _native()
+    d, l0, wp, bp, saved = _run_double_fwd(c, with_workspace)
+    n_psqt = c["n_psqt"]
+    l0q = torch.full((B, L1), float("nan"), device=_dev())
+    wp2, bp2, saved2 = torch.empty_like(wp), torch.empty_like(bp), torch.empty_like(saved)
+    nbytes = lib.nnueft_fwd_workspace_bytes(B, K, R, L1, n_psqt) if with_workspace else 0
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=_dev())
+    scale, eps, post_mul = 127.0, 1e-5, 0.75
+    nat.check(lib.nnueft_double_fwd_act(d["us"].data_ptr(), d["them"].data_ptr(), d["widx"].data_ptr(),
+                                        d["bidx"].data_ptr(), d["psqt_idx"].data_ptr(), d["W"].data_ptr(),
+                                        d["bias"].data_ptr(), c["max_act"], l0q.data_ptr(), wp2.data_ptr(),
+                                        bp2.data_ptr(), saved2.data_ptr(), B, K, R, L1, n_psqt,
+                                        ws.data_ptr() if with_workspace else None, nbytes, scale, eps, post_mul,
+                                        _stream()), "double_fwd_act")
+    assert torch.equal(wp, wp2) and torch.equal(bp, bp2) and torch.equal(saved, saved2)
+    want = oracle_cpu.act_fake_quantize(l0.cpu().numpy(), scale, eps, post_mul)
+    assert np.array_equal(l0q.cpu().numpy(), want)
+    assert lib.nnueft_double_fwd_act(d["us"].data_ptr(), d["them"].data_ptr(), d["widx"].data_ptr(),
+                                     d["bidx"].data_ptr(), d["psqt_idx"].data_ptr(), d["W"].data_ptr(),
+                                     d["bias"].data_ptr(), c["max_act"], l0q.data_ptr(), wp2.data_ptr(),
+                                     bp2.data_ptr(), saved2.data_ptr(), B, K, R, L1, n_psqt, None, 0, 0.0, eps,
+                                     post_mul, _stream()) == -1      # scale must be positive
+
+
+@pytest.mark.parametrize("with_workspace", [False, True], ids=["plain", "l2blocked"])
+@pytest.mark.parametrize("B,L1,R,K,kw", DOUBLE_SHAPES)
 def test_double_forward(oracle_cpu, B, L1, R, K, kw, with_workspace):
     c = double_case(400 + B, B, L1, R, K, **kw)
     _, l0, wp, bp, saved = _run_double_fwd(c, with_workspace)
