@@ -119,12 +119,12 @@ __global__ __launch_bounds__(64) void k_bwd_rows(const float* __restrict__ us, c
                                                  const float* __restrict__ grad_bpsqt,
                                                  const float* __restrict__ saved, float* __restrict__ G,
                                                  float* __restrict__ partial, int B, int L1, int n_psqt, int group,
-                                                 int ntiles) {
+                                                 int ntiles, int nslices) {
     // `group` lanes share a tile (64 for wide rows; narrow rows put 64 / group tiles into one wave)
     const int lane = threadIdx.x;
-    const int tile = blockIdx.x * (64 / group) + lane / group;
+    const int s = blockIdx.x % nslices;          // launched 1-D: the slices of a tile are neighbours
+    const int tile = (blockIdx.x / nslices) * (64 / group) + lane / group;
     const int ql = lane % group;
-    const int s = blockIdx.y;
     if (tile >= ntiles) return;
     const int h = L1 >> 1;
     const int hv = h / VW;
@@ -788,13 +788,15 @@ int launch_bwd_rows(const float* us, const float* them, const int64_t* psqt_idx,
     int group = 64;
     while (group > 8 && group / 2 >= hv) group /= 2;   // lanes per tile: 64, 32, 16 or 8
     const int tiles_per_wave = 64 / group;
-    const dim3 grid((ntiles + tiles_per_wave - 1) / tiles_per_wave, max(1, (hv + group - 1) / group));
+    const int nslices = max(1, (hv + group - 1) / group);
+    if ((long long)((ntiles + tiles_per_wave - 1) / tiles_per_wave) * nslices > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
+    const dim3 grid((unsigned)((ntiles + tiles_per_wave - 1) / tiles_per_wave) * nslices);
     if (vec)
         hipLaunchKernelGGL(k_bwd_rows<4>, grid, dim3(64), 0, st, us, them, psqt_idx, bias, max_act, grad_l0,
-                           grad_wpsqt, grad_bpsqt, saved, G, partial, B, L1, n_psqt, group, ntiles);
+                           grad_wpsqt, grad_bpsqt, saved, G, partial, B, L1, n_psqt, group, ntiles, nslices);
     else
         hipLaunchKernelGGL(k_bwd_rows<1>, grid, dim3(64), 0, st, us, them, psqt_idx, bias, max_act, grad_l0,
-                           grad_wpsqt, grad_bpsqt, saved, G, partial, B, L1, n_psqt, group, ntiles);
+                           grad_wpsqt, grad_bpsqt, saved, G, partial, B, L1, n_psqt, group, ntiles, nslices);
     NNUEFT_LAUNCH_CHECK();
     return 0;
 }
