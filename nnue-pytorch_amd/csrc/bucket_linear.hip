@@ -250,6 +250,77 @@ __global__ __launch_bounds__(KS * 64) void k_bucket_fwd(const float* __restrict_
     }
 }
 
+// The same for wide layers (in % (64 KS) == 0), with the tile of x taken through LDS.  The MFMA
+// operand wants one row of x per lane, which as a global load touches 32 rows x 32 bytes per
+// instruction; here a wave loads 4 rows x 256 contiguous bytes per instruction, parks 32 rows x 64
+// columns in its own LDS strip and reads the operand layout back from there.  The terms of every
+// dot product meet in the same order as in k_bucket_fwd, so the two kernels give the same bits.
+template <int KS>
+__global__ __launch_bounds__(KS * 64) void k_bucket_fwd_lds(const float* __restrict__ x, const float* __restrict__ W,
+                                                             const float* __restrict__ bias, float* __restrict__ y,
+                                                             const uint32_t* __restrict__ order,
+                                                             const uint32_t* __restrict__ ntiles,
+                                                             const uint32_t* __restrict__ tiles, int in, int out) {
+    constexpr int CK = 64;          // columns per step
+    constexpr int LD = CK + 4;      // padded row of the strip, floats
+    constexpr int kStrip = 32 * LD;
+    constexpr int kRed = KS > 1 ? (KS - 1) * 16 * 64 : 1;
+    __shared__ __attribute__((aligned(16))) float lds[KS * kStrip > kRed ? KS * kStrip : kRed];
+    const int t = blockIdx.x;
+    if ((uint32_t)t >= *ntiles) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t start = tiles[2 * t], info = tiles[2 * t + 1];
+    const int n = (int)(info & 255u), bk = (int)(info >> 8);
+    const int r = lane & 31, h = lane >> 5;
+    const int kw = in / KS;
+    const int srow = lane >> 4, scol = 4 * (lane & 15);
+    const float* xs[8];
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const int i = srow + 4 * it;
+        xs[it] = x + (size_t)order[start + (i < n ? i : 0)] * in + wave * kw + scol;
+    }
+    const bool jok = r < out;
+    const float* wb = W + ((size_t)bk * out + (jok ? r : 0)) * in + wave * kw + 4 * h;
+    float* strip = lds + wave * kStrip;
+    f32x16 acc = {0};
+    for (int k = 0; k < kw; k += CK) {
+        vecf<4> v[8], b[8];
+#pragma unroll
+        for (int it = 0; it < 8; ++it) v[it] = ldv4_stream(xs[it] + k);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) b[u] = ldv<4>(wb + k + 8 * u);
+#pragma unroll
+        for (int it = 0; it < 8; ++it) stv<4>(strip + (srow + 4 * it) * LD + scol, v[it]);
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const vecf<4> a = ldv<4>(strip + r * LD + 8 * u + 4 * h);
+            if (!jok) b[u] = vzero<4>();
+            acc = mfma4(a, b[u], acc);
+        }
+        __syncthreads();
+    }
+    if (KS > 1) {
+        if (wave > 0) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) lds[((wave - 1) * 16 + v) * 64 + lane] = acc[v];
+        }
+        __syncthreads();
+        if (wave > 0) return;
+        for (int w = 0; w < KS - 1; ++w)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[v] = acc[v] + lds[(w * 16 + v) * 64 + lane];
+    }
+    if (!jok) return;
+    const float bj = bias[bk * out + r];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int i = acc_row(v, lane);
+        if (i < n) y[(size_t)order[start + i] * out + r] = acc[v] + bj;
+    }
+}
+
 // gx[pos, c0 + 32 q + j] = sum_o gy[pos, o] * W_b[o, c0 + 32 q + j].  Workgroup = (tile, column range);
 // lanes 0-31 supply outputs o = 0..15, lanes 32-63 o = 16..31.
 __global__ __launch_bounds__(64) void k_bucket_bwd_x(const float* __restrict__ gy, const float* __restrict__ W,
@@ -438,7 +509,10 @@ extern "C" int nnueft_bucket_linear_fwd(const float* x, const int64_t* bucket, c
     const uint32_t* order = (const uint32_t*)(ws + L.order);
     const uint32_t* ntiles = (const uint32_t*)(ws + L.ntiles);
     const uint32_t* tiles = (const uint32_t*)(ws + L.tiles);
-    if (in % 256 == 0)
+    if (in % 512 == 0 && in >= 1024 && aligned16(x) && aligned16(W))
+        hipLaunchKernelGGL(k_bucket_fwd_lds<8>, dim3(L.max_tiles), dim3(512), 0, st, x, W, bias, y, order, ntiles,
+                           tiles, in, out);
+    else if (in % 256 == 0)
         hipLaunchKernelGGL(k_bucket_fwd<8>, dim3(L.max_tiles), dim3(512), 0, st, x, W, bias, y, order, ntiles, tiles, in,
                            out);
     else if (in % 128 == 0)

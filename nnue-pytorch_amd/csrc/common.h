@@ -88,6 +88,15 @@ __device__ __forceinline__ void stv_stream<1>(float* p, const vecf<1>& x) {
 #endif
 }
 
+// Streaming load of 4 floats: data read once, not to displace what the kernel keeps in L2.
+__device__ __forceinline__ vecf<4> ldv4_stream(const float* p) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    const f4 v = __builtin_nontemporal_load(reinterpret_cast<const f4*>(p));
+    vecf<4> r;
+    r.v[0] = v.x; r.v[1] = v.y; r.v[2] = v.z; r.v[3] = v.w;
+    return r;
+}
+
 template <int VW>
 __device__ __forceinline__ vecf<VW> vzero() {
     vecf<VW> r;
