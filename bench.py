@@ -6,9 +6,10 @@ A step is one pass of the hot path over one synthetic batch: the fused two-persp
 function the trainer calls.  Inputs are resident in HBM before the timed region.
 
 Prints ONE JSON line: positions/s for the workload BASELINE.json's metric is quoted on (L1=3072,
-B=16384, HalfKAv2_hm lists, 24576-row table), the roofline of the forward kernel from HIP event
-timings, and the reference's CPU path (torch embedding_bag composition) timed on the host cores
-on a bounded sample of the same workload.
+B=16384, HalfKAv2_hm lists, 24576-row table), the roofline of the backward entry point (the dominant
+launch of the step; `roofline_forward` is the forward's) from HIP event timings, and the reference's
+CPU path (torch embedding_bag composition) timed on the host cores on a bounded sample of the same
+workload.
 """
 import argparse
 import json
@@ -22,10 +23,13 @@ sys.path.insert(0, os.path.join(ROOT, "nnue-pytorch_amd"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
-# Bytes that crossed the L2 boundary per call of nnueft_double_fwd (FETCH_SIZE x2.0 + WRITE_SIZE x1.0 summed over
-# its kernels, the scale being what the same counters read for a 1 GiB torch.add):
-# profiles/nnueft_double_fwd_L1_3072_B16384_pmc.txt
-MEASURED_FWD_TRAFFIC = {"ft_fwd_bwd_L1_3072_B16384": 1.48e9}
+# Bytes that crossed the L2 boundary per call of an entry point (FETCH_SIZE x2.0 + WRITE_SIZE x1.0 summed over its
+# kernels, the scale being what the same counters read for a 1 GiB torch.add), uniform positions:
+# profiles/ft_fwd_bwd_L1_3072_B16384_pmc.txt
+MEASURED_TRAFFIC = {
+    ("ft_fwd_bwd_L1_3072_B16384", "forward"): 1.46e9,
+    ("ft_fwd_bwd_L1_3072_B16384", "deterministic"): 2.68e9,
+}
 
 WORKLOADS = {
     # name: (L1, B)
@@ -446,7 +450,8 @@ def main():
 
         from nnueft.sparse_linear_functions import _aux_stream_ptr
 
-        aux_stream = _aux_stream_ptr(dev)      # what FusedDoubleFtFunction passes
+        # the entry point as FusedDoubleFtFunction calls it under this sort placement
+        aux_stream = _aux_stream_ptr(dev) if args.sort_placement == "backward" else None
 
         def bwd_det():
             rc = lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT,
@@ -505,13 +510,28 @@ def main():
             "index_scheme": "HalfKAv2_hm, seeded random positions", "positions": args.positions,
             "sort_placement": args.sort_placement,
         },
-        "roofline": {
+        "roofline_forward": {
             "kernel": "nnueft_double_fwd: k_acc_blocked (the gather, ~3/4 of the time) + k_mix + pair sort",
             "bound": "hbm", "achieved": fwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": fwd_gbs / HBM_PEAK_GBS, "traffic": MEASURED_FWD_TRAFFIC.get(args.workload),
+            "frac": fwd_gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get((args.workload, "forward")),
             "algorithmic_bytes_per_launch": fwd_bytes, "avg_launch_ms": fwd_ms,
         },
     }
+    # the dominant launch of the step is the backward entry point (about two thirds of it); both gathers are
+    # served from L2, so `achieved` (algorithmic bytes) can exceed the HBM peak while `traffic` stays far below
+    if head_mode in bwd_ms:
+        _, bwd_bytes = algorithmic_bytes(L1, B, sum_a, head_mode)
+        bwd_gbs = bwd_bytes / (bwd_ms[head_mode] * 1e-3) / 1e9
+        out["roofline"] = {
+            "kernel": ("nnueft_double_bwd_det: k_seg_reduce (the gather of the upstream rows, ~60 % of the time) + "
+                       "k_bwd_rows + index sort + bias chain") if head_mode == "deterministic"
+            else "nnueft_double_bwd_atomic: k_double_bwd_atomic (+ the zero fill of the dense gradient)",
+            "bound": "hbm", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get((args.workload, head_mode)),
+            "algorithmic_bytes_per_launch": bwd_bytes, "avg_launch_ms": bwd_ms[head_mode],
+        }
+    else:
+        out["roofline"] = out["roofline_forward"]
     step_stats = {}
     for mode in modes:
         if mode not in results:
