@@ -101,11 +101,12 @@ def test_full_model_trains_on_gpu():
     torch.testing.assert_close(a, b, atol=2e-4, rtol=1e-3)
 
 
-@pytest.mark.parametrize("backend", ["aot_eager", "inductor"])
+@pytest.mark.parametrize("backend", ["aot_eager", "inductor", "cudagraphs"])
 def test_model_under_torch_compile_on_gpu(backend):
-    """The reference compiles the model (train.py:296).  The launchers are opaque to dynamo
-    (torch.compiler.disable), so the graph breaks around the HIP kernels and the results are those
-    of the eager module, deterministic backward included."""
+    """The reference compiles the model (train.py:296; "inductor" or "cudagraphs", config.py:63-64).  The
+    launchers are opaque to dynamo (torch.compiler.disable), so the graph breaks around the HIP kernels
+    and the results are those of the eager module, deterministic backward included.  With "cudagraphs"
+    the stretches between the launchers are captured and replayed: four calls, each checked."""
     old = nnueft.get_backward_mode()
     nnueft.set_backward_mode("deterministic")
     try:
@@ -117,7 +118,7 @@ def test_model_under_torch_compile_on_gpu(backend):
         model.zero_grad()
         torch._dynamo.reset()
         cm = torch.compile(model, backend=backend)
-        for _ in range(2):      # second call: the cached graph
+        for _ in range(4 if backend == "cudagraphs" else 2):      # from the second call on: the cached graph
             model.zero_grad()
             o = cm(*batch)
             o.sum().backward()
