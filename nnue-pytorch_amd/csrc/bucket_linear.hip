@@ -284,15 +284,21 @@ __global__ __launch_bounds__(KS * 64) void k_bucket_fwd_lds(const float* __restr
     const float* wb = W + ((size_t)bk * out + (jok ? r : 0)) * in + wave * kw + 4 * h;
     float* strip = lds + wave * kStrip;
     f32x16 acc = {0};
-    for (int k = 0; k < kw; k += CK) {
-        vecf<4> v[8], b[8];
+    // the activations of step k + 1 (from HBM) are requested before the matrix operations of step k;
+    // the weights (L2-resident) are requested at the top of their own step
+    vecf<4> v[8], b[8];
 #pragma unroll
-        for (int it = 0; it < 8; ++it) v[it] = ldv4_stream(xs[it] + k);
+    for (int it = 0; it < 8; ++it) v[it] = ldv4_stream(xs[it]);
+    for (int k = 0; k < kw; k += CK) {
 #pragma unroll
         for (int u = 0; u < 8; ++u) b[u] = ldv<4>(wb + k + 8 * u);
 #pragma unroll
         for (int it = 0; it < 8; ++it) stv<4>(strip + (srow + 4 * it) * LD + scol, v[it]);
         __syncthreads();
+        if (k + CK < kw) {
+#pragma unroll
+            for (int it = 0; it < 8; ++it) v[it] = ldv4_stream(xs[it] + k + CK);
+        }
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const vecf<4> a = ldv<4>(strip + r * LD + 8 * u + 4 * h);
@@ -373,6 +379,10 @@ constexpr int kBwdWaves = 8;
 #ifndef NNUEFT_BWDW_PF
 #define NNUEFT_BWDW_PF 32
 #endif
+#ifndef NNUEFT_BWDW_COLS
+#define NNUEFT_BWDW_COLS 64
+#endif
+constexpr int kBwdCols = NNUEFT_BWDW_COLS;   // 64 or 32 columns per workgroup
 __global__ __launch_bounds__(kBwdWaves * 64) void k_bucket_bwd_w(const float* __restrict__ x,
                                                                  const float* __restrict__ gy,
                                                                  float* __restrict__ gW, float* __restrict__ gbias,
@@ -384,8 +394,8 @@ __global__ __launch_bounds__(kBwdWaves * 64) void k_bucket_bwd_w(const float* __
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
     const uint32_t beg = bucket_off[bk], end = bucket_off[bk + 1];
     const bool ook = r < out;
-    const int c0 = 64 * q + r;
-    const bool c1ok = c0 + 32 < in;
+    const int c0 = kBwdCols * q + r;
+    const bool c1ok = kBwdCols == 64 && c0 + 32 < in;
     f32x16 acc0 = {0}, acc1 = {0};
     float bsum = 0.0f;
     for (uint32_t e0 = beg + 64u * wave; e0 < end; e0 += 64u * kBwdWaves) {
@@ -549,7 +559,7 @@ extern "C" int nnueft_bucket_linear_bwd(const float* x, const int64_t* bucket, c
                            (const uint32_t*)(ws + L.ntiles), (const uint32_t*)(ws + L.tiles), in, out, nsplit);
         NNUEFT_LAUNCH_CHECK();
     }
-    hipLaunchKernelGGL(k_bucket_bwd_w, dim3((in + 63) / 64, count), dim3(kBwdWaves * 64), 0, st, x, gy, gW, gbias,
+    hipLaunchKernelGGL(k_bucket_bwd_w, dim3((in + kBwdCols - 1) / kBwdCols, count), dim3(kBwdWaves * 64), 0, st, x, gy, gW, gbias,
                        order, (const uint32_t*)(ws + L.bucket_off), in, out);
     NNUEFT_LAUNCH_CHECK();
     return 0;

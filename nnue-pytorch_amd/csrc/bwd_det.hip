@@ -26,7 +26,10 @@
 
 namespace {
 
-constexpr int kChunk = 128;        // positions per sort chunk
+#ifndef NNUEFT_SORT_CHUNK
+#define NNUEFT_SORT_CHUNK 128
+#endif
+constexpr int kChunk = NNUEFT_SORT_CHUNK;        // positions per sort chunk
 #ifndef NNUEFT_SEG_U
 #define NNUEFT_SEG_U 8
 #endif
