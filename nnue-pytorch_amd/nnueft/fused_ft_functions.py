@@ -112,10 +112,14 @@ def _launch_double_bwd(us, them, white_indices, black_indices, psqt_indices, bia
 class FusedDoubleFtFunction(autograd.Function):
     @staticmethod
     def forward(ctx, us, them, white_indices, black_indices, psqt_indices, weight, bias, max_ft_activation, l1_size,
-                act_grid=None):
-        """act_grid (not part of the reference's signature): None, or (scale, eps, post_mul): l0 comes out as
-        (floor(l0 * scale + eps) / scale) * post_mul, the activation grid and correction factor that
-        ComposedFeatureTransformer applies next, with a straight-through gradient."""
+                *extra):
+        """The reference's nine arguments, and optionally a tenth, act_grid: None, or (scale, eps, post_mul):
+        l0 then comes out as (floor(l0 * scale + eps) / scale) * post_mul, the activation grid and
+        correction factor that ComposedFeatureTransformer applies next, with a straight-through gradient."""
+        if len(extra) > 1:
+            raise TypeError("FusedDoubleFtFunction takes nine arguments and optionally act_grid")
+        act_grid = extra[0] if extra else None
+        ctx.n_extra = len(extra)
         ctx.act_grid = None if act_grid is None else tuple(float(v) for v in act_grid)
         ctx.max_ft_activation = float(max_ft_activation)
         ctx.l1_size = int(l1_size)
@@ -192,4 +196,4 @@ class FusedDoubleFtFunction(autograd.Function):
                 ctx.sort_placement != "inline",
             )
 
-        return None, None, None, None, None, grad_weight, grad_bias, None, None, None
+        return (None, None, None, None, None, grad_weight, grad_bias, None, None) + (None,) * ctx.n_extra

@@ -300,6 +300,39 @@ def test_sort_placements_give_the_same_bits(oracle_cpu, on_stream):
         nnueft.set_sort_placement("elsewhere")
 
 
+def test_fused_function_with_nine_and_ten_arguments(oracle_cpu):
+    """The reference calls FusedDoubleFtFunction.apply with nine arguments; the tenth (the activation
+    grid applied inside the forward) is this build's.  Both forms differentiate, and the grid is the
+    oracle's, with a straight-through gradient scaled by its post-multiplier."""
+    from nnueft.fused_ft_functions import FusedDoubleFtFunction
+
+    nnueft.set_backward_mode("deterministic")
+    c = double_case(53, 700, 256, 900, binary_side=True)
+    t = {k: torch.from_numpy(c[k]).to(DEV) for k in ("us", "them", "widx", "bidx", "psqt_idx", "W", "bias")}
+    grads = [torch.from_numpy(c[k]).to(DEV) for k in ("g_l0", "g_wp", "g_bp")]
+    got = {}
+    for extra in ((), ((127.0, 1e-5, 0.5),), (None,)):
+        W = t["W"].clone().requires_grad_()
+        bias = t["bias"].clone().requires_grad_()
+        out = FusedDoubleFtFunction.apply(t["us"], t["them"], t["widx"], t["bidx"], t["psqt_idx"], W, bias,
+                                          c["max_act"], 256, *extra)
+        torch.autograd.backward(list(out), grads)
+        got[extra] = (out[0].detach().cpu().numpy(), W.grad.cpu().numpy(), bias.grad.cpu().numpy())
+    plain, grid, none = got[()], got[((127.0, 1e-5, 0.5),)], got[(None,)]
+    for a, b in zip(plain, none):
+        assert np.array_equal(a, b)
+    assert np.array_equal(grid[0], oracle_cpu.act_fake_quantize(plain[0], 127.0, 1e-5, 0.5))
+    # straight-through: the gradient of the plain call with the upstream gradient of l0 halved
+    W = t["W"].clone().requires_grad_()
+    bias = t["bias"].clone().requires_grad_()
+    out = FusedDoubleFtFunction.apply(t["us"], t["them"], t["widx"], t["bidx"], t["psqt_idx"], W, bias, c["max_act"], 256)
+    torch.autograd.backward(list(out), [grads[0] * 0.5, grads[1], grads[2]])
+    assert np.array_equal(grid[1], W.grad.cpu().numpy()) and np.array_equal(grid[2], bias.grad.cpu().numpy())
+    with pytest.raises(TypeError):
+        FusedDoubleFtFunction.apply(t["us"], t["them"], t["widx"], t["bidx"], t["psqt_idx"], W, bias, c["max_act"],
+                                    256, None, None)
+
+
 def test_abi_rejects_bad_arguments():
     lib = _native.load()
     x = torch.zeros(64, device=DEV)
