@@ -253,7 +253,13 @@ __global__ __launch_bounds__(256) void k_chunk_hist(const int32_t* __restrict__ 
     }
     __syncthreads();
     uint32_t* dst = cnt + (size_t)c * R + r0;
-    for (int j = threadIdx.x; j < nr; j += 256) dst[j] = lds_u32[j];
+    if ((R & 3) == 0 && (r0 & 3) == 0 && (nr & 3) == 0) {
+        const uint4* src4 = reinterpret_cast<const uint4*>(lds_u32);
+        uint4* dst4 = reinterpret_cast<uint4*>(dst);
+        for (int j = threadIdx.x; j < (nr >> 2); j += 256) dst4[j] = src4[j];
+    } else {
+        for (int j = threadIdx.x; j < nr; j += 256) dst[j] = lds_u32[j];
+    }
 }
 
 // Per table row: chunk counts -> exclusive offsets; total and white share.
@@ -454,8 +460,32 @@ __global__ __launch_bounds__(256) void k_fill(const int32_t* __restrict__ widx, 
     int pos0, npos, p;
     const int32_t* ix = chunk_indices(widx, bidx, c, cpp, B, K, &pos0, &npos, &p);
     const uint32_t* coff = cnt + (size_t)c * R + r0;
-    {
-        // cursors = segment offset + offset of this chunk inside the segment; loads batched 8 deep
+    // cursors = segment offset + offset of this chunk inside the segment.  The workgroup waits for
+    // every batch of loads, so the batches are made as large as registers allow: four rows per load
+    // where the two arrays are 16-byte aligned, twelve loads of each array in flight per thread.
+    if ((R & 3) == 0 && (r0 & 3) == 0 && (nr & 3) == 0) {
+        constexpr int PF = 12;
+        const uint4* so4 = reinterpret_cast<const uint4*>(seg_off + r0);
+        const uint4* co4 = reinterpret_cast<const uint4*>(coff);
+        uint4* lds4 = reinterpret_cast<uint4*>(lds_u32);
+        const int nr4 = nr >> 2;
+        for (int j0 = threadIdx.x; j0 < nr4; j0 += 256 * PF) {
+            uint4 a[PF], b[PF];
+#pragma unroll
+            for (int u = 0; u < PF; ++u) {
+                const int j = j0 + u * 256;
+                if (j < nr4) {
+                    a[u] = so4[j];
+                    b[u] = co4[j];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < PF; ++u) {
+                const int j = j0 + u * 256;
+                if (j < nr4) lds4[j] = make_uint4(a[u].x + b[u].x, a[u].y + b[u].y, a[u].z + b[u].z, a[u].w + b[u].w);
+            }
+        }
+    } else {
         constexpr int PF = 8;
         for (int j0 = threadIdx.x; j0 < nr; j0 += 256 * PF) {
             uint32_t a[PF], b[PF];
