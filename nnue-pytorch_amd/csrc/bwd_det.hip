@@ -206,7 +206,7 @@ __global__ __launch_bounds__(64) void k_bias_final(const float* __restrict__ par
         for (int i = threadIdx.x; i < kXcd * kSchedQueues; i += 64) sched[kSchedCtr + i * 32] = 0;
     const int c = blockIdx.x * 64 + threadIdx.x;
     if (c >= out_cols) return;
-    constexpr int PF = 32;
+    constexpr int PF = 64;
     float total = 0.0f;
     int t = 0;
     for (; t + PF <= ntiles; t += PF) {
@@ -247,9 +247,14 @@ __global__ __launch_bounds__(256) void k_chunk_hist(const int32_t* __restrict__ 
     for (int j = threadIdx.x; j < nr; j += 256) lds_u32[j] = 0;
     __syncthreads();
     const int nslots = npos * K;
-    for (int i = threadIdx.x; i < nslots; i += 256) {
-        const int r = ix[i] - r0;
-        if (r >= 0 && r < nr) atomicAdd(&lds_u32[r], 1u);
+    constexpr int PF = 16;   // index loads in flight per thread: a chunk of 128 lists of 32 is one batch
+    for (int i0 = threadIdx.x; i0 < nslots; i0 += 256 * PF) {
+        int rr[PF];
+#pragma unroll
+        for (int u = 0; u < PF; ++u) rr[u] = i0 + u * 256 < nslots ? ix[i0 + u * 256] - r0 : -1;
+#pragma unroll
+        for (int u = 0; u < PF; ++u)
+            if (rr[u] >= 0 && rr[u] < nr) atomicAdd(&lds_u32[rr[u]], 1u);
     }
     __syncthreads();
     uint32_t* dst = cnt + (size_t)c * R + r0;
@@ -356,13 +361,14 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
     __syncthreads();
     for (int base = 0; base < R; base += cap) {
         const int n = min(cap, R - base);
-        // coalesced loads, 8 in flight per thread
-        for (int i0 = tid; i0 < n; i0 += kScanThreads * 8) {
-            uint32_t v[8];
+        // coalesced loads, 24 in flight per thread (a 24 576-row table is one batch)
+        constexpr int PFS = 24;
+        for (int i0 = tid; i0 < n; i0 += kScanThreads * PFS) {
+            uint32_t v[PFS];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = (i0 + u * kScanThreads < n) ? seg_off[base + i0 + u * kScanThreads] : 0;
+            for (int u = 0; u < PFS; ++u) v[u] = (i0 + u * kScanThreads < n) ? seg_off[base + i0 + u * kScanThreads] : 0;
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
+            for (int u = 0; u < PFS; ++u)
                 if (i0 + u * kScanThreads < n) stage[i0 + u * kScanThreads] = v[u];
         }
         __syncthreads();
