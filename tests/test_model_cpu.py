@@ -246,3 +246,11 @@ def test_bucket_linear_oracle_equals_wide_layer_and_selection(oracle_cpu, B, n_i
     assert np.allclose(gx, tx.grad.numpy(), rtol=1e-5, atol=1e-5)
     assert np.allclose(gW, tW.grad.numpy(), rtol=1e-5, atol=1e-5)
     assert np.allclose(gb, tb.grad.numpy(), rtol=1e-5, atol=1e-5)
+
+
+def test_synthetic_training_loop_on_cpu():
+    """The thin loop (host batches -> prefetcher -> model -> loss -> RangerLite) on the CPU path."""
+    from nnueft import train_synthetic
+
+    losses, rate = train_synthetic.run(steps=14, batch_size=256, l1=64, device="cpu", lr=2e-3)
+    assert len(losses) == 14 and all(np.isfinite(losses)) and losses[-1] < losses[0] and rate > 0
