@@ -328,6 +328,32 @@ int nnueft_ranger_lite_update_adam(float* p, const float* grad, float* grad_ma, 
                                    float beta1, float one_minus_beta1, float lr_div_bc1, float eps,
                                    float wd_factor, int update_variance, float* lookahead_params,
                                    float lookahead_alpha, void* stream);
+/*
+ * The same update for several tensors in one launch (a launch costs a few microseconds whatever the
+ * tensor's size, and a model has many small ones).  `tensors` is a host array of `count` records,
+ * copied into the kernel's arguments 16 at a time; every record carries its own hyperparameters, since
+ * parameter groups may differ.  neg_grad_ma == NULL selects the plain first moment (beta1,
+ * one_minus_beta1 as in nnueft_ranger_lite_update_adam), otherwise the pair (beta1 = beta1^2,
+ * one_minus_beta1 = 1 - beta1^2; odd_step = step & 1).  Element for element the arithmetic of the
+ * single-tensor entry points.
+ */
+typedef struct nnueft_ranger_args {
+    float* p;
+    const float* grad;
+    float* grad_ma;
+    float* neg_grad_ma;
+    float* variance_ma;
+    float* lookahead_params;   /* NULL: no lookahead merge in this call */
+    long long n;
+    float beta2, one_minus_beta2, bias_correction2;
+    float beta1, one_minus_beta1;
+    float one_plus_pnm, pnm_factor, noise_norm;
+    float lr_div_bc1, eps, wd_factor, lookahead_alpha, one_minus_lookahead_alpha;
+    int odd_step;
+    int update_variance;
+} nnueft_ranger_args;
+int nnueft_ranger_lite_update_multi(const nnueft_ranger_args* tensors, int count, void* stream);
+
 int nnueft_ranger_lite_update_variance(const float* grad, float* variance_ma, long long n, float beta2,
                                        float one_minus_beta2, void* stream);
 int nnueft_ranger_lite_lookahead_merge(float* p, float* lookahead_params, long long n, float alpha,

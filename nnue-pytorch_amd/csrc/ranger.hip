@@ -7,21 +7,8 @@
 
 namespace {
 
-struct RangerArgs {
-    float* p;
-    const float* grad;
-    float* grad_ma;
-    float* neg_grad_ma;     // null: plain first moment
-    float* variance_ma;
-    float* slow;            // null: no lookahead merge in this call
-    long long n;
-    float beta2, one_minus_beta2, bias_correction2;
-    float beta1, one_minus_beta1;          // for the pair: beta1^2 and 1 - beta1^2
-    float one_plus_pnm, pnm_factor, noise_norm;
-    float lr_div_bc1, eps, wd_factor, alpha, one_minus_alpha;
-    int odd_step;           // the pair: which buffer is the positive one this step
-    int update_variance;    // 0: variance_ma was updated before (two-phase step)
-};
+// One tensor's update; the layout is the public nnueft_ranger_args of the header.
+typedef nnueft_ranger_args RangerArgs;
 
 __device__ __forceinline__ void ranger_one(const RangerArgs& a, float& p, float g, float& gm, float& ngm, float& vm,
                                            float& slow) {
@@ -42,8 +29,8 @@ __device__ __forceinline__ void ranger_one(const RangerArgs& a, float& p, float 
     float np = p;
     if (a.wd_factor != 0.0f) np = np * (1.0f - a.wd_factor);
     np = np - a.lr_div_bc1 * (dir / denom);
-    if (a.slow) {
-        np = np * a.alpha + slow * a.one_minus_alpha;
+    if (a.lookahead_params) {
+        np = np * a.lookahead_alpha + slow * a.one_minus_lookahead_alpha;
         slow = np;
     }
     p = np;
@@ -58,7 +45,7 @@ __global__ __launch_bounds__(256) void k_ranger_update(RangerArgs a) {
         vecf<VW> p = ldv<VW>(a.p + o), g = ldv<VW>(a.grad + o), gm = ldv<VW>(a.grad_ma + o);
         vecf<VW> vm = ldv<VW>(a.variance_ma + o);
         vecf<VW> ngm = a.neg_grad_ma ? ldv<VW>(a.neg_grad_ma + o) : vzero<VW>();
-        vecf<VW> slow = a.slow ? ldv<VW>(a.slow + o) : vzero<VW>();
+        vecf<VW> slow = a.lookahead_params ? ldv<VW>(a.lookahead_params + o) : vzero<VW>();
 #pragma unroll
         for (int k = 0; k < VW; ++k) ranger_one(a, p.v[k], g.v[k], gm.v[k], ngm.v[k], vm.v[k], slow.v[k]);
         stv<VW>(a.p + o, p);
@@ -70,22 +57,48 @@ __global__ __launch_bounds__(256) void k_ranger_update(RangerArgs a) {
         } else {
             stv<VW>(a.grad_ma + o, gm);
         }
-        if (a.slow) stv<VW>(a.slow + o, slow);
+        if (a.lookahead_params) stv<VW>(a.lookahead_params + o, slow);
     }
     if (VW > 1) {
         // tail of fewer than VW elements
         const long long i = nvec * VW + (long long)blockIdx.x * 256 + threadIdx.x;
         if (i < a.n) {
-            float ngm = a.neg_grad_ma ? a.neg_grad_ma[i] : 0.0f, slow = a.slow ? a.slow[i] : 0.0f;
+            float ngm = a.neg_grad_ma ? a.neg_grad_ma[i] : 0.0f, slow = a.lookahead_params ? a.lookahead_params[i] : 0.0f;
             float p = a.p[i], gm = a.grad_ma[i], vm = a.variance_ma[i];
             ranger_one(a, p, a.grad[i], gm, ngm, vm, slow);
             a.p[i] = p;
             if (a.update_variance) a.variance_ma[i] = vm;
             if (a.neg_grad_ma && !a.odd_step) a.neg_grad_ma[i] = ngm;
             else a.grad_ma[i] = gm;
-            if (a.slow) a.slow[i] = slow;
+            if (a.lookahead_params) a.lookahead_params[i] = slow;
         }
     }
+}
+
+// Several small tensors in one launch: workgroup -> tensor through the running count of workgroups,
+// then one element per thread.  A launch costs a few microseconds whatever the tensor's size, and a
+// model has many small tensors (biases, the layers of the stacks).
+constexpr int kMultiMax = 16;
+struct RangerMulti {
+    RangerArgs t[kMultiMax];
+    unsigned first[kMultiMax + 1];   // first workgroup of every tensor
+    int count;
+};
+
+__global__ __launch_bounds__(256) void k_ranger_update_multi(RangerMulti m) {
+    int k = 0;
+    while (k + 1 < m.count && blockIdx.x >= m.first[k + 1]) ++k;
+    const RangerArgs& a = m.t[k];
+    const long long i = (long long)(blockIdx.x - m.first[k]) * 256 + threadIdx.x;
+    if (i >= a.n) return;
+    float ngm = a.neg_grad_ma ? a.neg_grad_ma[i] : 0.0f, slow = a.lookahead_params ? a.lookahead_params[i] : 0.0f;
+    float p = a.p[i], gm = a.grad_ma[i], vm = a.variance_ma[i];
+    ranger_one(a, p, a.grad[i], gm, ngm, vm, slow);
+    a.p[i] = p;
+    if (a.update_variance) a.variance_ma[i] = vm;
+    if (a.neg_grad_ma && !a.odd_step) a.neg_grad_ma[i] = ngm;
+    else a.grad_ma[i] = gm;
+    if (a.lookahead_params) a.lookahead_params[i] = slow;
 }
 
 template <int VW>
@@ -140,7 +153,7 @@ int launch_update(RangerArgs a, hipStream_t st) {
     if (a.n <= 0) return NNUEFT_E_ARG;
     if (!a.p || !a.grad || !a.grad_ma || !a.variance_ma) return NNUEFT_E_ARG;
     const bool vec = aligned16(a.p) && aligned16(a.grad) && aligned16(a.grad_ma) && aligned16(a.variance_ma) &&
-                     (!a.neg_grad_ma || aligned16(a.neg_grad_ma)) && (!a.slow || aligned16(a.slow)) && a.n >= 4;
+                     (!a.neg_grad_ma || aligned16(a.neg_grad_ma)) && (!a.lookahead_params || aligned16(a.lookahead_params)) && a.n >= 4;
     if (vec) hipLaunchKernelGGL(k_ranger_update<4>, dim3(grid_for(a.n / 4)), dim3(256), 0, st, a);
     else hipLaunchKernelGGL(k_ranger_update<1>, dim3(grid_for(a.n)), dim3(256), 0, st, a);
     NNUEFT_LAUNCH_CHECK();
@@ -159,12 +172,12 @@ extern "C" int nnueft_ranger_lite_update_pnm(float* p, const float* grad, float*
     if (!neg_grad_ma) return NNUEFT_E_ARG;
     RangerArgs a{};
     a.p = p; a.grad = grad; a.grad_ma = grad_ma; a.neg_grad_ma = neg_grad_ma; a.variance_ma = variance_ma;
-    a.slow = lookahead_params; a.n = n;
+    a.lookahead_params = lookahead_params; a.n = n;
     a.beta2 = beta2; a.one_minus_beta2 = one_minus_beta2; a.bias_correction2 = bias_correction2;
     a.beta1 = beta1_sq; a.one_minus_beta1 = one_minus_beta1_sq;
     a.one_plus_pnm = one_plus_pnm; a.pnm_factor = pnm_factor; a.noise_norm = noise_norm;
     a.lr_div_bc1 = lr_div_bc1; a.eps = eps; a.wd_factor = wd_factor;
-    a.alpha = lookahead_alpha; a.one_minus_alpha = 1.0f - lookahead_alpha;
+    a.lookahead_alpha = lookahead_alpha; a.one_minus_lookahead_alpha = 1.0f - lookahead_alpha;
     a.odd_step = (int)(step & 1LL); a.update_variance = update_variance != 0;
     return launch_update(a, (hipStream_t)stream);
 }
@@ -176,13 +189,36 @@ extern "C" int nnueft_ranger_lite_update_adam(float* p, const float* grad, float
                                               float lookahead_alpha, void* stream) {
     RangerArgs a{};
     a.p = p; a.grad = grad; a.grad_ma = grad_ma; a.neg_grad_ma = nullptr; a.variance_ma = variance_ma;
-    a.slow = lookahead_params; a.n = n;
+    a.lookahead_params = lookahead_params; a.n = n;
     a.beta2 = beta2; a.one_minus_beta2 = one_minus_beta2; a.bias_correction2 = bias_correction2;
     a.beta1 = beta1; a.one_minus_beta1 = one_minus_beta1;
     a.lr_div_bc1 = lr_div_bc1; a.eps = eps; a.wd_factor = wd_factor;
-    a.alpha = lookahead_alpha; a.one_minus_alpha = 1.0f - lookahead_alpha;
+    a.lookahead_alpha = lookahead_alpha; a.one_minus_lookahead_alpha = 1.0f - lookahead_alpha;
     a.update_variance = update_variance != 0;
     return launch_update(a, (hipStream_t)stream);
+}
+
+extern "C" int nnueft_ranger_lite_update_multi(const nnueft_ranger_args* tensors, int count, void* stream) {
+    if (count <= 0 || !tensors) return NNUEFT_E_ARG;
+    for (int i = 0; i < count; ++i) {
+        const nnueft_ranger_args& a = tensors[i];
+        if (a.n <= 0 || !a.p || !a.grad || !a.grad_ma || !a.variance_ma) return NNUEFT_E_ARG;
+        if ((a.n + 255) / 256 > 0x0fffffffLL) return NNUEFT_E_UNSUPPORTED;
+    }
+    for (int i0 = 0; i0 < count; i0 += kMultiMax) {
+        RangerMulti m{};
+        m.count = min(kMultiMax, count - i0);
+        unsigned blocks = 0;
+        for (int k = 0; k < m.count; ++k) {
+            m.t[k] = tensors[i0 + k];
+            m.first[k] = blocks;
+            blocks += (unsigned)((m.t[k].n + 255) / 256);
+        }
+        m.first[m.count] = blocks;
+        hipLaunchKernelGGL(k_ranger_update_multi, dim3(blocks), dim3(256), 0, (hipStream_t)stream, m);
+        NNUEFT_LAUNCH_CHECK();
+    }
+    return 0;
 }
 
 extern "C" int nnueft_ranger_lite_update_variance(const float* grad, float* variance_ma, long long n, float beta2,

@@ -12,6 +12,17 @@ _PKG = os.path.dirname(os.path.abspath(__file__))
 # NNUEFT_LIBRARY points at another build of the same library (kernel tuning)
 LIB_PATH = os.environ.get("NNUEFT_LIBRARY") or os.path.join(_PKG, "libnnueft.so")
 
+class RangerArgs(ctypes.Structure):
+    """nnueft_ranger_args of the header, field for field."""
+
+    _fields_ = [(n, c_void_p) for n in ("p", "grad", "grad_ma", "neg_grad_ma", "variance_ma", "lookahead_params")] + \
+               [("n", c_longlong)] + \
+               [(n, c_float) for n in ("beta2", "one_minus_beta2", "bias_correction2", "beta1", "one_minus_beta1",
+                                       "one_plus_pnm", "pnm_factor", "noise_norm", "lr_div_bc1", "eps", "wd_factor",
+                                       "lookahead_alpha", "one_minus_lookahead_alpha")] + \
+               [("odd_step", c_int), ("update_variance", c_int)]
+
+
 # name -> (restype, argtypes); mirrors include/nnueft.h one to one
 PROTOTYPES = {
     "nnueft_version": (c_int, []),
@@ -63,6 +74,7 @@ PROTOTYPES = {
     "nnueft_ranger_lite_update_adam": (
         c_int, [c_void_p] * 4 + [c_longlong] + [c_float] * 7 + [c_float, c_int, c_void_p, c_float, c_void_p],
     ),
+    "nnueft_ranger_lite_update_multi": (c_int, [ctypes.POINTER(RangerArgs), c_int, c_void_p]),
     "nnueft_ranger_lite_update_variance": (c_int, [c_void_p] * 2 + [c_longlong] + [c_float] * 2 + [c_void_p]),
     "nnueft_ranger_lite_lookahead_merge": (c_int, [c_void_p] * 2 + [c_longlong, c_float, c_void_p]),
 }

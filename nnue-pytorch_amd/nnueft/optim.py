@@ -24,6 +24,8 @@ from .sparse_linear_functions import _stream_ptr
 
 
 class RangerLite(torch.optim.Optimizer):
+    MULTI_TENSOR_BELOW = 1 << 20      # elements; smaller tensors are updated several per launch
+
     def __init__(self, params, lr=1.0, weight_decay=0.0, betas=(0.9, 0.999), eps=1e-7, pnm_activate=True,
                  pnm_momentum=1.0, lookahead_active=True, lookahead_mergetime=5, lookahead_blending_alpha=0.5,
                  normloss_active=True, normloss_factor=1e-4, use_legacy_scoping_bug=False):
@@ -124,6 +126,8 @@ class RangerLite(torch.optim.Optimizer):
                 self.lookahead_step = 0
                 merge = True
 
+        # tensors below this size share launches (a launch costs a few microseconds whatever the size)
+        small = {}
         for p, group in active:
             state = self.state[p]
             beta1, beta2 = group["betas"]
@@ -132,6 +136,28 @@ class RangerLite(torch.optim.Optimizer):
             wd_factor = decay * lr / variance_norm if (decay and variance_norm is not None) else 0.0
             bc2 = 1.0 - beta2 ** step
             slow = state["lookahead_params"].data_ptr() if merge else None
+            if p.numel() < self.MULTI_TENSOR_BELOW:
+                a = _native.RangerArgs()
+                a.p, a.grad, a.grad_ma = p.data_ptr(), p.grad.data_ptr(), state["grad_ma"].data_ptr()
+                a.variance_ma, a.lookahead_params, a.n = state["variance_ma"].data_ptr(), slow, p.numel()
+                a.beta2, a.one_minus_beta2, a.bias_correction2 = beta2, 1.0 - beta2, bc2
+                a.eps, a.wd_factor = eps, wd_factor
+                a.lookahead_alpha, a.one_minus_lookahead_alpha = self.lookahead_alpha, 1.0 - self.lookahead_alpha
+                a.update_variance = 0 if needs_norm else 1
+                if self.pnm_active:
+                    pnm = group["pnm_momentum"]
+                    a.neg_grad_ma = state["neg_grad_ma"].data_ptr()
+                    a.beta1, a.one_minus_beta1 = beta1 * beta1, 1.0 - beta1 * beta1
+                    a.one_plus_pnm, a.pnm_factor = 1.0 + pnm, pnm
+                    a.noise_norm = math.sqrt((1.0 + pnm) ** 2 + pnm ** 2)
+                    a.lr_div_bc1 = lr / (1.0 - beta1 ** (((step + 1) // 2) * 2))
+                    a.odd_step = step & 1
+                else:
+                    a.neg_grad_ma = None
+                    a.beta1, a.one_minus_beta1 = beta1, 1.0 - beta1
+                    a.lr_div_bc1 = lr / (1.0 - beta1 ** step)
+                small.setdefault(p.device, []).append(a)
+                continue
             with torch.cuda.device(p.device):
                 if self.pnm_active:
                     pnm = group["pnm_momentum"]
@@ -149,6 +175,11 @@ class RangerLite(torch.optim.Optimizer):
                         p.numel(), beta2, 1.0 - beta2, bc2, beta1, 1.0 - beta1, lr / bc1, eps, wd_factor,
                         0 if needs_norm else 1, slow, self.lookahead_alpha, _stream_ptr(p.device))
                     _native.check(rc, "nnueft_ranger_lite_update_adam")
+        for device, records in small.items():
+            arr = (_native.RangerArgs * len(records))(*records)
+            with torch.cuda.device(device):
+                rc = lib.nnueft_ranger_lite_update_multi(arr, len(records), _stream_ptr(device))
+            _native.check(rc, "nnueft_ranger_lite_update_multi")
 
     def _step_torch(self):
         """The reference's Python path (ranger_lite.py:589-735) in torch ops."""

@@ -117,3 +117,30 @@ def test_class_on_gpu_follows_its_cpu_path(kw):
         if "lookahead_params" in oc.state[a]:
             torch.testing.assert_close(b.detach().cpu(), oc.state[a]["lookahead_params"], rtol=2e-5, atol=2e-6)
     og.train()
+
+
+@pytest.mark.parametrize("kw", [dict(), dict(pnm_activate=False), dict(weight_decay=0.05)], ids=["default", "adam", "decay"])
+def test_multi_tensor_launch_gives_the_bits_of_single_launches(kw):
+    """Small tensors are updated several per launch; the arithmetic per element is the same, so two
+    optimizers that differ only in that threshold stay equal bit for bit (20 tensors: two launches)."""
+    g0 = torch.Generator().manual_seed(5)
+    shapes = [(257,), (3, 70), (1,), (64, 33)] * 5
+    one = [torch.nn.Parameter(torch.randn(*s, generator=g0).to(DEV)) for s in shapes]
+    many = [torch.nn.Parameter(p.detach().clone()) for p in one]
+    wd = kw.pop("weight_decay", 0.0)
+    groups = lambda ps: [{"params": ps[:7], "lr": 1e-2, "weight_decay": wd}, {"params": ps[7:], "lr": 3e-3, "betas": (0.8, 0.99)}]
+    o1 = RangerLite(groups(one), normloss_active=False, **kw)
+    o1.MULTI_TENSOR_BELOW = 0
+    o2 = RangerLite(groups(many), normloss_active=False, **kw)
+    for s in range(7):
+        gen = torch.Generator().manual_seed(200 + s)
+        for a, b in zip(one, many):
+            a.grad = torch.randn(a.shape, generator=gen).to(DEV)
+            b.grad = a.grad.clone()
+        o1.step()
+        o2.step()
+    for a, b in zip(one, many):
+        assert torch.equal(a, b)
+        for key, x in o1.state[a].items():
+            if torch.is_tensor(x):
+                assert torch.equal(x, o2.state[b][key])
