@@ -20,8 +20,11 @@ constexpr int kOrderThreads = 1024;
 constexpr int kTile = 32;
 constexpr int kMaxCount = 64;
 
+constexpr size_t kPartialBytes = 1 << 20;   // partial weight gradients of narrow layers (k_bucket_bwd_w in splits)
+constexpr int kBwdSplits = 8;
+
 struct BucketLayout {
-    size_t order, bucket_off, ntiles, tiles, end;
+    size_t order, bucket_off, ntiles, tiles, partial, end;
     int max_tiles;
 };
 
@@ -39,6 +42,8 @@ bool bucket_layout(int B, int count, BucketLayout* L) {
     off += 256;
     L->tiles = off;
     off += up256((size_t)L->max_tiles * 2 * sizeof(uint32_t));
+    L->partial = off;
+    off += kPartialBytes;
     L->end = off;
     return true;
 }
@@ -388,9 +393,14 @@ __global__ __launch_bounds__(kBwdWaves * 64) void k_bucket_bwd_w(const float* __
                                                                  float* __restrict__ gW, float* __restrict__ gbias,
                                                                  const uint32_t* __restrict__ order,
                                                                  const uint32_t* __restrict__ bucket_off, int in,
-                                                                 int out) {
+                                                                 int out, int nsplit, int rows_total) {
+    // nsplit > 1: workgroup z takes every nsplit-th group of kBwdWaves runs and writes its sums to
+    // gW + z * rows_total * in (gbias + z * rows_total): partial results that k_bucket_bwd_w_sum adds up
+    // in the order of z.  A narrow layer has too few (bucket, column block) pairs to fill the chip.
     __shared__ float red[(kBwdWaves - 1) * 33 * 64];
-    const int bk = blockIdx.y, q = blockIdx.x;
+    const int bk = blockIdx.y, q = blockIdx.x, z = blockIdx.z;
+    gW += (size_t)z * rows_total * in;
+    gbias += (size_t)z * rows_total;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
     const uint32_t beg = bucket_off[bk], end = bucket_off[bk + 1];
     const bool ook = r < out;
@@ -398,7 +408,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void k_bucket_bwd_w(const float* __
     const bool c1ok = kBwdCols == 64 && c0 + 32 < in;
     f32x16 acc0 = {0}, acc1 = {0};
     float bsum = 0.0f;
-    for (uint32_t e0 = beg + 64u * wave; e0 < end; e0 += 64u * kBwdWaves) {
+    for (uint32_t e0 = beg + 64u * (uint32_t)(z * kBwdWaves + wave); e0 < end; e0 += 64u * kBwdWaves * (uint32_t)nsplit) {
         const uint32_t mine = e0 + lane < end ? order[e0 + lane] : 0xffffffffu;
         constexpr int PF = NNUEFT_BWDW_PF;
 #pragma unroll
@@ -458,6 +468,28 @@ __global__ __launch_bounds__(kBwdWaves * 64) void k_bucket_bwd_w(const float* __
         // even-position sums sit in lanes 0-31, odd ones in lanes 32-63
         const float other = __shfl_xor(bsum, 32);
         if (h == 0 && ook) gbias[bk * out + r] = bsum + other;
+    }
+}
+
+// gW[i] = chain over the splits of part[z, i], likewise gbias; one thread per element.
+__global__ __launch_bounds__(256) void k_bucket_bwd_w_sum(const float* __restrict__ part_w,
+                                                          const float* __restrict__ part_b, float* __restrict__ gW,
+                                                          float* __restrict__ gbias, int nw, int nb, int nsplit) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < nw) {
+        float v[kBwdSplits];
+#pragma unroll
+        for (int z = 0; z < kBwdSplits; ++z) v[z] = z < nsplit ? part_w[(size_t)z * nw + i] : 0.0f;
+        float t = v[0];
+#pragma unroll
+        for (int z = 1; z < kBwdSplits; ++z)
+            if (z < nsplit) t = t + v[z];
+        gW[i] = t;
+    } else if (i - nw < nb) {
+        const int j = i - nw;
+        float t = part_b[j];
+        for (int z = 1; z < nsplit; ++z) t = t + part_b[(size_t)z * nb + j];
+        gbias[j] = t;
     }
 }
 
@@ -559,8 +591,24 @@ extern "C" int nnueft_bucket_linear_bwd(const float* x, const int64_t* bucket, c
                            (const uint32_t*)(ws + L.ntiles), (const uint32_t*)(ws + L.tiles), in, out, nsplit);
         NNUEFT_LAUNCH_CHECK();
     }
-    hipLaunchKernelGGL(k_bucket_bwd_w, dim3((in + kBwdCols - 1) / kBwdCols, count), dim3(kBwdWaves * 64), 0, st, x, gy, gW, gbias,
-                       order, (const uint32_t*)(ws + L.bucket_off), in, out);
+    const int colblocks = (in + kBwdCols - 1) / kBwdCols;
+    const int rows_total = count * out;
+    const size_t part_floats = (size_t)kBwdSplits * rows_total * ((size_t)in + 1);
+    if (colblocks * count < 128 && part_floats * sizeof(float) <= kPartialBytes) {
+        // narrow layer: eight workgroups per (bucket, column block), partial sums, then their chain
+        float* part_w = (float*)(ws + L.partial);
+        float* part_b = part_w + (size_t)kBwdSplits * rows_total * in;
+        hipLaunchKernelGGL(k_bucket_bwd_w, dim3(colblocks, count, kBwdSplits), dim3(kBwdWaves * 64), 0, st, x, gy, part_w,
+                           part_b, order, (const uint32_t*)(ws + L.bucket_off), in, out, kBwdSplits, rows_total);
+        NNUEFT_LAUNCH_CHECK();
+        const int nw = rows_total * in, nb = rows_total;
+        hipLaunchKernelGGL(k_bucket_bwd_w_sum, dim3((nw + nb + 255) / 256), dim3(256), 0, st, part_w, part_b, gW, gbias,
+                           nw, nb, kBwdSplits);
+        NNUEFT_LAUNCH_CHECK();
+        return 0;
+    }
+    hipLaunchKernelGGL(k_bucket_bwd_w, dim3(colblocks, count, 1), dim3(kBwdWaves * 64), 0, st, x, gy, gW, gbias, order,
+                       (const uint32_t*)(ws + L.bucket_off), in, out, 1, rows_total);
     NNUEFT_LAUNCH_CHECK();
     return 0;
 }
