@@ -20,7 +20,7 @@ constexpr int kOrderThreads = 1024;
 constexpr int kTile = 32;
 constexpr int kMaxCount = 64;
 
-constexpr size_t kPartialBytes = 1 << 20;   // partial weight gradients of narrow layers (k_bucket_bwd_w in splits)
+constexpr size_t kPartialBytes = 8 << 20;   // partial weight gradients of narrow layers (k_bucket_bwd_w in splits)
 constexpr int kBwdSplits = 8;
 
 struct BucketLayout {
@@ -387,6 +387,9 @@ constexpr int kBwdWaves = 8;
 #ifndef NNUEFT_BWDW_COLS
 #define NNUEFT_BWDW_COLS 64
 #endif
+#ifndef NNUEFT_BWDW_WIDE_SPLITS
+#define NNUEFT_BWDW_WIDE_SPLITS 2
+#endif
 constexpr int kBwdCols = NNUEFT_BWDW_COLS;   // 64 or 32 columns per workgroup
 __global__ __launch_bounds__(kBwdWaves * 64) void k_bucket_bwd_w(const float* __restrict__ x,
                                                                  const float* __restrict__ gy,
@@ -593,17 +596,19 @@ extern "C" int nnueft_bucket_linear_bwd(const float* x, const int64_t* bucket, c
     }
     const int colblocks = (in + kBwdCols - 1) / kBwdCols;
     const int rows_total = count * out;
-    const size_t part_floats = (size_t)kBwdSplits * rows_total * ((size_t)in + 1);
-    if (colblocks * count < 128 && part_floats * sizeof(float) <= kPartialBytes) {
-        // narrow layer: eight workgroups per (bucket, column block), partial sums, then their chain
+    // too few (bucket, column block) pairs to fill the chip: several workgroups per pair, partial sums,
+    // then their chain
+    int nsplit = colblocks * count < 128 ? kBwdSplits : (colblocks * count < 1024 ? NNUEFT_BWDW_WIDE_SPLITS : 1);
+    while (nsplit > 1 && (size_t)nsplit * rows_total * ((size_t)in + 1) * sizeof(float) > kPartialBytes) nsplit >>= 1;
+    if (nsplit > 1) {
         float* part_w = (float*)(ws + L.partial);
-        float* part_b = part_w + (size_t)kBwdSplits * rows_total * in;
-        hipLaunchKernelGGL(k_bucket_bwd_w, dim3(colblocks, count, kBwdSplits), dim3(kBwdWaves * 64), 0, st, x, gy, part_w,
-                           part_b, order, (const uint32_t*)(ws + L.bucket_off), in, out, kBwdSplits, rows_total);
+        float* part_b = part_w + (size_t)nsplit * rows_total * in;
+        hipLaunchKernelGGL(k_bucket_bwd_w, dim3(colblocks, count, nsplit), dim3(kBwdWaves * 64), 0, st, x, gy, part_w,
+                           part_b, order, (const uint32_t*)(ws + L.bucket_off), in, out, nsplit, rows_total);
         NNUEFT_LAUNCH_CHECK();
         const int nw = rows_total * in, nb = rows_total;
         hipLaunchKernelGGL(k_bucket_bwd_w_sum, dim3((nw + nb + 255) / 256), dim3(256), 0, st, part_w, part_b, gW, gbias,
-                           nw, nb, kBwdSplits);
+                           nw, nb, nsplit);
         NNUEFT_LAUNCH_CHECK();
         return 0;
     }
