@@ -462,9 +462,23 @@ class ComposedFeatureTransformer(nn.Module):
                                     q.fake_quantize_weights(merged[:, self.l1_size:], "ft_psqt_weight")], dim=1)
         b = self.bias[:self.l1_size]
         if fake_quantize_weights:
-            b = q.fake_quantize_weights(b, "ft_bias")
-        bias = torch.cat([b, torch.zeros_like(self.bias[self.l1_size:], dtype=b.dtype)], dim=0)
+            if b.is_cuda and b.dtype == torch.float32 and _native.available():
+                # one launch instead of the five elementwise ops of fake_quantize_weights (same bits)
+                s = q.weight_scales_dict["ft_bias"]
+                b = _table_merge(b.view(1, -1), None, self.l1_size, s, s, True).view(-1)
+            else:
+                b = q.fake_quantize_weights(b, "ft_bias")
+        bias = torch.cat([b, self._psqt_bias_zeros(b)], dim=0)
         return merged, bias
+
+    def _psqt_bias_zeros(self, like):
+        """The PSQT part of the bias is held at zero; the zeros are made once per device and dtype."""
+        n = self.bias.shape[0] - self.l1_size
+        z = getattr(self, "_zeros_cache", None)
+        if z is None or z.device != like.device or z.dtype != like.dtype or z.shape[0] != n:
+            z = torch.zeros(n, dtype=like.dtype, device=like.device)
+            object.__setattr__(self, "_zeros_cache", z)     # not a parameter, not a buffer, not in the state dict
+        return z
 
     @torch.no_grad()
     def coalesce(self):
