@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # profiles/ft_fwd_bwd_L1_3072_B16384_pmc.txt
 MEASURED_TRAFFIC = {
     ("ft_fwd_bwd_L1_3072_B16384", "forward"): 1.46e9,
-    ("ft_fwd_bwd_L1_3072_B16384", "deterministic"): 2.68e9,
+    ("ft_fwd_bwd_L1_3072_B16384", "deterministic"): 2.69e9,
 }
 
 WORKLOADS = {
