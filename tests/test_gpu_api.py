@@ -346,6 +346,21 @@ def test_abi_rejects_bad_arguments():
     assert lib.nnueft_sparse_bwd_det(p, p, p, p, 4, 8, 10, 8, 0, 1 << 20, st) == -2  # workspace missing
     assert lib.nnueft_sparse_bwd_det(p, p, p, p, 4, 8, 10, 8, p + 4, 1 << 20, st) == -2  # misaligned
     assert lib.nnueft_ft_int16_fwd(p, p, p, p, p, p, p, p, p, 4, 8, 10, 8, 8, 70000, 9, 0, None, 0, st) == -1   # clip_max
+    # the entry points around the operator reject what they cannot run, before any launch
+    assert lib.nnueft_det_sort(p, p, 4, 8, 10, 8, 2, p, 16, st) == -2                # sorted block too small
+    assert lib.nnueft_det_sort(p, p, 4, 8, 10, 8, 2, p + 4, 1 << 20, st) == -2       # misaligned
+    assert lib.nnueft_det_sort(p, None, 4, 8, 10, 8, 2, p, 1 << 20, st) == -1        # two lists asked, one given
+    assert lib.nnueft_det_sort_bytes(4, 8, 10, 8, 3) == 0                            # one or two perspectives
+    assert lib.nnueft_double_bwd_det(p, p, p, p, p, p, 1.0, p, p, p, p, p, p, 4, 8, 10, 8, 0, p, 1 << 30, p + 4, st,
+                                     None) == -2                                      # sorted lists misaligned
+    assert lib.nnueft_ranger_lite_update_multi(None, 0, st) == -1
+    assert lib.nnueft_sqr_crelu_fwd(p, p, p, 4, 1, 127.0, 1e-5, 1.0, 1.0, 1, st) == -1     # skip value needs 2 columns
+    assert lib.nnueft_sqr_crelu_fwd(p, p, None, 4, 4, 0.0, 1e-5, 1.0, 1.0, 1, st) == -1    # grid without a scale
+    assert lib.nnueft_stack_output_fwd(p, p, p, p, p, p, 4, 0, 600, 1, st) == -1           # output grid without den
+    assert lib.nnueft_sf_loss_fwd(p, p, p, p, p, p, 4, 270.0, 0.0, 270.0, 380.0, 2.5, 0.0, 0.0, 0.5, 4000.0, 4000.0,
+                                  0.85, 1.0, st) == -1                                # scaling must be positive
+    assert lib.nnueft_batch_unpack(p, p, p, None, 4, st) == -1
+    assert lib.nnueft_bucket_linear_fwd(p, p, p, p, p, 4, 48, 8, 8, p, 1 << 30, 0, st) == -3   # in % 32 != 0
     with pytest.raises(RuntimeError, match="invalid argument"):
         _native.check(-1, "x")
     torch.cuda.synchronize()
