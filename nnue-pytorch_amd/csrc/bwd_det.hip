@@ -109,6 +109,12 @@ bool det_layout(int B, int K, int R, int out_cols, int n_persp, DetLayout* L) {
     return true;
 }
 
+template <int VW>
+__device__ __forceinline__ vecf<VW> ldv_once(const float* p) {
+    if constexpr (VW == 4) return ldv4_stream(p);
+    else return ldv<VW>(p);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Upstream rows of the two sparse-linear outputs of a position, and the bias partial sums.
 // One wave per (tile of NNUEFT_BIAS_TILE positions, column slice); a lane keeps its columns and
@@ -146,10 +152,11 @@ __global__ __launch_bounds__(64) void k_bwd_rows(const float* __restrict__ us, c
             const float u = us[b], t = them[b];
             const float* sw = saved + (size_t)b * L1;
             const float* sb = saved + ((size_t)B + b) * L1;
-            const vecf<VW> sw0 = ldv<VW>(sw + c), sw1 = ldv<VW>(sw + h + c);
-            const vecf<VW> sb0 = ldv<VW>(sb + c), sb1 = ldv<VW>(sb + h + c);
-            const vecf<VW> g0 = ldv<VW>(grad_l0 + (size_t)b * L1 + c);
-            const vecf<VW> g1 = ldv<VW>(grad_l0 + (size_t)b * L1 + h + c);
+            // read once: streaming loads, so they do not displace the rows the next kernel gathers
+            const vecf<VW> sw0 = ldv_once<VW>(sw + c), sw1 = ldv_once<VW>(sw + h + c);
+            const vecf<VW> sb0 = ldv_once<VW>(sb + c), sb1 = ldv_once<VW>(sb + h + c);
+            const vecf<VW> g0 = ldv_once<VW>(grad_l0 + (size_t)b * L1 + c);
+            const vecf<VW> g1 = ldv_once<VW>(grad_l0 + (size_t)b * L1 + h + c);
             vecf<VW> gw0, gw1, gb0, gb1;
 #pragma unroll
             for (int i = 0; i < VW; ++i) {
