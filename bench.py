@@ -329,7 +329,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--optimizer", default="rangerlite", choices=["rangerlite", "adam"],
                     help="full_step workload only")
-    ap.add_argument("--compile", default="", choices=["", "inductor", "aot_eager"],
+    ap.add_argument("--compile", default="", choices=["", "inductor", "aot_eager", "cudagraphs"],
                     help="full_step workload only: torch.compile the model with this backend, as the reference's "
                          "train.py does (the kernels of this build stay opaque to it); off by default")
     ap.add_argument("--sort-placement", default="inline", choices=["inline", "backward", "forward"],

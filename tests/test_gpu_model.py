@@ -101,12 +101,16 @@ def test_full_model_trains_on_gpu():
     torch.testing.assert_close(a, b, atol=2e-4, rtol=1e-3)
 
 
+@pytest.mark.parametrize("whole_model", [True, False], ids=["model", "modules"])
 @pytest.mark.parametrize("backend", ["aot_eager", "inductor", "cudagraphs"])
-def test_model_under_torch_compile_on_gpu(backend):
-    """The reference compiles the model (train.py:296; "inductor" or "cudagraphs", config.py:63-64).  The
-    launchers are opaque to dynamo (torch.compiler.disable), so the graph breaks around the HIP kernels
-    and the results are those of the eager module, deterministic backward included.  With "cudagraphs"
-    the stretches between the launchers are captured and replayed: four calls, each checked."""
+def test_model_under_torch_compile_on_gpu(backend, whole_model):
+    """The reference compiles the model (train.py:296; "inductor" or "cudagraphs", config.py:63-64).
+    whole_model: torch.compile(model) leaves NNUEModel.forward as it is (it is marked not to be traced).
+    Otherwise a function over the feature transformer and the layer stacks is compiled, as when the
+    operator sits under other modules: the launchers are opaque to dynamo (torch.compiler.disable), the
+    graph breaks around the HIP kernels, and the stretches between them are compiled (captured and
+    replayed with "cudagraphs": four calls, each checked).  Either way the results are the eager ones,
+    deterministic backward included."""
     old = nnueft.get_backward_mode()
     nnueft.set_backward_mode("deterministic")
     try:
@@ -117,13 +121,19 @@ def test_model_under_torch_compile_on_gpu(backend):
         ref = {n: p.grad.clone() for n, p in model.named_parameters()}
         model.zero_grad()
         torch._dynamo.reset()
-        cm = torch.compile(model, backend=backend)
+
+        def modules(us, them, white, black, piece_count):
+            psqt, ls = model.calculate_buckets(piece_count)
+            l0, wp, bp = model.input(us, them, white, black, psqt, True, True)
+            return model.layer_stacks(l0, ls, True, True) + (wp - bp) * (us - 0.5)
+
+        cm = torch.compile(model if whole_model else modules, backend=backend)
         for _ in range(4 if backend == "cudagraphs" else 2):      # from the second call on: the cached graph
             model.zero_grad()
             o = cm(*batch)
             o.sum().backward()
             torch.testing.assert_close(o, out, atol=1e-5, rtol=1e-5)
-            if backend == "aot_eager":   # same kernels upstream, so the same bits (inductor fuses the layer stacks)
+            if whole_model or backend == "aot_eager":   # same kernels upstream, so the same bits
                 assert torch.equal(model.input.features[0].weight.grad, ref["input.features.0.weight"])
             for n, p in model.named_parameters():
                 torch.testing.assert_close(p.grad, ref[n], atol=1e-4, rtol=1e-4)
