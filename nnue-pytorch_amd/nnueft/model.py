@@ -434,6 +434,8 @@ class ComposedFeatureTransformer(nn.Module):
         self.num_outputs = l1_size + num_psqt_buckets
         self.features = nn.ModuleList([cls(self.num_outputs) for cls in feature_classes])
         self.bias = nn.Parameter(torch.empty(self.num_outputs))
+        # moves with the module, stays out of the state dict (checkpoints are the reference's)
+        self.register_buffer("psqt_bias_zeros", torch.zeros(num_psqt_buckets), persistent=False)
         self.NUM_INPUTS = sum(f.NUM_INPUTS for f in self.features)
         self.MAX_ACTIVE_FEATURES = sum(f.MAX_ACTIVE_FEATURES for f in self.features)
         self.NUM_REAL_FEATURES = sum(f.NUM_REAL_FEATURES for f in self.features)
@@ -468,7 +470,8 @@ class ComposedFeatureTransformer(nn.Module):
                 b = _table_merge(b.view(1, -1), None, self.l1_size, s, s, True).view(-1)
             else:
                 b = q.fake_quantize_weights(b, "ft_bias")
-        bias = torch.cat([b, self._psqt_bias_zeros(b)], dim=0)
+        # the PSQT part of the bias is held at zero
+        bias = torch.cat([b, self.psqt_bias_zeros.to(b.dtype)], dim=0)
         return merged, bias
 
     def _psqt_bias_zeros(self, like):
