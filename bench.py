@@ -440,7 +440,8 @@ def main():
     if args.only != "fwd":
         g_l0, g_wp, g_bp = t["g_l0"], t["g_wp"], t["g_bp"]
         oc = L1 + N_PSQT
-        nbytes = lib.nnueft_det_workspace_bytes(B, K_, R_ROWS, oc, 2)
+        row_split = lib.nnueft_row_split()
+        nbytes = lib.nnueft_det_workspace_bytes(B, K_, R_ROWS, oc, 2, row_split)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
         gW = torch.empty(R_ROWS, oc, device=dev)
         gb = torch.empty(oc, device=dev)
@@ -454,7 +455,7 @@ def main():
         aux_stream = _aux_stream_ptr(dev) if args.sort_placement == "backward" else None
 
         def bwd_det():
-            rc = lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT,
+            rc = lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT, row_split,
                                            ws.data_ptr(), nbytes, None, stream, aux_stream)
             assert rc == 0
 
@@ -474,13 +475,13 @@ def main():
             lists = torch.empty(sbytes, dtype=torch.uint8, device=dev)
 
             def sort_only():
-                rc = lib.nnueft_det_sort(t["white"].data_ptr(), t["black"].data_ptr(), B, K_, R_ROWS, oc, 2,
+                rc = lib.nnueft_det_sort(t["white"].data_ptr(), t["black"].data_ptr(), B, K_, R_ROWS, oc, 2, row_split,
                                          lists.data_ptr(), sbytes, stream)
                 assert rc == 0
 
             def bwd_presorted():
                 rc = lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT,
-                                               ws.data_ptr(), nbytes, lists.data_ptr(), stream, None)
+                                               row_split, ws.data_ptr(), nbytes, lists.data_ptr(), stream, None)
                 assert rc == 0
 
             _, bwd_ms["sort"] = time_steps(sort_only, max(args.steps, 10), args.warmup)

@@ -4,7 +4,11 @@
  * C ABI.  Every pointer is a DEVICE pointer owned by the caller unless stated otherwise; the
  * library never allocates, frees or retains memory.  `stream` is a hipStream_t passed as void*
  * (NULL = the default stream); all work is enqueued on it and the call returns without waiting.
- * The library keeps no global state and may be called from several host threads.
+ * The library may be called from several host threads.  What it keeps between calls: per device,
+ * a few facts queried once (LDS size, number of XCDs); per host thread and device, two events for
+ * the two-stream backward.
+ * After the first call on a device an entry point makes no calls but kernel launches and event
+ * record / wait, so it can be recorded by a stream capture (make that first call before capturing).
  *
  * Return value: 0 on success, a negative NNUEFT_E_* code for a rejected argument, or a positive
  * hipError_t when a launch failed.  nnueft_error_string() describes either.
@@ -21,9 +25,11 @@
  *                  +0 over the slots naming that row in ascending (position, slot) order; then
  *                  white chain + black chain.  This is the order of torch's CPU embedding_bag
  *                  backward, i.e. of the reference's CPU path.
- *                  Exception, for speed on batches where a few rows are named by a large part of
- *                  the positions: a table row named by more than nnueft_row_split() slots of the
- *                  batch (both perspectives together) is summed window by window.  Window w holds
+ *                  With row_split = 0 that holds for every row (the strict order: bit for bit the
+ *                  reference's CPU path).  With row_split > 0, for speed on batches where a few rows are
+ *                  named by a large part of the positions, a table row named by more than row_split
+ *                  slots of the batch (both perspectives together) is summed window by window
+ *                  (nnueft_row_split() is the value this build is tuned for).  Window w holds
  *                  positions [w * nnueft_row_window(B), (w + 1) * nnueft_row_window(B)); per
  *                  perspective, each window's slots are chained from +0 as above, the window sums
  *                  are chained from +0 in ascending w, and the two perspectives are added.  Such
@@ -42,7 +48,7 @@
 extern "C" {
 #endif
 
-#define NNUEFT_VERSION 1
+#define NNUEFT_VERSION 2
 
 #define NNUEFT_E_ARG (-1)         /* null pointer, non-positive or inconsistent dimension, odd L1 */
 #define NNUEFT_E_WORKSPACE (-2)   /* workspace missing, misaligned (256 B) or smaller than nnueft_det_workspace_bytes() */
@@ -54,10 +60,18 @@ const char* nnueft_error_string(int code);
 /* Positions per tile of the deterministic bias-gradient order. */
 int nnueft_bias_tile(void);
 
-/* Deterministic weight-gradient order: rows named by more slots than nnueft_row_split() are summed
- * in windows of nnueft_row_window(B) positions (see "Summation order" above). */
+/* Deterministic weight-gradient order: the `row_split` argument of the deterministic entry points.
+ * 0: every row in the strict order.  n > 0: rows named by more than n slots are summed in windows of
+ * nnueft_row_window(B) positions (see "Summation order" above).  nnueft_row_split() returns the
+ * threshold the kernels are tuned for (512); any non-negative value is accepted. */
 int nnueft_row_split(void);
 int nnueft_row_window(int B);
+
+/* Accelerator dies (XCDs, each with an L2 of its own) of the current device, 0 if the runtime does
+ * not say; negative on error.  The L2-blocked kernels are laid out for 8: on a device that presents
+ * another number, nnueft_double_fwd and nnueft_ft_int16_fwd take their unblocked kernels (same
+ * results), and the deterministic backward keeps its results but loses its cache blocking. */
+int nnueft_device_xcds(void);
 
 /*
  * out[b,:] = (sum_k W[idx[b,k],:]) + bias.
@@ -81,9 +95,10 @@ int nnueft_sparse_bwd_atomic(const int32_t* idx, const float* gout, float* gW, f
 /*
  * Bytes of scratch the deterministic backward entry points need (256-B aligned device memory,
  * contents irrelevant on entry, garbage on exit).  n_persp = 1 for nnueft_sparse_bwd_det,
- * 2 for nnueft_double_bwd_det.  Returns 0 for invalid dimensions.
+ * 2 for nnueft_double_bwd_det; row_split as passed to them (the window sums of split rows are
+ * sized for the worst case, so row_split = 0 needs the least).  Returns 0 for invalid dimensions.
  */
-size_t nnueft_det_workspace_bytes(int B, int K, int R, int out_cols, int n_persp);
+size_t nnueft_det_workspace_bytes(int B, int K, int R, int out_cols, int n_persp, int row_split);
 
 /*
  * Same gradient as nnueft_sparse_bwd_atomic in the fixed order stated at the top: a stable
@@ -93,7 +108,7 @@ size_t nnueft_det_workspace_bytes(int B, int K, int R, int out_cols, int n_persp
  * reference's CPU path (torch embedding_bag backward, sparse_linear_functions.py:43-50).
  */
 int nnueft_sparse_bwd_det(const int32_t* idx, const float* gout, float* gW, float* gbias,
-                          int B, int K, int R, int out_cols,
+                          int B, int K, int R, int out_cols, int row_split,
                           void* workspace, size_t workspace_bytes, void* stream);
 
 /*
@@ -160,9 +175,11 @@ int nnueft_double_bwd_atomic(const float* us, const float* them, const int32_t* 
  * Same gradient in the fixed order stated at the top; gW and gbias are fully written.
  * No counterpart in the reference's GPU code; the order is that of autograd through the
  * reference's CPU composition (double_ft_functions.py:62-80).
- * sorted_lists: NULL, or the block nnueft_det_sort wrote for these index lists and sizes (typically
- * while the forward pass ran: the sort reads nothing but the lists); the call then skips its own
- * sort.  The block stays valid for further calls.
+ * sorted_lists: NULL, or the block nnueft_det_sort wrote for these index lists, sizes and row_split
+ * (typically while the forward pass ran: the sort reads nothing but the lists); the call then skips
+ * its own sort.  The block stays valid for further calls, one at a time: it holds the task counters
+ * of the reduction, which the call's last kernel rewinds, so two reductions that overlap on one
+ * block (two streams, two threads) race on them.
  * aux_stream: NULL, or a second stream of the same device.
  *   With sorted_lists NULL: sorting the index lists and computing the upstream rows are independent;
  *   given a second stream the call runs the sort there, beside the other work on `stream`, and
@@ -177,7 +194,7 @@ int nnueft_double_bwd_det(const float* us, const float* them, const int32_t* wid
                           const int64_t* psqt_idx, const float* bias, float max_act,
                           const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt,
                           const float* saved, float* gW, float* gbias,
-                          int B, int K, int R, int L1, int n_psqt,
+                          int B, int K, int R, int L1, int n_psqt, int row_split,
                           void* workspace, size_t workspace_bytes, void* sorted_lists, void* stream,
                           void* aux_stream);
 
@@ -185,11 +202,24 @@ int nnueft_double_bwd_det(const float* us, const float* them, const int32_t* wid
  * The part of the deterministic backward that depends on the index lists only: the stable sort of
  * the (table row, position) pairs and the work split of the reduction.  sorted_lists: device
  * memory of nnueft_det_sort_bytes(...) bytes, 256-byte aligned; pass it to nnueft_double_bwd_det
- * with the same lists and sizes.  n_persp = 2: both lists; 1: widx only (bidx ignored).
+ * with the same lists, sizes and row_split.  n_persp = 2: both lists; 1: widx only (bidx ignored).
  */
 size_t nnueft_det_sort_bytes(int B, int K, int R, int out_cols, int n_persp);
 int nnueft_det_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, int out_cols, int n_persp,
-                    void* sorted_lists, size_t sorted_bytes, void* stream);
+                    int row_split, void* sorted_lists, size_t sorted_bytes, void* stream);
+
+/*
+ * The reduction stage of the deterministic backward on its own: gW[r, :] = the chains stated at the
+ * top over the upstream rows G f32[n_persp, B, out_cols] (G[p, b] is what position b contributes to
+ * every table row its list p names), given the block nnueft_det_sort wrote for the lists.  For
+ * callers that make the upstream rows themselves and for timing the stage; nnueft_sparse_bwd_det is
+ * nnueft_det_sort + this with G = gout, nnueft_double_bwd_det computes G first.  gW fully written.
+ * workspace: nnueft_det_workspace_bytes(...) bytes (only the window sums of split rows are used).
+ * No counterpart in the reference.
+ */
+int nnueft_det_reduce_rows(const float* G, float* gW, int B, int K, int R, int out_cols, int n_persp,
+                           int row_split, void* workspace, size_t workspace_bytes, void* sorted_lists,
+                           void* stream);
 
 /*
  * merged[r, c] = q(W[r, c] + V[r % vrows, c]): the table the gather reads, from the real weights

@@ -21,6 +21,8 @@
 //                   one window's upstream rows
 //   k_split_combine the window sums of a split row: chain over the windows, white + black
 //   k_bias_final    chain over the tile partial sums
+#include <atomic>
+
 #include "gather.h"
 #include "internal.h"
 
@@ -46,7 +48,6 @@ constexpr int kWavesPerXcd = NNUEFT_SEG_WAVES;  // persistent waves per XCD in t
 #define NNUEFT_LONG_ROW 256
 #endif
 constexpr int kLongRow = NNUEFT_LONG_ROW;  // table rows named by at least this many slots are reduced first
-static_assert(NNUEFT_ROW_SPLIT >= NNUEFT_LONG_ROW, "split rows are skipped where long rows are");
 #ifndef NNUEFT_RUN_U
 #define NNUEFT_RUN_U 16
 #endif
@@ -70,12 +71,15 @@ struct DetLayout {
     int wch;     // chunks per window of a split row
     int nwin;    // windows
     int max_split;   // most rows that can be split
+    int row_split;   // the threshold this layout was made for
 };
 
 inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-bool det_layout(int B, int K, int R, int out_cols, int n_persp, DetLayout* L) {
-    if (B <= 0 || K <= 0 || R <= 0 || out_cols <= 0 || (n_persp != 1 && n_persp != 2)) return false;
+// row_split: a table row named by more slots than this is summed window by window; 0 = no row is.
+bool det_layout(int B, int K, int R, int out_cols, int n_persp, int row_split, DetLayout* L) {
+    if (B <= 0 || K <= 0 || R <= 0 || out_cols <= 0 || (n_persp != 1 && n_persp != 2) || row_split < 0) return false;
+    L->row_split = row_split;
     L->cpp = (B + kChunk - 1) / kChunk;
     L->nchunks = n_persp * L->cpp;
     L->ntiles = (B + NNUEFT_BIAS_TILE - 1) / NNUEFT_BIAS_TILE;
@@ -102,7 +106,9 @@ bool det_layout(int B, int K, int R, int out_cols, int n_persp, DetLayout* L) {
     const int wpos = nnueft_window_positions(B);
     L->wch = wpos / kChunk;
     L->nwin = (B + wpos - 1) / wpos;
-    L->max_split = (int)(((long long)n_persp * B * K) / (NNUEFT_ROW_SPLIT + 1));
+    const long long most = row_split > 0 ? ((long long)n_persp * B * K) / ((long long)row_split + 1) : 0;
+    if (most > 0x3fffffffLL) return false;
+    L->max_split = (int)most;
     L->runs = off;
     off += up256((size_t)L->max_split * n_persp * L->nwin * out_cols * sizeof(float));
     L->end = off;
@@ -211,6 +217,7 @@ __global__ __launch_bounds__(64) void k_bias_final(const float* __restrict__ par
     // another reduction (a second backward through the same graph)
     if (sched && blockIdx.x == 0)
         for (int i = threadIdx.x; i < kXcd * kSchedQueues; i += 64) sched[kSchedCtr + i * 32] = 0;
+    if (!partial) return;   // the rows-only reduction: nothing but the rewind
     const int c = blockIdx.x * 64 + threadIdx.x;
     if (c >= out_cols) return;
     constexpr int PF = 64;
@@ -276,7 +283,8 @@ __global__ __launch_bounds__(256) void k_chunk_hist(const int32_t* __restrict__ 
 
 // Per table row: chunk counts -> exclusive offsets; total and white share.
 __global__ __launch_bounds__(64) void k_col_scan(uint32_t* __restrict__ cnt, uint32_t* __restrict__ wcount,
-                                                 uint32_t* __restrict__ seg_off, int R, int cpp, int nchunks) {
+                                                 uint32_t* __restrict__ seg_off, int R, int cpp, int nchunks,
+                                                 uint32_t row_split) {
     const int r = blockIdx.x * 64 + threadIdx.x;
     if (r >= R) return;
     constexpr int PF = 16;
@@ -301,7 +309,7 @@ __global__ __launch_bounds__(64) void k_col_scan(uint32_t* __restrict__ cnt, uin
     }
     if (nchunks == cpp) white = run;
     wcount[r] = white;
-    seg_off[r] = run > (uint32_t)NNUEFT_ROW_SPLIT ? (run | kSplitFlag) : run;
+    seg_off[r] = (row_split != 0 && run > row_split) ? (run | kSplitFlag) : run;
 }
 
 // floor(kXcd * w / denom) for w < denom, without a 64-bit division
@@ -592,6 +600,7 @@ struct RunPlan {
     float* runs;           // [split row, perspective, window, out_cols] window sums
     int R, cpp, nchunks, wch, nwin, n_persp;
     int nslices, slice_v;  // 64-lane slices
+    uint32_t row_split;    // rows named by more slots than this are the split ones (0: none)
 };
 
 // Persistent waves.  A wave takes tasks from its home queue of its XCD, then from the XCD's other
@@ -659,7 +668,9 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
             r = lo + (u - (uint32_t)s * nreg);
         }
         const uint32_t beg = seg_off[r], end = seg_off[r + 1];
-        if (t >= long_end && end - beg >= (uint32_t)kLongRow) continue;   // long or split: done elsewhere
+        // long or split: done elsewhere
+        if (t >= long_end && (end - beg >= (uint32_t)kLongRow || (rp.row_split != 0 && end - beg > rp.row_split)))
+            continue;
         seg_reduce_task<VW, NQ, kRowsUnroll>(G, list, beg, beg + wcount[r], end, gW + (size_t)r * out_cols, s, lane,
                                              out_cols, slice_v, two_persp);
     }
@@ -699,10 +710,7 @@ __global__ __launch_bounds__(64) void k_split_combine(const uint32_t* __restrict
 }
 
 // Table rows per sort pass and whether the chunk's index lists are staged in LDS by k_fill.
-bool lds_plan(int R, int K, int* range_out, int* stage_out, size_t* hist_bytes, size_t* fill_bytes) {
-    int dev = 0, max_lds = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return false;
-    if (hipDeviceGetAttribute(&max_lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess) return false;
+bool lds_plan(int max_lds, int R, int K, int* range_out, int* stage_out, size_t* hist_bytes, size_t* fill_bytes) {
     if (max_lds < 16 * 1024) return false;
     const size_t stage_bytes = (size_t)kChunk * K * sizeof(int32_t);
     const int stage = stage_bytes <= (size_t)max_lds / 4;
@@ -719,6 +727,29 @@ bool lds_plan(int R, int K, int* range_out, int* stage_out, size_t* hist_bytes, 
     return true;
 }
 
+// The three sort kernels may ask for all of a workgroup's LDS; that permission is a property of
+// the loaded kernel on a device, so it is given once per device, on the first sort there.
+constexpr int kMaxDevices = 64;
+std::atomic<int> g_lds_allowed[kMaxDevices];
+
+int allow_full_lds(int device, int max_lds) {
+    if (device < 0 || device >= kMaxDevices) return NNUEFT_E_UNSUPPORTED;
+    if (g_lds_allowed[device].load(std::memory_order_acquire) == max_lds) return 0;
+    if (max_lds > 48 * 1024) {
+        const void* kernels[3] = {(const void*)k_row_scan, (const void*)k_chunk_hist, (const void*)k_fill};
+        for (const void* k : kernels) {
+            // what a kernel declares statically comes out of the same budget
+            hipFuncAttributes fa{};
+            hipError_t e = hipFuncGetAttributes(&fa, k);
+            if (e != hipSuccess) return (int)e;
+            e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, max_lds - (int)fa.sharedSizeBytes);
+            if (e != hipSuccess) return (int)e;
+        }
+    }
+    g_lds_allowed[device].store(max_lds, std::memory_order_release);
+    return 0;
+}
+
 // The sort: everything the reduction needs to know about the index lists (it reads no gradient).
 // `sorted` is the block [L.sort_begin, L.sort_end) of the layout, wherever the caller keeps it.
 int det_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, char* sorted, const DetLayout& L,
@@ -731,29 +762,23 @@ int det_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, char
     uint32_t* sched = (uint32_t*)(ws + L.sched);
     uint32_t* list = (uint32_t*)(ws + L.list);
 
+    int device = 0;
+    const nnueft_dev::DeviceInfo* info = nullptr;
+    int rc = nnueft_dev::device_info(&device, &info);
+    if (rc) return rc;
     int range = 0, stage = 0;
     size_t hist_bytes = 0, fill_bytes = 0;
-    if (!lds_plan(R, K, &range, &stage, &hist_bytes, &fill_bytes)) return NNUEFT_E_UNSUPPORTED;
+    if (!lds_plan(info->max_lds, R, K, &range, &stage, &hist_bytes, &fill_bytes)) return NNUEFT_E_UNSUPPORTED;
     const int nranges = (R + range - 1) / range;
     // rows the single-workgroup row scan stages in LDS at a time (`range` fits by construction)
     const int scan_cap = max(kScanThreads, min(range, (R + kScanThreads - 1) / kScanThreads * kScanThreads));
-    if ((size_t)scan_cap * sizeof(uint32_t) > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void*)k_row_scan, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)(scan_cap * sizeof(uint32_t)));
-        if (e != hipSuccess) return (int)e;
-    }
-    if (fill_bytes > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void*)k_chunk_hist, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)hist_bytes);
-        if (e != hipSuccess) return (int)e;
-        e = hipFuncSetAttribute((const void*)k_fill, hipFuncAttributeMaxDynamicSharedMemorySize, (int)fill_bytes);
-        if (e != hipSuccess) return (int)e;
-    }
+    rc = allow_full_lds(device, info->max_lds);
+    if (rc) return rc;
     hipLaunchKernelGGL(k_chunk_hist, dim3(L.nchunks, nranges), dim3(256), hist_bytes, st, widx, bidx, cnt, B, K, R,
                        L.cpp, range);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_col_scan, dim3((R + 63) / 64), dim3(64), 0, st, cnt, wcount, seg_off, R, L.cpp,
-                       L.nchunks);
+                       L.nchunks, (uint32_t)L.row_split);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_row_scan, dim3(1), dim3(kScanThreads), (size_t)scan_cap * sizeof(uint32_t), st, seg_off,
                        long_rows, sched, R, scan_cap);
@@ -797,6 +822,7 @@ int det_reduce(const float* G, float* gW, float* gbias, int B, int R, int out_co
     rp.n_persp = n_persp;
     rp.nslices = (nv + 63) / 64;
     rp.slice_v = ((nv + rp.nslices - 1) / rp.nslices + line_v - 1) / line_v * line_v;
+    rp.row_split = (uint32_t)L.row_split;
     if ((long long)L.max_split * rp.nslices * NNUEFT_ROW_WINDOWS > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
 #define SEG_LAUNCH(VW_, NQ_)                                                                                      \
     hipLaunchKernelGGL((k_seg_reduce<VW_, NQ_>), dim3(kXcd * kWavesPerXcd), dim3(64), 0, st, G, list, seg_off,      \
@@ -816,7 +842,7 @@ int det_reduce(const float* G, float* gW, float* gbias, int B, int R, int out_co
         NNUEFT_LAUNCH_CHECK();
     }
 
-    return nnueft_det::launch_bias_final(partial, gbias, B, out_cols, sched, st);
+    return nnueft_det::launch_bias_final(gbias ? partial : nullptr, gbias, B, out_cols, sched, st);
 }
 
 }  // namespace
@@ -857,36 +883,50 @@ int launch_bias_final(const float* partial, float* gbias, int B, int out_cols, u
 
 }  // namespace nnueft_det
 
-extern "C" size_t nnueft_det_workspace_bytes(int B, int K, int R, int out_cols, int n_persp) {
+extern "C" size_t nnueft_det_workspace_bytes(int B, int K, int R, int out_cols, int n_persp, int row_split) {
     DetLayout L;
-    if (!det_layout(B, K, R, out_cols, n_persp, &L)) return 0;
+    if (!det_layout(B, K, R, out_cols, n_persp, row_split, &L)) return 0;
     return L.end;
 }
 
 extern "C" size_t nnueft_det_sort_bytes(int B, int K, int R, int out_cols, int n_persp) {
     DetLayout L;
-    if (!det_layout(B, K, R, out_cols, n_persp, &L)) return 0;
+    if (!det_layout(B, K, R, out_cols, n_persp, 0, &L)) return 0;
     return L.sort_end - L.sort_begin;
 }
 
 extern "C" int nnueft_det_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, int out_cols,
-                               int n_persp, void* sorted_lists, size_t sorted_bytes, void* stream) {
+                               int n_persp, int row_split, void* sorted_lists, size_t sorted_bytes, void* stream) {
     if (!widx || (n_persp == 2 && !bidx)) return NNUEFT_E_ARG;
     if ((long long)B * K > 0x3fffffffLL || (long long)B > 0x3fffffffLL) return NNUEFT_E_UNSUPPORTED;
     DetLayout L;
-    if (!det_layout(B, K, R, out_cols, n_persp, &L)) return NNUEFT_E_ARG;
+    if (!det_layout(B, K, R, out_cols, n_persp, row_split, &L)) return NNUEFT_E_ARG;
     if (!sorted_lists || !aligned256(sorted_lists) || sorted_bytes < L.sort_end - L.sort_begin)
         return NNUEFT_E_WORKSPACE;
     return det_sort(widx, n_persp == 2 ? bidx : widx, B, K, R, (char*)sorted_lists, L, (hipStream_t)stream);
 }
 
+extern "C" int nnueft_det_reduce_rows(const float* G, float* gW, int B, int K, int R, int out_cols, int n_persp,
+                                      int row_split, void* workspace, size_t workspace_bytes, void* sorted_lists,
+                                      void* stream) {
+    if (!G || !gW) return NNUEFT_E_ARG;
+    if ((long long)B * K > 0x3fffffffLL || (long long)B > 0x3fffffffLL) return NNUEFT_E_UNSUPPORTED;
+    DetLayout L;
+    if (!det_layout(B, K, R, out_cols, n_persp, row_split, &L)) return NNUEFT_E_ARG;
+    if (!workspace || !aligned256(workspace) || workspace_bytes < L.end) return NNUEFT_E_WORKSPACE;
+    if (!sorted_lists || !aligned256(sorted_lists)) return NNUEFT_E_WORKSPACE;
+    return det_reduce(G, gW, nullptr, B, R, out_cols, n_persp, (char*)workspace, (char*)sorted_lists, L,
+                      (hipStream_t)stream);
+}
+
 extern "C" int nnueft_sparse_bwd_det(const int32_t* idx, const float* gout, float* gW, float* gbias, int B, int K,
-                                     int R, int out_cols, void* workspace, size_t workspace_bytes, void* stream) {
-    if (B <= 0 || K <= 0 || R <= 0 || out_cols <= 0) return NNUEFT_E_ARG;
+                                     int R, int out_cols, int row_split, void* workspace, size_t workspace_bytes,
+                                     void* stream) {
+    if (B <= 0 || K <= 0 || R <= 0 || out_cols <= 0 || row_split < 0) return NNUEFT_E_ARG;
     if (!idx || !gout || !gW || !gbias) return NNUEFT_E_ARG;
     if ((long long)B * K > 0x7fffffffLL || (long long)B > 0x3fffffffLL) return NNUEFT_E_UNSUPPORTED;
     DetLayout L;
-    if (!det_layout(B, K, R, out_cols, 1, &L)) return NNUEFT_E_ARG;
+    if (!det_layout(B, K, R, out_cols, 1, row_split, &L)) return NNUEFT_E_ARG;
     if (!workspace || !aligned256(workspace) || workspace_bytes < L.end) return NNUEFT_E_WORKSPACE;
     hipStream_t st = (hipStream_t)stream;
     char* ws = (char*)workspace;
@@ -902,70 +942,63 @@ extern "C" int nnueft_double_bwd_det(const float* us, const float* them, const i
                                      const int64_t* psqt_idx, const float* bias, float max_act,
                                      const float* grad_l0,
                                      const float* grad_wpsqt, const float* grad_bpsqt, const float* saved,
-                                     float* gW, float* gbias, int B, int K, int R, int L1, int n_psqt,
+                                     float* gW, float* gbias, int B, int K, int R, int L1, int n_psqt, int row_split,
                                      void* workspace, size_t workspace_bytes, void* sorted_lists, void* stream,
                                      void* aux_stream) {
-    if (B <= 0 || K <= 0 || R <= 0 || L1 <= 0 || (L1 & 1) || n_psqt < 0) return NNUEFT_E_ARG;
+    if (B <= 0 || K <= 0 || R <= 0 || L1 <= 0 || (L1 & 1) || n_psqt < 0 || row_split < 0) return NNUEFT_E_ARG;
     if (!us || !them || !widx || !bidx || !psqt_idx || !bias || !grad_l0 || !grad_wpsqt || !grad_bpsqt || !saved ||
         !gW || !gbias)
         return NNUEFT_E_ARG;
     if ((long long)B * K > 0x3fffffffLL || (long long)B > 0x3fffffffLL) return NNUEFT_E_UNSUPPORTED;
     const int out_cols = L1 + n_psqt;
     DetLayout L;
-    if (!det_layout(B, K, R, out_cols, 2, &L)) return NNUEFT_E_ARG;
+    if (!det_layout(B, K, R, out_cols, 2, row_split, &L)) return NNUEFT_E_ARG;
     if (!workspace || !aligned256(workspace) || workspace_bytes < L.end) return NNUEFT_E_WORKSPACE;
+    if (sorted_lists && !aligned256(sorted_lists)) return NNUEFT_E_WORKSPACE;
     hipStream_t st = (hipStream_t)stream;
     char* ws = (char*)workspace;
     float* G = (float*)(ws + L.G);
+    float* partial = (float*)(ws + L.partial);
     // The sort reads only the index lists, the upstream rows only the activations: with a second
     // stream they run side by side and meet before the reduction.
     hipStream_t aux = (hipStream_t)aux_stream;
+    const bool two_streams = aux && aux != st;
+    hipEvent_t forked = nullptr, joined = nullptr;
+    if (two_streams) {
+        int device = 0;
+        const nnueft_dev::DeviceInfo* info = nullptr;
+        int rc = nnueft_dev::device_info(&device, &info);
+        if (rc == 0) rc = nnueft_dev::thread_events(device, &forked, &joined);
+        if (rc) return rc;
+    }
     if (sorted_lists) {
         // the caller ran nnueft_det_sort on these lists already; if on aux_stream, it may still be
         // running there: only the reduction has to wait for it, the upstream rows do not
-        if (!aligned256(sorted_lists)) return NNUEFT_E_WORKSPACE;
-        int rc = nnueft_det::launch_bwd_rows(us, them, psqt_idx, bias, max_act, grad_l0, grad_wpsqt, grad_bpsqt,
-                                             saved, G, (float*)(ws + L.partial), B, L1, n_psqt, st);
+        const int rc = nnueft_det::launch_bwd_rows(us, them, psqt_idx, bias, max_act, grad_l0, grad_wpsqt, grad_bpsqt,
+                                                   saved, G, partial, B, L1, n_psqt, st);
         if (rc) return rc;
-        if (aux && aux != st) {
-            hipEvent_t sorted = nullptr;
-            hipError_t e = hipEventCreateWithFlags(&sorted, hipEventDisableTiming);
-            if (e == hipSuccess) e = hipEventRecord(sorted, aux);
-            if (e == hipSuccess) e = hipStreamWaitEvent(st, sorted, 0);
-            if (sorted) (void)hipEventDestroy(sorted);
+        if (two_streams) {
+            hipError_t e = hipEventRecord(joined, aux);
+            if (e == hipSuccess) e = hipStreamWaitEvent(st, joined, 0);
             if (e != hipSuccess) return (int)e;
         }
         return det_reduce(G, gW, gbias, B, R, out_cols, 2, ws, (char*)sorted_lists, L, st);
     }
-    hipEvent_t forked = nullptr, sorted = nullptr;
-    if (aux && aux != st) {
-        hipError_t e = hipEventCreateWithFlags(&forked, hipEventDisableTiming);
-        if (e == hipSuccess) e = hipEventCreateWithFlags(&sorted, hipEventDisableTiming);
-        if (e == hipSuccess) e = hipEventRecord(forked, st);
+    if (two_streams) {
+        hipError_t e = hipEventRecord(forked, st);
         if (e == hipSuccess) e = hipStreamWaitEvent(aux, forked, 0);
-        if (e != hipSuccess) {
-            if (forked) (void)hipEventDestroy(forked);
-            if (sorted) (void)hipEventDestroy(sorted);
-            return (int)e;
-        }
-    } else {
-        aux = st;
+        if (e != hipSuccess) return (int)e;
     }
-    int rc = det_sort(widx, bidx, B, K, R, ws + L.sort_begin, L, aux);
-    if (rc == 0 && aux != st) {
-        hipError_t e = hipEventRecord(sorted, aux);
-        if (e != hipSuccess) rc = (int)e;
+    int rc = det_sort(widx, bidx, B, K, R, ws + L.sort_begin, L, two_streams ? aux : st);
+    if (two_streams) {
+        // always rejoin, also after a failed launch: the caller's stream must not run ahead of the other one
+        hipError_t e = hipEventRecord(joined, aux);
+        if (e == hipSuccess) e = hipStreamWaitEvent(st, joined, 0);
+        if (rc == 0 && e != hipSuccess) rc = (int)e;
     }
     if (rc == 0)
         rc = nnueft_det::launch_bwd_rows(us, them, psqt_idx, bias, max_act, grad_l0, grad_wpsqt, grad_bpsqt, saved, G,
-                                         (float*)(ws + L.partial), B, L1, n_psqt, st);
-    if (aux != st) {
-        // always rejoin, also after a failed launch: the caller's stream must not run ahead of the other one
-        const hipError_t e = hipStreamWaitEvent(st, sorted, 0);
-        if (rc == 0 && e != hipSuccess) rc = (int)e;
-        (void)hipEventDestroy(forked);
-        (void)hipEventDestroy(sorted);
-    }
+                                         partial, B, L1, n_psqt, st);
     if (rc) return rc;
     return det_reduce(G, gW, gbias, B, R, out_cols, 2, ws, ws + L.sort_begin, L, st);
 }

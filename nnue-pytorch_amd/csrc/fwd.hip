@@ -206,8 +206,12 @@ int double_fwd(const float* us, const float* them, const int32_t* widx, const in
     if (workspace) {
         if (!aligned256(workspace) || workspace_bytes < nnueft_blocked::pair_sort_workspace(B, R, 0))
             return NNUEFT_E_WORKSPACE;
-        // the L2-blocked path needs 16-byte rows; other shapes take the plain kernel below
-        if (vec && (long long)B <= 0x3fffffffLL)
+        // the L2-blocked path needs 16-byte rows and the XCD layout it is made for; other shapes and
+        // devices take the plain kernel below
+        const nnueft_dev::DeviceInfo* info = nullptr;
+        const int rc_dev = nnueft_dev::device_info(nullptr, &info);
+        if (rc_dev) return rc_dev;
+        if (vec && (long long)B <= 0x3fffffffLL && nnueft_blocked::blocked_layout_fits(*info))
             return nnueft_blocked::double_fwd_blocked(us, them, widx, bidx, psqt_idx, W, bias, max_act, l0, wpsqt,
                                                       bpsqt, saved, B, K, R, L1, n_psqt, workspace, st, act);
     }

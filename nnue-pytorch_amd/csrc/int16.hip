@@ -336,7 +336,10 @@ extern "C" int nnueft_ft_int16_fwd(const int32_t* widx, const int32_t* bidx, con
         Int16Layout L;
         if (!int16_layout(B, R, L1, table_block_rows, &L)) return NNUEFT_E_ARG;
         if (!aligned256(workspace) || workspace_bytes < L.end) return NNUEFT_E_WORKSPACE;
-        if (vec && (long long)B <= 0x3fffffffLL) {
+        const nnueft_dev::DeviceInfo* info = nullptr;
+        const int rc_dev = nnueft_dev::device_info(nullptr, &info);
+        if (rc_dev) return rc_dev;
+        if (vec && (long long)B <= 0x3fffffffLL && nnueft_blocked::blocked_layout_fits(*info)) {
             char* ws = (char*)workspace;
             int16_t* accW = (int16_t*)(ws + L.accW);
             const uint32_t* order = nullptr;

@@ -10,9 +10,28 @@ struct ActGrid {
     int on;
 };
 
+namespace nnueft_dev {
+
+// What the launchers need to know about a device; queried once per device and process.
+struct DeviceInfo {
+    int max_lds;   // most LDS a workgroup can ask for, bytes
+    int xcds;      // accelerator dies (each with an L2 of its own) the device presents; 0 = unknown
+};
+// The current device and its facts.  Returns 0, a negative NNUEFT_E_* or a positive hipError_t.
+int device_info(int* device, const DeviceInfo** info);
+// Two events without timing that belong to the calling thread and `device`, created on first use and
+// kept, for ordering a second stream against the caller's (record / wait only on the launch path).
+int thread_events(int device, hipEvent_t* fork, hipEvent_t* join);
+
+}  // namespace nnueft_dev
+
 namespace nnueft_blocked {
 
-constexpr int kXcd = 8;   // XCDs of the device; workgroup id % kXcd is the XCD a workgroup lands on
+// XCDs the blocked kernels are laid out for; workgroup id % kXcd is the XCD a workgroup lands on
+// (workgroups are dealt to the XCDs round-robin).  Results never depend on it; on a device that
+// presents another number of XCDs the entry points take the unblocked kernels where they have them.
+constexpr int kXcd = 8;
+inline bool blocked_layout_fits(const nnueft_dev::DeviceInfo& d) { return d.xcds == kXcd || d.xcds == 0; }
 
 // Pair sort: order[] = ids (perspective * B + position) of the 2B index lists of a batch grouped by
 // the table block they name (block_rows_hint rows per block, 0 = 768).  `ws` needs pair_sort_workspace() bytes; returns the order array

@@ -32,8 +32,9 @@ PROTOTYPES = {
     "nnueft_row_window": (c_int, [c_int]),
     "nnueft_sparse_fwd": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_void_p]),
     "nnueft_sparse_bwd_atomic": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_void_p]),
-    "nnueft_det_workspace_bytes": (c_size_t, [c_int] * 5),
-    "nnueft_sparse_bwd_det": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
+    "nnueft_device_xcds": (c_int, []),
+    "nnueft_det_workspace_bytes": (c_size_t, [c_int] * 6),
+    "nnueft_sparse_bwd_det": (c_int, [c_void_p] * 4 + [c_int] * 5 + [c_void_p, c_size_t, c_void_p]),
     "nnueft_fwd_workspace_bytes": (c_size_t, [c_int] * 5),
     "nnueft_double_fwd": (
         c_int,
@@ -46,10 +47,11 @@ PROTOTYPES = {
     "nnueft_double_bwd_atomic": (c_int, [c_void_p] * 6 + [c_float] + [c_void_p] * 6 + [c_int] * 5 + [c_void_p]),
     "nnueft_double_bwd_det": (
         c_int,
-        [c_void_p] * 6 + [c_float] + [c_void_p] * 6 + [c_int] * 5 + [c_void_p, c_size_t, c_void_p, c_void_p, c_void_p],
+        [c_void_p] * 6 + [c_float] + [c_void_p] * 6 + [c_int] * 6 + [c_void_p, c_size_t, c_void_p, c_void_p, c_void_p],
     ),
     "nnueft_det_sort_bytes": (c_size_t, [c_int] * 5),
-    "nnueft_det_sort": (c_int, [c_void_p] * 2 + [c_int] * 5 + [c_void_p, c_size_t, c_void_p]),
+    "nnueft_det_sort": (c_int, [c_void_p] * 2 + [c_int] * 6 + [c_void_p, c_size_t, c_void_p]),
+    "nnueft_det_reduce_rows": (c_int, [c_void_p] * 2 + [c_int] * 6 + [c_void_p, c_size_t, c_void_p, c_void_p]),
     "nnueft_table_merge": (c_int, [c_void_p] * 3 + [c_int] * 4 + [c_float] * 2 + [c_int, c_void_p]),
     "nnueft_table_virtual_grad": (c_int, [c_void_p] * 2 + [c_int] * 3 + [c_void_p]),
     "nnueft_int16_workspace_bytes": (c_size_t, [c_int] * 5),

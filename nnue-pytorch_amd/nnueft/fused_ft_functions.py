@@ -9,8 +9,9 @@ Differences that a caller can observe:
     keeps the clamped mixed values, fused_ft_kernel.py:95-99); the backward recomputes the mix from
     them, so the clamp passes gradient at exactly 0 and exactly max like torch.clamp does in the
     reference's CPU path;
-  * NNUEFT_BACKWARD=deterministic (or set_backward_mode) selects a backward whose result does
-    not depend on scheduling.
+  * the backward mode (NNUEFT_BACKWARD or set_backward_mode): "deterministic" (default) and
+    "deterministic_strict" give results that do not depend on scheduling, the strict one bit for bit
+    the weight gradient of the reference's CPU path; "atomic" is the reference's GPU scheme.
 """
 import torch
 from torch import autograd
@@ -50,7 +51,7 @@ def _launch_double_fwd(us, them, white_indices, black_indices, psqt_indices, wei
 
 
 @torch.compiler.disable(recursive=False)
-def _launch_det_sort(white_indices, black_indices, num_rows, output_size):
+def _launch_det_sort(white_indices, black_indices, num_rows, output_size, row_split):
     """The sort of the deterministic backward reads nothing but the index lists, so it starts here, in
     the forward pass, on a second stream, and is long done when the backward pass wants it.
     Returns the sorted lists, an opaque byte tensor that is complete once the second stream has run."""
@@ -62,7 +63,7 @@ def _launch_det_sort(white_indices, black_indices, num_rows, output_size):
     cur, aux = torch.cuda.current_stream(device), _aux_stream(device)
     aux.wait_stream(cur)                     # the lists and buf are ordered on the caller's stream
     rc = lib.nnueft_det_sort(white_indices.data_ptr(), black_indices.data_ptr(), B, K, num_rows, output_size, 2,
-                             buf.data_ptr(), nbytes, aux.cuda_stream)
+                             row_split, buf.data_ptr(), nbytes, aux.cuda_stream)
     _native.check(rc, "nnueft_det_sort")
     for t in (buf, white_indices, black_indices):
         t.record_stream(aux)                 # their memory is not handed out again before the sort has run
@@ -82,18 +83,19 @@ def _launch_double_bwd(us, them, white_indices, black_indices, psqt_indices, bia
         psqt_indices.data_ptr(), bias.data_ptr(), float(max_ft_activation),
         grad_l0.data_ptr(), grad_wpsqt.data_ptr(), grad_bpsqt.data_ptr(), saved.data_ptr(),
     )
-    if mode == "deterministic":
+    if mode != "atomic":
         grad_weight = torch.empty(num_rows, output_size, dtype=torch.float32, device=device)
         grad_bias = torch.empty(output_size, dtype=torch.float32, device=device)
         if B == 0:
             return grad_weight.zero_(), grad_bias.zero_()
-        nbytes = lib.nnueft_det_workspace_bytes(B, K, num_rows, output_size, 2)
+        row_split = _slf.row_split_of(mode)
+        nbytes = lib.nnueft_det_workspace_bytes(B, K, num_rows, output_size, 2, row_split)
         ws = _workspace(nbytes, device)
         # presorted: the lists sorted during the forward pass on the second stream; the entry point makes
         # its reduction (not its first kernel) wait for that stream
         sorted_ptr = presorted.data_ptr() if presorted is not None else None
         rc = lib.nnueft_double_bwd_det(
-            *head, grad_weight.data_ptr(), grad_bias.data_ptr(), B, K, num_rows, l1_size, n_psqt,
+            *head, grad_weight.data_ptr(), grad_bias.data_ptr(), B, K, num_rows, l1_size, n_psqt, row_split,
             ws.data_ptr(), nbytes, sorted_ptr, _stream_ptr(device),
             _aux_stream_ptr(device) if second_stream else None,
         )
@@ -166,9 +168,10 @@ class FusedDoubleFtFunction(autograd.Function):
         with torch.cuda.device(device):
             # first, so that it runs beside the forward kernel
             ctx.presorted = None
-            if (ctx.sort_placement == "forward" and ctx.backward_mode == "deterministic" and batch_size > 0
+            if (ctx.sort_placement == "forward" and ctx.backward_mode != "atomic" and batch_size > 0
                     and (ctx.needs_input_grad[5] or ctx.needs_input_grad[6])):
-                ctx.presorted = _launch_det_sort(white_indices, black_indices, weight.shape[0], weight.shape[1])
+                ctx.presorted = _launch_det_sort(white_indices, black_indices, weight.shape[0], weight.shape[1],
+                                                 _slf.row_split_of(ctx.backward_mode))
 
             _launch_double_fwd(
                 us, them, white_indices, black_indices, psqt_indices, weight, bias,

@@ -19,17 +19,30 @@ from . import _native
 
 _HAS_CUPY_KERNELS = _native.available()
 
-# "atomic" (reference semantics, unordered fp32 atomics) or "deterministic" (sort + segmented reduction)
 # "deterministic": sort + segmented reduction (any result of it is one the reference's unordered atomics
-# could have produced, and on MI355X it is five times faster); "atomic": the reference's scheme
+#     could have produced, the same bits on every run, and on MI355X it is five times faster than atomics).
+#     Table rows named by more than nnueft_row_split() slots of a batch are summed window by window,
+#     which differs from the reference's CPU path in the last bits of those rows.
+# "deterministic_strict": the same with every row summed in one chain: bit for bit the weight gradient of
+#     the reference's CPU path (torch embedding_bag backward under autograd); slower on batches where a
+#     few table rows are named by thousands of positions.
+# "atomic": the reference's GPU scheme, unordered fp32 atomics.
+BACKWARD_MODES = ("atomic", "deterministic", "deterministic_strict")
 _BACKWARD_MODE = os.environ.get("NNUEFT_BACKWARD", "deterministic")
+if _BACKWARD_MODE not in BACKWARD_MODES:
+    raise ValueError(f"NNUEFT_BACKWARD={_BACKWARD_MODE!r}: expected one of {BACKWARD_MODES}")
 
 
 def set_backward_mode(mode: str) -> None:
     global _BACKWARD_MODE
-    if mode not in ("atomic", "deterministic"):
+    if mode not in BACKWARD_MODES:
         raise ValueError(f"Invalid backward mode: {mode}")
     _BACKWARD_MODE = mode
+
+
+def row_split_of(mode: str) -> int:
+    """The row_split argument of the deterministic entry points for a backward mode."""
+    return 0 if mode == "deterministic_strict" else _native.load().nnueft_row_split()
 
 
 def get_backward_mode() -> str:
@@ -116,16 +129,17 @@ def _launch_sparse_bwd(feature_indices, grad_output, num_rows, mode):
     B, K = feature_indices.shape
     out_cols = grad_output.shape[1]
     device = grad_output.device
-    if mode == "deterministic":
+    if mode != "atomic":
         weight_grad = torch.empty(num_rows, out_cols, dtype=torch.float32, device=device)
         bias_grad = torch.empty(out_cols, dtype=torch.float32, device=device)
         if B == 0:
             return weight_grad.zero_(), bias_grad.zero_()
-        nbytes = lib.nnueft_det_workspace_bytes(B, K, num_rows, out_cols, 1)
+        row_split = row_split_of(mode)
+        nbytes = lib.nnueft_det_workspace_bytes(B, K, num_rows, out_cols, 1, row_split)
         ws = _workspace(nbytes, device)
         rc = lib.nnueft_sparse_bwd_det(
             feature_indices.data_ptr(), grad_output.data_ptr(), weight_grad.data_ptr(), bias_grad.data_ptr(),
-            B, K, num_rows, out_cols, ws.data_ptr(), nbytes, _stream_ptr(device),
+            B, K, num_rows, out_cols, row_split, ws.data_ptr(), nbytes, _stream_ptr(device),
         )
         _native.check(rc, "nnueft_sparse_bwd_det")
     else:

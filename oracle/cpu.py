@@ -42,8 +42,14 @@ def bias_tile() -> int:
 
 
 def row_split() -> int:
-    """Most slots that may name a table row before its gradient is summed window by window."""
+    """Default threshold: most slots that may name a table row before its gradient is summed window by
+    window.  sparse_bwd / double_bwd take row_split=None for this value, 0 for the strict order (no row
+    is split: the order of the reference's CPU path) or any other threshold."""
     return int(lib().nnueft_oracle_row_split())
+
+
+def _rs(threshold) -> int:
+    return row_split() if threshold is None else int(threshold)
 
 
 def row_window(B: int) -> int:
@@ -61,13 +67,13 @@ def sparse_fwd(idx, W, bias):
     return out
 
 
-def sparse_bwd(idx, gout, R):
+def sparse_bwd(idx, gout, R, row_split=None):
     idx, gout = _c(idx, np.int32), _c(gout, np.float32)
     B, K = idx.shape
     oc = gout.shape[1]
     gW = np.empty((R, oc), np.float32)
     gb = np.empty((oc,), np.float32)
-    rc = lib().nnueft_oracle_sparse_bwd(_p(idx), _p(gout), _p(gW), _p(gb), B, K, R, oc)
+    rc = lib().nnueft_oracle_sparse_bwd(_p(idx), _p(gout), _p(gW), _p(gb), B, K, R, oc, _rs(row_split))
     assert rc == 0
     return gW, gb
 
@@ -106,7 +112,8 @@ def double_bwd_rows(us, them, psqt_idx, bias, max_act, grad_l0, grad_wpsqt, grad
     return G
 
 
-def double_bwd(us, them, widx, bidx, psqt_idx, bias, max_act, grad_l0, grad_wpsqt, grad_bpsqt, saved, R, n_psqt):
+def double_bwd(us, them, widx, bidx, psqt_idx, bias, max_act, grad_l0, grad_wpsqt, grad_bpsqt, saved, R, n_psqt,
+               row_split=None):
     us, them = _c(us, np.float32).reshape(-1), _c(them, np.float32).reshape(-1)
     widx, bidx = _c(widx, np.int32), _c(bidx, np.int32)
     psqt_idx = _c(psqt_idx, np.int64)
@@ -121,7 +128,7 @@ def double_bwd(us, them, widx, bidx, psqt_idx, bias, max_act, grad_l0, grad_wpsq
     gb = np.empty((oc,), np.float32)
     rc = lib().nnueft_oracle_double_bwd(_p(us), _p(them), _p(widx), _p(bidx), _p(psqt_idx), _p(bias),
                                         ctypes.c_float(max_act), _p(grad_l0), _p(gwp), _p(gbp), _p(saved),
-                                        _p(gW), _p(gb), B, K, R, L1, n_psqt)
+                                        _p(gW), _p(gb), B, K, R, L1, n_psqt, _rs(row_split))
     assert rc == 0
     return gW, gb
 

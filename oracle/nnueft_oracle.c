@@ -35,8 +35,10 @@
  *             (position, slot) order; the two perspectives' chains are then added
  *             (white + black).  torch's CPU embedding_bag backward followed by autograd's
  *             accumulation of the two uses of `weight` produces exactly this.
- *             Exception (this build's own order): a table row named by more than
- *             NNUEFT_ORACLE_ROW_SPLIT slots of the batch, both perspectives together, is summed
+ *             That is the order for every row when row_split = 0 (the strict order).
+ *             With row_split > 0 (this build's own order; NNUEFT_ORACLE_ROW_SPLIT is the default the
+ *             kernels are tuned for): a table row named by more than
+ *             row_split slots of the batch, both perspectives together, is summed
  *             window by window: window w = positions [w*W, (w+1)*W), W = nnueft_oracle_row_window(B);
  *             per perspective each window's slots are chained from +0, the window sums are
  *             chained from +0 in ascending w, then white + black.  torch agrees with such a row
@@ -95,9 +97,10 @@ int nnueft_oracle_sparse_fwd(const int32_t* idx, const float* W, const float* bi
     return 0;
 }
 
-/* split_id[r] = ordinal of row r among the rows named by more than NNUEFT_ORACLE_ROW_SPLIT slots
- * of idx_a and idx_b together (idx_b may be NULL), -1 for the others.  Returns how many. */
-static int find_split_rows(const int32_t* idx_a, const int32_t* idx_b, int B, int K, int R, int32_t* split_id)
+/* split_id[r] = ordinal of row r among the rows named by more than row_split slots of idx_a and
+ * idx_b together (idx_b may be NULL), -1 for the others; row_split = 0: no row.  Returns how many. */
+static int find_split_rows(const int32_t* idx_a, const int32_t* idx_b, int B, int K, int R, int row_split,
+                           int32_t* split_id)
 {
     int64_t* count = (int64_t*)calloc((size_t)R, sizeof(int64_t));
     if (!count) return -1;
@@ -108,7 +111,7 @@ static int find_split_rows(const int32_t* idx_a, const int32_t* idx_b, int B, in
             if (valid(idx[i], R)) count[idx[i]]++;
     }
     int n = 0;
-    for (int r = 0; r < R; ++r) split_id[r] = count[r] > NNUEFT_ORACLE_ROW_SPLIT ? n++ : -1;
+    for (int r = 0; r < R; ++r) split_id[r] = (row_split > 0 && count[r] > row_split) ? n++ : -1;
     free(count);
     return n;
 }
@@ -172,12 +175,13 @@ static void bias_tiled(const float* V1, const float* V2, size_t stride, float* g
 
 /* gW[r,:] = chain over slots naming r of gout[b,:]; gbias = tiled column sum of gout. */
 int nnueft_oracle_sparse_bwd(const int32_t* idx, const float* gout, float* gW, float* gbias,
-                             int B, int K, int R, int out_cols)
+                             int B, int K, int R, int out_cols, int row_split)
 {
+    if (row_split < 0) return -1;
     memset(gW, 0, (size_t)R * out_cols * sizeof(float));
     int32_t* split_id = (int32_t*)malloc(sizeof(int32_t) * (size_t)R);
     if (!split_id) return -2;
-    const int nsplit = find_split_rows(idx, NULL, B, K, R, split_id);
+    const int nsplit = find_split_rows(idx, NULL, B, K, R, row_split, split_id);
     if (nsplit < 0) { free(split_id); return -2; }
     const int window = nnueft_oracle_row_window(B);
     int nblk = (out_cols + COLBLK - 1) / COLBLK;
@@ -309,9 +313,10 @@ int nnueft_oracle_double_bwd(const float* us, const float* them,
                              const float* bias, float max_act,
                              const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt,
                              const float* saved, float* gW, float* gbias,
-                             int B, int K, int R, int L1, int n_psqt)
+                             int B, int K, int R, int L1, int n_psqt, int row_split)
 {
     const int out_cols = L1 + n_psqt;
+    if (row_split < 0) return -1;
     float* G = (float*)malloc(sizeof(float) * 2 * (size_t)B * out_cols);
     float* accb = (float*)calloc((size_t)R * out_cols, sizeof(float));
     if (!G || !accb) { free(G); free(accb); return -2; }
@@ -320,7 +325,7 @@ int nnueft_oracle_double_bwd(const float* us, const float* them,
     if (rc) { free(G); free(accb); return rc; }
     memset(gW, 0, (size_t)R * out_cols * sizeof(float));
     int32_t* split_id = (int32_t*)malloc(sizeof(int32_t) * (size_t)R);
-    const int nsplit = split_id ? find_split_rows(widx, bidx, B, K, R, split_id) : -1;
+    const int nsplit = split_id ? find_split_rows(widx, bidx, B, K, R, row_split, split_id) : -1;
     if (nsplit < 0) { free(G); free(accb); free(split_id); return -2; }
     const int window = nnueft_oracle_row_window(B);
     int nblk = (out_cols + COLBLK - 1) / COLBLK;

@@ -39,7 +39,7 @@ def test_binding_covers_every_declared_symbol():
 
 def test_host_only_entry_points():
     lib = _native.load()
-    assert lib.nnueft_version() == 1
+    assert lib.nnueft_version() == 2
     assert lib.nnueft_bias_tile() == 32
     # the constants of the deterministic order are the oracle's
     from oracle import cpu as oracle_cpu
@@ -53,12 +53,15 @@ def test_host_only_entry_points():
     for code in (-1, -2, -3):
         assert lib.nnueft_error_string(code).startswith(b"nnueft:")
     # workspace size: monotone, 256-byte granular, zero for nonsense
-    a = lib.nnueft_det_workspace_bytes(16384, 32, 24576, 3080, 2)
-    b = lib.nnueft_det_workspace_bytes(16384, 32, 24576, 3080, 1)
+    a = lib.nnueft_det_workspace_bytes(16384, 32, 24576, 3080, 2, 512)
+    b = lib.nnueft_det_workspace_bytes(16384, 32, 24576, 3080, 1, 512)
+    strict = lib.nnueft_det_workspace_bytes(16384, 32, 24576, 3080, 2, 0)
     assert a > b > 0 and a % 256 == 0 and b % 256 == 0
-    assert a >= 2 * 16384 * 3080 * 4          # holds the two upstream rows of every position
-    assert lib.nnueft_det_workspace_bytes(0, 32, 10, 8, 1) == 0
-    assert lib.nnueft_det_workspace_bytes(4, 32, 10, 8, 3) == 0
+    assert a > strict >= 2 * 16384 * 3080 * 4   # holds the two upstream rows of every position; no window sums
+    assert lib.nnueft_det_workspace_bytes(16384, 32, 24576, 3080, 2, 256) > a      # more rows can be split
+    assert lib.nnueft_det_workspace_bytes(0, 32, 10, 8, 1, 512) == 0
+    assert lib.nnueft_det_workspace_bytes(4, 32, 10, 8, 3, 512) == 0
+    assert lib.nnueft_det_workspace_bytes(4, 32, 10, 8, 1, -1) == 0
 
 
 def test_check_raises_with_the_library_message():

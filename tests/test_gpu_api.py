@@ -135,6 +135,162 @@ def test_deterministic_backward_bits_equal_the_reference_cpu_path():
     torch.testing.assert_close(bg.grad.cpu(), bc.grad, atol=1e-4, rtol=1e-4)
 
 
+def _strict_vs_reference_cpu_path(L1, B, seed, **batch_kw):
+    """Forward and strict-order deterministic backward on the GPU against torch CPU autograd of the
+    reference's composition (oracle/ref_torch.py) on the same inputs; returns the two weight gradients."""
+    n_psqt, R = 8, hk.NUM_INPUTS
+    assert B * 32 >= 32768        # from this many slots per list on, torch's CPU backward adds in (position, slot) order
+    us, them, white, black, pc = hk.synthetic_batch(B, seed, **batch_kw)
+    g = torch.Generator().manual_seed(seed)
+    cpu = [torch.from_numpy(a) for a in (us, them, white, black, (pc - 1) // 4)]
+    W0 = torch.randn(R, L1 + n_psqt, generator=g) * 0.01
+    b0 = torch.randn(L1 + n_psqt, generator=g) * 0.01
+    grads = [torch.randn(B, L1, generator=g), torch.randn(B, 1, generator=g), torch.randn(B, 1, generator=g)]
+    max_act = 255.0 / 256.0
+    Wc, bc = W0.clone().requires_grad_(), b0.clone().requires_grad_()
+    out_c = ref_torch.double_feature_transform(*cpu, Wc, bc, max_act, L1)
+    torch.autograd.backward(list(out_c), grads)
+    nnueft.set_backward_mode("deterministic_strict")
+    Wg, bg = W0.to(DEV).requires_grad_(), b0.to(DEV).requires_grad_()
+    out_g = double_feature_transform(*[a.to(DEV) for a in cpu], Wg, bg, max_act, L1, "fused")
+    torch.autograd.backward(list(out_g), [x.to(DEV) for x in grads])
+    for a, b in zip(out_g, out_c):
+        assert torch.equal(a.detach().cpu(), b.detach())
+    torch.testing.assert_close(bg.grad.cpu(), bc.grad, atol=1e-4, rtol=1e-4)
+    counts = np.bincount(np.concatenate([white[white >= 0], black[black >= 0]]), minlength=R)
+    return Wg.grad.cpu(), Wc.grad, counts
+
+
+def test_strict_deterministic_backward_bits_equal_the_reference_cpu_path_at_config_1():
+    """BASELINE.json config 1 at full size (L1=1024, B=8192; 262144 slots per list): the strict mode's weight
+    gradient is torch CPU autograd's, bit for bit, rows named by more than nnueft_row_split() slots included."""
+    g_gpu, g_cpu, counts = _strict_vs_reference_cpu_path(1024, 8192, 1235)
+    assert (counts > _native.load().nnueft_row_split()).sum() >= 1       # rows the default mode would split
+    assert torch.equal(g_gpu, g_cpu)
+
+
+def test_strict_deterministic_backward_bits_equal_the_reference_cpu_path_on_game_like_lists():
+    """The same on lists with the bucket statistics of game positions: a few hundred table rows are named by
+    thousands of slots each."""
+    g_gpu, g_cpu, counts = _strict_vs_reference_cpu_path(256, 8192, 1236, game_like=True)
+    split = counts > _native.load().nnueft_row_split()
+    assert split.sum() >= 30 and counts.max() > 2000
+    assert torch.equal(g_gpu, g_cpu)
+    # the default mode on the same inputs: the same bits on the rows it leaves whole, rounding apart on the others
+    nnueft.set_backward_mode("deterministic")
+    us, them, white, black, pc = hk.synthetic_batch(8192, 1236, game_like=True)
+    g = torch.Generator().manual_seed(1236)
+    W0 = torch.randn(hk.NUM_INPUTS, 264, generator=g) * 0.01
+    b0 = torch.randn(264, generator=g) * 0.01
+    grads = [torch.randn(8192, 256, generator=g), torch.randn(8192, 1, generator=g), torch.randn(8192, 1, generator=g)]
+    Wg, bg = W0.to(DEV).requires_grad_(), b0.to(DEV).requires_grad_()
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    out = double_feature_transform(t(us), t(them), t(white), t(black), t((pc - 1) // 4), Wg, bg, 255.0 / 256.0, 256,
+                                   "fused")
+    torch.autograd.backward(list(out), [x.to(DEV) for x in grads])
+    windowed = Wg.grad.cpu()
+    whole = torch.from_numpy(~split)
+    assert torch.equal(windowed[whole], g_cpu[whole])
+    torch.testing.assert_close(windowed, g_cpu, atol=1e-4, rtol=1e-3)
+
+
+def test_reduce_rows_stage_equals_the_sparse_backward(oracle_cpu):
+    """nnueft_det_sort + nnueft_det_reduce_rows on G = gout is the weight gradient of nnueft_sparse_bwd_det."""
+    lib = _native.load()
+    B, K, R, oc = 3000, 32, 900, 264
+    c = sparse_case(41, B, oc, R, K, allow_holes=True)
+    c["idx"][np.random.default_rng(1).random((B, K)) < 0.1] = 17          # a row beyond the split threshold
+    idx, g = torch.from_numpy(c["idx"]).to(DEV), torch.from_numpy(c["g"]).to(DEV)
+    st = torch.cuda.current_stream().cuda_stream
+    for rs in (lib.nnueft_row_split(), 0):
+        nbytes = lib.nnueft_det_workspace_bytes(B, K, R, oc, 1, rs)
+        sbytes = lib.nnueft_det_sort_bytes(B, K, R, oc, 1)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
+        lists = torch.empty(sbytes, dtype=torch.uint8, device=DEV)
+        gW = torch.full((R, oc), float("nan"), device=DEV)
+        _native.check(lib.nnueft_det_sort(idx.data_ptr(), None, B, K, R, oc, 1, rs, lists.data_ptr(), sbytes, st), "sort")
+        for _ in range(2):        # the sorted block serves a second reduction
+            gW.fill_(float("nan"))
+            _native.check(lib.nnueft_det_reduce_rows(g.data_ptr(), gW.data_ptr(), B, K, R, oc, 1, rs, ws.data_ptr(),
+                                                     nbytes, lists.data_ptr(), st), "reduce_rows")
+            rW, _ = oracle_cpu.sparse_bwd(c["idx"], c["g"], R, row_split=rs)
+            assert np.array_equal(gW.cpu().numpy(), rW)
+
+
+def test_forward_and_deterministic_backward_under_graph_capture():
+    """The launch path of the operator inside one captured HIP graph: forward + deterministic backward (sort
+    inline, workspaces allocated before the capture), replayed with eager work and synchronisations between the
+    replays; every replay must give the bits of the eager run, also after the inputs changed in place."""
+    lib = _native.load()
+    L1, B, K, R, n_psqt = 256, 4096, 32, hk.NUM_INPUTS, 8
+    oc = L1 + n_psqt
+    rs = lib.nnueft_row_split()
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    batches = []
+    for seed in (50, 51):
+        us, them, white, black, pc = hk.synthetic_batch(B, seed, game_like=(seed == 51))
+        batches.append([t(us), t(them), t(white), t(black), t((pc - 1) // 4)])
+    g = torch.Generator().manual_seed(3)
+    W = (torch.randn(R, oc, generator=g) * 0.02).to(DEV)
+    bias = (torch.randn(oc, generator=g) * 0.02).to(DEV)
+    g_l0, g_wp, g_bp = (torch.randn(B, L1, generator=g).to(DEV), torch.randn(B, 1, generator=g).to(DEV),
+                        torch.randn(B, 1, generator=g).to(DEV))
+    cur = [x.clone() for x in batches[0]]            # the graph's input buffers
+    fbytes = lib.nnueft_fwd_workspace_bytes(B, K, R, L1, n_psqt)
+    dbytes = lib.nnueft_det_workspace_bytes(B, K, R, oc, 2, rs)
+    fws = torch.empty(fbytes, dtype=torch.uint8, device=DEV)
+    dws = torch.empty(dbytes, dtype=torch.uint8, device=DEV)
+
+    def outputs():
+        return (torch.empty(B, L1, device=DEV), torch.empty(B, device=DEV), torch.empty(B, device=DEV),
+                torch.empty(2, B, L1, device=DEV), torch.empty(R, oc, device=DEV), torch.empty(oc, device=DEV))
+
+    def launch(o, stream):
+        l0, wp, bp, saved, gW, gb = o
+        us, them, white, black, psqt = cur
+        _native.check(lib.nnueft_double_fwd(us.data_ptr(), them.data_ptr(), white.data_ptr(), black.data_ptr(),
+                                            psqt.data_ptr(), W.data_ptr(), bias.data_ptr(), 255.0 / 256.0, l0.data_ptr(),
+                                            wp.data_ptr(), bp.data_ptr(), saved.data_ptr(), B, K, R, L1, n_psqt,
+                                            fws.data_ptr(), fbytes, stream), "fwd")
+        _native.check(lib.nnueft_double_bwd_det(us.data_ptr(), them.data_ptr(), white.data_ptr(), black.data_ptr(),
+                                                psqt.data_ptr(), bias.data_ptr(), 255.0 / 256.0, g_l0.data_ptr(),
+                                                g_wp.data_ptr(), g_bp.data_ptr(), saved.data_ptr(), gW.data_ptr(),
+                                                gb.data_ptr(), B, K, R, L1, n_psqt, rs, dws.data_ptr(), dbytes, None,
+                                                stream, None), "bwd")
+
+    eager = []
+    for b in batches:                                  # also the first calls on the device, outside any capture
+        for dst, src in zip(cur, b):
+            dst.copy_(src)
+        o = outputs()
+        launch(o, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        eager.append([x.clone() for x in o])
+    assert not torch.equal(eager[0][4], eager[1][4])
+
+    captured = outputs()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            launch(captured, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    for replay in range(4):
+        which = replay % 2
+        for dst, src in zip(cur, batches[which]):
+            dst.copy_(src)
+        for x in captured:
+            x.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(captured, eager[which]):
+            assert torch.equal(got, want), f"replay {replay} differs from the eager run"
+        # the program's own eager work between replays
+        launch(outputs(), torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+
+
 FULL = [(1024, 8192), (128, 16384), (3072, 16384)]   # BASELINE.json configs 1-3
 
 
@@ -342,17 +498,19 @@ def test_abi_rejects_bad_arguments():
     assert lib.nnueft_sparse_fwd(0, p, p, p, 4, 8, 10, 8, st) == -1                 # null pointer
     assert lib.nnueft_double_fwd(p, p, p, p, p, p, p, 1.0, p, p, p, p, 4, 8, 10, 7, 1, None, 0, st) == -1    # odd L1
     assert lib.nnueft_double_fwd(p, p, p, p, p, p, p, 1.0, p, p, p, p, 4, 8, 10, 8, 0, p, 8, st) == -2       # workspace too small
-    assert lib.nnueft_sparse_bwd_det(p, p, p, p, 4, 8, 10, 8, p, 16, st) == -2      # workspace too small
-    assert lib.nnueft_sparse_bwd_det(p, p, p, p, 4, 8, 10, 8, 0, 1 << 20, st) == -2  # workspace missing
-    assert lib.nnueft_sparse_bwd_det(p, p, p, p, 4, 8, 10, 8, p + 4, 1 << 20, st) == -2  # misaligned
+    assert lib.nnueft_sparse_bwd_det(p, p, p, p, 4, 8, 10, 8, 512, p, 16, st) == -2      # workspace too small
+    assert lib.nnueft_sparse_bwd_det(p, p, p, p, 4, 8, 10, 8, 512, 0, 1 << 20, st) == -2  # workspace missing
+    assert lib.nnueft_sparse_bwd_det(p, p, p, p, 4, 8, 10, 8, 0, p + 4, 1 << 20, st) == -2  # misaligned
+    assert lib.nnueft_sparse_bwd_det(p, p, p, p, 4, 8, 10, 8, -1, p, 1 << 20, st) == -1   # negative row_split
     assert lib.nnueft_ft_int16_fwd(p, p, p, p, p, p, p, p, p, 4, 8, 10, 8, 8, 70000, 9, 0, None, 0, st) == -1   # clip_max
     # the entry points around the operator reject what they cannot run, before any launch
-    assert lib.nnueft_det_sort(p, p, 4, 8, 10, 8, 2, p, 16, st) == -2                # sorted block too small
-    assert lib.nnueft_det_sort(p, p, 4, 8, 10, 8, 2, p + 4, 1 << 20, st) == -2       # misaligned
-    assert lib.nnueft_det_sort(p, None, 4, 8, 10, 8, 2, p, 1 << 20, st) == -1        # two lists asked, one given
+    assert lib.nnueft_det_sort(p, p, 4, 8, 10, 8, 2, 512, p, 16, st) == -2                # sorted block too small
+    assert lib.nnueft_det_sort(p, p, 4, 8, 10, 8, 2, 0, p + 4, 1 << 20, st) == -2       # misaligned
+    assert lib.nnueft_det_sort(p, None, 4, 8, 10, 8, 2, 512, p, 1 << 20, st) == -1        # two lists asked, one given
+    assert lib.nnueft_det_reduce_rows(p, p, 4, 8, 10, 8, 2, 512, p, 1 << 30, None, st) == -2   # no sorted lists
     assert lib.nnueft_det_sort_bytes(4, 8, 10, 8, 3) == 0                            # one or two perspectives
-    assert lib.nnueft_double_bwd_det(p, p, p, p, p, p, 1.0, p, p, p, p, p, p, 4, 8, 10, 8, 0, p, 1 << 30, p + 4, st,
-                                     None) == -2                                      # sorted lists misaligned
+    assert lib.nnueft_double_bwd_det(p, p, p, p, p, p, 1.0, p, p, p, p, p, p, 4, 8, 10, 8, 0, 512, p, 1 << 30, p + 4,
+                                     st, None) == -2                                      # sorted lists misaligned
     assert lib.nnueft_ranger_lite_update_multi(None, 0, st) == -1
     assert lib.nnueft_sqr_crelu_fwd(p, p, p, 4, 1, 127.0, 1e-5, 1.0, 1.0, 1, st) == -1     # skip value needs 2 columns
     assert lib.nnueft_sqr_crelu_fwd(p, p, None, 4, 4, 0.0, 1e-5, 1.0, 1.0, 1, st) == -1    # grid without a scale

@@ -38,6 +38,23 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
+# The row_split argument of the deterministic entry points under test: the library's default unless a
+# test asks for another through the `row_split` fixture (0 = strict order, no row is split).
+_RS_OVERRIDE = None
+
+
+def RS(lib):
+    return lib.nnueft_row_split() if _RS_OVERRIDE is None else _RS_OVERRIDE
+
+
+@pytest.fixture(params=[None, 0, 100, 3000], ids=["split_default", "strict", "split_100", "split_3000"])
+def row_split(request):
+    global _RS_OVERRIDE
+    _RS_OVERRIDE = request.param
+    yield request.param
+    _RS_OVERRIDE = None
+
+
 SPARSE_SHAPES = [
     # B, out_cols, R, K
     (16, 128, 10, 32),      # reference tests/test_feature_transformer.py:36-40 (duplicates)
@@ -73,7 +90,7 @@ def test_sparse_backward_atomic(oracle_cpu, B, out_cols, R, K):
     gb = torch.zeros(out_cols, device=_dev())
     nat.check(lib.nnueft_sparse_bwd_atomic(idx.data_ptr(), g.data_ptr(), gW.data_ptr(), gb.data_ptr(), B, K, R,
                                            out_cols, _stream()), "sparse_bwd_atomic")
-    rW, rb = oracle_cpu.sparse_bwd(c["idx"], c["g"], R)
+    rW, rb = oracle_cpu.sparse_bwd(c["idx"], c["g"], R, row_split=_RS_OVERRIDE)
     assert _rel_err(gW.cpu().numpy(), rW) <= 1e-4
     assert _rel_err(gb.cpu().numpy(), rb) <= 1e-4
 
@@ -83,15 +100,15 @@ def test_sparse_backward_deterministic(oracle_cpu, B, out_cols, R, K):
     c = sparse_case(300 + B, B, out_cols, R, K, allow_holes=True)
     nat, lib = _native()
     idx, g = _t(c["idx"]), _t(c["g"])
-    nbytes = lib.nnueft_det_workspace_bytes(B, K, R, out_cols, 1)
+    nbytes = lib.nnueft_det_workspace_bytes(B, K, R, out_cols, 1, RS(lib))
     assert nbytes > 0
     ws = torch.empty(nbytes, dtype=torch.uint8, device=_dev())
     # poison the outputs: every element must be written
     gW = torch.full((R, out_cols), float("nan"), device=_dev())
     gb = torch.full((out_cols,), float("nan"), device=_dev())
     nat.check(lib.nnueft_sparse_bwd_det(idx.data_ptr(), g.data_ptr(), gW.data_ptr(), gb.data_ptr(), B, K, R,
-                                        out_cols, ws.data_ptr(), nbytes, _stream()), "sparse_bwd_det")
-    rW, rb = oracle_cpu.sparse_bwd(c["idx"], c["g"], R)
+                                        out_cols, RS(lib), ws.data_ptr(), nbytes, _stream()), "sparse_bwd_det")
+    rW, rb = oracle_cpu.sparse_bwd(c["idx"], c["g"], R, row_split=_RS_OVERRIDE)
     assert np.array_equal(gW.cpu().numpy(), rW)
     assert np.array_equal(gb.cpu().numpy(), rb)
 
@@ -189,35 +206,35 @@ def test_double_backward(oracle_cpu, B, L1, R, K, kw, mode):
         nat.check(lib.nnueft_double_bwd_atomic(*head, gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt, _stream()),
                   "double_bwd_atomic")
     else:
-        nbytes = lib.nnueft_det_workspace_bytes(B, K, R, out_cols, 2)
+        nbytes = lib.nnueft_det_workspace_bytes(B, K, R, out_cols, 2, RS(lib))
         ws = torch.empty(nbytes, dtype=torch.uint8, device=_dev())
         gW = torch.full((R, out_cols), float("nan"), device=_dev())
         gb = torch.full((out_cols,), float("nan"), device=_dev())
-        nat.check(lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt, ws.data_ptr(),
+        nat.check(lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt, RS(lib), ws.data_ptr(),
                                             nbytes, None, _stream(), None), "double_bwd_det")
         # the same with the sort on a second stream
         gW2 = torch.full((R, out_cols), float("nan"), device=_dev())
         gb2 = torch.full((out_cols,), float("nan"), device=_dev())
         aux = torch.cuda.Stream()
-        nat.check(lib.nnueft_double_bwd_det(*head, gW2.data_ptr(), gb2.data_ptr(), B, K, R, L1, n_psqt, ws.data_ptr(),
+        nat.check(lib.nnueft_double_bwd_det(*head, gW2.data_ptr(), gb2.data_ptr(), B, K, R, L1, n_psqt, RS(lib), ws.data_ptr(),
                                             nbytes, None, _stream(), aux.cuda_stream), "double_bwd_det")
         assert torch.equal(gW, gW2) and torch.equal(gb, gb2)
         # the same with lists sorted beforehand, used twice
         sbytes = lib.nnueft_det_sort_bytes(B, K, R, out_cols, 2)
         assert 0 < sbytes < nbytes
         lists = torch.full((sbytes,), 0x5A, dtype=torch.uint8, device=_dev())
-        nat.check(lib.nnueft_det_sort(d["widx"].data_ptr(), d["bidx"].data_ptr(), B, K, R, out_cols, 2,
+        nat.check(lib.nnueft_det_sort(d["widx"].data_ptr(), d["bidx"].data_ptr(), B, K, R, out_cols, 2, RS(lib),
                                       lists.data_ptr(), sbytes, _stream()), "det_sort")
         for _ in range(2):
             gW2.fill_(float("nan"))
             gb2.fill_(float("nan"))
             ws.fill_(0xC3)
-            nat.check(lib.nnueft_double_bwd_det(*head, gW2.data_ptr(), gb2.data_ptr(), B, K, R, L1, n_psqt,
+            nat.check(lib.nnueft_double_bwd_det(*head, gW2.data_ptr(), gb2.data_ptr(), B, K, R, L1, n_psqt, RS(lib),
                                                 ws.data_ptr(), nbytes, lists.data_ptr(), _stream(), None),
                       "double_bwd_det")
             assert torch.equal(gW, gW2) and torch.equal(gb, gb2)
     rW, rb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["bias"], c["max_act"],
-                                   c["g_l0"], c["g_wp"], c["g_bp"], saved.cpu().numpy(), R, n_psqt)
+                                   c["g_l0"], c["g_wp"], c["g_bp"], saved.cpu().numpy(), R, n_psqt, row_split=_RS_OVERRIDE)
     gW, gb = gW.cpu().numpy(), gb.cpu().numpy()
     if mode == "atomic":
         assert _rel_err(gW, rW) <= 1e-4
@@ -247,7 +264,7 @@ def _skewed_double_case(seed, B, L1, castled, fold=0):
 
 @pytest.mark.parametrize("B,L1,castled,fold", [(4096, 64, 1.0, 0), (6000, 256, 0.6, 96), (16384, 128, 0.5, 200),
                                                 (3000, 1024, 0.9, 40), (16384, 64, -1, 0), (5000, 3072, -1, 0)])
-def test_double_backward_deterministic_with_split_rows(oracle_cpu, B, L1, castled, fold):
+def test_double_backward_deterministic_with_split_rows(oracle_cpu, row_split, B, L1, castled, fold):
     c = _skewed_double_case(900 + B, B, L1, castled, fold)
     nat, lib = _native()
     R, K, n_psqt = c["R"], c["K"], c["n_psqt"]
@@ -256,24 +273,24 @@ def test_double_backward_deterministic_with_split_rows(oracle_cpu, B, L1, castle
     assert (counts > lib.nnueft_row_split()).sum() >= (8 if fold else 2) and B > lib.nnueft_row_window(B)
     d, l0, wp, bp, saved = _run_double_fwd(c)
     g_l0, g_wp, g_bp = _t(c["g_l0"]), _t(c["g_wp"]), _t(c["g_bp"])
-    nbytes = lib.nnueft_det_workspace_bytes(B, K, R, out_cols, 2)
+    nbytes = lib.nnueft_det_workspace_bytes(B, K, R, out_cols, 2, RS(lib))
     ws = torch.empty(nbytes, dtype=torch.uint8, device=_dev())
     gW = torch.full((R, out_cols), float("nan"), device=_dev())
     gb = torch.full((out_cols,), float("nan"), device=_dev())
     nat.check(lib.nnueft_double_bwd_det(d["us"].data_ptr(), d["them"].data_ptr(), d["widx"].data_ptr(),
                                         d["bidx"].data_ptr(), d["psqt_idx"].data_ptr(), d["bias"].data_ptr(),
                                         c["max_act"], g_l0.data_ptr(), g_wp.data_ptr(), g_bp.data_ptr(),
-                                        saved.data_ptr(), gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt,
+                                        saved.data_ptr(), gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt, RS(lib),
                                         ws.data_ptr(), nbytes, None, _stream(), torch.cuda.Stream().cuda_stream),
               "double_bwd_det")
     rW, rb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["bias"], c["max_act"],
-                                   c["g_l0"], c["g_wp"], c["g_bp"], saved.cpu().numpy(), R, n_psqt)
+                                   c["g_l0"], c["g_wp"], c["g_bp"], saved.cpu().numpy(), R, n_psqt, row_split=_RS_OVERRIDE)
     assert np.array_equal(gW.cpu().numpy(), rW)
     assert np.array_equal(gb.cpu().numpy(), rb)
     # lists sorted beforehand: same bits, also on the second use of the sorted block
     sbytes = lib.nnueft_det_sort_bytes(B, K, R, out_cols, 2)
     lists = torch.empty(sbytes, dtype=torch.uint8, device=_dev())
-    nat.check(lib.nnueft_det_sort(d["widx"].data_ptr(), d["bidx"].data_ptr(), B, K, R, out_cols, 2,
+    nat.check(lib.nnueft_det_sort(d["widx"].data_ptr(), d["bidx"].data_ptr(), B, K, R, out_cols, 2, RS(lib),
                                   lists.data_ptr(), sbytes, _stream()), "det_sort")
     for _ in range(2):
         gW2 = torch.full((R, out_cols), float("nan"), device=_dev())
@@ -281,7 +298,7 @@ def test_double_backward_deterministic_with_split_rows(oracle_cpu, B, L1, castle
         nat.check(lib.nnueft_double_bwd_det(d["us"].data_ptr(), d["them"].data_ptr(), d["widx"].data_ptr(),
                                             d["bidx"].data_ptr(), d["psqt_idx"].data_ptr(), d["bias"].data_ptr(),
                                             c["max_act"], g_l0.data_ptr(), g_wp.data_ptr(), g_bp.data_ptr(),
-                                            saved.data_ptr(), gW2.data_ptr(), gb2.data_ptr(), B, K, R, L1, n_psqt,
+                                            saved.data_ptr(), gW2.data_ptr(), gb2.data_ptr(), B, K, R, L1, n_psqt, RS(lib),
                                             ws.data_ptr(), nbytes, lists.data_ptr(), _stream(), None),
                   "double_bwd_det")
         assert torch.equal(gW, gW2) and torch.equal(gb, gb2)
@@ -290,20 +307,20 @@ def test_double_backward_deterministic_with_split_rows(oracle_cpu, B, L1, castle
 # (the last two tables are taller than the row scan stages at once: several passes, totals summed first)
 @pytest.mark.parametrize("B,out_cols,R,K", [(5000, 72, 40, 16), (9000, 37, 300, 8), (20000, 264, 64, 4),
                                             (3000, 8, 70001, 8), (2500, 12, 40000, 16)])
-def test_sparse_backward_deterministic_with_split_rows(oracle_cpu, B, out_cols, R, K):
+def test_sparse_backward_deterministic_with_split_rows(oracle_cpu, row_split, B, out_cols, R, K):
     c = sparse_case(950 + B, B, out_cols, R, K, allow_holes=True)
     rng = np.random.default_rng(B)
     c["idx"][rng.random((B, K)) < 0.3] = 3      # one row named by a third of all slots
     nat, lib = _native()
     assert B > lib.nnueft_row_window(B)
     idx, g = _t(c["idx"]), _t(c["g"])
-    nbytes = lib.nnueft_det_workspace_bytes(B, K, R, out_cols, 1)
+    nbytes = lib.nnueft_det_workspace_bytes(B, K, R, out_cols, 1, RS(lib))
     ws = torch.empty(nbytes, dtype=torch.uint8, device=_dev())
     gW = torch.full((R, out_cols), float("nan"), device=_dev())
     gb = torch.full((out_cols,), float("nan"), device=_dev())
     nat.check(lib.nnueft_sparse_bwd_det(idx.data_ptr(), g.data_ptr(), gW.data_ptr(), gb.data_ptr(), B, K, R,
-                                        out_cols, ws.data_ptr(), nbytes, _stream()), "sparse_bwd_det")
-    rW, rb = oracle_cpu.sparse_bwd(c["idx"], c["g"], R)
+                                        out_cols, RS(lib), ws.data_ptr(), nbytes, _stream()), "sparse_bwd_det")
+    rW, rb = oracle_cpu.sparse_bwd(c["idx"], c["g"], R, row_split=_RS_OVERRIDE)
     assert np.array_equal(gW.cpu().numpy(), rW)
     assert np.array_equal(gb.cpu().numpy(), rb)
 
@@ -315,7 +332,7 @@ def test_deterministic_backward_repeats_bitwise():
     B, K, R, L1, n_psqt = 300, 32, 600, 256, 8
     d, l0, wp, bp, saved = _run_double_fwd(c)
     g_l0, g_wp, g_bp = _t(c["g_l0"]), _t(c["g_wp"]), _t(c["g_bp"])
-    nbytes = lib.nnueft_det_workspace_bytes(B, K, R, L1 + n_psqt, 2)
+    nbytes = lib.nnueft_det_workspace_bytes(B, K, R, L1 + n_psqt, 2, RS(lib))
     outs = []
     for fill in (0.0, 123.0):
         ws = torch.full((nbytes,), int(fill) % 251, dtype=torch.uint8, device=_dev())
@@ -325,7 +342,7 @@ def test_deterministic_backward_repeats_bitwise():
                                             d["bidx"].data_ptr(), d["psqt_idx"].data_ptr(), d["bias"].data_ptr(),
                                             c["max_act"],
                                             g_l0.data_ptr(), g_wp.data_ptr(), g_bp.data_ptr(), saved.data_ptr(),
-                                            gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt, ws.data_ptr(), nbytes,
+                                            gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt, RS(lib), ws.data_ptr(), nbytes,
                                             None, _stream(), None), "double_bwd_det")
         outs.append((gW.cpu().numpy().copy(), gb.cpu().numpy().copy()))
     assert np.array_equal(outs[0][0], outs[1][0])

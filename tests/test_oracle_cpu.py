@@ -227,6 +227,71 @@ def test_double_backward_split_counts_both_perspectives_together(oracle_cpu):
     assert gW[2, L1] == BIG + 212.0
 
 
+def test_row_split_argument_selects_the_order(oracle_cpu):
+    B, K, R = 4096, 2, 5
+    W = oracle_cpu.row_window(B)
+    # 600 slots: position 0 carries 2**24, 299 ones follow in window 0, 300 ones in window 1
+    pos = np.r_[0:300, W:W + 300]
+    idx, g = _ones_after_big(B, K, R, 3, pos)
+    # strict order (0) and a threshold the row stays below: one plain chain, every 1.0 lost
+    for rs in (0, 600, 3000):
+        assert oracle_cpu.sparse_bwd(idx, g, R, row_split=rs)[0][3, 0] == BIG
+    # any threshold below the row's slot count splits it, the default included
+    for rs in (None, 512, 599, 100, 1):
+        assert oracle_cpu.sparse_bwd(idx, g, R, row_split=rs)[0][3, 0] == BIG + 300.0
+    # the same for the two-perspective gradient (300 white + 300 black slots, PSQT column)
+    widx = np.full((B, K), -1, np.int32)
+    bidx = np.full((B, K), -1, np.int32)
+    widx[np.r_[0:1, W:W + 299], 0] = 2
+    bidx[np.r_[0:1, W:W + 299], 0] = 2
+    one, zero = np.ones((B, 1), np.float32), np.zeros((B, 1), np.float32)
+    g_wp = np.ones((B, 1), np.float32)
+    g_wp[0, 0] = BIG
+    args = (one, zero, widx, bidx, np.zeros(B, np.int64), np.zeros(10, np.float32), 127.0, np.zeros((B, 8), np.float32),
+            g_wp, one, np.zeros((2, B, 8), np.float32), 4, 2)
+    assert oracle_cpu.double_bwd(*args, row_split=0)[0][2, 8] == BIG + 300.0          # white: ones lost; black: 300
+    assert oracle_cpu.double_bwd(*args, row_split=599)[0][2, 8] == BIG + 300.0 + 300.0  # white: 2**24 + 299 -> ties to even
+
+
+@pytest.mark.parametrize("B,oc,R,K", [(4096, 24, 500, 16), (3000, 40, 300, 32)])
+def test_strict_order_bits_equal_torch_cpu_autograd_with_crowded_rows(oracle_cpu, B, oc, R, K):
+    """row_split = 0 is the reference's CPU path for every row, also for rows named by thousands of slots
+    (which the default order sums window by window and therefore rounds differently)."""
+    assert B * K >= 32768
+    c = sparse_case(14, B, oc, R, K)
+    rng = np.random.default_rng(B)
+    c["idx"][rng.random((B, K)) < 0.25] = 5          # one row named by a quarter of all slots
+    assert (c["idx"] == 5).sum() > 8 * oracle_cpu.row_split()
+    W = torch.from_numpy(c["W"]).requires_grad_()
+    bias = torch.from_numpy(c["bias"]).requires_grad_()
+    ref_torch.sparse_linear(torch.from_numpy(c["idx"]), W, bias).backward(torch.from_numpy(c["g"]))
+    strict, _ = oracle_cpu.sparse_bwd(c["idx"], c["g"], R, row_split=0)
+    assert np.array_equal(strict, W.grad.numpy())
+    windowed, _ = oracle_cpu.sparse_bwd(c["idx"], c["g"], R)
+    assert not np.array_equal(windowed[5], strict[5])                  # the crowded row: another order
+    assert np.allclose(windowed[5], strict[5], rtol=1e-4, atol=1e-3)    # ... the same sum to rounding
+    counts = np.bincount(c["idx"][c["idx"] >= 0], minlength=R)
+    short = counts <= oracle_cpu.row_split()                           # rows the default order leaves whole
+    assert np.array_equal(windowed[short], strict[short])
+
+
+def test_strict_order_double_bits_equal_torch_cpu_autograd_with_crowded_rows(oracle_cpu):
+    from nnueft import halfka_v2_hm as hk
+
+    B, L1, R = 2048, 32, hk.NUM_INPUTS
+    c = double_case(23, B, L1, R, 32, halfka=True, weight_scale=0.05, max_act=255 / 256)
+    us, them, widx, bidx, pc = hk.synthetic_batch(B, 23, castled_kings=0.9)
+    c.update(us=us, them=them, widx=widx, bidx=bidx, psqt_idx=((pc - 1) // 4).astype(np.int64))
+    counts = np.bincount(np.concatenate([widx[widx >= 0], bidx[bidx >= 0]]), minlength=R)
+    assert counts.max() > 2 * oracle_cpu.row_split() and B * 32 >= 32768
+    W, bias, outs = _torch_double(c, need_grad=True)
+    torch.autograd.backward(list(outs), [torch.from_numpy(c[k]) for k in ("g_l0", "g_wp", "g_bp")])
+    _, _, _, saved = oracle_cpu.double_fwd(us, them, widx, bidx, c["psqt_idx"], c["W"], c["bias"], c["max_act"], L1)
+    gW, _ = oracle_cpu.double_bwd(us, them, widx, bidx, c["psqt_idx"], c["bias"], c["max_act"], c["g_l0"], c["g_wp"],
+                                  c["g_bp"], saved, R, c["n_psqt"], row_split=0)
+    assert np.array_equal(gW, W.grad.numpy())
+
+
 def test_bias_gradient_tile_order_brute_force(oracle_cpu):
     tile = oracle_cpu.bias_tile()
     rng = np.random.default_rng(2)
