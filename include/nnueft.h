@@ -5,8 +5,8 @@
  * library never allocates, frees or retains memory.  `stream` is a hipStream_t passed as void*
  * (NULL = the default stream); all work is enqueued on it and the call returns without waiting.
  * The library may be called from several host threads.  What it keeps between calls: per device,
- * a few facts queried once (LDS size, number of XCDs); per host thread and device, two events for
- * the two-stream backward.
+ * a few facts queried once (LDS size, number of XCDs) and the fixed scratch array of
+ * nnueft_double_fwd_noalloc; per host thread and device, two events for the two-stream backward.
  * After the first call on a device an entry point makes no calls but kernel launches and event
  * record / wait, so it can be recorded by a stream capture (make that first call before capturing).
  *
@@ -53,6 +53,7 @@ extern "C" {
 #define NNUEFT_E_ARG (-1)         /* null pointer, non-positive or inconsistent dimension, odd L1 */
 #define NNUEFT_E_WORKSPACE (-2)   /* workspace missing, misaligned (256 B) or smaller than nnueft_det_workspace_bytes() */
 #define NNUEFT_E_UNSUPPORTED (-3) /* a dimension beyond what the kernels index (see each entry point) */
+#define NNUEFT_E_SCRATCH (-4)     /* sizes beyond what the library's own fixed scratch memory holds (nnueft_double_fwd_noalloc) */
 
 int nnueft_version(void);
 const char* nnueft_error_string(int code);
@@ -158,6 +159,23 @@ int nnueft_double_fwd_act(const float* us, const float* them, const int32_t* wid
                           int B, int K, int R, int L1, int n_psqt,
                           void* workspace, size_t workspace_bytes,
                           float act_scale, float act_eps, float act_post_mul, void* stream);
+
+/*
+ * nnueft_double_fwd for callers that cannot allocate device memory or size a workspace (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the scratch memory of the
+ * L2-blocked gather (pair order, keys, per-workgroup histograms) is a fixed array inside the library,
+ * one copy per GPU, 2 MiB, held until the process ends.  Same arguments and results as
+ * nnueft_double_fwd minus the workspace; no counterpart in the reference.  The call allocates and
+ * frees nothing.  Limit: nnueft_fwd_workspace_bytes(B, K, R, L1, n_psqt) <= 2 MiB (B = 65536 with a
+ * 24576-row table fits), beyond it NNUEFT_E_SCRATCH.  All calls on one GPU share that GPU's array:
+ * calls that overlap in time on one GPU (two streams, two threads) race on it; calls on one stream
+ * are ordered and safe.  The first call on a device looks up the array's address (not a stream
+ * operation: make one call on each device before capturing a graph there).
+ */
+int nnueft_double_fwd_noalloc(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+                              const int64_t* psqt_idx, const float* W, const float* bias, float max_act,
+                              float* l0, float* wpsqt, float* bpsqt, float* saved,
+                              int B, int K, int R, int L1, int n_psqt, void* stream);
 
 /*
  * Gradient of nnueft_double_fwd with respect to W and bias, floating-point atomics.

@@ -13,6 +13,9 @@ extern "C" const char* nnueft_error_string(int code) {
         case NNUEFT_E_ARG: return "nnueft: invalid argument (null pointer, bad dimension or odd L1)";
         case NNUEFT_E_WORKSPACE: return "nnueft: workspace missing, not 256-byte aligned or too small";
         case NNUEFT_E_UNSUPPORTED: return "nnueft: dimension beyond what the kernels index";
+        case NNUEFT_E_SCRATCH:
+            return "nnueft: sizes beyond the library's fixed scratch memory (2 MiB: pass a workspace to "
+                   "nnueft_double_fwd instead)";
         default: break;
     }
     if (code > 0) return hipGetErrorString((hipError_t)code);

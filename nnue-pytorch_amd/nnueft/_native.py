@@ -44,6 +44,7 @@ PROTOTYPES = {
         c_int,
         [c_void_p] * 7 + [c_float] + [c_void_p] * 4 + [c_int] * 5 + [c_void_p, c_size_t] + [c_float] * 3 + [c_void_p],
     ),
+    "nnueft_double_fwd_noalloc": (c_int, [c_void_p] * 7 + [c_float] + [c_void_p] * 4 + [c_int] * 5 + [c_void_p]),
     "nnueft_double_bwd_atomic": (c_int, [c_void_p] * 6 + [c_float] + [c_void_p] * 6 + [c_int] * 5 + [c_void_p]),
     "nnueft_double_bwd_det": (
         c_int,

@@ -50,7 +50,7 @@ def test_host_only_entry_points():
         assert lib.nnueft_row_window(B) == oracle_cpu.row_window(B)
     assert lib.nnueft_row_window(0) == 0
     assert lib.nnueft_error_string(0) == b"success"
-    for code in (-1, -2, -3):
+    for code in (-1, -2, -3, -4):
         assert lib.nnueft_error_string(code).startswith(b"nnueft:")
     # workspace size: monotone, 256-byte granular, zero for nonsense
     a = lib.nnueft_det_workspace_bytes(16384, 32, 24576, 3080, 2, 512)

@@ -508,6 +508,8 @@ def test_abi_rejects_bad_arguments():
     assert lib.nnueft_det_sort(p, p, 4, 8, 10, 8, 2, 0, p + 4, 1 << 20, st) == -2       # misaligned
     assert lib.nnueft_det_sort(p, None, 4, 8, 10, 8, 2, 512, p, 1 << 20, st) == -1        # two lists asked, one given
     assert lib.nnueft_det_reduce_rows(p, p, 4, 8, 10, 8, 2, 512, p, 1 << 30, None, st) == -2   # no sorted lists
+    assert lib.nnueft_double_fwd_noalloc(p, p, p, p, p, p, p, 1.0, p, p, p, p, 4, 8, 10, 7, 1, st) == -1      # odd L1
+    assert lib.nnueft_double_fwd_noalloc(p, p, p, p, p, p, p, 1.0, p, p, p, p, 1 << 20, 8, 24576, 8, 0, st) == -4   # beyond the fixed scratch
     assert lib.nnueft_det_sort_bytes(4, 8, 10, 8, 3) == 0                            # one or two perspectives
     assert lib.nnueft_double_bwd_det(p, p, p, p, p, p, 1.0, p, p, p, p, p, p, 4, 8, 10, 8, 0, 512, p, 1 << 30, p + 4,
                                      st, None) == -2                                      # sorted lists misaligned
