@@ -6,14 +6,17 @@ A step is one pass of the hot path over one synthetic batch: the fused two-persp
 function the trainer calls.  Inputs are resident in HBM before the timed region.
 
 Prints ONE JSON line: positions/s for the workload BASELINE.json's metric is quoted on (L1=3072,
-B=16384, HalfKAv2_hm lists, 24576-row table), the roofline of the backward entry point (the dominant
-launch of the step; `roofline_forward` is the forward's) from HIP event timings, and the reference's
-CPU path (torch embedding_bag composition) timed on the host cores on a bounded sample of the same
-workload.
+B=16384, HalfKAv2_hm lists, 24576-row table); the roofline of the dominant kernel (k_seg_reduce, the
+segmented reduction of the deterministic backward) from HIP event timings of the entry point that
+launches it alone, against three bounds (algorithmic bytes against the L2 line rate that serves them,
+the bytes that must cross HBM, and the counter-measured traffic read from profiles/); the same for the
+two entry points and the step; and the reference's CPU path (torch embedding_bag composition) timed on
+the host cores on the same workload.
 """
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -22,14 +25,10 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "nnue-pytorch_amd"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
-
-# Bytes that crossed the L2 boundary per call of an entry point (FETCH_SIZE x2.0 + WRITE_SIZE x1.0 summed over its
-# kernels, the scale being what the same counters read for a 1 GiB torch.add), uniform positions:
-# profiles/ft_fwd_bwd_L1_3072_B16384_pmc.txt
-MEASURED_TRAFFIC = {
-    ("ft_fwd_bwd_L1_3072_B16384", "forward"): 1.46e9,
-    ("ft_fwd_bwd_L1_3072_B16384", "deterministic"): 2.69e9,
-}
+# L2: 8 XCDs x 16 channels, one 128-byte line per channel and clock, at the published peak engine clock
+L2_CHANNELS = 128
+L2_LINE_BYTES = 128
+ENGINE_CLOCK_GHZ = 2.4
 
 WORKLOADS = {
     # name: (L1, B)
@@ -38,11 +37,16 @@ WORKLOADS = {
     "ft_fwd_bwd_L1_128_B16384": (128, 16384),       # config 2
     "ft_int16_fwd_L1_3072_B65536": (3072, 65536),   # config 5: quantized forward only
     "full_step_L1_3072_B16384": (3072, 16384),      # config 4: FT + layer stacks + loss + optimizer
+    "ref_microbench_L1_264_B8192": (264, 8192),     # the reference's own tests/bench_feature_transformer.py
 }
 R_ROWS = 24576
 N_PSQT = 8
 K_SLOTS = 32
+MAX_ACT = 255.0 / 256.0
 
+
+# ------------------------------------------------------------------------------------------------
+# byte counts
 
 def algorithmic_bytes(L1, B, sum_a, mode):
     """Logical bytes of one step, no reuse between positions assumed (a = active rows of both lists)."""
@@ -57,13 +61,78 @@ def algorithmic_bytes(L1, B, sum_a, mode):
     return fwd, bwd
 
 
+def seg_reduce_bytes(L1, B, sum_a):
+    """k_seg_reduce's part of the deterministic backward's formula: (algorithmic, of which gathered rows,
+    compulsory).  Algorithmic: one upstream row per slot + the slot's list entry + every table row written
+    once.  Compulsory: the upstream rows once, the list, the dense gradient."""
+    oc = L1 + N_PSQT
+    gathered = sum_a * oc * 4
+    alg = gathered + sum_a * 4 + R_ROWS * oc * 4
+    comp = 2 * B * oc * 4 + sum_a * 4 + (R_ROWS + 1) * 8 + R_ROWS * oc * 4
+    return alg, gathered, comp
+
+
+def compulsory_bytes(L1, B, sum_a):
+    """Bytes that have to cross HBM once per kernel that reads or writes them, with this decomposition into
+    kernels and nothing kept in a cache between kernels: per entry point."""
+    oc = L1 + N_PSQT
+    lists = 2 * B * K_SLOTS * 4
+    saved = 2 * B * L1 * 4
+    small = B * 24
+    fwd = {
+        "pair sort": lists + 3 * 2 * B * 4,
+        "k_acc_blocked": R_ROWS * oc * 4 + lists + saved,             # table once, row sums written
+        "k_mix": saved + B * L1 * 4 + small,                          # row sums read, l0 written
+    }
+    nchunks = 2 * ((B + 127) // 128)
+    bwd = {
+        "k_bwd_rows": saved + B * L1 * 4 + 2 * B * oc * 4 + small,    # row sums + grad_l0 read, upstream rows written
+        "sort": 2 * lists + 3 * nchunks * R_ROWS * 4 + sum_a * 4,     # lists twice, chunk counts w/r/w, sorted list
+        "k_seg_reduce": seg_reduce_bytes(L1, B, sum_a)[2],
+        "bias": 2 * (B // 32) * oc * 4,
+    }
+    return fwd, bwd
+
+
+def read_profile_traffic(workload, positions):
+    """Counter-measured bytes per dispatch (FETCH_SIZE, WRITE_SIZE scaled by a copy kernel of known size) from the
+    tracked summary profiles/<workload>[_game_like]_pmc.txt: lines `traffic <kernel> fetched_bytes=N written_bytes=N`."""
+    name = workload + ("_game_like" if positions == "game" else "") + "_pmc.txt"
+    path = os.path.join(ROOT, "profiles", name)
+    out = {}
+    if not os.path.exists(path):
+        return out, None
+    for line in open(path):
+        m = re.match(r"traffic\s+(\S+)\s+fetched_bytes=(\d+)\s+written_bytes=(\d+)", line)
+        if m:
+            out[m.group(1)] = (int(m.group(2)), int(m.group(3)))
+    return out, os.path.relpath(path, ROOT)
+
+
+def sum_traffic(traffic, kernels):
+    """Total of the named kernels (prefix match on the kernel name), or None when one is missing."""
+    total = 0
+    for k in kernels:
+        hit = [v for name, v in traffic.items() if name.startswith(k)]
+        if not hit:
+            return None
+        total += sum(f + w for f, w in hit)
+    return total
+
+
+FWD_KERNELS = ("k_pair_hist", "k_pair_scan", "k_pair_scatter", "k_acc_blocked", "k_mix")
+BWD_KERNELS = ("k_bwd_rows", "k_chunk_hist", "k_col_scan", "k_row_scan", "k_fill", "k_seg_reduce", "k_split_combine",
+               "k_bias_final")
+
+
+# ------------------------------------------------------------------------------------------------
+# inputs
+
 def make_inputs(L1, B, seed, device, positions="uniform"):
-    import numpy as np
     import torch
     from nnueft import halfka_v2_hm as hk
 
     us, them, white, black, pc = hk.synthetic_batch(B, seed, game_like=(positions == "game"))
-    rng = np.random.default_rng(seed)
     oc = L1 + N_PSQT
     g = torch.Generator(device="cpu").manual_seed(seed)
     W = (torch.randn(R_ROWS, oc, generator=g) * 0.01)
@@ -77,47 +146,88 @@ def make_inputs(L1, B, seed, device, positions="uniform"):
         "g_bp": torch.randn(B, 1, generator=g),
     }
     sum_a = int((white >= 0).sum() + (black >= 0).sum())
-    del rng
     if device is not None:
         t = {k: v.to(device) for k, v in t.items()}
     return t, sum_a
 
 
-def cpu_baseline(L1, B_full, seed, budget_s=20.0):
-    """The reference's CPU path (oracle.ref_torch) on a sample of the workload's positions."""
+def host_threads():
+    """Threads for the CPU leg: the cores this process may run on, and not more than the share the job was given
+    (OMP_NUM_THREADS is that share where a scheduler sets it; on a shared host the affinity mask alone overstates it)."""
+    affinity = len(os.sched_getaffinity(0))
+    share = os.environ.get("OMP_NUM_THREADS", "")
+    threads = min(affinity, int(share)) if share.isdigit() and int(share) > 0 else affinity
+    return affinity, threads
+
+
+def cpu_baseline(workloads, seed, budget_s=12.0):
+    """The reference's CPU path (oracle.ref_torch: the torch embedding_bag composition, autograd backward) on the
+    whole batch of each workload: 3 warm-up steps, then at least 10 timed steps (fewer only when `budget_s` runs out)."""
     import torch
     from oracle import ref_torch
 
-    cores = len(os.sched_getaffinity(0))
-    cores = min(cores, 16) if os.environ.get("GRAFT_REPO_ROOT") else cores
-    torch.set_num_threads(cores)
-    B = min(B_full, 4096)
-    t, _ = make_inputs(L1, B_full, seed, None)
-    sl = slice(0, B)
-    W = t["W"].clone().requires_grad_()
-    bias = t["bias"].clone().requires_grad_()
+    affinity, threads = host_threads()
+    torch.set_num_threads(threads)
+    runs = []
+    for name in workloads:
+        L1, B = WORKLOADS[name]
+        t, _ = make_inputs(L1, B, seed, None)
+        W = t["W"].clone().requires_grad_()
+        bias = t["bias"].clone().requires_grad_()
 
-    def step():
-        W.grad = None
-        bias.grad = None
-        out = ref_torch.double_feature_transform(t["us"][sl], t["them"][sl], t["white"][sl], t["black"][sl],
-                                                 t["psqt_idx"][sl], W, bias, 255.0 / 256.0, L1)
-        torch.autograd.backward(list(out), [t["g_l0"][sl], t["g_wp"][sl], t["g_bp"][sl]])
+        def step():
+            W.grad = None
+            bias.grad = None
+            out = ref_torch.double_feature_transform(t["us"], t["them"], t["white"], t["black"], t["psqt_idx"], W,
+                                                     bias, MAX_ACT, L1)
+            torch.autograd.backward(list(out), [t["g_l0"], t["g_wp"], t["g_bp"]])
 
-    step()  # warm-up
-    n, t0 = 0, time.perf_counter()
-    while True:
-        step()
-        n += 1
-        el = time.perf_counter() - t0
-        if el > budget_s or n >= 8:
-            break
+        for _ in range(3):
+            step()
+        n, t0 = 0, time.perf_counter()
+        while True:
+            step()
+            n += 1
+            el = time.perf_counter() - t0
+            if (n >= 10 and el > 2.0) or el > budget_s:
+                break
+        runs.append({"workload": name, "positions_per_s": B * n / el, "ms_per_step": el / n * 1e3, "steps": n,
+                     "warmup": 3, "batch": B})
+    head = runs[0]
     return {
-        "value": B * n / el, "unit": "positions/s", "cores": cores, "kind": "port",
-        "sample": f"first {B} positions of the {B_full}-position batch, same 24576x{L1 + N_PSQT} table, "
-                  f"{n} fwd+bwd steps of the torch embedding_bag composition (autograd backward), 1 warm-up",
+        "value": head["positions_per_s"], "unit": "positions/s", "cores": threads, "kind": "port",
+        "affinity_cores": affinity, "threads_used": threads,
+        "sample": f"the whole {head['batch']}-position batch of {head['workload']} (same seeded lists, 24576-row table), "
+                  f"{head['steps']} fwd+bwd steps of the torch embedding_bag composition with autograd backward after 3 "
+                  f"warm-ups, torch.set_num_threads({threads}) of {affinity} cores in the affinity mask",
+        "runs": runs,
     }
 
+
+def time_steps(fn, steps, warmup):
+    """(wall ms per call, HIP-event ms per call); events on torch's current stream, the one every launch here uses."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall / steps * 1e3, e0.elapsed_time(e1) / steps
+
+
+def l2_peak_gbs():
+    return L2_CHANNELS * L2_LINE_BYTES * ENGINE_CLOCK_GHZ
+
+
+# ------------------------------------------------------------------------------------------------
+# other workloads
 
 def run_int16(args, lib, dev):
     """Quantized forward (BASELINE.json config 5): int16 gather-accumulate, clip, product >> 9 -> u8."""
@@ -154,21 +264,14 @@ def run_int16(args, lib, dev):
         x_u8, psqt = quantized.ft_int16_forward(wi, bi, stm, w16, b16, p32, pi)
         return quantized.stack_int8_forward(x_u8, pi, *stack_q) + psqt
 
-    def timed(fn):
-        for _ in range(args.warmup):
-            fn()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(args.steps):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / args.steps
-
-    ms = timed(step)
-    ms_chain = timed(chain)
-    alg = sum_a * L1 * 2 + B * (2 * K_SLOTS * 4 + L1)
+    _, ms = time_steps(step, args.steps, args.warmup)
+    _, ms_chain = time_steps(chain, args.steps, args.warmup)
+    gathered = sum_a * L1 * 2
+    alg = gathered + B * (2 * K_SLOTS * 4 + L1)
+    # table once, lists by both kernels, white sums written and read, u8 out
+    comp = R * L1 * 2 + R * N_PSQT * 4 + 2 * B * K_SLOTS * 4 * 2 + 2 * B * L1 * 2 + B * L1
+    l2_peak = l2_peak_gbs()
+    gbs = alg / (ms * 1e-3) / 1e9
     print(json.dumps({
         "metric": "quantized FT forward positions/sec (int16 accumulate, L1=3072, B=65536)",
         "value": B / (ms * 1e-3), "unit": "positions/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -177,9 +280,14 @@ def run_int16(args, lib, dev):
         "config": {"workload": args.workload, "L1": L1, "batch": B, "table_rows": R,
                    "active_rows_per_position": sum_a / B,
                    "with_int8_layer_stacks_ms": ms_chain, "with_int8_layer_stacks_positions_per_s": B / (ms_chain * 1e-3)},
-        "roofline": {"kernel": "nnueft_ft_int16_fwd", "bound": "hbm", "achieved": alg / (ms * 1e-3) / 1e9,
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "traffic": None, "algorithmic_bytes_per_launch": alg, "avg_launch_ms": ms},
+        "roofline": {"kernel": "nnueft_ft_int16_fwd: k_acc16_white + k_black_mix16 (+ pair sort)", "bound": "l2",
+                     "achieved": gbs, "peak": l2_peak, "unit": "GB/s", "frac": gbs / l2_peak, "traffic": None,
+                     "algorithmic_bytes_per_launch": alg, "avg_launch_ms": ms,
+                     "achieved_over_hbm_peak": gbs / HBM_PEAK_GBS,
+                     "note": "the gathered rows are served from the per-XCD L2s (blocked gather), so the algorithmic "
+                             "rate is held against the L2 line rate; the HBM-side figure is roofline_compulsory"},
+        "roofline_compulsory": {"bound": "hbm", "bytes_per_launch": comp, "achieved": comp / (ms * 1e-3) / 1e9,
+                                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": comp / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
         "cpu_baseline": None,
     }))
 
@@ -241,6 +349,60 @@ def run_full_step(args, dev):
     }))
 
 
+def run_ref_microbench(args, dev):
+    """The reference's own micro-benchmark, tests/bench_feature_transformer.py:22-25,57-133: B=8192, row width 264,
+    24 sorted random indices over the whole table + 8 pads per list; the bare sparse-linear function under
+    clamp/mean/backward, then the composed feature transformer (fake-quantized weights and activations) with the
+    fused backend.  Same loop, same positions/s figure it prints."""
+    import torch
+    import nnueft
+    from nnueft import model as M
+    from nnueft.sparse_linear_functions import SparseLinearFunction
+
+    stride, B = WORKLOADS[args.workload]
+    nnueft.set_backward_mode(args.backward)
+    torch.manual_seed(0)
+    quant = M.QuantizationManager(M.QuantizationConfig())
+    ft = M.ComposedFeatureTransformer(M.get_feature_cls("HalfKAv2_hm^"), stride, num_psqt_buckets=8,
+                                      quantization=quant).to(dev)
+    n_in, k = ft.NUM_INPUTS, ft.MAX_ACTIVE_FEATURES
+
+    def fake_indices():
+        r = torch.randint(0, n_in, (B, k * 3 // 4), dtype=torch.int32, device=dev)
+        r, _ = torch.sort(r, dim=1)
+        return torch.cat([r, torch.full((B, k // 4), -1, dtype=torch.int32, device=dev)], dim=1)
+
+    i0, i1 = fake_indices(), fake_indices()
+    us = torch.randint(0, 2, (B, 1), device=dev).float()
+    them = 1.0 - us
+    psqt = (torch.randint(1, 32, (B,), dtype=torch.int64, device=dev) - 1) // 4
+    weight = torch.randn(n_in, stride, device=dev, requires_grad=True)
+    bias = torch.randn(stride, device=dev, requires_grad=True)
+
+    def direct():
+        out = torch.clamp(SparseLinearFunction.apply(i0, weight, bias), 0.0, 1.0)
+        out.mean().backward()
+
+    def composed():
+        l0, wp, bp = ft(us, them, i0, i1, psqt, fake_quantize_acts=True, fake_quantize_weights=True, backend="fused")
+        (l0.sum() + wp.sum() + bp.sum()).backward()
+
+    iters, warm = max(args.steps, 64), max(args.warmup, 10)
+    ms_direct, _ = time_steps(direct, iters, warm)
+    ms_composed, _ = time_steps(composed, iters, warm)
+    print(json.dumps({
+        "metric": "reference micro-benchmark (tests/bench_feature_transformer.py): positions/sec, B=8192, row width 264",
+        "value": B / (ms_composed * 1e-3), "unit": "positions/s", "n_gpus": 1, "steps": iters, "warmup": warm,
+        "ms_per_step": ms_composed, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "batch": B, "row_width": stride, "backward": args.backward,
+                   "indices": "24 sorted uniform indices over the whole table + 8 pads per list",
+                   "composed_feature_transformer_fused": {"ms": ms_composed, "positions_per_s": B / (ms_composed * 1e-3)},
+                   "direct_sparse_linear_function": {"ms": ms_direct, "positions_per_s": B / (ms_direct * 1e-3)}},
+        "roofline": None, "cpu_baseline": None,
+    }))
+
+
 def run_handoff(args, dev):
     """The step before the path: batches in host memory laid out as the loader leaves them, staged and
     copied to the GPU by nnueft.batch_handoff, feeding the same forward+backward step.  Reports the cost
@@ -283,8 +445,7 @@ def run_handoff(args, dev):
         us, them, white, black, outcome, score, piece_count = t
         W.grad = None
         bias.grad = None
-        out = double_feature_transform(us, them, white, black, (piece_count - 1) // 4, W, bias, 255.0 / 256.0, L1,
-                                       "fused")
+        out = double_feature_transform(us, them, white, black, (piece_count - 1) // 4, W, bias, MAX_ACT, L1, "fused")
         torch.autograd.backward(list(out), [g_l0, g_p, g_p])
 
     def rate(source, n):
@@ -318,146 +479,135 @@ def run_handoff(args, dev):
     }))
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="ft_fwd_bwd_L1_3072_B16384", choices=sorted(WORKLOADS))
-    ap.add_argument("--backward", default="deterministic", choices=["deterministic", "atomic"],
-                    help="backward mode the headline value is measured with (the other one is reported beside it)")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--optimizer", default="rangerlite", choices=["rangerlite", "adam"],
-                    help="full_step workload only")
-    ap.add_argument("--compile", default="", choices=["", "inductor", "aot_eager", "cudagraphs"],
-                    help="full_step workload only: torch.compile the model with this backend, as the reference's "
-                         "train.py does (the kernels of this build stay opaque to it); off by default")
-    ap.add_argument("--sort-placement", default="inline", choices=["inline", "backward", "forward"],
-                    help="where the index sort of the deterministic backward runs (nnueft.set_sort_placement); "
-                         "the default is the library's")
-    ap.add_argument("--positions", default="uniform", choices=["uniform", "game"],
-                    help="uniform: kings and pieces uniform over the board (the headline workload); game: piece "
-                         "placement statistics of real game positions, where one or two king buckets hold a large "
-                         "part of the batch (halfka_v2_hm.game_like_positions); a default run times both")
-    ap.add_argument("--only", default="", choices=["", "fwd", "det", "atomic", "copy", "handoff"],
-                    help="run only this part (for profiling runs); 'copy' launches a plain elementwise kernel "
-                         "reading and writing 1 GiB each, the yardstick the FETCH_SIZE/WRITE_SIZE counters are scaled by")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
-        sys.exit(2)
+# ------------------------------------------------------------------------------------------------
+# the feature-transformer workloads (configs 1-3)
 
+def bound_block(kernel, ms, alg_bytes, gathered_bytes, comp_bytes, traffic_bytes, l2_peak, note=None):
+    """One launch against its three yardsticks."""
+    s = ms * 1e-3
+    alg_gbs = alg_bytes / s / 1e9
+    out = {
+        "kernel": kernel, "avg_launch_ms": ms,
+        # the algorithmic bytes are served by L2 (the gathers are blocked for it), so that is the bound they are held to
+        "bound": "l2", "achieved": alg_gbs, "peak": l2_peak, "unit": "GB/s", "frac": alg_gbs / l2_peak,
+        "algorithmic_bytes_per_launch": alg_bytes, "achieved_over_hbm_peak": alg_gbs / HBM_PEAK_GBS,
+        "l2_lines_per_clock_per_channel": gathered_bytes / s / 1e9 / l2_peak if gathered_bytes else None,
+        "traffic": traffic_bytes,
+        "traffic_GBs": traffic_bytes / s / 1e9 if traffic_bytes else None,
+        "traffic_frac_of_hbm_peak": traffic_bytes / s / 1e9 / HBM_PEAK_GBS if traffic_bytes else None,
+    }
+    if note:
+        out["note"] = note
+    comp = {"kernel": kernel, "bound": "hbm", "bytes_per_launch": comp_bytes, "achieved": comp_bytes / s / 1e9,
+            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": comp_bytes / s / 1e9 / HBM_PEAK_GBS,
+            "ms_at_peak": comp_bytes / (HBM_PEAK_GBS * 1e9) * 1e3}
+    return out, comp
+
+
+def run_ft(args, lib, dev):
     import torch
     import nnueft
-    from nnueft import _native
     from nnueft.double_ft_functions import double_feature_transform
 
-    nnueft.set_sort_placement(args.sort_placement)
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU", file=sys.stderr)
-        sys.exit(2)
-    lib = _native.load()  # raises if libnnueft.so is missing: there is no fallback
-    dev = torch.device("cuda:0")
-    if args.workload.startswith("ft_int16"):
-        run_int16(args, lib, dev)
-        return
-    if args.workload.startswith("full_step"):
-        run_full_step(args, dev)
-        return
-    if args.only == "copy":
-        n = (1 << 30) // 4
-        src = torch.ones(n, device=dev)
-        dst = torch.empty(n, device=dev)
-        for _ in range(args.warmup + args.steps):
-            torch.add(src, 1.0, out=dst)
-        torch.cuda.synchronize()
-        print(json.dumps({"calibration": "torch.add(src, 1.0, out=dst)", "read_bytes": n * 4, "write_bytes": n * 4,
-                          "launches": args.warmup + args.steps}))
-        return
-    if args.only == "handoff":
-        run_handoff(args, dev)
-        return
     L1, B = WORKLOADS[args.workload]
+    oc = L1 + N_PSQT
     seed = 1234 + 3
     t, sum_a = make_inputs(L1, B, seed, dev, args.positions)
     W = t["W"].requires_grad_()
     bias = t["bias"].requires_grad_()
-    max_act = 255.0 / 256.0
+    l2_peak = l2_peak_gbs()
 
     def step(mode, t=t):
         nnueft.set_backward_mode(mode)
         W.grad = None
         bias.grad = None
         out = double_feature_transform(t["us"], t["them"], t["white"], t["black"], t["psqt_idx"], W, bias,
-                                       max_act, L1, "fused")
+                                       MAX_ACT, L1, "fused")
         torch.autograd.backward(list(out), [t["g_l0"], t["g_wp"], t["g_bp"]])
 
-    def time_steps(fn, steps, warmup):
-        for _ in range(warmup):
-            fn()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        t0 = time.perf_counter()
-        e0.record()
-        for _ in range(steps):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        return wall / steps * 1e3, e0.elapsed_time(e1) / steps
-
+    all_modes = ("deterministic", "deterministic_strict", "atomic")
+    modes = [args.backward] + [m for m in all_modes if m != args.backward]
+    only_mode = {"det": "deterministic", "strict": "deterministic_strict", "atomic": "atomic"}.get(args.only)
+    if only_mode:
+        modes = [only_mode]
     results = {}
-    modes = [args.backward] + [m for m in ("deterministic", "atomic") if m != args.backward]
-    if args.only in ("det", "atomic"):
-        modes = ["deterministic" if args.only == "det" else "atomic"]
-    if args.only != "fwd":
+    if args.only not in ("fwd", "reduce"):
         for mode in modes:
-            ms_wall, ms_ev = time_steps(lambda: step(mode), args.steps, args.warmup)
+            ms_wall, _ = time_steps(lambda: step(mode), args.steps, args.warmup)
             results[mode] = ms_wall
 
-    # the forward kernel alone (one launch per call), HIP events on the launch stream
-    B_, K_ = t["white"].shape
+    # the entry points alone, HIP events on the launch stream
+    K_ = K_SLOTS
     l0 = torch.empty(B, L1, device=dev)
     wp = torch.empty(B, 1, device=dev)
     bp = torch.empty(B, 1, device=dev)
     saved = torch.empty(2, B, L1, device=dev)
-    fwd_ws_bytes = lib.nnueft_fwd_workspace_bytes(B, K_SLOTS, R_ROWS, L1, N_PSQT)
+    fwd_ws_bytes = lib.nnueft_fwd_workspace_bytes(B, K_, R_ROWS, L1, N_PSQT)
     fwd_ws = torch.empty(fwd_ws_bytes, dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
     Wd, bd = W.detach(), bias.detach()
+    n_entry = max(args.steps, 10)
 
     def fwd_only():
         rc = lib.nnueft_double_fwd(t["us"].data_ptr(), t["them"].data_ptr(), t["white"].data_ptr(),
                                    t["black"].data_ptr(), t["psqt_idx"].data_ptr(), Wd.data_ptr(), bd.data_ptr(),
-                                   max_act, l0.data_ptr(), wp.data_ptr(), bp.data_ptr(), saved.data_ptr(),
+                                   MAX_ACT, l0.data_ptr(), wp.data_ptr(), bp.data_ptr(), saved.data_ptr(),
                                    B, K_, R_ROWS, L1, N_PSQT, fwd_ws.data_ptr(), fwd_ws_bytes, stream)
         assert rc == 0
 
-    _, fwd_ms = time_steps(fwd_only, max(args.steps, 10), args.warmup)
+    _, fwd_ms = time_steps(fwd_only, n_entry, args.warmup)
 
-    # the backward entry points alone
     bwd_ms = {}
     if args.only != "fwd":
         g_l0, g_wp, g_bp = t["g_l0"], t["g_wp"], t["g_bp"]
-        oc = L1 + N_PSQT
-        row_split = lib.nnueft_row_split()
-        nbytes = lib.nnueft_det_workspace_bytes(B, K_, R_ROWS, oc, 2, row_split)
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
         gW = torch.empty(R_ROWS, oc, device=dev)
         gb = torch.empty(oc, device=dev)
         head = (t["us"].data_ptr(), t["them"].data_ptr(), t["white"].data_ptr(), t["black"].data_ptr(),
-                t["psqt_idx"].data_ptr(), bd.data_ptr(), max_act, g_l0.data_ptr(), g_wp.data_ptr(), g_bp.data_ptr(),
+                t["psqt_idx"].data_ptr(), bd.data_ptr(), MAX_ACT, g_l0.data_ptr(), g_wp.data_ptr(), g_bp.data_ptr(),
                 saved.data_ptr())
 
-        from nnueft.sparse_linear_functions import _aux_stream_ptr
+        from nnueft.sparse_linear_functions import _aux_stream_ptr, row_split_of
 
         # the entry point as FusedDoubleFtFunction calls it under this sort placement
         aux_stream = _aux_stream_ptr(dev) if args.sort_placement == "backward" else None
 
-        def bwd_det():
-            rc = lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT, row_split,
-                                           ws.data_ptr(), nbytes, None, stream, aux_stream)
-            assert rc == 0
+        def det_entry(row_split):
+            nbytes = lib.nnueft_det_workspace_bytes(B, K_, R_ROWS, oc, 2, row_split)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            sbytes = lib.nnueft_det_sort_bytes(B, K_, R_ROWS, oc, 2)
+            lists = torch.empty(sbytes, dtype=torch.uint8, device=dev)
+            G = torch.randn(2, B, oc, device=dev)
+
+            def whole():
+                rc = lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT,
+                                               row_split, ws.data_ptr(), nbytes, None, stream, aux_stream)
+                assert rc == 0
+
+            def sort_only():
+                rc = lib.nnueft_det_sort(t["white"].data_ptr(), t["black"].data_ptr(), B, K_, R_ROWS, oc, 2,
+                                         row_split, lists.data_ptr(), sbytes, stream)
+                assert rc == 0
+
+            def presorted():
+                rc = lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT,
+                                               row_split, ws.data_ptr(), nbytes, lists.data_ptr(), stream, None)
+                assert rc == 0
+
+            def reduce_only():
+                # the segmented reduction alone: k_seg_reduce, then the window sums of split rows (k_split_combine)
+                # and the rewind of the task counters, a few microseconds together
+                rc = lib.nnueft_det_reduce_rows(G.data_ptr(), gW.data_ptr(), B, K_, R_ROWS, oc, 2, row_split,
+                                                ws.data_ptr(), nbytes, lists.data_ptr(), stream)
+                assert rc == 0
+
+            out = {}
+            if args.only != "reduce":
+                _, out["entry"] = time_steps(whole, n_entry, args.warmup)
+            _, out["sort"] = time_steps(sort_only, n_entry, args.warmup)
+            if args.only != "reduce":
+                _, out["presorted"] = time_steps(presorted, n_entry, args.warmup)
+            _, out["reduce"] = time_steps(reduce_only, n_entry, args.warmup)
+            return out
 
         def bwd_atomic():
             gW.zero_()
@@ -465,30 +615,18 @@ def main():
             rc = lib.nnueft_double_bwd_atomic(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT, stream)
             assert rc == 0
 
-        for name, fn in (("deterministic", bwd_det), ("atomic", bwd_atomic)):
-            if name in modes:
-                _, bwd_ms[name] = time_steps(fn, max(args.steps, 10), args.warmup)
+        fwd_only()   # `saved` holds this batch's row sums
+        for mode in (["deterministic"] if args.only == "reduce" else modes):
+            if mode == "atomic":
+                _, ms = time_steps(bwd_atomic, n_entry, args.warmup)
+                bwd_ms[mode] = {"entry": ms}
+            else:
+                bwd_ms[mode] = det_entry(row_split_of(mode))
 
-        if "deterministic" in modes:
-            # with the lists sorted beforehand, as in the step above (the sort runs beside the forward)
-            sbytes = lib.nnueft_det_sort_bytes(B, K_, R_ROWS, oc, 2)
-            lists = torch.empty(sbytes, dtype=torch.uint8, device=dev)
-
-            def sort_only():
-                rc = lib.nnueft_det_sort(t["white"].data_ptr(), t["black"].data_ptr(), B, K_, R_ROWS, oc, 2, row_split,
-                                         lists.data_ptr(), sbytes, stream)
-                assert rc == 0
-
-            def bwd_presorted():
-                rc = lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT,
-                                               row_split, ws.data_ptr(), nbytes, lists.data_ptr(), stream, None)
-                assert rc == 0
-
-            _, bwd_ms["sort"] = time_steps(sort_only, max(args.steps, 10), args.warmup)
-            _, bwd_ms["deterministic_presorted"] = time_steps(bwd_presorted, max(args.steps, 10), args.warmup)
-
+    # ---- report
+    traffic, traffic_file = read_profile_traffic(args.workload, args.positions)
     fwd_bytes, _ = algorithmic_bytes(L1, B, sum_a, "atomic")
-    fwd_gbs = fwd_bytes / (fwd_ms * 1e-3) / 1e9
+    comp_fwd, comp_bwd = compulsory_bytes(L1, B, sum_a)
     head_mode = modes[0]
     ms_step = results.get(head_mode, float("nan"))
     out = {
@@ -511,57 +649,135 @@ def main():
             "index_scheme": "HalfKAv2_hm, seeded random positions", "positions": args.positions,
             "sort_placement": args.sort_placement,
         },
-        "roofline_forward": {
-            "kernel": "nnueft_double_fwd: k_acc_blocked (the gather, ~3/4 of the time) + k_mix + pair sort",
-            "bound": "hbm", "achieved": fwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": fwd_gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get((args.workload, "forward")),
-            "algorithmic_bytes_per_launch": fwd_bytes, "avg_launch_ms": fwd_ms,
-        },
+        "peaks": {"hbm_GBs": HBM_PEAK_GBS, "l2_GBs": l2_peak,
+                  "l2": f"{L2_CHANNELS} channels x {L2_LINE_BYTES} B per clock at {ENGINE_CLOCK_GHZ} GHz",
+                  "traffic_source": traffic_file},
     }
-    # the dominant launch of the step is the backward entry point (about two thirds of it); both gathers are
-    # served from L2, so `achieved` (algorithmic bytes) can exceed the HBM peak while `traffic` stays far below
-    if head_mode in bwd_ms:
-        _, bwd_bytes = algorithmic_bytes(L1, B, sum_a, head_mode)
-        bwd_gbs = bwd_bytes / (bwd_ms[head_mode] * 1e-3) / 1e9
-        out["roofline"] = {
-            "kernel": ("nnueft_double_bwd_det: k_seg_reduce (the gather of the upstream rows, ~60 % of the time) + "
-                       "k_bwd_rows + index sort + bias chain") if head_mode == "deterministic"
-            else "nnueft_double_bwd_atomic: k_double_bwd_atomic (+ the zero fill of the dense gradient)",
-            "bound": "hbm", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get((args.workload, head_mode)),
-            "algorithmic_bytes_per_launch": bwd_bytes, "avg_launch_ms": bwd_ms[head_mode],
-        }
+    fwd_block, fwd_comp = bound_block(
+        "nnueft_double_fwd: k_acc_blocked (the gather, ~3/4 of the time) + k_mix + pair sort", fwd_ms, fwd_bytes,
+        sum_a * oc * 4, sum(comp_fwd.values()), sum_traffic(traffic, FWD_KERNELS), l2_peak)
+    out["roofline_forward"] = fwd_block
+    out["roofline_forward_compulsory"] = fwd_comp
+    det = bwd_ms.get("deterministic") or bwd_ms.get("deterministic_strict")
+    if det:
+        alg, gathered, comp = seg_reduce_bytes(L1, B, sum_a)
+        seg_traffic = sum_traffic(traffic, ("k_seg_reduce", "k_split_combine"))
+        out["roofline"], out["roofline_compulsory"] = bound_block(
+            "k_seg_reduce<4,3> (timed through nnueft_det_reduce_rows, which launches it with k_split_combine and the "
+            "rewind of the task counters, a few microseconds, behind it)", det["reduce"], alg, gathered, comp,
+            seg_traffic, l2_peak,
+            note="dominant kernel of the step; it gathers one upstream row per slot through L2 (blocked by king bucket "
+                 "and column slice), so `achieved` (algorithmic bytes) is held against the L2 line rate; against HBM "
+                 "see roofline_compulsory (bytes that must cross HBM once) and `traffic` (counter-measured)")
+    elif "atomic" in bwd_ms:
+        _, bwd_bytes = algorithmic_bytes(L1, B, sum_a, "atomic")
+        gbs = bwd_bytes / (bwd_ms["atomic"]["entry"] * 1e-3) / 1e9
+        out["roofline"] = {"kernel": "k_double_bwd_atomic<4> (+ the zero fill of the dense gradient)", "bound": "hbm",
+                           "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                           "traffic": None, "algorithmic_bytes_per_launch": bwd_bytes,
+                           "avg_launch_ms": bwd_ms["atomic"]["entry"]}
     else:
-        out["roofline"] = out["roofline_forward"]
+        out["roofline"], out["roofline_compulsory"] = fwd_block, fwd_comp
     step_stats = {}
     for mode in modes:
         if mode not in results:
             continue
         fb, bb = algorithmic_bytes(L1, B, sum_a, mode)
         ms = results[mode]
-        step_stats[mode] = {
-            "ms_per_step": ms, "positions_per_s": B / (ms * 1e-3),
-            "algorithmic_GBs": (fb + bb) / (ms * 1e-3) / 1e9,
-            "frac_of_hbm_peak": (fb + bb) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            "backward_entry_ms": bwd_ms.get(mode),
-            "backward_algorithmic_GBs": bb / (bwd_ms[mode] * 1e-3) / 1e9 if mode in bwd_ms else None,
-        }
-        if mode == "deterministic" and "sort" in bwd_ms:
-            step_stats[mode]["sort_entry_ms"] = bwd_ms["sort"]
-            step_stats[mode]["backward_presorted_entry_ms"] = bwd_ms["deterministic_presorted"]
+        st = {"ms_per_step": ms, "positions_per_s": B / (ms * 1e-3), "algorithmic_GBs": (fb + bb) / (ms * 1e-3) / 1e9}
+        if mode != "atomic":
+            comp_step = sum(comp_fwd.values()) + sum(comp_bwd.values())
+            st["compulsory_bytes"] = comp_step
+            st["compulsory_frac_of_hbm_peak"] = comp_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS
+            tr = sum_traffic(traffic, FWD_KERNELS + BWD_KERNELS) if mode == "deterministic" else None
+            st["traffic_bytes"] = tr
+            st["traffic_frac_of_hbm_peak"] = tr / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS if tr else None
+        else:
+            st["algorithmic_frac_of_hbm_peak"] = st["algorithmic_GBs"] / HBM_PEAK_GBS
+        if mode in bwd_ms:
+            e = bwd_ms[mode]
+            st["backward_entry_ms"] = e.get("entry")
+            if "sort" in e:
+                st.update(sort_entry_ms=e["sort"], backward_presorted_entry_ms=e.get("presorted"),
+                          reduce_stage_ms=e["reduce"])
+        step_stats[mode] = st
     out["step"] = step_stats
     if not args.only and args.positions == "uniform":
-        # the same step on game-like index lists (not the headline: a robustness figure)
+        # the same step on game-like index lists (not the headline: what real training data looks like)
         tg, sum_g = make_inputs(L1, B, seed, dev, "game")
-        ms_g, _ = time_steps(lambda: step(head_mode, tg), args.steps, args.warmup)
-        out["game_like_positions"] = {"ms_per_step": ms_g, "positions_per_s": B / (ms_g * 1e-3),
-                                      "active_rows_per_position": sum_g / B, "backward": head_mode}
+        game = {"active_rows_per_position": sum_g / B}
+        for mode in ("deterministic", "deterministic_strict"):
+            ms_g, _ = time_steps(lambda: step(mode, tg), args.steps, args.warmup)
+            game[mode] = {"ms_per_step": ms_g, "positions_per_s": B / (ms_g * 1e-3)}
+        out["game_like_positions"] = game
         del tg
     if not args.no_cpu_baseline and not args.only:
-        out["cpu_baseline"] = cpu_baseline(L1, B, seed)
+        names = [args.workload] + (["ft_fwd_bwd_L1_1024_B8192"] if args.workload != "ft_fwd_bwd_L1_1024_B8192" else [])
+        out["cpu_baseline"] = cpu_baseline(names, seed)
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="ft_fwd_bwd_L1_3072_B16384", choices=sorted(WORKLOADS))
+    ap.add_argument("--backward", default="deterministic", choices=["deterministic", "deterministic_strict", "atomic"],
+                    help="backward mode the headline value is measured with (the others are reported beside it)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--optimizer", default="rangerlite", choices=["rangerlite", "adam"],
+                    help="full_step workload only")
+    ap.add_argument("--compile", default="", choices=["", "inductor", "aot_eager", "cudagraphs"],
+                    help="full_step workload only: torch.compile the model with this backend, as the reference's "
+                         "train.py does (the kernels of this build stay opaque to it); off by default")
+    ap.add_argument("--sort-placement", default="inline", choices=["inline", "backward", "forward"],
+                    help="where the index sort of the deterministic backward runs (nnueft.set_sort_placement); "
+                         "the default is the library's")
+    ap.add_argument("--positions", default="uniform", choices=["uniform", "game"],
+                    help="uniform: kings and pieces uniform over the board (the headline workload); game: piece "
+                         "placement statistics of real game positions, where one or two king buckets hold a large "
+                         "part of the batch (halfka_v2_hm.game_like_positions); a default run times both")
+    ap.add_argument("--only", default="", choices=["", "fwd", "det", "strict", "atomic", "reduce", "copy", "handoff"],
+                    help="run only this part (for profiling runs); 'reduce' the segmented reduction alone; 'copy' "
+                         "launches a plain elementwise kernel reading and writing 1 GiB each, the yardstick the "
+                         "FETCH_SIZE/WRITE_SIZE counters are scaled by")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import nnueft
+    from nnueft import _native
+
+    nnueft.set_sort_placement(args.sort_placement)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    lib = _native.load()  # raises if libnnueft.so is missing: there is no fallback
+    dev = torch.device("cuda:0")
+    if args.workload.startswith("ft_int16"):
+        run_int16(args, lib, dev)
+    elif args.workload.startswith("full_step"):
+        run_full_step(args, dev)
+    elif args.workload.startswith("ref_microbench"):
+        run_ref_microbench(args, dev)
+    elif args.only == "copy":
+        n = (1 << 30) // 4
+        src = torch.ones(n, device=dev)
+        dst = torch.empty(n, device=dev)
+        for _ in range(args.warmup + args.steps):
+            torch.add(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "torch.add(src, 1.0, out=dst)", "read_bytes": n * 4, "write_bytes": n * 4,
+                          "launches": args.warmup + args.steps}))
+    elif args.only == "handoff":
+        run_handoff(args, dev)
+    else:
+        run_ft(args, lib, dev)
 
 
 if __name__ == "__main__":

@@ -122,7 +122,7 @@ def random_positions(batch_size: int, seed: int, min_other: int = 2, max_other: 
 def game_like_positions(batch_size: int, seed: int):
     """Seeded synthetic positions with the piece placement statistics of real game positions.
 
-    game_like_stats.npz (written by make_game_like_stats.py from the reference's sample data) holds,
+    game_like_stats.npz (written by tests/golden/make_game_like_stats.py from the reference's sample data) holds,
     per piece kind and square, how often it occurs from white's point of view with white's king
     mirrored onto files e-h: one table for each of white's three most common king buckets, one for
     the rest.  A position draws its class, the kings from their rows of the class's table, and

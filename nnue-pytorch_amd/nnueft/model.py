@@ -474,15 +474,6 @@ class ComposedFeatureTransformer(nn.Module):
         bias = torch.cat([b, self.psqt_bias_zeros.to(b.dtype)], dim=0)
         return merged, bias
 
-    def _psqt_bias_zeros(self, like):
-        """The PSQT part of the bias is held at zero; the zeros are made once per device and dtype."""
-        n = self.bias.shape[0] - self.l1_size
-        z = getattr(self, "_zeros_cache", None)
-        if z is None or z.device != like.device or z.dtype != like.dtype or z.shape[0] != n:
-            z = torch.zeros(n, dtype=like.dtype, device=like.device)
-            object.__setattr__(self, "_zeros_cache", z)     # not a parameter, not a buffer, not in the state dict
-        return z
-
     @torch.no_grad()
     def coalesce(self):
         for f in self.features:
@@ -804,6 +795,35 @@ class NNUEModel(nn.Module):
             return _StackOutput.apply(lin, skip, wpsqt, bpsqt, us, den, mult, fake_quantize_acts)
         return self.layer_stacks(l0_, ls_indices, fake_quantize_acts, fake_quantize_weights) + (wpsqt - bpsqt) * (us - 0.5)
 
+    def weight_clipping_config(self):
+        """The layer-stack weights and the range the quantization scheme leaves them
+        (QuantizationManager.generate_weight_clipping_config, model/quantize.py:150-172)."""
+        ls, m = self.layer_stacks, self.quantization.max_hidden_weight
+        return [
+            {"params": [ls.l1.linear.weight], "min_weight": -m[0], "max_weight": m[0],
+             "virtual_params": ls.l1.factorized_linear.weight},
+            {"params": [ls.l2.linear.weight], "min_weight": -m[1], "max_weight": m[1]},
+            {"params": [ls.output.linear.weight], "min_weight": -m[2], "max_weight": m[2]},
+        ]
+
+    @torch.no_grad()
+    def clip_weights(self, include_input: bool):
+        """Clamp the layer-stack weights to what their int8 image can hold (model/model.py:42-72; the
+        reference's trainer calls it after every batch, trainer/callbacks.py:70-85).  Where a layer has
+        shared (factorised) weights, the sum of the two is what gets exported, so the bounds of the real
+        weights move by the shared ones."""
+        if include_input:
+            self.input.clip_weights(self.quantization)
+        for group in self.weight_clipping_config():
+            lo, hi = group["min_weight"], group["max_weight"]
+            for p in group["params"]:
+                if "virtual_params" in group:
+                    v = group["virtual_params"]
+                    spread = v.repeat(p.shape[0] // v.shape[0], p.shape[1] // v.shape[1])
+                    p.data.copy_(torch.minimum(torch.maximum(p.data, lo - spread), hi - spread))
+                else:
+                    p.data.clamp_(lo, hi)
+
     @torch.no_grad()
     def zero_virtual_weights(self):
         self.input.zero_virtual_weights()
@@ -835,9 +855,14 @@ def remap_tablebase_score(score, base: float, scale: float, decay: float):
 
 def sf_loss(scorenet, score, outcome, p: LossParams, actual_lambda):
     """Win-rate-model loss; `scorenet` is the net output times nnue2score (model/nnue.py:39-70)."""
-    if _fused_tail_applies(scorenet) and score.dtype == torch.float32 and outcome.dtype == torch.float32 \
+    # the fused kernels take one lambda for the batch, as a host number, and device pointers for the rest; a
+    # per-sample lambda tensor (the reference's jittered schedule, model/lambda_utils.py:69-83) or tensors that
+    # live elsewhere go through the torch formula below
+    if _fused_tail_applies(scorenet) and isinstance(actual_lambda, (int, float)) \
+            and score.is_cuda and outcome.is_cuda and score.device == scorenet.device == outcome.device \
+            and score.dtype == torch.float32 and outcome.dtype == torch.float32 \
             and scorenet.numel() > 0 and score.shape == scorenet.shape == outcome.shape:
-        return _SfLoss.apply(scorenet, score, outcome, p, actual_lambda)
+        return _SfLoss.apply(scorenet, score, outcome, p, float(actual_lambda))
     score = remap_tablebase_score(score, p.tb_remap_base, p.tb_remap_scale, p.tb_remap_decay)
 
     def win_rate(x, offset, scaling):

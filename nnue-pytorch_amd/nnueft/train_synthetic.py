@@ -61,6 +61,7 @@ def run(steps: int = 50, batch_size: int = 16384, l1: int = 1024, lr: float = 8.
         loss = M.sf_loss(out * model.quantization.nnue2score, score, outcome, params, lam)
         loss.backward()
         opt.step()
+        model.clip_weights(include_input=False)      # the trainer's WeightClipper, after every batch
         losses.append(loss.detach())
         if log_every and step % log_every == 0:
             print(f"step {step:5d}  loss {float(losses[-1]):.6f}", flush=True)

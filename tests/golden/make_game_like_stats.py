@@ -8,7 +8,9 @@ common king buckets of white and one for all others, since where the pieces stan
 where the king went.  Nothing of the positions themselves is kept.
 nnueft.halfka_v2_hm.game_like_positions() draws synthetic positions from the tables.
 
-    python nnue-pytorch_amd/nnueft/make_game_like_stats.py /root/reference/.pgo/small.binpack
+    python tests/golden/make_game_like_stats.py /root/reference/.pgo/small.binpack
+
+writes nnue-pytorch_amd/nnueft/game_like_stats.npz (the package ships the statistics, not this script).
 """
 import ctypes
 import os
@@ -17,7 +19,9 @@ import sys
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-sys.path.insert(0, os.path.join(HERE, "..", ".."))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+OUT = os.path.join(ROOT, "nnue-pytorch_amd", "nnueft", "game_like_stats.npz")
+sys.path.insert(0, ROOT)
 from oracle import loader_ref as lr  # noqa: E402
 
 
@@ -74,7 +78,7 @@ def main(path):
         share[c] = len(sel) / n_pos
         v = sel[sel >= 0] % 768
         freq[c] = (np.bincount(v, minlength=768) / max(len(sel), 1)).reshape(12, 64)
-    np.savez_compressed(os.path.join(HERE, "game_like_stats.npz"), freq=freq, share=share, buckets=top.astype(np.int32),
+    np.savez_compressed(OUT, freq=freq, share=share, buckets=top.astype(np.int32),
                         positions=np.int64(n_pos))
     print("positions", n_pos, "classes", top, share, "pieces per position", freq.sum((1, 2)))
 

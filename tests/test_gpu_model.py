@@ -353,3 +353,107 @@ def test_synthetic_training_loop_on_gpu():
         nnueft.set_backward_mode(old)
     assert all(np.isfinite(a)) and a[-1] < a[0] and rate > 0
     assert a == b
+
+
+@pytest.mark.parametrize("L2", [32, 16], ids=["L2_32", "L2_15plus1"])
+def test_config_4_full_size_step(oracle_cpu, L2):
+    """BASELINE.json config 4 at its real size: L1=3072 feature transformer, 8 bucketed layer stacks
+    (3072 -> L2 -> 32 -> 1; L2=32 is the reference's default, 16 = 15+1 the configuration's literal), B=16384,
+    RangerLite.  (a) the feature transformer of the first step, outputs and gradients, bit-equal to the oracle on
+    the same merged table; (b) the bucketed first layer at in=3072, B=16384 against the oracle, 1e-5 of the largest
+    magnitude; (c) three optimizer steps, losses finite and identical on a second run from the same seed."""
+    from nnueft.optim import RangerLite
+
+    old = nnueft.get_backward_mode()
+    nnueft.set_backward_mode("deterministic")
+    L1, B, R, n_psqt = 3072, 16384, hk.NUM_INPUTS, 8
+    host = hk.synthetic_batch(B, 1238)
+    us, them, white, black, pc = [torch.from_numpy(a).to(DEV) for a in host]
+    psqt_np = ((host[4] - 1) // 4).astype(np.int64)
+    g = torch.Generator().manual_seed(1238)
+    score = (torch.randn(B, 1, generator=g) * 400).clamp(-3000, 3000).to(DEV)
+    outcome = (torch.randint(0, 3, (B, 1), generator=g).float() / 2).to(DEV)
+
+    def fresh():
+        torch.manual_seed(0)
+        m = M.NNUEModel("HalfKAv2_hm^", M.ModelConfig(L1=L1, L2=L2, L3=32)).to(DEV)
+        with torch.no_grad():      # shared weights off zero, so that the merge has something to add
+            m.input.features[0].virtual_weight.normal_(0, 0.003)
+            m.input.features[0].weight[:, :L1].normal_(0, 0.01)
+            m.input.bias[:L1].normal_(0, 0.01)
+        return m
+
+    try:
+        model = fresh()
+        q = model.quantization
+        # (a) the feature transformer of step 1
+        merged, bias = model.input.merged_weight_and_bias(True)
+        l0, wp, bp = model.input(us, them, white, black, (pc - 1) // 4, True, True)
+        Wn, bn = merged.detach().cpu().numpy(), bias.detach().cpu().numpy()
+        feat = model.input.features[0]
+        assert np.array_equal(Wn, oracle_cpu.table_merge(feat.weight.detach().cpu().numpy(),
+                                                         feat.virtual_weight.detach().cpu().numpy(), L1))
+        r_l0, r_wp, r_bp, r_saved = oracle_cpu.double_fwd(host[0], host[1], host[2], host[3], psqt_np, Wn, bn,
+                                                          q.max_ft_activation, L1)
+        r_l0 = oracle_cpu.act_fake_quantize(r_l0, q.hidden_quantized_one, M.FAKE_QUANTIZE_EPS, q.l0_correction_factor)
+        assert np.array_equal(l0.detach().cpu().numpy(), r_l0)
+        assert np.array_equal(wp.detach().cpu().numpy(), r_wp) and np.array_equal(bp.detach().cpu().numpy(), r_bp)
+        up = [torch.randn(B, L1, generator=g), torch.randn(B, 1, generator=g), torch.randn(B, 1, generator=g)]
+        torch.autograd.backward([l0, wp, bp], [t.to(DEV) for t in up])
+        r_gW, r_gb = oracle_cpu.double_bwd(host[0], host[1], host[2], host[3], psqt_np, bn, q.max_ft_activation,
+                                           up[0].numpy() * np.float32(q.l0_correction_factor), up[1].numpy(),
+                                           up[2].numpy(), r_saved, R, n_psqt)
+        assert np.array_equal(feat.weight.grad.cpu().numpy(), r_gW)                     # straight-through
+        assert np.array_equal(feat.virtual_weight.grad.cpu().numpy(), oracle_cpu.table_virtual_grad(r_gW, 768))
+        assert np.array_equal(model.input.bias.grad.cpu().numpy()[:L1], r_gb[:L1])
+        del merged, l0, wp, bp, r_gW, r_saved, Wn
+        model.zero_grad(set_to_none=True)
+
+        # (b) the first bucketed layer on this model's own activations
+        ls = model.layer_stacks
+        with torch.no_grad():
+            x = model.input(us, them, white, black, (pc - 1) // 4, True, True)[0]
+        bucket = (pc - 1) // 4
+        w, b_ = ls.l1._params_one_pass(True)
+        out_f = ls.l1.linear.out_features // 8
+        xg = x.clone().requires_grad_()
+        wg = w.detach().clone().requires_grad_()
+        bg = b_.detach().clone().requires_grad_()
+        y = M._BucketLinear.apply(xg, bucket, wg, bg, out_f, 8, None)
+        gy = torch.randn(B, out_f, generator=g)
+        y.backward(gy.to(DEV))
+        xn, wn, bucket_n = x.cpu().numpy(), wg.detach().cpu().numpy(), bucket.cpu().numpy()
+        ref = oracle_cpu.bucket_linear_fwd(xn, bucket_n, wn, bg.detach().cpu().numpy(), out_f, 8)
+        tol = lambda r: 1e-5 * max(float(np.abs(r).max()), 1e-30)
+        assert np.abs(y.detach().cpu().numpy() - ref).max() <= tol(ref)
+        rx, rW, rb = oracle_cpu.bucket_linear_bwd(xn, bucket_n, wn, gy.numpy(), out_f, 8)
+        assert np.abs(xg.grad.cpu().numpy() - rx).max() <= tol(rx)
+        assert np.abs(wg.grad.cpu().numpy() - rW).max() <= tol(rW)
+        assert np.abs(bg.grad.cpu().numpy() - rb).max() <= tol(rb)
+        del x, xg, y, rx, rW, xn
+
+        # (c) three steps, twice
+        def run(model):
+            opt = RangerLite(M.optimizer_param_groups(model, lr=8.75e-4), normloss_active=False)
+            losses = []
+            for _ in range(3):
+                opt.zero_grad(set_to_none=True)
+                out = model(us, them, white, black, pc)
+                loss = M.sf_loss(out * model.quantization.nnue2score, score, outcome, M.LossParams(), 0.75)
+                loss.backward()
+                for name, prm in model.named_parameters():
+                    assert prm.grad is not None, name
+                opt.step()
+                model.clip_weights(include_input=False)
+                losses.append(float(loss))
+            for name, prm in model.named_parameters():
+                assert torch.isfinite(prm).all(), name
+            return losses
+
+        a = run(model)
+        del model
+        torch.cuda.empty_cache()
+        b = run(fresh())
+        assert all(np.isfinite(a)) and a == b
+    finally:
+        nnueft.set_backward_mode(old)

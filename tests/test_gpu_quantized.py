@@ -32,6 +32,37 @@ def test_stack_int8_against_oracle(oracle_cpu, B, L1, L2, L3, count):
     assert len(np.unique(want)) > min(B, 20) // 2
 
 
+def test_config_5_end_to_end_at_full_size(oracle_cpu):
+    """BASELINE.json config 5 as a whole at its real size: L1=3072, B=65536, exported numbering (22528 rows); the
+    int16 feature transformer, then the int8 layer stacks of a quantized model (L2=32 and the literal 15+1), every
+    output bit-equal to the CPU integer evaluation of the same quantized tensors."""
+    L1, B, R = 3072, 65536, hk.NUM_INPUTS_EXPORT
+    us, them, white, black, pc = hk.synthetic_batch(B, 1239, fold_kings=True)
+    g = torch.Generator().manual_seed(5)
+    W = torch.randn(R, L1 + 8, generator=g) * 0.02
+    W[:, L1:] = torch.randn(R, 8, generator=g) * 0.5
+    bias = torch.randn(L1 + 8, generator=g) * 0.1
+    w16, b16, p32 = quantized.quantize_feature_transformer(W, bias, L1)
+    stm = (1 - us[:, 0]).astype(np.uint8)
+    bucket = ((pc - 1) // 4).astype(np.int64)
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    x_u8, psqt = quantized.ft_int16_forward(t(white), t(black), t(stm), w16.to(DEV), b16.to(DEV), p32.to(DEV), t(bucket))
+    r_x, r_ps = oracle_cpu.ft_int16_fwd(white, black, stm, w16.numpy(), b16.numpy(), p32.numpy(), bucket)
+    assert np.array_equal(x_u8.cpu().numpy(), r_x) and np.array_equal(psqt.cpu().numpy(), r_ps)
+    for L2 in (32, 16):
+        torch.manual_seed(5 + L2)
+        stacks = M.LayerStacks(8, M.ModelConfig(L1=L1, L2=L2, L3=32), M.QuantizationManager(M.QuantizationConfig()))
+        with torch.no_grad():
+            stacks.l1.linear.weight.mul_(0.5)
+            stacks.l1.factorized_linear.weight.normal_(0, 0.004)
+        stack = quantized.quantize_layer_stacks(stacks)
+        out = quantized.stack_int8_forward(x_u8, t(bucket), *[s.to(DEV) for s in stack])
+        want = oracle_cpu.stack_int8_fwd(r_x, bucket, *[s.numpy() for s in stack], L2, 32, 8)
+        assert np.array_equal(out.cpu().numpy(), want)
+        total = out.cpu().numpy().astype(np.int64) + r_ps
+        assert len(np.unique(total)) > 1000 and np.abs(out.cpu().numpy()).max() > 0
+
+
 def test_quantized_chain_tracks_the_float_model(oracle_cpu):
     """Export a float model (weights on the quantization grid so that nothing is lost in the export),
     evaluate it with the integer kernels, compare with its own fake-quantized float forward."""

@@ -254,3 +254,71 @@ def test_synthetic_training_loop_on_cpu():
 
     losses, rate = train_synthetic.run(steps=14, batch_size=256, l1=64, device="cpu", lr=2e-3)
     assert len(losses) == 14 and all(np.isfinite(losses)) and losses[-1] < losses[0] and rate > 0
+
+
+def test_loss_with_a_per_sample_lambda_tensor():
+    """The reference's jittered lambda schedule hands sf_loss one lambda per sample (model/lambda_utils.py:69-83);
+    the loss must take it (through the torch formula) and agree with per-sample evaluation."""
+    p = M.LossParams()
+    g = torch.Generator().manual_seed(1)
+    net = torch.randn(6, 1, generator=g) * 300
+    score = torch.randn(6, 1, generator=g) * 400
+    outcome = torch.tensor([[0.0], [0.5], [1.0], [1.0], [0.0], [0.5]])
+    lam = torch.tensor([[1.0], [0.75], [0.5], [0.0], [0.9], [0.3]])
+    got = M.sf_loss(net, score, outcome, p, lam)
+    each = torch.stack([M.sf_loss(net[i:i + 1], score[i:i + 1], outcome[i:i + 1], p, float(lam[i])) for i in range(6)])
+    assert float(got) == pytest.approx(float(each.mean()), rel=1e-6)     # weights are 1 at w1 = 0
+    assert float(M.sf_loss(net, score, outcome, p, torch.tensor(0.75))) == \
+        pytest.approx(float(M.sf_loss(net, score, outcome, p, 0.75)), rel=1e-6)
+
+
+def test_clip_weights_bounds_what_gets_exported():
+    """NNUEModel.clip_weights (model/model.py:42-72): the layer-stack weights end inside the range of their int8
+    image; for the first layer the bound applies to real + shared weight, which is what the export sums."""
+    torch.manual_seed(5)
+    m = M.NNUEModel("HalfKAv2_hm^", M.ModelConfig(L1=64, L2=16, L3=32))
+    ls, q = m.layer_stacks, m.quantization
+    with torch.no_grad():
+        ls.l1.linear.weight.normal_(0, 3.0)
+        ls.l1.factorized_linear.weight.normal_(0, 0.5)
+        ls.l2.linear.weight.normal_(0, 5.0)
+        ls.output.linear.weight.normal_(0, 5.0)
+    before_input = m.input.features[0].weight.clone()
+    m.clip_weights(include_input=True)
+    assert torch.equal(m.input.features[0].weight, before_input)          # HalfKAv2_hm clips nothing
+    v = ls.l1.factorized_linear.weight
+    total = ls.l1.linear.weight + v.repeat(ls.l1.linear.weight.shape[0] // v.shape[0], 1)
+    total = total.detach()
+    assert float(total.abs().max()) <= q.max_hidden_weight[0] * (1 + 1e-6)
+    assert float((total.abs() - q.max_hidden_weight[0]).abs().min()) < 1e-6      # and the bound is reached
+    assert float(ls.l2.linear.weight.detach().abs().max()) == pytest.approx(q.max_hidden_weight[1])
+    assert float(ls.output.linear.weight.detach().abs().max()) == pytest.approx(q.max_hidden_weight[2])
+    assert q.max_hidden_weight == pytest.approx([127 / 128, 127 / 64, 127 / 128])   # weights x128 / x64 / x128
+
+
+def test_train_clip_write_read_round_trip():
+    """A few optimizer steps with a large learning rate push layer-stack weights past the int8 range; without the
+    clip the writer refuses the net, with it the file reads back to the model's quantized tensors."""
+    import io
+
+    from nnueft import serialize as S
+    from nnueft.optim import RangerLite
+
+    torch.manual_seed(9)
+    m = M.NNUEModel("HalfKAv2_hm^", M.ModelConfig(L1=64, L2=15, L3=32))
+    opt = RangerLite(M.optimizer_param_groups(m, lr=0.8), normloss_active=False)
+    us, them, white, black, pc = [torch.from_numpy(a) for a in hk.synthetic_batch(64, 8)]
+    g = torch.Generator().manual_seed(2)
+    score, outcome = torch.randn(64, 1, generator=g) * 400, torch.full((64, 1), 0.5)
+    for _ in range(4):
+        opt.zero_grad()
+        loss = M.sf_loss(m(us, them, white, black, pc) * 600.0, score, outcome, M.LossParams(), 1.0)
+        loss.backward()
+        opt.step()
+    assert float(m.layer_stacks.l2.linear.weight.detach().abs().max()) > m.quantization.max_hidden_weight[1]
+    with pytest.raises(RuntimeError, match="out of bounds"):
+        S.NNUEWriter(m, "unclipped")
+    m.clip_weights(include_input=True)
+    buf = bytes(S.NNUEWriter(m, "clipped").buf)
+    back = S.NNUEReader(io.BytesIO(buf), "HalfKAv2_hm^", M.ModelConfig(L1=64, L2=15, L3=32)).model
+    assert bytes(S.NNUEWriter(back, "clipped").buf) == buf
