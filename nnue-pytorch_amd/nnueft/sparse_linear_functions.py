@@ -41,8 +41,13 @@ def set_backward_mode(mode: str) -> None:
 
 
 def row_split_of(mode: str) -> int:
-    """The row_split argument of the deterministic entry points for a backward mode."""
-    return 0 if mode == "deterministic_strict" else _native.load().nnueft_row_split()
+    """The row_split argument of the deterministic entry points for a backward mode.  NNUEFT_ROW_SPLIT in the
+    environment replaces the library's threshold for the "deterministic" mode (kernel tuning: the threshold is
+    part of the summation order, so results change in the last bits of the rows it moves across)."""
+    if mode == "deterministic_strict":
+        return 0
+    override = os.environ.get("NNUEFT_ROW_SPLIT", "")
+    return int(override) if override.isdigit() else _native.load().nnueft_row_split()
 
 
 def get_backward_mode() -> str:
