@@ -52,6 +52,10 @@ constexpr int kLongRow = NNUEFT_LONG_ROW;  // table rows named by at least this 
 #define NNUEFT_RUN_U 16
 #endif
 constexpr int kRunUnroll = NNUEFT_RUN_U;   // rows in flight per lane in the chain of one window of a split row
+#ifndef NNUEFT_NARROW_AVG
+#define NNUEFT_NARROW_AVG 64
+#endif
+constexpr int kNarrowAvg = NNUEFT_NARROW_AVG;   // slots per row of a XCD's row range from which it is walked in 64-lane slices
 constexpr uint32_t kSplitFlag = 0x80000000u;   // on a row's slot count between k_col_scan and k_row_scan
 
 // Work split of the segmented reduction, written by k_row_scan (uint32 words).
@@ -626,7 +630,12 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
     const uint32_t lo = sched[kSchedRowLo + xcd], hi = sched[kSchedRowLo + xcd + 1];
     const uint32_t nreg = hi - lo;
     const uint32_t long_end = run_tasks + my_long * (uint32_t)nslices;
-    const uint32_t ntasks = long_end + nreg * (uint32_t)nslices;
+    // A range whose rows are named by many slots each belongs to a table block that a large part of
+    // the batch sits in: one wide slice of all those positions' upstream rows would not fit the L2,
+    // so such a range is walked in 64-lane slices (the results do not depend on the slicing).
+    const bool narrow = nreg > 0 && (seg_off[hi] - seg_off[lo]) / nreg > (uint32_t)kNarrowAvg && rp.nslices > nslices;
+    const uint32_t walk_slices = narrow ? (uint32_t)rp.nslices : (uint32_t)nslices;
+    const uint32_t ntasks = long_end + nreg * walk_slices;
     static_assert(kQueues <= kSchedQueues, "counters per XCD");
     const int home = (blockIdx.x / kXcd) % kQueues;
 
@@ -671,8 +680,12 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
         // long or split: done elsewhere
         if (t >= long_end && (end - beg >= (uint32_t)kLongRow || (rp.row_split != 0 && end - beg > rp.row_split)))
             continue;
-        seg_reduce_task<VW, NQ, kRowsUnroll>(G, list, beg, beg + wcount[r], end, gW + (size_t)r * out_cols, s, lane,
-                                             out_cols, slice_v, two_persp);
+        if (t >= long_end && narrow)
+            seg_reduce_task<VW, 1, kRunUnroll>(G, list, beg, beg + wcount[r], end, gW + (size_t)r * out_cols, s, lane,
+                                               out_cols, rp.slice_v, two_persp);
+        else
+            seg_reduce_task<VW, NQ, kRowsUnroll>(G, list, beg, beg + wcount[r], end, gW + (size_t)r * out_cols, s,
+                                                 lane, out_cols, slice_v, two_persp);
     }
   }
 }
