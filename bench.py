@@ -548,7 +548,7 @@ def run_ft(args, lib, dev):
     Wd, bd = W.detach(), bias.detach()
     n_entry = max(args.steps, 10)
 
-    def fwd_only():
+    def fwd_only(stream=stream):
         rc = lib.nnueft_double_fwd(t["us"].data_ptr(), t["them"].data_ptr(), t["white"].data_ptr(),
                                    t["black"].data_ptr(), t["psqt_idx"].data_ptr(), Wd.data_ptr(), bd.data_ptr(),
                                    MAX_ACT, l0.data_ptr(), wp.data_ptr(), bp.data_ptr(), saved.data_ptr(),
@@ -578,10 +578,24 @@ def run_ft(args, lib, dev):
             lists = torch.empty(sbytes, dtype=torch.uint8, device=dev)
             G = torch.randn(2, B, oc, device=dev)
 
-            def whole():
+            def whole(stream=stream, aux_stream=aux_stream):
                 rc = lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT,
                                                row_split, ws.data_ptr(), nbytes, None, stream, aux_stream)
                 assert rc == 0
+
+            def graph_replay():
+                """Forward + this backward captured once into a HIP graph (every buffer allocated beforehand), then
+                replayed: what is left of the step when the host launches one graph instead of ~16 kernels."""
+                side = torch.cuda.Stream()
+                side.wait_stream(torch.cuda.current_stream())
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.stream(side):
+                    with torch.cuda.graph(graph, stream=side):
+                        cap = torch.cuda.current_stream().cuda_stream
+                        fwd_only(cap)
+                        whole(cap, None)
+                torch.cuda.current_stream().wait_stream(side)
+                return time_steps(graph.replay, n_entry, args.warmup)[0]
 
             def sort_only():
                 rc = lib.nnueft_det_sort(t["white"].data_ptr(), t["black"].data_ptr(), B, K_, R_ROWS, oc, 2,
@@ -603,6 +617,8 @@ def run_ft(args, lib, dev):
             out = {}
             if args.only != "reduce":
                 _, out["entry"] = time_steps(whole, n_entry, args.warmup)
+                if args.graph:
+                    out["graph_replay"] = graph_replay()
             _, out["sort"] = time_steps(sort_only, n_entry, args.warmup)
             if args.only != "reduce":
                 _, out["presorted"] = time_steps(presorted, n_entry, args.warmup)
@@ -700,6 +716,8 @@ def run_ft(args, lib, dev):
             if "sort" in e:
                 st.update(sort_entry_ms=e["sort"], backward_presorted_entry_ms=e.get("presorted"),
                           reduce_stage_ms=e["reduce"])
+            if "graph_replay" in e:
+                st["fwd_bwd_graph_replay_ms"] = e["graph_replay"]
         step_stats[mode] = st
     out["step"] = step_stats
     if not args.only and args.positions == "uniform":
@@ -740,6 +758,9 @@ def main():
                     help="uniform: kings and pieces uniform over the board (the headline workload); game: piece "
                          "placement statistics of real game positions, where one or two king buckets hold a large "
                          "part of the batch (halfka_v2_hm.game_like_positions); a default run times both")
+    ap.add_argument("--graph", action="store_true",
+                    help="also capture forward + deterministic backward (through the C ABI, buffers allocated beforehand) "
+                         "into one HIP graph and time its replay")
     ap.add_argument("--only", default="", choices=["", "fwd", "det", "strict", "atomic", "reduce", "copy", "handoff"],
                     help="run only this part (for profiling runs); 'reduce' the segmented reduction alone; 'copy' "
                          "launches a plain elementwise kernel reading and writing 1 GiB each, the yardstick the "
