@@ -1003,15 +1003,17 @@ extern "C" int nnueft_double_bwd_det(const float* us, const float* them, const i
         if (e != hipSuccess) return (int)e;
     }
     int rc = det_sort(widx, bidx, B, K, R, ws + L.sort_begin, L, two_streams ? aux : st);
-    if (two_streams) {
-        // always rejoin, also after a failed launch: the caller's stream must not run ahead of the other one
-        hipError_t e = hipEventRecord(joined, aux);
-        if (e == hipSuccess) e = hipStreamWaitEvent(st, joined, 0);
-        if (rc == 0 && e != hipSuccess) rc = (int)e;
-    }
+    hipError_t sorted = hipSuccess;
+    if (two_streams) sorted = hipEventRecord(joined, aux);
+    // the upstream rows go onto the caller's stream before it is made to wait for the sort
     if (rc == 0)
         rc = nnueft_det::launch_bwd_rows(us, them, psqt_idx, bias, max_act, grad_l0, grad_wpsqt, grad_bpsqt, saved, G,
                                          partial, B, L1, n_psqt, st);
+    if (two_streams) {
+        // always rejoin, also after a failed launch: the caller's stream must not run ahead of the other one
+        if (sorted == hipSuccess) sorted = hipStreamWaitEvent(st, joined, 0);
+        if (rc == 0 && sorted != hipSuccess) rc = (int)sorted;
+    }
     if (rc) return rc;
     return det_reduce(G, gW, gbias, B, R, out_cols, 2, ws, ws + L.sort_begin, L, st);
 }

@@ -27,10 +27,29 @@ _HAS_CUPY_KERNELS = _native.available()
 BACKWARD_TILE_SIZE = 4
 
 
+_XCDS_CHECKED = set()
+
+
+def _warn_once_about_xcds(lib, device) -> None:
+    """The blocked kernels are laid out for 8 XCDs; on a device that presents another number (a partitioned
+    GPU) the library takes slower paths with the same results.  Say so once per device."""
+    key = torch.device(device).index
+    if key in _XCDS_CHECKED:
+        return
+    _XCDS_CHECKED.add(key)
+    n = lib.nnueft_device_xcds()
+    if n not in (0, 8):
+        import warnings
+
+        warnings.warn(f"nnueft: device {device} presents {n} XCDs; the L2-blocked kernels are laid out for 8 and are "
+                      "not used (results are the same, the gathers run two to three times slower)")
+
+
 @torch.compiler.disable(recursive=False)
 def _launch_double_fwd(us, them, white_indices, black_indices, psqt_indices, weight, bias, max_ft_activation,
                        l1_size, l0_, wpsqt, bpsqt, saved, act_grid=None):
     lib = _native.load()
+    _warn_once_about_xcds(lib, weight.device)
     B, K = white_indices.shape
     R, out_cols = weight.shape
     nbytes = lib.nnueft_fwd_workspace_bytes(B, K, R, l1_size, out_cols - l1_size)

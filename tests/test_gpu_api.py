@@ -489,6 +489,11 @@ def test_fused_function_with_nine_and_ten_arguments(oracle_cpu):
                                     256, None, None)
 
 
+def test_device_presents_the_xcd_layout_the_blocked_kernels_are_made_for():
+    # MI355X in its default partition mode: 8 XCDs (0 = the runtime does not say; the blocked kernels then run too)
+    assert _native.load().nnueft_device_xcds() in (0, 8)
+
+
 def test_abi_rejects_bad_arguments():
     lib = _native.load()
     x = torch.zeros(64, device=DEV)
