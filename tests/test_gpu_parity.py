@@ -262,8 +262,11 @@ def _skewed_double_case(seed, B, L1, castled, fold=0):
     return c
 
 
+# (the last case is wide and crowded enough for the XCDs that own the crowded king buckets to walk their row
+# ranges in 64-lane slices)
 @pytest.mark.parametrize("B,L1,castled,fold", [(4096, 64, 1.0, 0), (6000, 256, 0.6, 96), (16384, 128, 0.5, 200),
-                                                (3000, 1024, 0.9, 40), (16384, 64, -1, 0), (5000, 3072, -1, 0)])
+                                                (3000, 1024, 0.9, 40), (16384, 64, -1, 0), (5000, 3072, -1, 0),
+                                                (16384, 1024, -1, 0)])
 def test_double_backward_deterministic_with_split_rows(oracle_cpu, row_split, B, L1, castled, fold):
     c = _skewed_double_case(900 + B, B, L1, castled, fold)
     nat, lib = _native()
