@@ -5,7 +5,8 @@ model/modules/feature_transformer/sparse_linear_functions.py; the CuPy kernels i
 (:85-99 forward, :118-134 backward) are replaced by libnnueft.so (hand-written HIP for gfx950).
 
 `_HAS_CUPY_KERNELS` keeps its name because callers and the reference's tests test it; here it
-means "libnnueft.so is loaded".  There is no silent fallback for device tensors: with
+means "libnnueft.so is loaded".  The launches are torch custom ops (nnueft/_ops.py), so torch.compile keeps
+them inside its graph (the reference's kernels break the graph around themselves).  There is no silent fallback for device tensors: with
 backend="auto", tensors on the GPU and no library, apply() raises.  The "torch" backend (and
 "auto" on CPU tensors) is the reference's device-agnostic embedding_bag path, unchanged.
 """
@@ -16,6 +17,7 @@ import torch.nn.functional as F
 from torch import autograd
 
 from . import _native
+from . import _ops
 
 _HAS_CUPY_KERNELS = _native.available()
 
@@ -40,18 +42,11 @@ def set_backward_mode(mode: str) -> None:
     _BACKWARD_MODE = mode
 
 
-def row_split_of(mode: str) -> int:
-    """The row_split argument of the deterministic entry points for a backward mode.  NNUEFT_ROW_SPLIT in the
-    environment replaces the library's threshold for the "deterministic" mode (kernel tuning: the threshold is
-    part of the summation order, so results change in the last bits of the rows it moves across)."""
-    if mode == "deterministic_strict":
-        return 0
-    override = os.environ.get("NNUEFT_ROW_SPLIT", "")
-    return int(override) if override.isdigit() else _native.load().nnueft_row_split()
-
-
 def get_backward_mode() -> str:
     return _BACKWARD_MODE
+
+
+row_split_of = _ops.row_split_of
 
 
 # Where the index sort of the fused deterministic backward runs (the results are the same bits):
@@ -76,33 +71,25 @@ def get_sort_placement() -> str:
     return _SORT_PLACEMENT
 
 
+# the launches of this file are torch custom ops (nnueft/_ops.py); these helpers serve the launchers of the
+# module layer, which dynamo steps around (opaque to it: traced, current_stream() is a torch.Stream proxy
+# without a raw handle)
 @torch.compiler.disable
 def _stream_ptr(device) -> int:
-    # opaque to dynamo: traced, current_stream() is a torch.Stream proxy without a raw handle
-    return torch.cuda.current_stream(device).cuda_stream
-
-
-_AUX_STREAMS = {}
+    return _ops.stream_ptr(device)
 
 
 @torch.compiler.disable
 def _aux_stream(device):
-    """A second stream per device (default priority) for work that is independent of what runs on the
-    caller's stream; whoever uses it orders it against the caller's stream with events."""
-    key = torch.device(device).index if torch.device(device).index is not None else torch.cuda.current_device()
-    if key not in _AUX_STREAMS:
-        _AUX_STREAMS[key] = torch.cuda.Stream(device=key)
-    return _AUX_STREAMS[key]
+    return _ops.aux_stream(device)
 
 
 @torch.compiler.disable
 def _aux_stream_ptr(device) -> int:
-    return _aux_stream(device).cuda_stream
+    return _ops.aux_stream(device).cuda_stream
 
 
-def _workspace(nbytes: int, device) -> torch.Tensor:
-    # torch's caching allocator hands out blocks aligned to 512 bytes
-    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+_workspace = _ops.workspace
 
 
 def _torch_sparse_linear(feature_indices, weight, bias):
@@ -114,48 +101,6 @@ def _torch_sparse_linear(feature_indices, weight, bias):
     offsets = torch.arange(0, batch_size * max_active, max_active, device=feature_indices.device)
     output = F.embedding_bag(safe_indices, weight, offsets, mode="sum", per_sample_weights=per_sample_weights)
     return output + bias
-
-
-@torch.compiler.disable(recursive=False)
-def _launch_sparse_fwd(feature_indices, weight, bias, output):
-    lib = _native.load()
-    B, K = feature_indices.shape
-    R, out_cols = weight.shape
-    rc = lib.nnueft_sparse_fwd(
-        feature_indices.data_ptr(), weight.data_ptr(), bias.data_ptr(), output.data_ptr(),
-        B, K, R, out_cols, _stream_ptr(weight.device),
-    )
-    _native.check(rc, "nnueft_sparse_fwd")
-
-
-@torch.compiler.disable(recursive=False)
-def _launch_sparse_bwd(feature_indices, grad_output, num_rows, mode):
-    lib = _native.load()
-    B, K = feature_indices.shape
-    out_cols = grad_output.shape[1]
-    device = grad_output.device
-    if mode != "atomic":
-        weight_grad = torch.empty(num_rows, out_cols, dtype=torch.float32, device=device)
-        bias_grad = torch.empty(out_cols, dtype=torch.float32, device=device)
-        if B == 0:
-            return weight_grad.zero_(), bias_grad.zero_()
-        row_split = row_split_of(mode)
-        nbytes = lib.nnueft_det_workspace_bytes(B, K, num_rows, out_cols, 1, row_split)
-        ws = _workspace(nbytes, device)
-        rc = lib.nnueft_sparse_bwd_det(
-            feature_indices.data_ptr(), grad_output.data_ptr(), weight_grad.data_ptr(), bias_grad.data_ptr(),
-            B, K, num_rows, out_cols, row_split, ws.data_ptr(), nbytes, _stream_ptr(device),
-        )
-        _native.check(rc, "nnueft_sparse_bwd_det")
-    else:
-        weight_grad = torch.zeros(num_rows, out_cols, dtype=torch.float32, device=device)
-        bias_grad = torch.zeros(out_cols, dtype=torch.float32, device=device)
-        rc = lib.nnueft_sparse_bwd_atomic(
-            feature_indices.data_ptr(), grad_output.data_ptr(), weight_grad.data_ptr(), bias_grad.data_ptr(),
-            B, K, num_rows, out_cols, _stream_ptr(device),
-        )
-        _native.check(rc, "nnueft_sparse_bwd_atomic")
-    return weight_grad, bias_grad
 
 
 class _CudaSparseLinearFunction(autograd.Function):
@@ -182,22 +127,15 @@ class _CudaSparseLinearFunction(autograd.Function):
         assert weight.is_contiguous()
         assert bias.is_contiguous()
 
-        output = torch.empty(
-            feature_indices.shape[0], weight.shape[1], dtype=torch.float32, device=feature_indices.device
-        )
-        with torch.cuda.device(weight.device):
-            _launch_sparse_fwd(feature_indices, weight, bias, output)
-        return output
+        return _ops.launch("sparse_fwd", feature_indices, weight, bias)
 
     @staticmethod
     def backward(ctx, grad_output):
         assert not ctx.needs_input_grad[0]
         grad_output = grad_output.contiguous()
         feature_indices, weight, _bias = ctx.saved_tensors
-        with torch.cuda.device(weight.device):
-            weight_grad, bias_grad = _launch_sparse_bwd(
-                feature_indices, grad_output, weight.shape[0], ctx.backward_mode
-            )
+        weight_grad, bias_grad = _ops.launch("sparse_bwd", feature_indices, grad_output, weight.shape[0],
+                                                             ctx.backward_mode)
         return None, weight_grad, bias_grad
 
 

@@ -291,6 +291,60 @@ def test_forward_and_deterministic_backward_under_graph_capture():
         torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("mode", ["deterministic", "atomic"])
+@pytest.mark.parametrize("backend", ["aot_eager", "inductor", "cudagraphs"])
+def test_operator_stays_inside_a_compiled_graph(backend, mode):
+    """The operator under plain torch modules, as when it is dropped under the reference's own
+    ComposedFeatureTransformer: table merge and fake quantization in torch ops, double_feature_transform, the
+    activation grid, a loss.  torch.compile with fullgraph=True raises on any graph break, so passing means
+    the launches are part of the compiled graph; with "cudagraphs" they are then inside the captured HIP graph
+    (no 'CUDA Graph is empty' warning), replayed four times and compared with the eager run every time."""
+    import warnings
+
+    nnueft.set_backward_mode(mode)
+    torch._dynamo.reset()
+    L1, B, R = 256, 2048, hk.NUM_INPUTS
+    g = torch.Generator().manual_seed(77)
+    W = (torch.randn(R, L1 + 8, generator=g) * 0.02).to(DEV).requires_grad_()
+    V = (torch.randn(768, L1 + 8, generator=g) * 0.005).to(DEV).requires_grad_()
+    bias = (torch.randn(L1 + 8, generator=g) * 0.02).to(DEV).requires_grad_()
+    target = torch.rand(B, 1, generator=g).to(DEV)
+
+    def step(us, them, white, black, psqt):
+        merged = W + V.repeat(R // 768, 1)
+        merged = merged + ((merged * 256.0).round() / 256.0 - merged).detach()          # fake quantization, STE
+        l0, wp, bp = double_feature_transform(us, them, white, black, psqt, merged, bias, 255.0 / 256.0, L1, "fused")
+        l0 = l0 + ((l0 * 127.0 + 1e-5).floor() / 127.0 - l0).detach()
+        out = l0.sum(dim=1, keepdim=True) * 0.01 + (wp - bp) * (us - 0.5)
+        return ((out.sigmoid() - target) ** 2).mean()
+
+    def grads(fn, batch):
+        for p in (W, V, bias):
+            p.grad = None
+        loss = fn(*batch)
+        loss.backward()
+        return [loss.detach().clone()] + [p.grad.clone() for p in (W, V, bias)]
+
+    batches = []
+    for seed in (61, 62):
+        us, them, white, black, pc = hk.synthetic_batch(B, seed)
+        batches.append([torch.from_numpy(a).to(DEV) for a in (us, them, white, black, (pc - 1) // 4)])
+    eager = [grads(step, b) for b in batches]
+    compiled = torch.compile(step, backend=backend, fullgraph=True)
+    with warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter("always")
+        for call in range(4):
+            got = grads(compiled, batches[call % 2])
+            want = eager[call % 2]
+            torch.testing.assert_close(got[0], want[0], atol=1e-6, rtol=1e-5)
+            if mode == "deterministic" and backend != "inductor":      # same ops around the operator: same bits
+                assert torch.equal(got[1], want[1])
+            for a, b in zip(got[1:], want[1:]):
+                torch.testing.assert_close(a, b, atol=1e-5, rtol=1e-4)
+    assert not [w for w in seen if "Graph is empty" in str(w.message)]
+    torch._dynamo.reset()
+
+
 FULL = [(1024, 8192), (128, 16384), (3072, 16384)]   # BASELINE.json configs 1-3
 
 
