@@ -610,7 +610,7 @@ struct RunPlan {
 // Persistent waves.  A wave takes tasks from its home queue of its XCD, then from the XCD's other
 // queues, until none is left (a counter only grows, so every wave leaves every loop).  Task order per XCD: the
 // windows of the split rows, (perspective, window) pair after pair of those dealt to it, slice by
-// slice; the long rows dealt to it (all slices of a row together); then its row range, slice by slice.
+// slice; the long rows dealt to it (the 64-lane slices of a row together); then its row range, slice by slice.
 template <int VW, int NQ>
 __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, const uint32_t* __restrict__ list,
                                                    const uint32_t* __restrict__ seg_off,
@@ -629,7 +629,10 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
     const uint32_t my_long = n_long > (uint32_t)xcd ? (n_long - xcd + kXcd - 1) / kXcd : 0;
     const uint32_t lo = sched[kSchedRowLo + xcd], hi = sched[kSchedRowLo + xcd + 1];
     const uint32_t nreg = hi - lo;
-    const uint32_t long_end = run_tasks + my_long * (uint32_t)nslices;
+    // long rows: 64-lane slices with kRunUnroll rows in flight (a chain of hundreds of slots is bound by how
+    // many of its loads are in flight; three times as many waves share the row)
+    const uint32_t long_slices = (uint32_t)rp.nslices;
+    const uint32_t long_end = run_tasks + my_long * long_slices;
     // A range whose rows are named by many slots each belongs to a table block that a large part of
     // the batch sits in: one wide slice of all those positions' upstream rows would not fit the L2,
     // so such a range is walked in 64-lane slices (the results do not depend on the slicing).
@@ -664,23 +667,23 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
             seg_reduce_task<VW, 1, kRunUnroll>(G, list, beg, end, end, dst, (int)s, lane, out_cols, rp.slice_v, 0);
             continue;
         }
-        uint32_t r;
-        int s;
         if (t < long_end) {
             const uint32_t u = t - run_tasks;
-            const uint32_t i = u / (uint32_t)nslices;
-            s = (int)(u - i * (uint32_t)nslices);
-            r = long_rows[xcd + i * kXcd];
-        } else {
-            const uint32_t u = t - long_end;
-            s = (int)(u / nreg);
-            r = lo + (u - (uint32_t)s * nreg);
+            const uint32_t i = u / long_slices;
+            const int s = (int)(u - i * long_slices);
+            const uint32_t r = long_rows[xcd + i * kXcd];
+            const uint32_t beg = seg_off[r], end = seg_off[r + 1];
+            seg_reduce_task<VW, 1, kRunUnroll>(G, list, beg, beg + wcount[r], end, gW + (size_t)r * out_cols, s, lane,
+                                               out_cols, rp.slice_v, two_persp);
+            continue;
         }
+        const uint32_t u = t - long_end;
+        const int s = (int)(u / nreg);
+        const uint32_t r = lo + (u - (uint32_t)s * nreg);
         const uint32_t beg = seg_off[r], end = seg_off[r + 1];
         // long or split: done elsewhere
-        if (t >= long_end && (end - beg >= (uint32_t)kLongRow || (rp.row_split != 0 && end - beg > rp.row_split)))
-            continue;
-        if (t >= long_end && narrow)
+        if (end - beg >= (uint32_t)kLongRow || (rp.row_split != 0 && end - beg > rp.row_split)) continue;
+        if (narrow)
             seg_reduce_task<VW, 1, kRunUnroll>(G, list, beg, beg + wcount[r], end, gW + (size_t)r * out_cols, s, lane,
                                                out_cols, rp.slice_v, two_persp);
         else

@@ -345,6 +345,34 @@ def test_operator_stays_inside_a_compiled_graph(backend, mode):
     torch._dynamo.reset()
 
 
+def test_custom_ops_pass_torch_opcheck():
+    """torch.library.opcheck on the operator's four launches: the declared schema (nothing mutated, nothing
+    aliased) and the shape functions against what the kernels really return."""
+    from nnueft import _ops  # noqa: F401
+
+    B, L1, R, K = 300, 64, 900, 32
+    c = double_case(5, B, L1, R, K, binary_side=True)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+    us, them, widx, bidx, psqt = t(c["us"]), t(c["them"]), t(c["widx"]), t(c["bidx"]), t(c["psqt_idx"])
+    W, bias = t(c["W"]), t(c["bias"])
+    checks = ("test_schema", "test_faketensor")
+    torch.library.opcheck(torch.ops.nnueft.sparse_fwd.default, (widx, W, bias), test_utils=checks)
+    g = torch.randn(B, L1 + 8, device=DEV)
+    for mode in ("deterministic", "deterministic_strict", "atomic"):
+        torch.library.opcheck(torch.ops.nnueft.sparse_bwd.default, (widx, g, R, mode), test_utils=checks)
+    fwd_args = (us, them, widx, bidx, psqt, W, bias, 0.99, L1, False, 1.0, 0.0, 1.0)
+    torch.library.opcheck(torch.ops.nnueft.double_fwd.default, fwd_args, test_utils=checks)
+    torch.library.opcheck(torch.ops.nnueft.double_fwd.default, fwd_args[:9] + (True, 127.0, 1e-5, 1.0), test_utils=checks)
+    l0, wp, bp, saved = torch.ops.nnueft.double_fwd(*fwd_args)
+    lists = torch.ops.nnueft.det_sort(widx, bidx, R, L1 + 8, 512)
+    torch.library.opcheck(torch.ops.nnueft.det_sort.default, (widx, bidx, R, L1 + 8, 512), test_utils=checks)
+    torch.cuda.synchronize()
+    for mode, presorted in (("deterministic", None), ("deterministic", lists), ("atomic", None)):
+        torch.library.opcheck(torch.ops.nnueft.double_bwd.default,
+                              (us, them, widx, bidx, psqt, bias, 0.99, torch.randn_like(l0), torch.randn_like(wp),
+                               torch.randn_like(bp), saved, R, L1, L1 + 8, mode, presorted, False), test_utils=checks)
+
+
 FULL = [(1024, 8192), (128, 16384), (3072, 16384)]   # BASELINE.json configs 1-3
 
 
