@@ -39,7 +39,7 @@ constexpr int kChunk = NNUEFT_SORT_CHUNK;        // positions per sort chunk
 #define NNUEFT_SEG_NQ 3
 #endif
 #ifndef NNUEFT_SEG_WAVES
-#define NNUEFT_SEG_WAVES 512
+#define NNUEFT_SEG_WAVES 320
 #endif
 constexpr int kRowsUnroll = NNUEFT_SEG_U;  // rows in flight per lane group in the segmented reduction
 using nnueft_blocked::kXcd;
@@ -51,7 +51,12 @@ constexpr int kLongRow = NNUEFT_LONG_ROW;  // table rows named by at least this 
 #ifndef NNUEFT_RUN_U
 #define NNUEFT_RUN_U 16
 #endif
-constexpr int kRunUnroll = NNUEFT_RUN_U;   // rows in flight per lane in the chain of one window of a split row
+constexpr int kRunUnroll = NNUEFT_RUN_U;
+#ifndef NNUEFT_TAIL_U
+#define NNUEFT_TAIL_U 8
+#endif
+constexpr int kTailUnroll = NNUEFT_TAIL_U;
+constexpr int kTailMax = 8;   // most trailing vectors that are handled that way  // slots in flight per lane where a wave reduces the last columns of many rows   // rows in flight per lane in the chain of one window of a split row
 #ifndef NNUEFT_NARROW_AVG
 #define NNUEFT_NARROW_AVG 64
 #endif
@@ -324,6 +329,26 @@ __device__ __forceinline__ int xcd_of(unsigned long long w, unsigned long long d
     return x;
 }
 
+// What a row's slots weigh less in its row range than their number: all of them for a split row (its windows
+// are tasks of their own).  A row named by kHeavyRow slots or more sits in a table block that much of the batch
+// names, where the upstream rows of a slice overflow the L2 and a slot costs a trip to memory: such slots count
+// kHeavyFactor times (a negative return), so the XCDs that own crowded blocks get shorter ranges.
+#ifndef NNUEFT_HEAVY_ROW
+#define NNUEFT_HEAVY_ROW 64
+#endif
+#ifndef NNUEFT_HEAVY_F
+#define NNUEFT_HEAVY_F 3
+#endif
+constexpr int kHeavyRow = NNUEFT_HEAVY_ROW;
+constexpr int kHeavyFactor = NNUEFT_HEAVY_F;
+__device__ __forceinline__ uint32_t slots_elsewhere(uint32_t raw) {
+    const uint32_t len = raw & ~kSplitFlag;
+    if (raw & kSplitFlag) return len;
+    // (wraps below zero: the caller subtracts it, which adds the surcharge)
+    if (len >= (uint32_t)kHeavyRow && len < (uint32_t)kLongRow) return 0u - len * (uint32_t)(kHeavyFactor - 1);
+    return 0u;
+}
+
 // Single workgroup: seg_off (holding per-row totals) -> exclusive offsets, seg_off[R] = grand total.
 // Also the work split of the segmented reduction: the split rows (flagged by k_col_scan), the other
 // rows named by >= kLongRow slots (their chains are long and start first), and kXcd contiguous row
@@ -338,7 +363,7 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
                                                            uint32_t* __restrict__ long_rows,
                                                            uint32_t* __restrict__ sched, int R, int cap) {
     extern __shared__ uint32_t stage[];   // `cap` row lengths, turned into offsets in place
-    // two running sums: all slots, slots of split rows
+    // two running sums: all slots, and what slots_elsewhere() takes off the weight of the row ranges
     __shared__ uint32_t wave_tot[2][kScanThreads / 64];
     __shared__ uint32_t carry_s[2], total_s[2], n_long_s, n_split_s;
     __shared__ uint32_t lo_s[kXcd + 1];
@@ -359,7 +384,7 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
         for (int i = tid; i < R; i += kScanThreads) {
             const uint32_t raw = seg_off[i];
             s0 += raw & ~kSplitFlag;
-            s1 += (raw & kSplitFlag) ? (raw & ~kSplitFlag) : 0u;
+            s1 += slots_elsewhere(raw);
         }
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) {
@@ -398,7 +423,7 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
         for (int i = i_beg; i < i_end; ++i) {
             const uint32_t raw = stage[i];
             local[0] += raw & ~kSplitFlag;
-            local[1] += (raw & kSplitFlag) ? (raw & ~kSplitFlag) : 0u;
+            local[1] += slots_elsewhere(raw);
         }
         uint32_t incl[2] = {local[0], local[1]};
 #pragma unroll
@@ -427,7 +452,8 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
             if (!one_pass) all[k] = total_s[k];
         }
         // XCD of a row = floor(kXcd * weight of the rows before it / weight of all rows), weight =
-        // kRowWeight + its slots unless it is split; a range begins where that number goes up
+        // kRowWeight + its slots (none for a split row, kHeavyFactor times for a heavy one); a range begins
+        // where that number goes up
         const unsigned long long denom = (unsigned long long)(all[0] - all[1]) + (unsigned long long)R * kRowWeight;
         int x_cur = 0;
         if (i_beg < i_end) {
@@ -442,10 +468,10 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
             // a row is in at most one of the two lists, so they cannot meet inside long_rows[0..R)
             if (raw & kSplitFlag) {
                 long_rows[R - 1 - (int)atomicAdd(&n_split_s, 1u)] = (uint32_t)(base + i);
-                run[1] += len;
             } else if (len >= (uint32_t)kLongRow) {
                 long_rows[atomicAdd(&n_long_s, 1u)] = (uint32_t)(base + i);
             }
+            run[1] += slots_elsewhere(raw);
             run[0] += len;
             const int r_next = base + i + 1;
             if (r_next < R) {
@@ -550,10 +576,12 @@ __global__ __launch_bounds__(256) void k_fill(const int32_t* __restrict__ widx, 
 // ---------------------------------------------------------------------------------------------
 // Segmented reduction.  list[seg_off[r] .. +wcount[r]) are the white-perspective rows of G naming
 // table row r, the rest of the segment the black ones.  gW[r] = white chain (+ black chain).
+// `pre`: the caller already holds list[beg + lane] of a segment of at most 64 slots in `pre_my`.
 template <int VW, int NQ, int U>
 __device__ __forceinline__ void seg_reduce_task(const float* __restrict__ G, const uint32_t* __restrict__ list,
                                                 uint32_t beg, uint32_t mid, uint32_t end, float* __restrict__ dst,
-                                                int s, int lane, int out_cols, int slice_v, int two_persp) {
+                                                int s, int lane, int out_cols, int slice_v, int two_persp,
+                                                bool pre = false, int pre_my = 0) {
     const int nv = out_cols / VW;
     int col[NQ];
     bool act[NQ];
@@ -569,12 +597,23 @@ __device__ __forceinline__ void seg_reduce_task(const float* __restrict__ G, con
     for (int p = 0; p < 2; ++p) {
 #pragma unroll
         for (int m = 0; m < NQ; ++m) acc[p][m] = vzero<VW>();
-        const uint32_t e_beg = p ? mid : beg, e_end = p ? end : mid;
-        for (uint32_t e0 = e_beg; e0 < e_end; e0 += 64) {
-            const uint32_t n = min(64u, e_end - e0);
-            const int my = lane < (int)n ? (int)list[e0 + lane] : 0;
-            const u64 mask = n >= 64 ? ~0ull : ((1ull << n) - 1ull);
-            chain_rows<VW, NQ, U>(acc[p], G, (size_t)out_cols, col, my, mask);
+    }
+    if (pre) {
+        const uint32_t nw = mid - beg, n = end - beg;
+        const u64 all = n >= 64 ? ~0ull : ((1ull << n) - 1ull);
+        const u64 white = nw >= 64 ? ~0ull : ((1ull << nw) - 1ull);
+        chain_rows<VW, NQ, U>(acc[0], G, (size_t)out_cols, col, pre_my, white);
+        chain_rows<VW, NQ, U>(acc[1], G, (size_t)out_cols, col, pre_my, all & ~white);
+    } else {
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const uint32_t e_beg = p ? mid : beg, e_end = p ? end : mid;
+            for (uint32_t e0 = e_beg; e0 < e_end; e0 += 64) {
+                const uint32_t n = min(64u, e_end - e0);
+                const int my = lane < (int)n ? (int)list[e0 + lane] : 0;
+                const u64 mask = n >= 64 ? ~0ull : ((1ull << n) - 1ull);
+                chain_rows<VW, NQ, U>(acc[p], G, (size_t)out_cols, col, my, mask);
+            }
         }
     }
 #pragma unroll
@@ -582,6 +621,58 @@ __device__ __forceinline__ void seg_reduce_task(const float* __restrict__ G, con
         if (!act[m]) continue;
         if (two_persp) vadd<VW>(acc[0][m], acc[1][m]);
         stv_stream<VW>(dst + col[m], acc[0][m]);
+    }
+}
+
+// The last few columns of a row (the 8 PSQT columns behind 3072 others) do not fill a slice of their own:
+// a wave that walked one row's list for them would pay a whole task for 32 bytes per slot.  Here a wave
+// takes 64 / g consecutive rows at once, g lanes per row, every lane group walking its own row's list
+// (U slots in flight per lane, the next U list entries fetched meanwhile).  Same chains, same order.
+template <int VW, int U>
+__device__ __forceinline__ void tail_rows_task(const float* __restrict__ G, const uint32_t* __restrict__ list,
+                                               const uint32_t* __restrict__ seg_off,
+                                               const uint32_t* __restrict__ wcount, float* __restrict__ gW,
+                                               uint32_t r0, uint32_t r1, int lane, int out_cols, int tail_v, int g,
+                                               int two_persp, uint32_t row_split) {
+    const int sub = lane % g;
+    const uint32_t row = r0 + (uint32_t)(lane / g);
+    bool on = row < r1 && sub < tail_v;
+    uint32_t bounds[3] = {0, 0, 0};
+    if (on) {
+        bounds[0] = seg_off[row];
+        bounds[2] = seg_off[row + 1];
+        bounds[1] = bounds[0] + wcount[row];
+        const uint32_t len = bounds[2] - bounds[0];
+        // long or split: done elsewhere, tail included
+        if (len >= (uint32_t)kLongRow || (row_split != 0 && len > row_split)) on = false;
+    }
+    if (!on) bounds[0] = bounds[1] = bounds[2] = 0;
+    const size_t col = (size_t)(out_cols / VW - tail_v + (on ? sub : 0)) * VW;
+    const float* src = G + col;
+    vecf<VW> acc[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        acc[p] = vzero<VW>();
+        uint32_t e = bounds[p];
+        const uint32_t e_end = bounds[p + 1];
+        uint32_t nid[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) nid[u] = e + u < e_end ? list[e + u] : 0u;
+        while (__any(e < e_end)) {
+            vecf<VW> v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[u] = e + u < e_end ? ldv<VW>(src + (size_t)nid[u] * out_cols) : vzero<VW>();
+#pragma unroll
+            for (int u = 0; u < U; ++u) nid[u] = e + U + u < e_end ? list[e + U + u] : 0u;
+            // a chain that started at +0 never holds -0, so adding the +0 of a lane that has run out changes no bit
+#pragma unroll
+            for (int u = 0; u < U; ++u) vadd<VW>(acc[p], v[u]);
+            e += U;
+        }
+    }
+    if (on) {
+        if (two_persp) vadd<VW>(acc[0], acc[1]);
+        stv_stream<VW>(gW + (size_t)row * out_cols + col, acc[0]);
     }
 }
 
@@ -604,6 +695,7 @@ struct RunPlan {
     float* runs;           // [split row, perspective, window, out_cols] window sums
     int R, cpp, nchunks, wch, nwin, n_persp;
     int nslices, slice_v;  // 64-lane slices
+    int tail_v, tail_g;    // trailing vectors of a row that tail_rows_task reduces (0: none), lanes per row there
     uint32_t row_split;    // rows named by more slots than this are the split ones (0: none)
 };
 
@@ -636,9 +728,12 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
     // A range whose rows are named by many slots each belongs to a table block that a large part of
     // the batch sits in: one wide slice of all those positions' upstream rows would not fit the L2,
     // so such a range is walked in 64-lane slices (the results do not depend on the slicing).
-    const bool narrow = nreg > 0 && (seg_off[hi] - seg_off[lo]) / nreg > (uint32_t)kNarrowAvg && rp.nslices > nslices;
-    const uint32_t walk_slices = narrow ? (uint32_t)rp.nslices : (uint32_t)nslices;
-    const uint32_t ntasks = long_end + nreg * walk_slices;
+    const uint32_t narrow_slices = (uint32_t)(rp.nslices - (rp.tail_v ? 1 : 0));   // the tail has tasks of its own
+    const bool narrow = nreg > 0 && (seg_off[hi] - seg_off[lo]) / nreg > (uint32_t)kNarrowAvg && narrow_slices > (uint32_t)nslices;
+    const uint32_t walk_slices = narrow ? narrow_slices : (uint32_t)nslices;
+    const uint32_t tail_rows = rp.tail_v ? 64u / (uint32_t)rp.tail_g : 1u;
+    const uint32_t tail_tasks = rp.tail_v ? (nreg + tail_rows - 1) / tail_rows : 0u;
+    const uint32_t ntasks = long_end + tail_tasks + nreg * walk_slices;
     static_assert(kQueues <= kSchedQueues, "counters per XCD");
     const int home = (blockIdx.x / kXcd) % kQueues;
 
@@ -677,18 +772,30 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
                                                out_cols, rp.slice_v, two_persp);
             continue;
         }
-        const uint32_t u = t - long_end;
+        uint32_t u = t - long_end;
+        if (u < tail_tasks) {   // first: they are few and each is a long chain of short steps
+            const uint32_t r0 = lo + u * tail_rows;
+            tail_rows_task<VW, kTailUnroll>(G, list, seg_off, wcount, gW, r0, hi, lane, out_cols, rp.tail_v, rp.tail_g,
+                                            two_persp, rp.row_split);
+            continue;
+        }
+        u -= tail_tasks;
         const int s = (int)(u / nreg);
         const uint32_t r = lo + (u - (uint32_t)s * nreg);
         const uint32_t beg = seg_off[r], end = seg_off[r + 1];
+        const uint32_t len = end - beg;
         // long or split: done elsewhere
-        if (end - beg >= (uint32_t)kLongRow || (rp.row_split != 0 && end - beg > rp.row_split)) continue;
+        if (len >= (uint32_t)kLongRow || (rp.row_split != 0 && len > rp.row_split)) continue;
+        // a segment of 64 slots at most: one load brings the white and the black part of the list
+        const bool pre = len <= 64u;
+        const int my = (pre && (uint32_t)lane < len) ? (int)list[beg + lane] : 0;
+        float* dst = gW + (size_t)r * out_cols;
         if (narrow)
-            seg_reduce_task<VW, 1, kRunUnroll>(G, list, beg, beg + wcount[r], end, gW + (size_t)r * out_cols, s, lane,
-                                               out_cols, rp.slice_v, two_persp);
+            seg_reduce_task<VW, 1, kRunUnroll>(G, list, beg, beg + wcount[r], end, dst, s, lane, out_cols, rp.slice_v,
+                                               two_persp, pre, my);
         else
-            seg_reduce_task<VW, NQ, kRowsUnroll>(G, list, beg, beg + wcount[r], end, gW + (size_t)r * out_cols, s,
-                                                 lane, out_cols, slice_v, two_persp);
+            seg_reduce_task<VW, NQ, kRowsUnroll>(G, list, beg, beg + wcount[r], end, dst, s, lane, out_cols, slice_v,
+                                                 two_persp, pre, my);
     }
   }
 }
@@ -821,10 +928,18 @@ int det_reduce(const float* G, float* gW, float* gbias, int B, int R, int out_co
     const int VWr = vec ? 4 : 1;
     const int nv = out_cols / VWr;
     const int NQ = nv > 64 ? NNUEFT_SEG_NQ : 1;
-    const int nslices = (nv + 64 * NQ - 1) / (64 * NQ);
+    // up to kTailMax vectors beyond a whole number of 64-lane slices are reduced many rows at a time
+    int tail_v = (nv > 64 && nv % 64 <= kTailMax) ? nv % 64 : 0;
+#ifdef NNUEFT_NO_TAIL
+    tail_v = 0;
+#endif
+    int tail_g = 1;
+    while (tail_g < tail_v) tail_g *= 2;
+    const int nv_main = nv - tail_v;
+    const int nslices = (nv_main + 64 * NQ - 1) / (64 * NQ);
     // equal slices, rounded up to whole 128-byte lines so no two waves share a cache line of a row
     const int line_v = 128 / (VWr * (int)sizeof(float));
-    const int slice_v = ((nv + nslices - 1) / nslices + line_v - 1) / line_v * line_v;
+    const int slice_v = ((nv_main + nslices - 1) / nslices + line_v - 1) / line_v * line_v;
     if ((long long)R * nslices > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
     const int two = n_persp == 2;
     RunPlan rp;
@@ -837,7 +952,10 @@ int det_reduce(const float* G, float* gW, float* gbias, int B, int R, int out_co
     rp.nwin = L.nwin;
     rp.n_persp = n_persp;
     rp.nslices = (nv + 63) / 64;
-    rp.slice_v = ((nv + rp.nslices - 1) / rp.nslices + line_v - 1) / line_v * line_v;
+    // (with a tail: whole 64-lane slices and the tail as the last one, which the row ranges leave out)
+    rp.slice_v = tail_v ? 64 : ((nv + rp.nslices - 1) / rp.nslices + line_v - 1) / line_v * line_v;
+    rp.tail_v = tail_v;
+    rp.tail_g = tail_g;
     rp.row_split = (uint32_t)L.row_split;
     if ((long long)L.max_split * rp.nslices * NNUEFT_ROW_WINDOWS > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
 #define SEG_LAUNCH(VW_, NQ_)                                                                                      \

@@ -11,16 +11,17 @@
 #define NNUEFT_BIAS_TILE 32
 // Deterministic weight gradient: a table row named by more slots than NNUEFT_ROW_SPLIT (both
 // perspectives together) is summed window by window, a window being nnueft_window_positions(B)
-// consecutive positions: at most NNUEFT_ROW_WINDOWS windows of at least NNUEFT_ROW_WINDOW_MIN
-// positions, a multiple of 128.
+// consecutive positions: as few windows as keep each at NNUEFT_ROW_WINDOW_MIN positions or fewer, at
+// most NNUEFT_ROW_WINDOWS of them, a multiple of 128.  (A window's upstream rows, one 1 KB slice of
+// each, are what a XCD's L2 has to hold while the split rows are reduced: 1 MB at 1024 positions.)
 #ifndef NNUEFT_ROW_SPLIT
 #define NNUEFT_ROW_SPLIT 512
 #endif
 #ifndef NNUEFT_ROW_WINDOWS
-#define NNUEFT_ROW_WINDOWS 8
+#define NNUEFT_ROW_WINDOWS 16
 #endif
 #ifndef NNUEFT_ROW_WINDOW_MIN
-#define NNUEFT_ROW_WINDOW_MIN 2048
+#define NNUEFT_ROW_WINDOW_MIN 1024
 #endif
 static inline int nnueft_window_positions(int B) {
     int nwin = (B + NNUEFT_ROW_WINDOW_MIN - 1) / NNUEFT_ROW_WINDOW_MIN;

@@ -65,13 +65,13 @@ int nnueft_oracle_bias_tile(void) { return NNUEFT_ORACLE_BIAS_TILE; }
 #define NNUEFT_ORACLE_ROW_SPLIT 512
 int nnueft_oracle_row_split(void) { return NNUEFT_ORACLE_ROW_SPLIT; }
 
-/* Window length: as few windows as hold at least 2048 positions each, at most 8, equal lengths
- * rounded up to a multiple of 128. */
+/* Window length: as few windows as keep every window at 1024 positions or fewer, at most 16 of them,
+ * equal lengths rounded up to a multiple of 128. */
 int nnueft_oracle_row_window(int B)
 {
-    int nwin = (B + 2047) / 2048;
+    int nwin = (B + 1023) / 1024;
     if (nwin < 1) nwin = 1;
-    if (nwin > 8) nwin = 8;
+    if (nwin > 16) nwin = 16;
     int w = (B + nwin - 1) / nwin;
     return (w + 127) / 128 * 128;
 }

@@ -115,9 +115,9 @@ BIG = float(2 ** 24)
 
 def test_row_window_lengths(oracle_cpu):
     assert oracle_cpu.row_split() == 512
-    # one window up to 2048 positions, then as few as hold >= 2048 each, at most 8, multiples of 128
-    assert [oracle_cpu.row_window(B) for B in (1, 100, 2048, 2049, 4096, 8192, 16384, 16385, 65536, 100000)] == \
-        [128, 128, 2048, 1152, 2048, 2048, 2048, 2176, 8192, 12544]
+    # one window up to 1024 positions, then as few as keep each at 1024 or fewer, at most 16, multiples of 128
+    assert [oracle_cpu.row_window(B) for B in (1, 100, 1024, 2048, 2049, 4096, 8192, 16384, 16385, 65536, 100000)] == \
+        [128, 128, 1024, 1024, 768, 1024, 1024, 1024, 1152, 4096, 6272]
 
 
 def _ones_after_big(B, K, R, row, positions):
@@ -132,7 +132,7 @@ def _ones_after_big(B, K, R, row, positions):
 def test_sparse_backward_split_row_sums_windows_separately(oracle_cpu):
     B, K, R = 4096, 2, 5
     W = oracle_cpu.row_window(B)
-    assert W == 2048
+    assert W == 1024
     # 600 slots > row_split: position 0 (2**24), 299 ones in window 0, 300 ones in window 1
     pos = np.r_[0:300, W:W + 300]
     idx, g = _ones_after_big(B, K, R, 3, pos)
@@ -155,7 +155,7 @@ def test_sparse_backward_split_row_sums_windows_separately(oracle_cpu):
 def test_sparse_backward_split_row_window_sums_are_chained_in_order(oracle_cpu):
     B, K, R = 8192, 1, 2
     W = oracle_cpu.row_window(B)
-    assert W == 2048
+    assert W == 1024
     # windows 0..3 hold 2**24, 200 ones, 200 ones, 200 ones: ((2**24 + 200) + 200) + 200, all exact
     pos = np.r_[0:1, W:W + 200, 2 * W:2 * W + 200, 3 * W:3 * W + 200]
     idx, g = _ones_after_big(B, K, R, 1, pos)
@@ -269,7 +269,7 @@ def test_strict_order_bits_equal_torch_cpu_autograd_with_crowded_rows(oracle_cpu
     assert np.array_equal(strict, W.grad.numpy())
     windowed, _ = oracle_cpu.sparse_bwd(c["idx"], c["g"], R)
     assert not np.array_equal(windowed[5], strict[5])                  # the crowded row: another order
-    assert np.allclose(windowed[5], strict[5], rtol=1e-4, atol=1e-3)    # ... the same sum to rounding
+    assert np.allclose(windowed[5], strict[5], rtol=1e-4, atol=1e-2)    # ... the same sum to rounding (24 000 addends)
     counts = np.bincount(c["idx"][c["idx"] >= 0], minlength=R)
     short = counts <= oracle_cpu.row_split()                           # rows the default order leaves whole
     assert np.array_equal(windowed[short], strict[short])
