@@ -18,9 +18,11 @@
 //                   large part of the batch has many) is cut at the window boundaries instead: one
 //                   task per (row, perspective, window, slice) writes that window's sum, and a XCD
 //                   takes whole (perspective, window) pairs, so what it gathers is one slice of
-//                   one window's upstream rows
-//   k_split_combine the window sums of a split row: chain over the windows, white + black
-//   k_bias_final    chain over the tile partial sums
+//                   one window's upstream rows.  The last columns of the rows (the 8 PSQT columns
+//                   behind a whole number of 64-lane slices) are reduced 32 rows per wave
+//   k_split_combine the window sums of a split row: chain over the windows, white + black; its first
+//                   workgroups chain the tile partial sums of the bias gradient
+//   k_bias_final    the same chain as a launch of its own where no row can be split (strict order)
 #include <atomic>
 
 #include "gather.h"
@@ -220,14 +222,14 @@ __global__ __launch_bounds__(256) void k_tile_colsum(const float* __restrict__ g
 
 // gbias[c] = chain over the tiles of partial[tile, c].  The adds are one dependent chain; the loads
 // are not, so they are issued a batch ahead.
-__global__ __launch_bounds__(64) void k_bias_final(const float* __restrict__ partial, float* __restrict__ gbias,
-                                                   int ntiles, int out_cols, uint32_t* __restrict__ sched) {
+__device__ __forceinline__ void bias_final_block(const float* __restrict__ partial, float* __restrict__ gbias,
+                                                 int ntiles, int out_cols, uint32_t* __restrict__ sched, int block) {
     // the last kernel of the backward also rewinds the task counters, so the sorted lists can serve
     // another reduction (a second backward through the same graph)
-    if (sched && blockIdx.x == 0)
+    if (sched && block == 0)
         for (int i = threadIdx.x; i < kXcd * kSchedQueues; i += 64) sched[kSchedCtr + i * 32] = 0;
     if (!partial) return;   // the rows-only reduction: nothing but the rewind
-    const int c = blockIdx.x * 64 + threadIdx.x;
+    const int c = block * 64 + threadIdx.x;
     if (c >= out_cols) return;
     constexpr int PF = 64;
     float total = 0.0f;
@@ -241,6 +243,11 @@ __global__ __launch_bounds__(64) void k_bias_final(const float* __restrict__ par
     }
     for (; t < ntiles; ++t) total = total + partial[(size_t)t * out_cols + c];
     gbias[c] = total;
+}
+
+__global__ __launch_bounds__(64) void k_bias_final(const float* __restrict__ partial, float* __restrict__ gbias,
+                                                   int ntiles, int out_cols, uint32_t* __restrict__ sched) {
+    bias_final_block(partial, gbias, ntiles, out_cols, sched, (int)blockIdx.x);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -803,16 +810,25 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
 // gW[r] of a split row = (chain over the windows of its white window sums) + (the same, black).
 // One wave per (split row, 64-lane slice); an empty window's sum is +0, which changes no bit of a
 // chain that started at +0.
+// The first `nbias` workgroups of slice 0 are the last step of the bias gradient instead (and rewind the task
+// counters): one launch less behind the reduction.
 template <int VW>
 __global__ __launch_bounds__(64) void k_split_combine(const uint32_t* __restrict__ long_rows,
-                                                      const uint32_t* __restrict__ sched,
-                                                      float* __restrict__ gW, int out_cols, RunPlan rp) {
+                                                      uint32_t* __restrict__ sched, float* __restrict__ gW,
+                                                      int out_cols, RunPlan rp, const float* __restrict__ partial,
+                                                      float* __restrict__ gbias, int ntiles, int nbias) {
     const int lane = threadIdx.x;
+    if (blockIdx.x < (unsigned)nbias) {
+        // (every workgroup reads n_split below; the rewind touches the task counters only)
+        if (blockIdx.y == 0) bias_final_block(partial, gbias, ntiles, out_cols, sched, (int)blockIdx.x);
+        return;
+    }
     const uint32_t n_split = sched[kSchedNSplit];
     const int q = blockIdx.y * 64 + lane;
     if (q >= out_cols / VW) return;
     const int col = q * VW;
-    for (uint32_t j = blockIdx.x; j < n_split; j += gridDim.x) {
+    const uint32_t stride = gridDim.x - (uint32_t)nbias;
+    for (uint32_t j = blockIdx.x - (uint32_t)nbias; j < n_split; j += stride) {
         const uint32_t r = long_rows[(uint32_t)rp.R - 1u - j];
         vecf<VW> tot = vzero<VW>();
         for (int p = 0; p < rp.n_persp; ++p) {
@@ -968,14 +984,19 @@ int det_reduce(const float* G, float* gW, float* gbias, int B, int R, int out_co
 #undef SEG_LAUNCH
     NNUEFT_LAUNCH_CHECK();
     if (L.max_split > 0) {
-        const dim3 cgrid((unsigned)min(L.max_split, 1024), (unsigned)rp.nslices);
+        const int nbias = (out_cols + 63) / 64;
+        const int ntiles = (B + NNUEFT_BIAS_TILE - 1) / NNUEFT_BIAS_TILE;
+        const float* part = gbias ? partial : nullptr;
+        const dim3 cgrid((unsigned)(nbias + min(L.max_split, 1024)), (unsigned)rp.nslices);
         if (vec)
-            hipLaunchKernelGGL(k_split_combine<4>, cgrid, dim3(64), 0, st, long_rows, sched, gW, out_cols, rp);
+            hipLaunchKernelGGL(k_split_combine<4>, cgrid, dim3(64), 0, st, long_rows, sched, gW, out_cols, rp, part,
+                               gbias, ntiles, nbias);
         else
-            hipLaunchKernelGGL(k_split_combine<1>, cgrid, dim3(64), 0, st, long_rows, sched, gW, out_cols, rp);
+            hipLaunchKernelGGL(k_split_combine<1>, cgrid, dim3(64), 0, st, long_rows, sched, gW, out_cols, rp, part,
+                               gbias, ntiles, nbias);
         NNUEFT_LAUNCH_CHECK();
+        return 0;
     }
-
     return nnueft_det::launch_bias_final(gbias ? partial : nullptr, gbias, B, out_cols, sched, st);
 }
 
@@ -983,13 +1004,18 @@ int det_reduce(const float* G, float* gW, float* gbias, int B, int R, int out_co
 
 namespace nnueft_det {
 
+constexpr long long kRowsScalarBelow = 2048;   // waves of 16-byte lanes below which k_bwd_rows uses 4-byte lanes
+
 int launch_bwd_rows(const float* us, const float* them, const int64_t* psqt_idx, const float* bias, float max_act,
                     const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt, const float* saved,
                     float* G, float* partial, int B, int L1, int n_psqt, hipStream_t st) {
     const int out_cols = L1 + n_psqt;
     const int ntiles = (B + NNUEFT_BIAS_TILE - 1) / NNUEFT_BIAS_TILE;
-    const bool vec = (L1 % 8 == 0) && (out_cols % 4 == 0) && aligned16(grad_l0) && aligned16(saved) &&
-                     aligned16(bias) && aligned16(G) && aligned16(partial);
+    bool vec = (L1 % 8 == 0) && (out_cols % 4 == 0) && aligned16(grad_l0) && aligned16(saved) &&
+               aligned16(bias) && aligned16(G) && aligned16(partial);
+    // a tile is one chain over its positions: with few tiles and narrow rows, 16-byte lanes leave most of the
+    // chip without a wave; 4-byte lanes give four times the waves (config 2: 128 -> 512 waves, 44 -> 30 us)
+    if (vec && (long long)ntiles * ((L1 / 8 + 63) / 64) < kRowsScalarBelow) vec = false;
     const int hv = (L1 / 2) / (vec ? 4 : 1);
     int group = 64;
     while (group > 8 && group / 2 >= hv) group /= 2;   // lanes per tile: 64, 32, 16 or 8
