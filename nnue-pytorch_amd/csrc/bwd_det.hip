@@ -366,21 +366,28 @@ __device__ __forceinline__ uint32_t slots_elsewhere(uint32_t raw) {
 #endif
 constexpr uint32_t kRowWeight = NNUEFT_ROW_WEIGHT;   // cost of a task that finds nothing to add, in slots
 constexpr int kScanThreads = 1024;
+constexpr int kLongClasses = 8;   // long rows by length: [kLongRow, 2 kLongRow), [2 kLongRow, 4 kLongRow), ...
+__device__ __forceinline__ int long_class(uint32_t len) {
+    const int c = (31 - __clz((int)(len / (uint32_t)kLongRow)));
+    return c < kLongClasses - 1 ? c : kLongClasses - 1;
+}
 __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict__ seg_off,
                                                            uint32_t* __restrict__ long_rows,
-                                                           uint32_t* __restrict__ sched, int R, int cap) {
+                                                           uint32_t* __restrict__ sched, int R, int cap,
+                                                           uint32_t row_split) {
     extern __shared__ uint32_t stage[];   // `cap` row lengths, turned into offsets in place
     // two running sums: all slots, and what slots_elsewhere() takes off the weight of the row ranges
     __shared__ uint32_t wave_tot[2][kScanThreads / 64];
-    __shared__ uint32_t carry_s[2], total_s[2], n_long_s, n_split_s;
+    __shared__ uint32_t carry_s[2], total_s[2], n_split_s;
+    __shared__ uint32_t long_cnt[kLongClasses];
     __shared__ uint32_t lo_s[kXcd + 1];
     const int tid = threadIdx.x;
     if (tid == 0) {
         carry_s[0] = 0;
         carry_s[1] = 0;
-        n_long_s = 0;
         n_split_s = 0;
     }
+    if (tid < kLongClasses) long_cnt[tid] = 0;
     if (tid <= kXcd) lo_s[tid] = (uint32_t)R;
     if (tid < kXcd * kSchedQueues) sched[kSchedCtr + tid * 32] = 0;
     // The row ranges need the two totals before the scan reaches the rows.  A table that fits the
@@ -476,7 +483,7 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
             if (raw & kSplitFlag) {
                 long_rows[R - 1 - (int)atomicAdd(&n_split_s, 1u)] = (uint32_t)(base + i);
             } else if (len >= (uint32_t)kLongRow) {
-                long_rows[atomicAdd(&n_long_s, 1u)] = (uint32_t)(base + i);
+                atomicAdd(&long_cnt[long_class(len)], 1u);
             }
             run[1] += slots_elsewhere(raw);
             run[0] += len;
@@ -496,10 +503,24 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
         for (int i = tid; i < n; i += kScanThreads) seg_off[base + i] = stage[i];
         __syncthreads();
     }
+    // The long rows, longest class first: their chains are the longest tasks of the reduction and are dealt to
+    // the XCDs in this order.
     if (tid == 0) {
         seg_off[R] = carry_s[0];
-        sched[kSchedNLong] = n_long_s;
+        uint32_t at = 0;
+        for (int c = kLongClasses - 1; c >= 0; --c) {
+            const uint32_t n = long_cnt[c];
+            long_cnt[c] = at;   // from here on the class's cursor
+            at += n;
+        }
+        sched[kSchedNLong] = at;
         sched[kSchedNSplit] = n_split_s;
+    }
+    __syncthreads();
+    for (int i = tid; i < R; i += kScanThreads) {
+        const uint32_t len = seg_off[i + 1] - seg_off[i];
+        if (len >= (uint32_t)kLongRow && !(row_split != 0 && len > row_split))
+            long_rows[atomicAdd(&long_cnt[long_class(len)], 1u)] = (uint32_t)i;
     }
     if (tid <= kXcd) sched[kSchedRowLo + tid] = lo_s[tid];
 }
@@ -920,7 +941,7 @@ int det_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, char
                        L.nchunks, (uint32_t)L.row_split);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_row_scan, dim3(1), dim3(kScanThreads), (size_t)scan_cap * sizeof(uint32_t), st, seg_off,
-                       long_rows, sched, R, scan_cap);
+                       long_rows, sched, R, scan_cap, (uint32_t)L.row_split);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_fill, dim3(L.nchunks, nranges), dim3(256), fill_bytes, st, widx, bidx, cnt, seg_off, list,
                        B, K, R, L.cpp, range, stage);
