@@ -475,6 +475,8 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
             if (base + i_beg == 0)
                 for (int k = 0; k <= x_cur; ++k) lo_s[k] = 0;
         }
+        // 8 w >= thr  <=>  the rows before this one weigh at least (x_cur + 1) eighths of the total
+        unsigned long long thr = (unsigned long long)(x_cur + 1) * denom;
         for (int i = i_beg; i < i_end; ++i) {
             const uint32_t raw = stage[i];
             const uint32_t len = raw & ~kSplitFlag;
@@ -489,10 +491,12 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
             run[0] += len;
             const int r_next = base + i + 1;
             if (r_next < R) {
-                const int x_next =
-                    xcd_of((unsigned long long)(run[0] - run[1]) + (unsigned long long)r_next * kRowWeight, denom);
-                for (int k = x_cur + 1; k <= x_next; ++k) lo_s[k] = (uint32_t)r_next;
-                x_cur = x_next;
+                const unsigned long long w8 =
+                    ((unsigned long long)(run[0] - run[1]) + (unsigned long long)r_next * kRowWeight) * kXcd;
+                while (x_cur < kXcd - 1 && w8 >= thr) {
+                    lo_s[++x_cur] = (uint32_t)r_next;
+                    thr += denom;
+                }
             }
         }
         __syncthreads();
@@ -517,8 +521,12 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
         sched[kSchedNSplit] = n_split_s;
     }
     __syncthreads();
+    const uint32_t total = carry_s[0];
     for (int i = tid; i < R; i += kScanThreads) {
-        const uint32_t len = seg_off[i + 1] - seg_off[i];
+        // (a table scanned in one pass still has its offsets staged in LDS)
+        const uint32_t a = one_pass ? stage[i] : seg_off[i];
+        const uint32_t b = i + 1 == R ? total : one_pass ? stage[i + 1] : seg_off[i + 1];
+        const uint32_t len = b - a;
         if (len >= (uint32_t)kLongRow && !(row_split != 0 && len > row_split))
             long_rows[atomicAdd(&long_cnt[long_class(len)], 1u)] = (uint32_t)i;
     }
