@@ -121,8 +121,8 @@ def sum_traffic(traffic, kernels):
 
 
 FWD_KERNELS = ("k_pair_hist", "k_pair_scan", "k_pair_scatter", "k_acc_blocked", "k_mix")
-BWD_KERNELS = ("k_bwd_rows", "k_chunk_hist", "k_col_scan", "k_row_scan", "k_fill", "k_seg_reduce", "k_split_combine",
-               "k_bias_final")
+# (the default order has no k_bias_final launch: the bias gradient's last step rides in k_split_combine)
+BWD_KERNELS = ("k_bwd_rows", "k_chunk_hist", "k_col_scan", "k_row_scan", "k_fill", "k_seg_reduce", "k_split_combine")
 
 
 # ------------------------------------------------------------------------------------------------
@@ -679,8 +679,8 @@ def run_ft(args, lib, dev):
         alg, gathered, comp = seg_reduce_bytes(L1, B, sum_a)
         seg_traffic = sum_traffic(traffic, ("k_seg_reduce", "k_split_combine"))
         out["roofline"], out["roofline_compulsory"] = bound_block(
-            "k_seg_reduce<4,3> (timed through nnueft_det_reduce_rows, which launches it with k_split_combine and the "
-            "rewind of the task counters, a few microseconds, behind it)", det["reduce"], alg, gathered, comp,
+            "k_seg_reduce<4,3> (timed through nnueft_det_reduce_rows, which launches it with k_split_combine, which also "
+            "rewinds the task counters, a few microseconds, behind it)", det["reduce"], alg, gathered, comp,
             seg_traffic, l2_peak,
             note="dominant kernel of the step; it gathers one upstream row per slot through L2 (blocked by king bucket "
                  "and column slice), so `achieved` (algorithmic bytes) is held against the L2 line rate; against HBM "
