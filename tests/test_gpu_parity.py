@@ -64,6 +64,11 @@ SPARSE_SHAPES = [
     (7, 3080, 500, 32),     # L1=3072 row width
     (9, 37, 50, 70),        # odd width (scalar path), K > 64
     (64, 272, 24576, 32),   # bench_feature_transformer.py:22-25 width, full table height
+    # widths a few columns beyond whole 64-lane slices (those columns are reduced many rows per wave):
+    (300, 131, 700, 32),    # scalar path, 3 columns over, rows with and without slots
+    (257, 70, 90, 16),      # scalar path, 6 over, every row named several times
+    (120, 260, 1000, 32),   # 16-byte path, 1 vector over
+    (90, 284, 333, 24),     # 16-byte path, 7 vectors over, range ends inside a group of rows
 ]
 
 
