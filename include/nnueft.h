@@ -133,9 +133,12 @@ size_t nnueft_fwd_workspace_bytes(int B, int K, int R, int L1, int n_psqt);
  * reference stores the clamped mixed values instead, fused_ft_kernel.py:95-99, and thereby loses
  * torch's clamp gradient at exactly 0 and exactly max.)  L1 must be even.
  * workspace: NULL, or nnueft_fwd_workspace_bytes() bytes.  With a workspace (and 16-byte aligned rows:
- * L1 % 8 == 0, (L1+n_psqt) % 4 == 0) the gather is blocked for the per-XCD L2 caches: positions are
- * grouped by the 768-row table block their lists name and each XCD works through its share one
- * column slice at a time.  Results are bit-identical with and without the workspace.
+ * L1 % 8 == 0, (L1+n_psqt) % 4 == 0) the positions are grouped by the 768-row table block their lists
+ * name.  Rows of 512 columns and more (L1 % 32 == 0, K <= 32, a table of at most 62 blocks) are then
+ * gathered out of LDS: a workgroup holds a tile of one block, 768 rows x 32 columns, and sums it for
+ * every list of the block.  Other shapes are blocked for the per-XCD L2 caches: each XCD works through
+ * its share of the grouped lists one column slice at a time.  Results are bit-identical with and
+ * without the workspace.
  */
 int nnueft_double_fwd(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                       const int64_t* psqt_idx, const float* W, const float* bias, float max_act,
@@ -166,8 +169,9 @@ int nnueft_double_fwd_act(const float* us, const float* them, const int32_t* wid
  * L2-blocked gather (pair order, keys, per-workgroup histograms) is a fixed array inside the library,
  * one copy per GPU, 2 MiB, held until the process ends.  Same arguments and results as
  * nnueft_double_fwd minus the workspace; no counterpart in the reference.  The call allocates and
- * frees nothing.  Limit: nnueft_fwd_workspace_bytes(B, K, R, L1, n_psqt) <= 2 MiB (B = 65536 with a
- * 24576-row table fits), beyond it NNUEFT_E_SCRATCH.  All calls on one GPU share that GPU's array:
+ * frees nothing.  Limit: the scratch of the L2-blocked gather, 2 * B * 8 bytes plus 4 bytes per
+ * (256 lists, table block), must fit 2 MiB (B = 65536 with a 24576-row table fits), beyond it
+ * NNUEFT_E_SCRATCH; the LDS-tiled gather is taken where its larger scratch fits as well.  All calls on one GPU share that GPU's array:
  * calls that overlap in time on one GPU (two streams, two threads) race on it; calls on one stream
  * are ordered and safe.  The first call on a device looks up the array's address (not a stream
  * operation: make one call on each device before capturing a graph there).

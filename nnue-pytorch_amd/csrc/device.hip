@@ -44,6 +44,8 @@ int device_info(int* device, const DeviceInfo** info) {
                 d.xcds = 0;
                 (void)hipGetLastError();
             }
+            e = hipDeviceGetAttribute(&d.cus, hipDeviceAttributeMultiprocessorCount, dev);
+            if (e != hipSuccess) return (int)e;
             s.info = d;
             s.ready = true;
         }

@@ -184,7 +184,7 @@ extern "C" int nnueft_sparse_fwd(const int32_t* idx, const float* W, const float
 
 extern "C" size_t nnueft_fwd_workspace_bytes(int B, int K, int R, int L1, int n_psqt) {
     if (B <= 0 || K <= 0 || R <= 0 || L1 <= 0 || n_psqt < 0) return 0;
-    return nnueft_blocked::pair_sort_workspace(B, R, 0);
+    return nnueft_tile::workspace(B, R);
 }
 
 extern "C" int nnueft_act_fake_quantize(const float* x, float* out, long long n, float scale, float eps,
@@ -211,6 +211,10 @@ int double_fwd(const float* us, const float* them, const int32_t* widx, const in
         const nnueft_dev::DeviceInfo* info = nullptr;
         const int rc_dev = nnueft_dev::device_info(nullptr, &info);
         if (rc_dev) return rc_dev;
+        // wide rows gather out of LDS tiles when the caller's workspace has room for that path's lists
+        if (vec && nnueft_tile::fits(*info, B, K, R, L1) && workspace_bytes >= nnueft_tile::workspace(B, R))
+            return nnueft_tile::double_fwd_tile(us, them, widx, bidx, psqt_idx, W, bias, max_act, l0, wpsqt, bpsqt,
+                                                saved, B, K, R, L1, n_psqt, workspace, st, act);
         if (vec && (long long)B <= 0x3fffffffLL && nnueft_blocked::blocked_layout_fits(*info))
             return nnueft_blocked::double_fwd_blocked(us, them, widx, bidx, psqt_idx, W, bias, max_act, l0, wpsqt,
                                                       bpsqt, saved, B, K, R, L1, n_psqt, workspace, st, act);

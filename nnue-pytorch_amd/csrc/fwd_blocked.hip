@@ -233,6 +233,26 @@ static inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 int table_block_rows(int R, int hint, int* nbins);
 
+int launch_scan(uint32_t* data, int n, hipStream_t st) {
+    hipLaunchKernelGGL(k_pair_scan, dim3(1), dim3(1024), 0, st, data, n);
+    NNUEFT_LAUNCH_CHECK();
+    return 0;
+}
+
+int launch_mix(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+               const int64_t* psqt_idx, const float* W, const float* bias, const float* saved, float max_act,
+               float* l0, float* wpsqt, float* bpsqt, int B, int K, int R, int L1, int n_psqt, hipStream_t st,
+               ActGrid act) {
+    const int hv = (L1 / 2) / 4;
+    const int mix_slices = (hv + 63) / 64;
+    if ((long long)B * mix_slices > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
+    const dim3 mix_grid((unsigned)B * mix_slices);
+    hipLaunchKernelGGL(k_mix<4>, mix_grid, dim3(64), 0, st, us, them, widx, bidx, psqt_idx, W, bias, saved, max_act,
+                       l0, wpsqt, bpsqt, B, K, R, L1, n_psqt, mix_slices, act);
+    NNUEFT_LAUNCH_CHECK();
+    return 0;
+}
+
 struct PairSortLayout {
     size_t order, keys, hist, end;
     int ngroups, nbins, block_rows;
@@ -269,8 +289,8 @@ int launch_pair_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int
     hipLaunchKernelGGL(k_pair_hist, dim3(L.ngroups), dim3(kPairThreads), 0, st, widx, bidx, keys, hist, B, K, R,
                        L.block_rows, L.nbins);
     NNUEFT_LAUNCH_CHECK();
-    hipLaunchKernelGGL(k_pair_scan, dim3(1), dim3(1024), 0, st, hist, L.ngroups * L.nbins);
-    NNUEFT_LAUNCH_CHECK();
+    const int rc_scan = launch_scan(hist, L.ngroups * L.nbins, st);
+    if (rc_scan) return rc_scan;
     hipLaunchKernelGGL(k_pair_scatter, dim3(L.ngroups), dim3(kPairThreads), 0, st, keys, hist, order, 2 * B,
                        L.nbins);
     NNUEFT_LAUNCH_CHECK();
@@ -311,14 +331,8 @@ int double_fwd_blocked(const float* us, const float* them, const int32_t* widx, 
                            saved, B, K, R, L1, out_cols, per_xcd);
     }
     NNUEFT_LAUNCH_CHECK();
-    const int hv = (L1 / 2) / 4;
-    const int mix_slices = (hv + 63) / 64;
-    if ((long long)B * mix_slices > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
-    const dim3 mix_grid((unsigned)B * mix_slices);
-    hipLaunchKernelGGL(k_mix<4>, mix_grid, dim3(64), 0, st, us, them, widx, bidx, psqt_idx, W, bias,
-                       saved, max_act, l0, wpsqt, bpsqt, B, K, R, L1, n_psqt, mix_slices, act);
-    NNUEFT_LAUNCH_CHECK();
-    return 0;
+    return launch_mix(us, them, widx, bidx, psqt_idx, W, bias, saved, max_act, l0, wpsqt, bpsqt, B, K, R, L1, n_psqt,
+                      st, act);
 }
 
 }  // namespace nnueft_blocked

@@ -45,7 +45,8 @@ extern "C" int nnueft_double_fwd_noalloc(const float* us, const float* them, con
                                          float* saved, int B, int K, int R, int L1, int n_psqt, void* stream) {
     if (B < 0 || K <= 0 || R <= 0 || L1 <= 0 || (L1 & 1) || n_psqt < 0) return NNUEFT_E_ARG;
     if (B == 0) return 0;
-    const size_t need = nnueft_fwd_workspace_bytes(B, K, R, L1, n_psqt);
+    // the L2-blocked path's scratch is what has to fit (the LDS-tiled path is taken when its lists fit too)
+    const size_t need = nnueft_blocked::pair_sort_workspace(B, R, 0);
     if (need == 0) return NNUEFT_E_ARG;
     if (need > kScratchBytes) return NNUEFT_E_SCRATCH;
     void* ptr = nullptr;

@@ -1,0 +1,506 @@
+// Forward, LDS-tiled variant: the gather reads the table out of LDS instead of through L2.
+//
+// All indices of one list name rows of a single 768-row block of the table (one king bucket).  A
+// workgroup keeps one tile of the table in LDS, 768 rows x 32 columns (96 KB), and the lists of up to
+// 512 (position, perspective) pairs of that block (32 KB, as 16-bit row numbers inside the block), and
+// sums the tile's columns for every pair: 8 lanes a pair, one 16-byte LDS read per row and lane, the
+// adds in slot order.  Every row of the table then crosses the CU's L1 once per chunk of pairs instead
+// of once per pair naming it (about 24 times in a batch of 16384 positions), which is what bounds the
+// gather through L2: a CU can only keep so many L1 misses pending.
+//
+//   k_tl_hist     one pair per thread: key (block, list length) counted per workgroup
+//   k_tl_binscan  per key, the counts of the workgroups become their exclusive prefix
+//   k_tl_lists    pairs to their slots, longest lists first inside a block and dealt to the block's
+//                 chunks in turn; writes the 16-bit lists, pair ids and the chunk table
+//   k_acc_tile    persistent workgroups, one per CU: units of (chunk, group of column tiles) handed out
+//                 per XCD; the tile for the next column group is fetched into registers while the
+//                 current one is summed; waves take tasks of 8 pairs from a counter in LDS
+//   k_mix         as in the L2-blocked path
+//
+// A list that names rows of more than one block (the interface allows it) is summed from global
+// memory by the same wave; results are bit-identical to the other forward kernels.
+#include <atomic>
+#include <cstdlib>
+
+#include "gather.h"
+#include "internal.h"
+
+namespace nnueft_tile {
+
+using nnueft_blocked::kXcd;
+
+constexpr int kRows = 768;                         // rows of a table block = rows of a tile
+constexpr int kTileCols = 32;                      // floats per tile row
+constexpr int kRowBytes = kTileCols * 4;
+constexpr int kTileBytes = (kRows + 1) * kRowBytes;   // + one row of zeros for the padding slots
+constexpr int kChunk = 512;                        // pairs whose lists a workgroup holds
+constexpr int kSlots = 32;                         // list slots the 16-bit lists hold
+constexpr int kLenBins = kSlots + 1;
+constexpr int kMaxBlocks = 62;
+constexpr int kBins = 2048;                        // LDS counters of the sort (kMaxBlocks * kLenBins + 1 used at most)
+static_assert(kMaxBlocks * kLenBins + 1 <= kBins, "sort bins");
+constexpr uint32_t kForeign = 63;                  // count field of a list that leaves its block
+constexpr int kAccThreads = 1024;
+constexpr int kSortThreads = 256;
+constexpr int kLdsBytes = kTileBytes + kChunk * kSlots * 2 + kChunk * 4 + 16;
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+
+struct Chunk {
+    int block, start, count, pad;
+};
+
+// What the sort and the gather share in the workspace.
+struct Layout {
+    size_t hist, total, lists, pidcnt, chunks, sched, end;
+    int ngroups, nblocks, nbins, max_chunks, nslots;
+};
+
+static inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+bool layout(int B, int R, Layout* L) {
+    if (B <= 0 || R <= 0) return false;
+    L->nblocks = (R + kRows - 1) / kRows;
+    if (L->nblocks > kMaxBlocks) return false;
+    L->nbins = L->nblocks * kLenBins + 1;   // + one empty bin: its offset is the end of the last block
+    L->ngroups = (2 * B + kSortThreads - 1) / kSortThreads;
+    L->max_chunks = (2 * B + kChunk - 1) / kChunk + L->nblocks;
+    L->nslots = 2 * B + L->max_chunks;     // a block's chunks are equally long, the last ones one pair short
+    size_t off = 0;
+    L->hist = off;
+    off += up256((size_t)L->ngroups * L->nbins * sizeof(uint32_t));
+    L->total = off;
+    off += up256((size_t)kBins * sizeof(uint32_t));
+    L->lists = off;
+    off += up256((size_t)L->nslots * kSlots * sizeof(uint16_t));
+    L->pidcnt = off;
+    off += up256((size_t)L->nslots * sizeof(uint32_t));
+    L->chunks = off;
+    off += up256((size_t)L->max_chunks * sizeof(Chunk));
+    L->sched = off;
+    off += up256((size_t)(kXcd + 1) * 32 * sizeof(uint32_t));
+    L->end = off;
+    return true;
+}
+
+size_t workspace(int B, int R) {
+    Layout L;
+    const size_t blocked = nnueft_blocked::pair_sort_workspace(B, R, 0);
+    if (!layout(B, R, &L)) return blocked;
+    return L.end > blocked ? L.end : blocked;
+}
+
+bool fits(const nnueft_dev::DeviceInfo& d, int B, int K, int R, int L1) {
+    Layout L;
+    return K <= kSlots && L1 % kTileCols == 0 && L1 >= 512 && (long long)2 * B < (1ll << 26) &&
+           d.max_lds >= kLdsBytes && d.xcds == kXcd && d.cus >= kXcd && layout(B, R, &L);
+}
+
+__device__ __forceinline__ const int32_t* pair_list(const int32_t* __restrict__ widx,
+                                                    const int32_t* __restrict__ bidx, int pair, int B, int K) {
+    const int p = pair >= B;
+    return (p ? bidx : widx) + (size_t)(pair - p * B) * K;
+}
+
+// A thread's view of one list: valid entries counted, the block of the first, whether all stay in it.
+struct ListFacts {
+    int cnt, block;
+    bool foreign;
+};
+
+// The list of a thread in registers: kSlots entries, -1 beyond K (16-byte loads when `vec`).
+struct ListRegs {
+    int v[kSlots];
+};
+
+__device__ __forceinline__ ListRegs load_list(const int32_t* __restrict__ ix, int K, bool vec) {
+    ListRegs l;
+    if (vec) {
+        const int4* p = reinterpret_cast<const int4*>(ix);
+#pragma unroll
+        for (int q = 0; q < kSlots / 4; ++q) {
+            const int4 t = 4 * q < K ? p[q] : make_int4(-1, -1, -1, -1);
+            l.v[4 * q] = t.x; l.v[4 * q + 1] = t.y; l.v[4 * q + 2] = t.z; l.v[4 * q + 3] = t.w;
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < kSlots; ++k) l.v[k] = k < K ? ix[k] : -1;
+    }
+    return l;
+}
+
+__device__ __forceinline__ ListFacts list_facts(const ListRegs& l, int R) {
+    ListFacts f{0, 0, false};
+    int first = -1;
+#pragma unroll
+    for (int k = 0; k < kSlots; ++k) {
+        const int r = l.v[k];
+        if (r >= 0 && r < R) {
+            const int b = r / kRows;
+            if (first < 0) first = b;
+            f.foreign |= b != first;
+            ++f.cnt;
+        }
+    }
+    f.block = first < 0 ? 0 : first;
+    return f;
+}
+
+__device__ __forceinline__ int sort_key(const ListFacts& f) { return f.block * kLenBins + (kSlots - f.cnt); }
+
+__global__ __launch_bounds__(kSortThreads) void k_tl_hist(const int32_t* __restrict__ widx,
+                                                          const int32_t* __restrict__ bidx,
+                                                          uint32_t* __restrict__ hist, int B, int K, int R,
+                                                          int nbins, int vec) {
+    __shared__ uint32_t bins[kBins];
+    const int tid = threadIdx.x;
+    const int n = blockIdx.x * kSortThreads + tid;
+    for (int i = tid; i < nbins; i += kSortThreads) bins[i] = 0;
+    __syncthreads();
+    if (n < 2 * B) atomicAdd(&bins[sort_key(list_facts(load_list(pair_list(widx, bidx, n, B, K), K, vec), R))], 1u);
+    __syncthreads();
+    for (int i = tid; i < nbins; i += kSortThreads) hist[(size_t)i * gridDim.x + blockIdx.x] = bins[i];
+}
+
+// Chunks of a block with n pairs: as few as keep each at kChunk pairs or fewer; pair i of the block
+// (longest list first) goes to chunk i % nc, so every chunk gets the same mix of list lengths.
+__device__ __forceinline__ int chunks_of(int n) { return (n + kChunk - 1) / kChunk; }
+
+// One wave per bin: the counts of the workgroups become their exclusive prefix, the sum goes to total[bin].
+__global__ __launch_bounds__(kSortThreads) void k_tl_binscan(uint32_t* __restrict__ hist, uint32_t* __restrict__ total,
+                                                             int nbins, int ngroups) {
+    const int lane = threadIdx.x & 63;
+    const int bin = blockIdx.x * (kSortThreads / 64) + (threadIdx.x >> 6);
+    if (bin >= nbins) return;
+    uint32_t* h = hist + (size_t)bin * ngroups;
+    uint32_t run = 0;
+    for (int g0 = 0; g0 < ngroups; g0 += 64) {
+        const int g = g0 + lane;
+        const uint32_t v = g < ngroups ? h[g] : 0;
+        uint32_t incl = v;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const uint32_t t = __shfl_up(incl, off);
+            if (lane >= off) incl += t;
+        }
+        if (g < ngroups) h[g] = run + incl - v;
+        run += __shfl(incl, 63);
+    }
+    if (lane == 0) total[bin] = run;
+}
+
+__global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __restrict__ widx,
+                                                           const int32_t* __restrict__ bidx,
+                                                           const uint32_t* __restrict__ hist,
+                                                           const uint32_t* __restrict__ total,
+                                                           uint16_t* __restrict__ lists,
+                                                           uint32_t* __restrict__ pidcnt, Chunk* __restrict__ chunks,
+                                                           uint32_t* __restrict__ sched, int B, int K, int R,
+                                                           int nblocks, int nbins, int vec) {
+    __shared__ uint32_t cursor[kBins];
+    __shared__ uint32_t wave_tot[kSortThreads / 64];
+    __shared__ uint32_t blk_start[kMaxBlocks + 1];
+    __shared__ uint32_t blk_base[kMaxBlocks + 1];   // first slot of the block's chunks; [nblocks] = chunks in all
+    const int tid = threadIdx.x;
+    const int n = blockIdx.x * kSortThreads + tid;
+    const int ngroups = gridDim.x;
+    // first slot of every bin: exclusive scan of the bin totals, kBins / kSortThreads consecutive bins a thread
+    {
+        constexpr int PER = kBins / kSortThreads;
+        static_assert(kBins % kSortThreads == 0, "bins per thread");
+        uint32_t v[PER];
+        uint32_t local = 0;
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const int i = tid * PER + u;
+            v[u] = i < nbins ? total[i] : 0;
+            local += v[u];
+        }
+        uint32_t incl = local;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const uint32_t t = __shfl_up(incl, off);
+            if ((tid & 63) >= off) incl += t;
+        }
+        if ((tid & 63) == 63) wave_tot[tid >> 6] = incl;
+        __syncthreads();
+        uint32_t run = incl - local;
+        for (int w = 0; w < (tid >> 6); ++w) run += wave_tot[w];
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const int i = tid * PER + u;
+            if (i < nbins) {
+                if (i % kLenBins == 0) blk_start[i / kLenBins] = run;
+                cursor[i] = run + hist[(size_t)i * ngroups + blockIdx.x];
+            }
+            run += v[u];
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t nchunks = 0;
+        for (int b = 0; b < nblocks; ++b) {
+            blk_base[b] = blk_start[b] + nchunks;
+            nchunks += (uint32_t)chunks_of((int)(blk_start[b + 1] - blk_start[b]));
+        }
+        blk_base[nblocks] = nchunks;
+    }
+    __syncthreads();
+    if (blockIdx.x == 0) {
+        // the chunk table, the number of chunks and the unit counters of the gather
+        for (int b = tid; b < nblocks; b += kSortThreads) {
+            const int nb = (int)(blk_start[b + 1] - blk_start[b]);
+            const int nc = chunks_of(nb);
+            const int len = nc ? (nb + nc - 1) / nc : 0;
+            const int first = (int)(blk_base[b] - blk_start[b]);
+            for (int j = 0; j < nc; ++j)
+                chunks[first + j] = Chunk{b, (int)blk_base[b] + j * len, (nb - j + nc - 1) / nc, 0};
+        }
+        if (tid <= kXcd) sched[tid * 32] = tid == kXcd ? blk_base[nblocks] : 0u;
+    }
+    if (n >= 2 * B) return;
+    const ListRegs l = load_list(pair_list(widx, bidx, n, B, K), K, vec);
+    const ListFacts f = list_facts(l, R);
+    const uint32_t slot = atomicAdd(&cursor[sort_key(f)], 1u);
+    const int nb = (int)(blk_start[f.block + 1] - blk_start[f.block]);
+    const int nc = chunks_of(nb);
+    const int len = (nb + nc - 1) / nc;
+    const int i = (int)(slot - blk_start[f.block]);
+    const size_t dst = (size_t)blk_base[f.block] + (size_t)(i % nc) * len + i / nc;
+    pidcnt[dst] = (uint32_t)n | ((f.foreign ? kForeign : (uint32_t)f.cnt) << 26);
+    // row numbers inside the block, valid entries first in slot order, the rest name the row of zeros
+    uint32_t w[kSlots / 2];
+    const int base = f.block * kRows;
+    bool prefix = true;   // the valid entries are the first cnt slots (what a loader writes)
+#pragma unroll
+    for (int k = 0; k < kSlots; ++k) prefix &= (k < f.cnt) == (l.v[k] >= 0 && l.v[k] < R);
+    if (f.foreign) {
+#pragma unroll
+        for (int q = 0; q < kSlots / 2; ++q) w[q] = (uint32_t)kRows | ((uint32_t)kRows << 16);
+    } else if (prefix) {
+#pragma unroll
+        for (int q = 0; q < kSlots / 2; ++q) {
+            const uint32_t lo = 2 * q < f.cnt ? (uint32_t)(l.v[2 * q] - base) : (uint32_t)kRows;
+            const uint32_t hi = 2 * q + 1 < f.cnt ? (uint32_t)(l.v[2 * q + 1] - base) : (uint32_t)kRows;
+            w[q] = lo | (hi << 16);
+        }
+    } else {
+#pragma unroll
+        for (int q = 0; q < kSlots / 2; ++q) w[q] = (uint32_t)kRows | ((uint32_t)kRows << 16);
+        int m = 0;
+#pragma unroll
+        for (int k = 0; k < kSlots; ++k) {
+            const int r = l.v[k];
+            if (r >= 0 && r < R) {
+                const uint32_t v = (uint32_t)(r - base);
+#pragma unroll
+                for (int q = 0; q <= k / 2; ++q)
+                    if (q == (m >> 1)) w[q] = (m & 1) ? ((w[q] & 0xffffu) | (v << 16)) : ((w[q] & 0xffff0000u) | v);
+                ++m;
+            }
+        }
+    }
+    u4* out = reinterpret_cast<u4*>(lists + dst * kSlots);
+#pragma unroll
+    for (int q = 0; q < kSlots / 8; ++q) out[q] = u4{w[4 * q], w[4 * q + 1], w[4 * q + 2], w[4 * q + 3]};
+}
+
+// (16-bit half of w) * bytes per tile row + off: the LDS address of a lane's piece of a row, one instruction.
+template <int HI>
+__device__ __forceinline__ uint32_t row_addr(uint32_t w, uint32_t off) {
+    uint32_t r;
+    const uint32_t stride = kRowBytes;
+    if (HI)
+        asm("v_mad_u32_u16 %0, %1, %2, %3 op_sel:[1,0,0,0]" : "=v"(r) : "v"(w), "s"(stride), "v"(off));
+    else
+        asm("v_mad_u32_u16 %0, %1, %2, %3 op_sel:[0,0,0,0]" : "=v"(r) : "v"(w), "s"(stride), "v"(off));
+    return r;
+}
+
+// saved[pair, columns of the tile] = chain from +0 over the pair's list, for every pair of the chunk.
+__global__ __launch_bounds__(kAccThreads) void k_acc_tile(const int32_t* __restrict__ widx,
+                                                          const int32_t* __restrict__ bidx,
+                                                          const uint16_t* __restrict__ lists,
+                                                          const uint32_t* __restrict__ pidcnt,
+                                                          const Chunk* __restrict__ chunks,
+                                                          uint32_t* __restrict__ sched, const float* __restrict__ W,
+                                                          float* __restrict__ acc, int B, int K, int R, int L1,
+                                                          int out_cols, int tiles_per_xcd, int tile_group) {
+    extern __shared__ float4 lds_raw[];
+    char* tb = reinterpret_cast<char*>(lds_raw);
+    u4* moff = reinterpret_cast<u4*>(tb + kTileBytes);                                   // kChunk * 4
+    uint32_t* mpid = reinterpret_cast<uint32_t*>(tb + kTileBytes + kChunk * kSlots * 2);  // kChunk
+    uint32_t* ctr = mpid + kChunk;       // [0] task counter, [1] the unit this workgroup works on next
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    constexpr int N4 = kRows * (kRowBytes / 16);
+    static_assert(N4 % kAccThreads == 0, "tile load");
+    constexpr int IT = N4 / kAccThreads;
+    const int x = blockIdx.x % kXcd;
+    const int ntiles = L1 / kTileCols;
+    const int groups = (tiles_per_xcd + tile_group - 1) / tile_group;
+    const int nunits = (int)sched[kXcd * 32] * groups;
+    uint32_t* unit_ctr = sched + x * 32;
+    const int g = lane >> 3, j = lane & 7;
+    const uint32_t lane_off = j * 16;
+    if (tid < kRowBytes / 16) reinterpret_cast<f4*>(tb)[kRows * (kRowBytes / 16) + tid] = f4{0.f, 0.f, 0.f, 0.f};
+    if (tid == 0) ctr[1] = atomicAdd(unit_ctr, 1u);
+
+    f4 v[IT];
+    while (true) {
+        __syncthreads();   // the previous unit is done with the lists and the tile; ctr[1] is written
+        const int unit = (int)ctr[1];
+        if (unit >= nunits) break;
+        const int ch = unit / groups;
+        const int tg = unit - ch * groups;
+        const Chunk C = chunks[ch];
+        const int q0 = tg * tile_group;
+        int q1 = min(q0 + tile_group, tiles_per_xcd);
+        q1 = min(q1, ntiles - x * tiles_per_xcd);
+        const int row0 = C.block * kRows;
+        const float* wb = W + (size_t)row0 * out_cols;
+        const int rows_here = min(kRows, R - row0);
+        const int ntasks = (C.count + 7) >> 3;
+        __syncthreads();   // everyone has read ctr[1]
+        if (tid == 0) ctr[1] = atomicAdd(unit_ctr, 1u);
+        {
+            const u4* ms = reinterpret_cast<const u4*>(lists + (size_t)C.start * kSlots);
+            for (int f = tid; f < C.count * 4; f += kAccThreads) moff[f] = ms[f];
+            if (tid < C.count) mpid[tid] = pidcnt[C.start + tid];
+        }
+#define NNUEFT_LOAD_TILE(c_)                                                                          \
+    {                                                                                                 \
+        const float* src = wb + (c_) * kTileCols;                                                     \
+        _Pragma("unroll") for (int i = 0; i < IT; ++i) {                                              \
+            const int f = tid + i * kAccThreads;                                                      \
+            const int row = f >> 3;                                                                   \
+            v[i] = row < rows_here                                                                    \
+                       ? *reinterpret_cast<const f4*>(src + (size_t)row * out_cols + (f & 7) * 4)     \
+                       : f4{0.f, 0.f, 0.f, 0.f};                                                      \
+        }                                                                                             \
+    }
+        if (q0 < q1) NNUEFT_LOAD_TILE(x * tiles_per_xcd + q0)
+        for (int q = q0; q < q1; ++q) {
+            const int c = x * tiles_per_xcd + q;
+            if (q != q0) __syncthreads();   // everyone is done reading the previous tile
+#pragma unroll
+            for (int i = 0; i < IT; ++i) {
+                const int f = tid + i * kAccThreads;
+                reinterpret_cast<f4*>(tb)[f] = v[i];
+            }
+            if (tid == 0) ctr[0] = 0;
+            __syncthreads();
+            if (q + 1 < q1) NNUEFT_LOAD_TILE(c + 1)
+            int task = 0;
+            if (lane == 0) task = (int)atomicAdd(ctr, 1u);
+            task = __builtin_amdgcn_readfirstlane(task);
+            while (task < ntasks) {
+                int nxt = 0;
+                if (lane == 0) nxt = (int)atomicAdd(ctr, 1u);
+                int s = task * 8 + g;
+                const bool valid = s < C.count;
+                if (!valid) s = task * 8;
+                const uint32_t pc = mpid[s];
+                const uint32_t field = pc >> 26;
+                const int pair = (int)(pc & 0x3ffffffu);
+                const int mx = __builtin_amdgcn_readfirstlane((int)field);   // lists are sorted longest first
+                f4 a = {0.f, 0.f, 0.f, 0.f};
+                if (__ballot(field == kForeign) != 0) {
+                    // some list of the task leaves its block: the wave's 8 pairs from global memory
+                    const int32_t* ix = pair_list(widx, bidx, pair, B, K);
+                    for (int k = 0; k < K; ++k) {
+                        const int r = ix[k];
+                        if (r >= 0 && r < R) a += *reinterpret_cast<const f4*>(W + (size_t)r * out_cols + c * kTileCols + j * 4);
+                    }
+                } else {
+                    uint32_t oo[kSlots / 2];
+#pragma unroll
+                    for (int i = 0; i < kSlots / 8; ++i) {
+                        const u4 t = moff[s * 4 + i];
+                        oo[4 * i] = t.x; oo[4 * i + 1] = t.y; oo[4 * i + 2] = t.z; oo[4 * i + 3] = t.w;
+                    }
+                    // blocks of four slots, the next block's reads issued before the current block's adds
+                    f4 r[2][4];
+#define NNUEFT_ISSUE(buf_, i_)                                                                   \
+    r[buf_][0] = *reinterpret_cast<const f4*>(tb + row_addr<0>(oo[2 * (i_)], lane_off));          \
+    r[buf_][1] = *reinterpret_cast<const f4*>(tb + row_addr<1>(oo[2 * (i_)], lane_off));          \
+    r[buf_][2] = *reinterpret_cast<const f4*>(tb + row_addr<0>(oo[2 * (i_) + 1], lane_off));      \
+    r[buf_][3] = *reinterpret_cast<const f4*>(tb + row_addr<1>(oo[2 * (i_) + 1], lane_off));
+                    NNUEFT_ISSUE(0, 0)
+#pragma unroll
+                    for (int i = 0; i < kSlots / 4; ++i) {
+                        if (i * 4 < mx) {
+                            if ((i + 1) * 4 < mx) { NNUEFT_ISSUE((i + 1) & 1, (i + 1) & 7) }
+#pragma unroll
+                            for (int h = 0; h < 4; ++h) a += r[i & 1][h];
+                        }
+                    }
+                }
+                if (valid)
+                    __builtin_nontemporal_store(a, reinterpret_cast<f4*>(acc + (size_t)pair * L1 + c * kTileCols + j * 4));
+                task = __builtin_amdgcn_readfirstlane(nxt);
+            }
+        }
+    }
+}
+
+// The gather may ask for most of a CU's LDS; that permission belongs to the loaded kernel on a device
+// and is given once per device.
+constexpr int kMaxDevices = 64;
+std::atomic<int> g_lds_allowed[kMaxDevices];
+
+int allow_lds(int device) {
+    if (device < 0 || device >= kMaxDevices) return NNUEFT_E_UNSUPPORTED;
+    if (g_lds_allowed[device].load(std::memory_order_acquire)) return 0;
+    const hipError_t e =
+        hipFuncSetAttribute((const void*)k_acc_tile, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    if (e != hipSuccess) return (int)e;
+    g_lds_allowed[device].store(1, std::memory_order_release);
+    return 0;
+}
+
+int double_fwd_tile(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+                    const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,
+                    float* wpsqt, float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt, void* ws,
+                    hipStream_t st, ActGrid act) {
+    Layout L;
+    if (!layout(B, R, &L)) return NNUEFT_E_UNSUPPORTED;
+    int device = 0;
+    const nnueft_dev::DeviceInfo* info = nullptr;
+    int rc = nnueft_dev::device_info(&device, &info);
+    if (rc) return rc;
+    rc = allow_lds(device);
+    if (rc) return rc;
+    char* base = (char*)ws;
+    uint32_t* hist = (uint32_t*)(base + L.hist);
+    uint16_t* lists = (uint16_t*)(base + L.lists);
+    uint32_t* pidcnt = (uint32_t*)(base + L.pidcnt);
+    Chunk* chunks = (Chunk*)(base + L.chunks);
+    uint32_t* sched = (uint32_t*)(base + L.sched);
+    uint32_t* total = (uint32_t*)(base + L.total);
+    const int vec = (K % 4 == 0) && aligned16(widx) && aligned16(bidx);
+    hipLaunchKernelGGL(k_tl_hist, dim3(L.ngroups), dim3(kSortThreads), 0, st, widx, bidx, hist, B, K, R, L.nbins, vec);
+    NNUEFT_LAUNCH_CHECK();
+    hipLaunchKernelGGL(k_tl_binscan, dim3((L.nbins + kSortThreads / 64 - 1) / (kSortThreads / 64)), dim3(kSortThreads), 0, st, hist,
+                       total, L.nbins, L.ngroups);
+    NNUEFT_LAUNCH_CHECK();
+    hipLaunchKernelGGL(k_tl_lists, dim3(L.ngroups), dim3(kSortThreads), 0, st, widx, bidx, hist, total, lists, pidcnt,
+                       chunks, sched, B, K, R, L.nblocks, L.nbins, vec);
+    NNUEFT_LAUNCH_CHECK();
+    const int out_cols = L1 + n_psqt;
+    const int ntiles = L1 / kTileCols;
+    const int tiles_per_xcd = (ntiles + kXcd - 1) / kXcd;
+    int tile_group = tiles_per_xcd < 6 ? tiles_per_xcd : 6;
+#ifdef NNUEFT_TUNE_ENV
+    if (const char* e = getenv("NNUEFT_TILE_GROUP")) tile_group = atoi(e) > 0 ? atoi(e) : tile_group;
+#endif
+    const int grid = info->cus / kXcd * kXcd;
+    hipLaunchKernelGGL(k_acc_tile, dim3(grid), dim3(kAccThreads), kLdsBytes, st, widx, bidx, lists, pidcnt, chunks,
+                       sched, W, saved, B, K, R, L1, out_cols, tiles_per_xcd, tile_group);
+    NNUEFT_LAUNCH_CHECK();
+    return nnueft_blocked::launch_mix(us, them, widx, bidx, psqt_idx, W, bias, saved, max_act, l0, wpsqt, bpsqt, B,
+                                      K, R, L1, n_psqt, st, act);
+}
+
+}  // namespace nnueft_tile

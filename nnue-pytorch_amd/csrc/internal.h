@@ -16,6 +16,7 @@ namespace nnueft_dev {
 struct DeviceInfo {
     int max_lds;   // most LDS a workgroup can ask for, bytes
     int xcds;      // accelerator dies (each with an L2 of its own) the device presents; 0 = unknown
+    int cus;       // compute units
 };
 // The current device and its facts.  Returns 0, a negative NNUEFT_E_* or a positive hipError_t.
 int device_info(int* device, const DeviceInfo** info);
@@ -40,12 +41,33 @@ size_t pair_sort_workspace(int B, int R, int block_rows_hint);
 int launch_pair_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, int block_rows_hint, void* ws,
                      hipStream_t st, const uint32_t** order);
 
+// In-place exclusive scan of data[0..n) (one workgroup); the second half of the forward (bias, mix, clamp,
+// product, psqt chains) over row sums saved[2, B, L1].
+int launch_scan(uint32_t* data, int n, hipStream_t st);
+int launch_mix(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+               const int64_t* psqt_idx, const float* W, const float* bias, const float* saved, float max_act,
+               float* l0, float* wpsqt, float* bpsqt, int B, int K, int R, int L1, int n_psqt, hipStream_t st,
+               ActGrid act);
+
 int double_fwd_blocked(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                        const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,
                        float* wpsqt, float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt, void* ws,
                        hipStream_t st, ActGrid act);
 
 }  // namespace nnueft_blocked
+
+namespace nnueft_tile {
+
+// Forward gather out of LDS-resident tiles of the table (one 768-row block x 32 columns).  fits(): whether
+// the shape and the device can take it; workspace(): bytes it needs (at least the L2-blocked path's).
+bool fits(const nnueft_dev::DeviceInfo& d, int B, int K, int R, int L1);
+size_t workspace(int B, int R);
+int double_fwd_tile(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+                    const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,
+                    float* wpsqt, float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt, void* ws,
+                    hipStream_t st, ActGrid act);
+
+}  // namespace nnueft_tile
 
 namespace nnueft_det {
 

@@ -129,6 +129,11 @@ DOUBLE_SHAPES = [
     (6, 6, 20, 5, dict(n_psqt=3)),             # h = 3: scalar path
     (6, 50, 20, 80, dict(n_psqt=8, allow_holes=True)),   # K > 64, holes inside the lists
     (130, 64, 30, 32, dict(n_psqt=0)),         # no psqt columns, more than one sort chunk
+    # rows wide enough for the LDS-tiled forward
+    (300, 512, 2000, 32, {}),                  # lists that leave their 768-row block (summed from global memory)
+    (700, 544, 24576, 32, dict(halfka=True, weight_scale=0.05, max_act=255 / 256)),   # 17 tiles over 8 XCDs
+    (1500, 512, 1000, 20, dict(allow_holes=True)),   # K < 32, holes, a last block of 232 rows
+    (2000, 576, 768, 32, dict(n_psqt=0)),      # one block, eight chunks of lists
 ]
 
 
