@@ -29,6 +29,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 L2_CHANNELS = 128
 L2_LINE_BYTES = 128
 ENGINE_CLOCK_GHZ = 2.4
+# LDS: 256 CUs, 256 bytes read per CU and clock
+LDS_PEAK_GBS = 256 * 256 * ENGINE_CLOCK_GHZ
 
 WORKLOADS = {
     # name: (L1, B)
@@ -79,11 +81,18 @@ def compulsory_bytes(L1, B, sum_a):
     lists = 2 * B * K_SLOTS * 4
     saved = 2 * B * L1 * 4
     small = B * 24
-    fwd = {
-        "pair sort": lists + 3 * 2 * B * 4,
-        "k_acc_blocked": R_ROWS * oc * 4 + lists + saved,             # table once, row sums written
-        "k_mix": saved + B * L1 * 4 + small,                          # row sums read, l0 written
-    }
+    if forward_path(L1) == "tile":
+        fwd = {
+            "list sort": 2 * lists + 2 * B * (64 + 4),                    # lists twice, 16-bit lists and pair ids written
+            "k_acc_tile": R_ROWS * oc * 4 + 2 * B * (64 + 4) + saved,     # table once, 16-bit lists, row sums written
+            "k_mix": saved + B * L1 * 4 + small,                          # row sums read, l0 written
+        }
+    else:
+        fwd = {
+            "pair sort": lists + 3 * 2 * B * 4,
+            "k_acc_blocked": R_ROWS * oc * 4 + lists + saved,             # table once, row sums written
+            "k_mix": saved + B * L1 * 4 + small,                          # row sums read, l0 written
+        }
     nchunks = 2 * ((B + 127) // 128)
     bwd = {
         "k_bwd_rows": saved + B * L1 * 4 + 2 * B * oc * 4 + small,    # row sums + grad_l0 read, upstream rows written
@@ -120,7 +129,17 @@ def sum_traffic(traffic, kernels):
     return total
 
 
-FWD_KERNELS = ("k_pair_hist", "k_pair_scan", "k_pair_scatter", "k_acc_blocked", "k_mix")
+def forward_path(L1):
+    """Which gather nnueft_double_fwd takes with a workspace: out of LDS tiles for wide rows, else blocked for L2."""
+    return "tile" if L1 >= 512 and L1 % 32 == 0 else "blocked"
+
+
+def fwd_kernels(L1):
+    if forward_path(L1) == "tile":
+        return ("k_tl_hist", "k_tl_binscan", "k_tl_lists", "k_acc_tile", "k_mix")
+    return ("k_pair_hist", "k_pair_scan", "k_pair_scatter", "k_acc_blocked", "k_mix")
+
+
 # (the default order has no k_bias_final launch: the bias gradient's last step rides in k_split_combine)
 BWD_KERNELS = ("k_bwd_rows", "k_chunk_hist", "k_col_scan", "k_row_scan", "k_fill", "k_seg_reduce", "k_split_combine")
 
@@ -669,9 +688,18 @@ def run_ft(args, lib, dev):
                   "l2": f"{L2_CHANNELS} channels x {L2_LINE_BYTES} B per clock at {ENGINE_CLOCK_GHZ} GHz",
                   "traffic_source": traffic_file},
     }
-    fwd_block, fwd_comp = bound_block(
-        "nnueft_double_fwd: k_acc_blocked (the gather, ~3/4 of the time) + k_mix + pair sort", fwd_ms, fwd_bytes,
-        sum_a * oc * 4, sum(comp_fwd.values()), sum_traffic(traffic, FWD_KERNELS), l2_peak)
+    if forward_path(L1) == "tile":
+        # the gather reads the table out of LDS tiles: its algorithmic bytes are LDS reads
+        fwd_block, fwd_comp = bound_block(
+            "nnueft_double_fwd: k_acc_tile (the gather out of LDS tiles, ~2/3 of the time) + k_mix + list sort", fwd_ms,
+            fwd_bytes, None, sum(comp_fwd.values()), sum_traffic(traffic, fwd_kernels(L1)), LDS_PEAK_GBS,
+            note="peak: 256 CUs x 256 B of LDS reads per clock at 2.4 GHz; 16-byte reads of whole 128-byte rows at "
+                 "random rows reach 69 TB/s, consecutive ones 124 TB/s (measured on this part)")
+        fwd_block["bound"] = "lds"
+    else:
+        fwd_block, fwd_comp = bound_block(
+            "nnueft_double_fwd: k_acc_blocked (the gather, ~3/4 of the time) + k_mix + pair sort", fwd_ms, fwd_bytes,
+            sum_a * oc * 4, sum(comp_fwd.values()), sum_traffic(traffic, fwd_kernels(L1)), l2_peak)
     out["roofline_forward"] = fwd_block
     out["roofline_forward_compulsory"] = fwd_comp
     det = bwd_ms.get("deterministic") or bwd_ms.get("deterministic_strict")
@@ -705,7 +733,7 @@ def run_ft(args, lib, dev):
             comp_step = sum(comp_fwd.values()) + sum(comp_bwd.values())
             st["compulsory_bytes"] = comp_step
             st["compulsory_frac_of_hbm_peak"] = comp_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS
-            tr = sum_traffic(traffic, FWD_KERNELS + BWD_KERNELS) if mode == "deterministic" else None
+            tr = sum_traffic(traffic, fwd_kernels(L1) + BWD_KERNELS) if mode == "deterministic" else None
             st["traffic_bytes"] = tr
             st["traffic_frac_of_hbm_peak"] = tr / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS if tr else None
         else:
