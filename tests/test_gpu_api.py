@@ -217,12 +217,15 @@ def test_reduce_rows_stage_equals_the_sparse_backward(oracle_cpu):
             assert np.array_equal(gW.cpu().numpy(), rW)
 
 
-def test_forward_and_deterministic_backward_under_graph_capture():
+@pytest.mark.parametrize("L1", [256, 1024], ids=["l2_blocked_forward", "lds_tiled_forward"])
+def test_forward_and_deterministic_backward_under_graph_capture(L1):
     """The launch path of the operator inside one captured HIP graph: forward + deterministic backward (sort
     inline, workspaces allocated before the capture), replayed with eager work and synchronisations between the
-    replays; every replay must give the bits of the eager run, also after the inputs changed in place."""
+    replays; every replay must give the bits of the eager run, also after the inputs changed in place.  Both
+    forward gathers: blocked for L2 (narrow rows) and out of LDS tiles (its unit counters live in the workspace
+    and are reset by the sort of every call)."""
     lib = _native.load()
-    L1, B, K, R, n_psqt = 256, 4096, 32, hk.NUM_INPUTS, 8
+    B, K, R, n_psqt = 4096, 32, hk.NUM_INPUTS, 8
     oc = L1 + n_psqt
     rs = lib.nnueft_row_split()
     t = lambda a: torch.from_numpy(a).to(DEV)
