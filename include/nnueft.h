@@ -164,6 +164,31 @@ int nnueft_double_fwd_act(const float* us, const float* them, const int32_t* wid
                           float act_scale, float act_eps, float act_post_mul, void* stream);
 
 /*
+ * The fused forward over a table that is never written to memory: W + V[row % virtual_rows], rounded to
+ * multiples of 1 / scale_ft (first L1 columns) and 1 / scale_psqt (the others) when fake_quantize is set.
+ * Replaces the table passes in front of the operator in ComposedFeatureTransformer.forward: the merge of
+ * real and virtual weights (features/halfka_v2_hm.py:68-69, `weight + virtual_weight.repeat(32, 1)`) and
+ * their fake quantization (composed_feature_transformer.py:61-76, model/quantize.py:47-56), each a pass over
+ * the whole table in the reference.  The merge happens where a tile of the table goes into LDS, with the
+ * operations of nnueft_table_merge in their order, so the outputs have the bits of nnueft_table_merge followed
+ * by nnueft_double_fwd / nnueft_double_fwd_act (act_on != 0: the activation grid as there).
+ * V f32[virtual_rows, L1 + n_psqt].  Only the LDS-tiled gather can do this: virtual_rows must be 768 and
+ * nnueft_double_fwd_virtual_fits() must return 1 for the sizes on the current device (rows of 512 columns and
+ * more, L1 % 32 == 0, K <= 32, 8 XCDs), else NNUEFT_E_UNSUPPORTED; the workspace is required
+ * (nnueft_fwd_workspace_bytes).  The backward entry points serve it unchanged: they never read the table;
+ * their weight gradient is that of the merged table (the gradient of W as it is, of V after
+ * nnueft_table_virtual_grad).
+ */
+int nnueft_double_fwd_virtual_fits(int B, int K, int R, int L1, int n_psqt, int virtual_rows);
+int nnueft_double_fwd_virtual(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+                              const int64_t* psqt_idx, const float* W, const float* V, const float* bias,
+                              float max_act, float* l0, float* wpsqt, float* bpsqt, float* saved,
+                              int B, int K, int R, int L1, int n_psqt, int virtual_rows,
+                              float scale_ft, float scale_psqt, int fake_quantize,
+                              void* workspace, size_t workspace_bytes,
+                              int act_on, float act_scale, float act_eps, float act_post_mul, void* stream);
+
+/*
  * nnueft_double_fwd for callers that cannot allocate device memory or size a workspace (code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the scratch memory of the
  * L2-blocked gather (pair order, keys, per-workgroup histograms) is a fixed array inside the library,

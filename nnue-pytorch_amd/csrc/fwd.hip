@@ -5,6 +5,8 @@
 // reads 64*VW*4 contiguous bytes of a gathered row (1 KiB with VW = 4).  The index list of the
 // position sits one slot per lane; the valid slots are walked through a ballot mask, so padding
 // costs nothing and no LDS is needed.
+#include <cmath>
+
 #include "gather.h"
 #include "internal.h"
 
@@ -195,7 +197,7 @@ namespace {
 int double_fwd(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0, float* wpsqt,
                float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt, void* workspace,
-               size_t workspace_bytes, void* stream, ActGrid act) {
+               size_t workspace_bytes, void* stream, ActGrid act, VirtualTable vt = VirtualTable{nullptr, 1.0f, 1.0f, 0, 0.0f}) {
     if (B < 0 || K <= 0 || R <= 0 || L1 <= 0 || (L1 & 1) || n_psqt < 0) return NNUEFT_E_ARG;
     if (B == 0) return 0;
     if (!us || !them || !widx || !bidx || !psqt_idx || !W || !bias || !l0 || !wpsqt || !bpsqt || !saved)
@@ -214,11 +216,13 @@ int double_fwd(const float* us, const float* them, const int32_t* widx, const in
         // wide rows gather out of LDS tiles when the caller's workspace has room for that path's lists
         if (vec && nnueft_tile::fits(*info, B, K, R, L1) && workspace_bytes >= nnueft_tile::workspace(B, R))
             return nnueft_tile::double_fwd_tile(us, them, widx, bidx, psqt_idx, W, bias, max_act, l0, wpsqt, bpsqt,
-                                                saved, B, K, R, L1, n_psqt, workspace, st, act);
+                                                saved, B, K, R, L1, n_psqt, workspace, st, act, vt);
+        if (vt.V) return NNUEFT_E_UNSUPPORTED;   // only the LDS-tiled gather merges on the fly
         if (vec && (long long)B <= 0x3fffffffLL && nnueft_blocked::blocked_layout_fits(*info))
             return nnueft_blocked::double_fwd_blocked(us, them, widx, bidx, psqt_idx, W, bias, max_act, l0, wpsqt,
                                                       bpsqt, saved, B, K, R, L1, n_psqt, workspace, st, act);
     }
+    if (vt.V) return NNUEFT_E_UNSUPPORTED;
     if (act.on) {
         // the plain kernels know nothing of the grid: run them, then the grid in place
         ActGrid off{};
@@ -261,4 +265,36 @@ extern "C" int nnueft_double_fwd_act(const float* us, const float* them, const i
     ActGrid act{act_scale, act_eps, act_post_mul, 1};
     return double_fwd(us, them, widx, bidx, psqt_idx, W, bias, max_act, l0, wpsqt, bpsqt, saved, B, K, R, L1, n_psqt,
                       workspace, workspace_bytes, stream, act);
+}
+
+// Whether nnueft_double_fwd_virtual can run these sizes on the current device (1) or not (0; negative: error).
+extern "C" int nnueft_double_fwd_virtual_fits(int B, int K, int R, int L1, int n_psqt, int virtual_rows) {
+    if (B <= 0 || K <= 0 || R <= 0 || L1 <= 0 || (L1 & 1) || n_psqt < 0) return 0;
+    const nnueft_dev::DeviceInfo* info = nullptr;
+    const int rc = nnueft_dev::device_info(nullptr, &info);
+    if (rc) return rc > 0 ? -rc - 1000 : rc;
+    const bool vec = (L1 % 8 == 0) && ((L1 + n_psqt) % 4 == 0);
+    return vec && virtual_rows == nnueft_tile::kBlockRows && nnueft_tile::fits(*info, B, K, R, L1) ? 1 : 0;
+}
+
+extern "C" int nnueft_double_fwd_virtual(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+                                         const int64_t* psqt_idx, const float* W, const float* V, const float* bias,
+                                         float max_act, float* l0, float* wpsqt, float* bpsqt, float* saved, int B,
+                                         int K, int R, int L1, int n_psqt, int virtual_rows, float scale_ft,
+                                         float scale_psqt, int fake_quantize, void* workspace, size_t workspace_bytes,
+                                         int act_on, float act_scale, float act_eps, float act_post_mul, void* stream) {
+    if (!V || virtual_rows != nnueft_tile::kBlockRows) return V ? NNUEFT_E_UNSUPPORTED : NNUEFT_E_ARG;
+    if (fake_quantize && (!(scale_ft > 0.0f) || !(scale_psqt > 0.0f))) return NNUEFT_E_ARG;
+    if (act_on && !(act_scale > 0.0f)) return NNUEFT_E_ARG;
+    if (!workspace) return NNUEFT_E_WORKSPACE;
+    if (!aligned16(V)) return NNUEFT_E_UNSUPPORTED;
+    ActGrid act{act_scale, act_eps, act_post_mul, act_on ? 1 : 0};
+    if (!act_on) act = ActGrid{};
+    // a power of two divides exactly as its reciprocal multiplies (1 / 2^k is exact and so is every product with it
+    // short of underflow, which a multiple of 2^-k of this size never meets)
+    int exp2 = 0;
+    const bool pow2 = fake_quantize && std::frexp(scale_ft, &exp2) == 0.5f && exp2 > -100 && exp2 < 100;
+    VirtualTable vt{V, scale_ft, scale_psqt, fake_quantize ? 1 : 0, pow2 ? 1.0f / scale_ft : 0.0f};
+    return double_fwd(us, them, widx, bidx, psqt_idx, W, bias, max_act, l0, wpsqt, bpsqt, saved, B, K, R, L1, n_psqt,
+                      workspace, workspace_bytes, stream, act, vt);
 }

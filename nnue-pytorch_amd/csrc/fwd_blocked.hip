@@ -170,7 +170,7 @@ __global__ __launch_bounds__(64) void k_mix(const float* __restrict__ us, const 
                                             const float* __restrict__ bias, const float* __restrict__ saved,
                                             float max_act, float* __restrict__ l0, float* __restrict__ wpsqt,
                                             float* __restrict__ bpsqt, int B, int K, int R, int L1, int n_psqt,
-                                            int nslices, ActGrid act) {
+                                            int nslices, ActGrid act, VirtualTable vt) {
     const int lane = threadIdx.x;
     // 1-D launch, the slices of a position next to each other: its rows are then read and written
     // at about the same time (a few per cent faster than position-fastest)
@@ -216,7 +216,12 @@ __global__ __launch_bounds__(64) void k_mix(const float* __restrict__ us, const 
                     const int my = (k0 + lane < K) ? ix[k0 + lane] : -1;
                     const bool ok = my >= 0 && my < R;
                     u64 mask = __ballot(ok);
-                    const float myps = ok ? W[(size_t)my * out_cols + L1 + pi] : 0.0f;
+                    float myps = ok ? W[(size_t)my * out_cols + L1 + pi] : 0.0f;
+                    if (ok && vt.V) {
+                        // the merged table's entry: W + V[row % 768], on the psqt grid when asked for
+                        myps = myps + vt.V[(size_t)(my % nnueft_tile::kBlockRows) * out_cols + L1 + pi];
+                        if (vt.quantize) myps = rintf(myps * vt.scale_psqt) / vt.scale_psqt;
+                    }
                     while (mask) ps[p] = ps[p] + bcast_f(myps, pop_lane(mask));
                 }
             }
@@ -242,13 +247,13 @@ int launch_scan(uint32_t* data, int n, hipStream_t st) {
 int launch_mix(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                const int64_t* psqt_idx, const float* W, const float* bias, const float* saved, float max_act,
                float* l0, float* wpsqt, float* bpsqt, int B, int K, int R, int L1, int n_psqt, hipStream_t st,
-               ActGrid act) {
+               ActGrid act, VirtualTable vt) {
     const int hv = (L1 / 2) / 4;
     const int mix_slices = (hv + 63) / 64;
     if ((long long)B * mix_slices > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
     const dim3 mix_grid((unsigned)B * mix_slices);
     hipLaunchKernelGGL(k_mix<4>, mix_grid, dim3(64), 0, st, us, them, widx, bidx, psqt_idx, W, bias, saved, max_act,
-                       l0, wpsqt, bpsqt, B, K, R, L1, n_psqt, mix_slices, act);
+                       l0, wpsqt, bpsqt, B, K, R, L1, n_psqt, mix_slices, act, vt);
     NNUEFT_LAUNCH_CHECK();
     return 0;
 }
@@ -332,7 +337,7 @@ int double_fwd_blocked(const float* us, const float* them, const int32_t* widx, 
     }
     NNUEFT_LAUNCH_CHECK();
     return launch_mix(us, them, widx, bidx, psqt_idx, W, bias, saved, max_act, l0, wpsqt, bpsqt, B, K, R, L1, n_psqt,
-                      st, act);
+                      st, act, VirtualTable{nullptr, 1.0f, 1.0f, 0, 0.0f});
 }
 
 }  // namespace nnueft_blocked

@@ -39,8 +39,13 @@ constexpr int kLenBins = kSlots + 1;
 constexpr int kMaxBlocks = 62;
 constexpr int kBins = 2048;                        // LDS counters of the sort (kMaxBlocks * kLenBins + 1 used at most)
 static_assert(kMaxBlocks * kLenBins + 1 <= kBins, "sort bins");
+static_assert(kRows == kBlockRows, "rows of a table block");
 constexpr uint32_t kForeign = 63;                  // count field of a list that leaves its block
-constexpr int kAccThreads = 1024;
+#ifndef NNUEFT_TILE_NT
+#define NNUEFT_TILE_NT 1024
+#endif
+constexpr int kAccThreads = NNUEFT_TILE_NT;
+constexpr int kAccThreadsVirtual = 768;
 constexpr int kSortThreads = 256;
 constexpr int kLdsBytes = kTileBytes + kChunk * kSlots * 2 + kChunk * 4 + 16;
 
@@ -318,15 +323,43 @@ __device__ __forceinline__ uint32_t row_addr(uint32_t w, uint32_t off) {
     return r;
 }
 
+// round(x * scale) / scale with round-half-to-even, as torch's mul / round / div (the table merge's grid)
+__device__ __forceinline__ float fq(float x, float scale) { return rintf(x * scale) / scale; }
+
+// One element of the table the gather sums: W[row] alone, or merged with the virtual weights of the row's place
+// in its block, W + V[row % virtual rows], on the fake-quantization grid when asked for; the same operations, in
+// the same order, as the separate merge pass (k_table_merge), so a forward over either gives the same bits.
+__device__ __forceinline__ f4 merged4(f4 w, f4 v, const VirtualTable& vt) {
+    w += v;
+    if (vt.quantize) {
+        if (vt.inv_scale_ft != 0.0f) {
+            w.x = rintf(w.x * vt.scale_ft) * vt.inv_scale_ft;
+            w.y = rintf(w.y * vt.scale_ft) * vt.inv_scale_ft;
+            w.z = rintf(w.z * vt.scale_ft) * vt.inv_scale_ft;
+            w.w = rintf(w.w * vt.scale_ft) * vt.inv_scale_ft;
+        } else {
+            w.x = fq(w.x, vt.scale_ft);
+            w.y = fq(w.y, vt.scale_ft);
+            w.z = fq(w.z, vt.scale_ft);
+            w.w = fq(w.w, vt.scale_ft);
+        }
+    }
+    return w;
+}
+
 // saved[pair, columns of the tile] = chain from +0 over the pair's list, for every pair of the chunk.
-__global__ __launch_bounds__(kAccThreads) void k_acc_tile(const int32_t* __restrict__ widx,
+// VIRT: the table is W + V[row % kRows] (see merged4); the tile is merged on its way into LDS.  That variant
+// runs with 768 threads: the tile of V waits in registers beside the tile of W.
+template <int NT, bool VIRT>
+__global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ widx,
                                                           const int32_t* __restrict__ bidx,
                                                           const uint16_t* __restrict__ lists,
                                                           const uint32_t* __restrict__ pidcnt,
                                                           const Chunk* __restrict__ chunks,
                                                           uint32_t* __restrict__ sched, const float* __restrict__ W,
                                                           float* __restrict__ acc, int B, int K, int R, int L1,
-                                                          int out_cols, int tiles_per_xcd, int tile_group) {
+                                                          int out_cols, int tiles_per_xcd, int tile_group,
+                                                          VirtualTable vt) {
     extern __shared__ float4 lds_raw[];
     char* tb = reinterpret_cast<char*>(lds_raw);
     u4* moff = reinterpret_cast<u4*>(tb + kTileBytes);                                   // kChunk * 4
@@ -335,8 +368,8 @@ __global__ __launch_bounds__(kAccThreads) void k_acc_tile(const int32_t* __restr
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     constexpr int N4 = kRows * (kRowBytes / 16);
-    static_assert(N4 % kAccThreads == 0, "tile load");
-    constexpr int IT = N4 / kAccThreads;
+    static_assert(N4 % NT == 0, "tile load");
+    constexpr int IT = N4 / NT;
     const int x = blockIdx.x % kXcd;
     const int ntiles = L1 / kTileCols;
     const int groups = (tiles_per_xcd + tile_group - 1) / tile_group;
@@ -348,6 +381,7 @@ __global__ __launch_bounds__(kAccThreads) void k_acc_tile(const int32_t* __restr
     if (tid == 0) ctr[1] = atomicAdd(unit_ctr, 1u);
 
     f4 v[IT];
+    f4 vv[VIRT ? IT : 1];
     while (true) {
         __syncthreads();   // the previous unit is done with the lists and the tile; ctr[1] is written
         const int unit = (int)ctr[1];
@@ -366,18 +400,22 @@ __global__ __launch_bounds__(kAccThreads) void k_acc_tile(const int32_t* __restr
         if (tid == 0) ctr[1] = atomicAdd(unit_ctr, 1u);
         {
             const u4* ms = reinterpret_cast<const u4*>(lists + (size_t)C.start * kSlots);
-            for (int f = tid; f < C.count * 4; f += kAccThreads) moff[f] = ms[f];
-            if (tid < C.count) mpid[tid] = pidcnt[C.start + tid];
+            for (int f = tid; f < C.count * 4; f += NT) moff[f] = ms[f];
+            for (int f = tid; f < C.count; f += NT) mpid[f] = pidcnt[C.start + f];
         }
 #define NNUEFT_LOAD_TILE(c_)                                                                          \
     {                                                                                                 \
         const float* src = wb + (c_) * kTileCols;                                                     \
         _Pragma("unroll") for (int i = 0; i < IT; ++i) {                                              \
-            const int f = tid + i * kAccThreads;                                                      \
+            const int f = tid + i * NT;                                                               \
             const int row = f >> 3;                                                                   \
             v[i] = row < rows_here                                                                    \
                        ? *reinterpret_cast<const f4*>(src + (size_t)row * out_cols + (f & 7) * 4)     \
                        : f4{0.f, 0.f, 0.f, 0.f};                                                      \
+            if (VIRT)                                                                                 \
+                vv[i] = row < rows_here ? *reinterpret_cast<const f4*>(vt.V + (size_t)row * out_cols + \
+                                                                       (c_) * kTileCols + (f & 7) * 4) \
+                                        : f4{0.f, 0.f, 0.f, 0.f};                                     \
         }                                                                                             \
     }
         if (q0 < q1) NNUEFT_LOAD_TILE(x * tiles_per_xcd + q0)
@@ -386,8 +424,8 @@ __global__ __launch_bounds__(kAccThreads) void k_acc_tile(const int32_t* __restr
             if (q != q0) __syncthreads();   // everyone is done reading the previous tile
 #pragma unroll
             for (int i = 0; i < IT; ++i) {
-                const int f = tid + i * kAccThreads;
-                reinterpret_cast<f4*>(tb)[f] = v[i];
+                const int f = tid + i * NT;
+                reinterpret_cast<f4*>(tb)[f] = VIRT ? merged4(v[i], vv[i], vt) : v[i];
             }
             if (tid == 0) ctr[0] = 0;
             __syncthreads();
@@ -411,7 +449,13 @@ __global__ __launch_bounds__(kAccThreads) void k_acc_tile(const int32_t* __restr
                     const int32_t* ix = pair_list(widx, bidx, pair, B, K);
                     for (int k = 0; k < K; ++k) {
                         const int r = ix[k];
-                        if (r >= 0 && r < R) a += *reinterpret_cast<const f4*>(W + (size_t)r * out_cols + c * kTileCols + j * 4);
+                        if (r >= 0 && r < R) {
+                            f4 w = *reinterpret_cast<const f4*>(W + (size_t)r * out_cols + c * kTileCols + j * 4);
+                            if (VIRT)
+                                w = merged4(w, *reinterpret_cast<const f4*>(vt.V + (size_t)(r % kRows) * out_cols +
+                                                                            c * kTileCols + j * 4), vt);
+                            a += w;
+                        }
                     }
                 } else {
                     uint32_t oo[kSlots / 2];
@@ -453,8 +497,11 @@ std::atomic<int> g_lds_allowed[kMaxDevices];
 int allow_lds(int device) {
     if (device < 0 || device >= kMaxDevices) return NNUEFT_E_UNSUPPORTED;
     if (g_lds_allowed[device].load(std::memory_order_acquire)) return 0;
-    const hipError_t e =
-        hipFuncSetAttribute((const void*)k_acc_tile, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    hipError_t e = hipFuncSetAttribute((const void*)k_acc_tile<kAccThreads, false>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute((const void*)k_acc_tile<kAccThreadsVirtual, true>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
     if (e != hipSuccess) return (int)e;
     g_lds_allowed[device].store(1, std::memory_order_release);
     return 0;
@@ -463,7 +510,7 @@ int allow_lds(int device) {
 int double_fwd_tile(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                     const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,
                     float* wpsqt, float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt, void* ws,
-                    hipStream_t st, ActGrid act) {
+                    hipStream_t st, ActGrid act, VirtualTable vt) {
     Layout L;
     if (!layout(B, R, &L)) return NNUEFT_E_UNSUPPORTED;
     int device = 0;
@@ -496,11 +543,17 @@ int double_fwd_tile(const float* us, const float* them, const int32_t* widx, con
     if (const char* e = getenv("NNUEFT_TILE_GROUP")) tile_group = atoi(e) > 0 ? atoi(e) : tile_group;
 #endif
     const int grid = info->cus / kXcd * kXcd;
-    hipLaunchKernelGGL(k_acc_tile, dim3(grid), dim3(kAccThreads), kLdsBytes, st, widx, bidx, lists, pidcnt, chunks,
-                       sched, W, saved, B, K, R, L1, out_cols, tiles_per_xcd, tile_group);
+    if (vt.V)
+        hipLaunchKernelGGL((k_acc_tile<kAccThreadsVirtual, true>), dim3(grid), dim3(kAccThreadsVirtual), kLdsBytes, st,
+                           widx, bidx, lists, pidcnt, chunks, sched, W, saved, B, K, R, L1, out_cols, tiles_per_xcd,
+                           tile_group, vt);
+    else
+        hipLaunchKernelGGL((k_acc_tile<kAccThreads, false>), dim3(grid), dim3(kAccThreads), kLdsBytes, st, widx, bidx,
+                           lists, pidcnt, chunks, sched, W, saved, B, K, R, L1, out_cols, tiles_per_xcd, tile_group,
+                           vt);
     NNUEFT_LAUNCH_CHECK();
     return nnueft_blocked::launch_mix(us, them, widx, bidx, psqt_idx, W, bias, saved, max_act, l0, wpsqt, bpsqt, B,
-                                      K, R, L1, n_psqt, st, act);
+                                      K, R, L1, n_psqt, st, act, vt);
 }
 
 }  // namespace nnueft_tile

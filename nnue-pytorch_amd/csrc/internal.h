@@ -10,6 +10,17 @@ struct ActGrid {
     int on;
 };
 
+// The virtual weights a forward may merge into the table on the fly: the table it sums is
+// W + V[row % 768] (V: f32 [768, L1 + n_psqt]), rounded to multiples of 1 / scale_ft (first L1 columns) and
+// 1 / scale_psqt (the rest) when `quantize` is set.  V == nullptr: the table is W as it is.
+struct VirtualTable {
+    const float* V;
+    float scale_ft, scale_psqt;
+    int quantize;
+    float inv_scale_ft;   // 1 / scale_ft when scale_ft is a power of two (dividing by it is then the same as
+                          // multiplying by this, bit for bit, at a fraction of the instructions), else 0
+};
+
 namespace nnueft_dev {
 
 // What the launchers need to know about a device; queried once per device and process.
@@ -47,7 +58,7 @@ int launch_scan(uint32_t* data, int n, hipStream_t st);
 int launch_mix(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                const int64_t* psqt_idx, const float* W, const float* bias, const float* saved, float max_act,
                float* l0, float* wpsqt, float* bpsqt, int B, int K, int R, int L1, int n_psqt, hipStream_t st,
-               ActGrid act);
+               ActGrid act, VirtualTable vt);
 
 int double_fwd_blocked(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                        const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,
@@ -60,12 +71,13 @@ namespace nnueft_tile {
 
 // Forward gather out of LDS-resident tiles of the table (one 768-row block x 32 columns).  fits(): whether
 // the shape and the device can take it; workspace(): bytes it needs (at least the L2-blocked path's).
+constexpr int kBlockRows = 768;   // rows of a table block (a king bucket of HalfKAv2_hm); also the virtual rows
 bool fits(const nnueft_dev::DeviceInfo& d, int B, int K, int R, int L1);
 size_t workspace(int B, int R);
 int double_fwd_tile(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                     const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,
                     float* wpsqt, float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt, void* ws,
-                    hipStream_t st, ActGrid act);
+                    hipStream_t st, ActGrid act, VirtualTable vt);
 
 }  // namespace nnueft_tile
 

@@ -44,6 +44,12 @@ PROTOTYPES = {
         c_int,
         [c_void_p] * 7 + [c_float] + [c_void_p] * 4 + [c_int] * 5 + [c_void_p, c_size_t] + [c_float] * 3 + [c_void_p],
     ),
+    "nnueft_double_fwd_virtual_fits": (c_int, [c_int] * 6),
+    "nnueft_double_fwd_virtual": (
+        c_int,
+        [c_void_p] * 8 + [c_float] + [c_void_p] * 4 + [c_int] * 6 + [c_float] * 2 + [c_int]
+        + [c_void_p, c_size_t] + [c_int] + [c_float] * 3 + [c_void_p],
+    ),
     "nnueft_double_fwd_noalloc": (c_int, [c_void_p] * 7 + [c_float] + [c_void_p] * 4 + [c_int] * 5 + [c_void_p]),
     "nnueft_double_bwd_atomic": (c_int, [c_void_p] * 6 + [c_float] + [c_void_p] * 6 + [c_int] * 5 + [c_void_p]),
     "nnueft_double_bwd_det": (

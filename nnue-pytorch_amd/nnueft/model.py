@@ -255,6 +255,93 @@ def _table_merge(weight, virtual, l1_size, scale_ft, scale_psqt, quantize):
     return _TableMerge.apply(weight, virtual, l1_size, scale_ft, scale_psqt, quantize)
 
 
+# FOLD_TABLE_MERGE: whether ComposedFeatureTransformer lets the forward kernel merge real and virtual weights on
+# their way into LDS (no merged table in memory, no merge pass) where the library can; False keeps the separate
+# pass.  Both give the same bits.
+FOLD_TABLE_MERGE = True
+
+
+@torch.compiler.disable(recursive=False)
+def _virtual_forward_fits(white_indices, weight, virtual, l1_size) -> bool:
+    if not (FOLD_TABLE_MERGE and weight.is_cuda and _native.available()):
+        return False
+    lib = _native.load()
+    B, K = white_indices.shape
+    R, cols = weight.shape
+    with torch.cuda.device(weight.device):
+        return B > 0 and lib.nnueft_double_fwd_virtual_fits(B, K, R, l1_size, cols - l1_size, virtual.shape[0]) == 1
+
+
+@torch.compiler.disable(recursive=False)
+def _launch_double_fwd_virtual(us, them, white_indices, black_indices, psqt_indices, weight, virtual, bias,
+                               max_ft_activation, l1_size, scale_ft, scale_psqt, quantize, act_grid):
+    lib = _native.load()
+    device = weight.device
+    B, K = white_indices.shape
+    R, cols = weight.shape
+    l0_ = torch.empty(B, l1_size, dtype=torch.float32, device=device)
+    wpsqt = torch.empty(B, 1, dtype=torch.float32, device=device)
+    bpsqt = torch.empty(B, 1, dtype=torch.float32, device=device)
+    row_sums = torch.empty(2, B, l1_size, dtype=torch.float32, device=device)
+    act = act_grid if act_grid is not None else (1.0, 0.0, 1.0)
+    with torch.cuda.device(device):
+        nbytes = lib.nnueft_fwd_workspace_bytes(B, K, R, l1_size, cols - l1_size)
+        ws = torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+        rc = lib.nnueft_double_fwd_virtual(
+            us.data_ptr(), them.data_ptr(), white_indices.data_ptr(), black_indices.data_ptr(),
+            psqt_indices.data_ptr(), weight.data_ptr(), virtual.data_ptr(), bias.data_ptr(), float(max_ft_activation),
+            l0_.data_ptr(), wpsqt.data_ptr(), bpsqt.data_ptr(), row_sums.data_ptr(), B, K, R, l1_size,
+            cols - l1_size, virtual.shape[0], float(scale_ft), float(scale_psqt), int(bool(quantize)),
+            ws.data_ptr(), nbytes, int(act_grid is not None), float(act[0]), float(act[1]), float(act[2]),
+            _stream_ptr(device))
+    _native.check(rc, "nnueft_double_fwd_virtual")
+    return l0_, wpsqt, bpsqt, row_sums
+
+
+class _FusedDoubleFtVirtual(torch.autograd.Function):
+    """FusedDoubleFtFunction over the table q(weight + virtual[row % 768]) without that table ever being
+    written: the forward kernel merges while it fills its LDS tiles.  The backward is FusedDoubleFtFunction's
+    (it never reads the table); the merge's straight-through gradient hands its weight gradient to `weight`
+    as it is and to `virtual` summed over the table blocks."""
+
+    @staticmethod
+    def forward(ctx, us, them, white_indices, black_indices, psqt_indices, weight, virtual, bias, max_ft_activation,
+                l1_size, scale_ft, scale_psqt, quantize, act_grid):
+        from . import sparse_linear_functions as _slf
+
+        ctx.act_grid = None if act_grid is None else tuple(float(v) for v in act_grid)
+        ctx.max_ft_activation = float(max_ft_activation)
+        ctx.l1_size = int(l1_size)
+        ctx.backward_mode = _slf.get_backward_mode()
+        ctx.sort_placement = _slf.get_sort_placement()
+        ctx.shape = tuple(weight.shape)
+        ctx.vrows = virtual.shape[0]
+        for t in (us, them, white_indices, black_indices, psqt_indices, weight, virtual, bias):
+            assert t.is_cuda and t.is_contiguous() and t.device == weight.device
+        assert weight.dtype == torch.float32 and virtual.dtype == torch.float32 and bias.dtype == torch.float32
+        assert virtual.shape[1] == weight.shape[1] == bias.shape[0]
+        l0_, wpsqt, bpsqt, row_sums = _launch_double_fwd_virtual(
+            us, them, white_indices, black_indices, psqt_indices, weight, virtual, bias, ctx.max_ft_activation,
+            ctx.l1_size, scale_ft, scale_psqt, quantize, ctx.act_grid)
+        ctx.save_for_backward(us, them, white_indices, black_indices, psqt_indices, bias, row_sums)
+        return l0_, wpsqt, bpsqt
+
+    @staticmethod
+    def backward(ctx, grad_l0, grad_wpsqt, grad_bpsqt):
+        from . import _ops
+
+        us, them, white_indices, black_indices, psqt_indices, bias, row_sums = ctx.saved_tensors
+        if ctx.act_grid is not None and ctx.act_grid[2] != 1.0:
+            grad_l0 = grad_l0 * ctx.act_grid[2]
+        second_stream = ctx.sort_placement != "inline" and not torch.compiler.is_compiling()
+        grad_weight, grad_bias = _ops.launch(
+            "double_bwd", us, them, white_indices, black_indices, psqt_indices, bias, ctx.max_ft_activation,
+            grad_l0, grad_wpsqt, grad_bpsqt, row_sums, ctx.shape[0], ctx.l1_size, ctx.shape[1], ctx.backward_mode,
+            None, second_stream)
+        grad_virtual = _launch_table_virtual_grad(grad_weight, ctx.vrows) if ctx.needs_input_grad[6] else None
+        return (None, None, None, None, None, grad_weight, grad_virtual, grad_bias, None, None, None, None, None, None)
+
+
 @torch.compiler.disable(recursive=False)
 def _launch_act_fake_quantize(x, scale, post_mul):
     lib = _native.load()
@@ -462,17 +549,7 @@ class ComposedFeatureTransformer(nn.Module):
             if fake_quantize_weights:
                 merged = torch.cat([q.fake_quantize_weights(merged[:, :self.l1_size], "ft_weight"),
                                     q.fake_quantize_weights(merged[:, self.l1_size:], "ft_psqt_weight")], dim=1)
-        b = self.bias[:self.l1_size]
-        if fake_quantize_weights:
-            if b.is_cuda and b.dtype == torch.float32 and _native.available():
-                # one launch instead of the five elementwise ops of fake_quantize_weights (same bits)
-                s = q.weight_scales_dict["ft_bias"]
-                b = _table_merge(b.view(1, -1), None, self.l1_size, s, s, True).view(-1)
-            else:
-                b = q.fake_quantize_weights(b, "ft_bias")
-        # the PSQT part of the bias is held at zero
-        bias = torch.cat([b, self.psqt_bias_zeros.to(b.dtype)], dim=0)
-        return merged, bias
+        return merged, self._merged_bias(fake_quantize_weights)
 
     @torch.no_grad()
     def coalesce(self):
@@ -505,10 +582,38 @@ class ComposedFeatureTransformer(nn.Module):
         for f in self.features:
             f.clip_weights(quantization)
 
+    def _merged_bias(self, fake_quantize_weights: bool):
+        q = self.quantization
+        b = self.bias[:self.l1_size]
+        if fake_quantize_weights:
+            if b.is_cuda and b.dtype == torch.float32 and _native.available():
+                # one launch instead of the five elementwise ops of fake_quantize_weights (same bits)
+                s = q.weight_scales_dict["ft_bias"]
+                b = _table_merge(b.view(1, -1), None, self.l1_size, s, s, True).view(-1)
+            else:
+                b = q.fake_quantize_weights(b, "ft_bias")
+        # the PSQT part of the bias is held at zero
+        return torch.cat([b, self.psqt_bias_zeros.to(b.dtype)], dim=0)
+
     def forward(self, us, them, white_indices, black_indices, psqt_indices, fake_quantize_acts: bool,
                 fake_quantize_weights: bool, backend: str = "auto"):
-        merged, bias = self.merged_weight_and_bias(fake_quantize_weights)
         q = self.quantization
+        only = self.features[0] if len(self.features) == 1 else None
+        if (only is not None and isinstance(only, HalfKav2Hm) and backend in ("auto", "fused")
+                and all(t.is_cuda for t in (us, them, white_indices, black_indices, psqt_indices, self.bias))
+                and white_indices.dtype == torch.int32 and white_indices.dim() == 2
+                and _virtual_forward_fits(white_indices, only.weight, only.virtual_weight, self.l1_size)):
+            # real + virtual weights (and their grid) merged inside the forward kernel: no pass over the table
+            act_grid = (q.hidden_quantized_one, FAKE_QUANTIZE_EPS, q.l0_correction_factor) if fake_quantize_acts else None
+            l0_, wpsqt, bpsqt = _FusedDoubleFtVirtual.apply(
+                us, them, white_indices, black_indices, psqt_indices, only.weight, only.virtual_weight,
+                self._merged_bias(fake_quantize_weights), q.max_ft_activation, self.l1_size,
+                q.weight_scales_dict["ft_weight"], q.weight_scales_dict["ft_psqt_weight"], fake_quantize_weights,
+                act_grid)
+            if not fake_quantize_acts and q.l0_correction_factor != 1.0:
+                l0_ = l0_ * q.l0_correction_factor
+            return l0_, wpsqt, bpsqt
+        merged, bias = self.merged_weight_and_bias(fake_quantize_weights)
         if (fake_quantize_acts and backend in ("auto", "fused") and merged.is_cuda and _native.available()
                 and all(t.is_cuda for t in (us, them, white_indices, black_indices, psqt_indices, bias))):
             # the activation grid and the correction factor inside the kernel that writes l0

@@ -34,6 +34,95 @@ def test_table_merge_and_virtual_grad(oracle_cpu, R, cols, L1, vrows, quantize):
     assert torch.equal(merged.detach().cpu(), t)
 
 
+@pytest.mark.parametrize("quantize", [True, False])
+@pytest.mark.parametrize("act_on", [True, False])
+@pytest.mark.parametrize("B,L1,lists", [(700, 512, "halfka"), (3000, 1024, "halfka"), (600, 544, "any")])
+def test_forward_over_the_virtual_table_equals_merge_then_forward(B, L1, lists, quantize, act_on):
+    """nnueft_double_fwd_virtual (real + virtual weights merged where the tile goes into LDS) against
+    nnueft_table_merge followed by nnueft_double_fwd / nnueft_double_fwd_act, through the C ABI: the same
+    bits in l0, the psqt outputs and the saved row sums.  "any": index lists that leave their table block
+    (those lists are summed from global memory, merged there too)."""
+    lib = _native.load()
+    K, R, n_psqt, vrows = 32, hk.NUM_INPUTS, 8, 768
+    oc = L1 + n_psqt
+    rng = np.random.default_rng(B + L1)
+    us, them, white, black, pc = hk.synthetic_batch(B, B + 1)
+    if lists == "any":
+        n = rng.integers(0, K + 1, size=(2, B))
+        idx = rng.integers(0, R, size=(2, B, K)).astype(np.int32)
+        idx[np.arange(K)[None, None, :] >= n[:, :, None]] = -1
+        white, black = idx[0].copy(), idx[1].copy()
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+    d_us, d_them, d_w, d_b, d_psqt = t(us), t(them), t(white), t(black), t(((pc - 1) // 4).astype(np.int64))
+    W = t((rng.standard_normal((R, oc)) * 0.05).astype(np.float32))
+    V = t((rng.standard_normal((vrows, oc)) * 0.05).astype(np.float32))
+    bias = t((rng.standard_normal(oc) * 0.05).astype(np.float32))
+    st = torch.cuda.current_stream().cuda_stream
+    assert lib.nnueft_double_fwd_virtual_fits(B, K, R, L1, n_psqt, vrows) == 1
+    assert lib.nnueft_double_fwd_virtual_fits(B, K, R, L1, n_psqt, 512) == 0
+    assert lib.nnueft_double_fwd_virtual_fits(B, K, R, 128, n_psqt, vrows) == 0
+    nbytes = lib.nnueft_fwd_workspace_bytes(B, K, R, L1, n_psqt)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
+    scale_ft, scale_psqt, act = 256.0, 9600.0, (127.0, 1e-5, 0.75)
+
+    def outs():
+        return [torch.full(s, float("nan"), device=DEV) for s in ((B, L1), (B, 1), (B, 1), (2, B, L1))]
+
+    got = outs()
+    _native.check(lib.nnueft_double_fwd_virtual(
+        d_us.data_ptr(), d_them.data_ptr(), d_w.data_ptr(), d_b.data_ptr(), d_psqt.data_ptr(), W.data_ptr(),
+        V.data_ptr(), bias.data_ptr(), 255.0 / 256.0, *[x.data_ptr() for x in got], B, K, R, L1, n_psqt, vrows,
+        scale_ft, scale_psqt, int(quantize), ws.data_ptr(), nbytes, int(act_on), *act, st), "double_fwd_virtual")
+    merged = torch.empty_like(W)
+    _native.check(lib.nnueft_table_merge(W.data_ptr(), V.data_ptr(), merged.data_ptr(), R, oc, L1, vrows, scale_ft,
+                                         scale_psqt, int(quantize), st), "table_merge")
+    want = outs()
+    head = (d_us.data_ptr(), d_them.data_ptr(), d_w.data_ptr(), d_b.data_ptr(), d_psqt.data_ptr(), merged.data_ptr(),
+            bias.data_ptr(), 255.0 / 256.0, *[x.data_ptr() for x in want], B, K, R, L1, n_psqt, ws.data_ptr(), nbytes)
+    if act_on:
+        _native.check(lib.nnueft_double_fwd_act(*head, *act, st), "double_fwd_act")
+    else:
+        _native.check(lib.nnueft_double_fwd(*head, st), "double_fwd")
+    torch.cuda.synchronize()
+    for a, b in zip(got, want):
+        assert not torch.isnan(a).any()
+        assert torch.equal(a, b)
+    # sizes the LDS-tiled gather does not take are refused, not run some other way
+    rc = lib.nnueft_double_fwd_virtual(
+        d_us.data_ptr(), d_them.data_ptr(), d_w.data_ptr(), d_b.data_ptr(), d_psqt.data_ptr(), W.data_ptr(),
+        V.data_ptr(), bias.data_ptr(), 255.0 / 256.0, *[x.data_ptr() for x in got], B, K, R, L1, n_psqt, 512,
+        scale_ft, scale_psqt, int(quantize), ws.data_ptr(), nbytes, int(act_on), *act, st)
+    assert rc != 0
+
+
+@pytest.mark.parametrize("fq_acts,fq_weights", [(True, True), (False, False)])
+def test_ft_module_with_the_merge_folded_into_the_forward(fq_acts, fq_weights):
+    """ComposedFeatureTransformer with the table merge inside the forward kernel against the same module with
+    the separate merge pass: outputs and every gradient (weight, virtual weight, bias) bit for bit."""
+    results = []
+    B, L1 = 2048, 512
+    batch = [torch.from_numpy(a).to(DEV) for a in hk.synthetic_batch(B, 16)]
+    us, them, white, black, pc = batch
+    psqt = (pc - 1) // 4
+    gl = None
+    old = M.FOLD_TABLE_MERGE
+    try:
+        for fold in (True, False):
+            M.FOLD_TABLE_MERGE = fold
+            model = _make_model(L1, 9).to(DEV)
+            out = model.input(us, them, white, black, psqt, fq_acts, fq_weights)
+            if gl is None:
+                gl = [torch.randn_like(o) for o in out]
+            torch.autograd.backward(list(out), gl)
+            f = model.input.features[0]
+            results.append([o.detach() for o in out] + [f.weight.grad, f.virtual_weight.grad, model.input.bias.grad])
+    finally:
+        M.FOLD_TABLE_MERGE = old
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    assert results[0][4].abs().sum() > 0
+
+
 def _make_model(L1, seed):
     torch.manual_seed(seed)
     model = M.NNUEModel("HalfKAv2_hm^", M.ModelConfig(L1=L1, L2=16, L3=32))
