@@ -33,10 +33,14 @@ constexpr int kRows = 768;                         // rows of a table block = ro
 constexpr int kTileCols = 32;                      // floats per tile row
 constexpr int kRowBytes = kTileCols * 4;
 constexpr int kTileBytes = (kRows + 1) * kRowBytes;   // + one row of zeros for the padding slots
-constexpr int kChunk = 512;                        // pairs whose lists a workgroup holds
 constexpr int kSlots = 32;                         // list slots the 16-bit lists hold
 constexpr int kLenBins = kSlots + 1;
+constexpr int kLenBins8 = kLenBins * kSlots;       // entries a chunk can get beyond its even share of a block
+constexpr int kChunk = 1536;                       // most pairs whose lists a workgroup holds
+constexpr int kListCap = 27648;                    // most list entries (padded, 16 bits each) it holds
+constexpr int kListSlack = kLenBins8;              // see chunks_of()
 constexpr int kMaxBlocks = 62;
+constexpr int kMaxChunks = 1024;                   // chunks whose places a workgroup of the sort keeps in LDS
 constexpr int kBins = 2048;                        // LDS counters of the sort (kMaxBlocks * kLenBins + 1 used at most)
 static_assert(kMaxBlocks * kLenBins + 1 <= kBins, "sort bins");
 static_assert(kRows == kBlockRows, "rows of a table block");
@@ -47,18 +51,23 @@ constexpr uint32_t kForeign = 63;                  // count field of a list that
 constexpr int kAccThreads = NNUEFT_TILE_NT;
 constexpr int kAccThreadsVirtual = 768;
 constexpr int kSortThreads = 256;
-constexpr int kLdsBytes = kTileBytes + kChunk * kSlots * 2 + kChunk * 4 + 16;
+constexpr int kLdsBytes = kTileBytes + (kListCap + 32) * 2 + kChunk * 4 + kChunk * 2 + 16;
 
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 
+// A chunk of a block's pairs: pairs [start, start + count) of pidcnt / loff, their lists in
+// lists[pool8 * 8 .. + n8 * 8) (every list padded to a multiple of 8 entries).
 struct Chunk {
-    int block, start, count, pad;
+    int block, start, count, pool8, n8, pad0, pad1, pad2;
 };
+
+// entries of a list of `cnt` slots in the pool
+__host__ __device__ __forceinline__ int padded(int cnt) { return (cnt + 7) & ~7; }
 
 // What the sort and the gather share in the workspace.
 struct Layout {
-    size_t hist, total, lists, pidcnt, chunks, sched, end;
+    size_t hist, total, lists, pidcnt, loff, chunks, sched, end;
     int ngroups, nblocks, nbins, max_chunks, nslots;
 };
 
@@ -70,7 +79,7 @@ bool layout(int B, int R, Layout* L) {
     if (L->nblocks > kMaxBlocks) return false;
     L->nbins = L->nblocks * kLenBins + 1;   // + one empty bin: its offset is the end of the last block
     L->ngroups = (2 * B + kSortThreads - 1) / kSortThreads;
-    L->max_chunks = (2 * B + kChunk - 1) / kChunk + L->nblocks;
+    L->max_chunks = (2 * B + 511) / 512 + 2 * L->nblocks + 2;
     L->nslots = 2 * B + L->max_chunks;     // a block's chunks are equally long, the last ones one pair short
     size_t off = 0;
     L->hist = off;
@@ -78,9 +87,11 @@ bool layout(int B, int R, Layout* L) {
     L->total = off;
     off += up256((size_t)kBins * sizeof(uint32_t));
     L->lists = off;
-    off += up256((size_t)L->nslots * kSlots * sizeof(uint16_t));
+    off += up256(((size_t)2 * B * kSlots + 64) * sizeof(uint16_t));
     L->pidcnt = off;
     off += up256((size_t)L->nslots * sizeof(uint32_t));
+    L->loff = off;
+    off += up256((size_t)L->nslots * sizeof(uint16_t));
     L->chunks = off;
     off += up256((size_t)L->max_chunks * sizeof(Chunk));
     L->sched = off;
@@ -99,7 +110,8 @@ size_t workspace(int B, int R) {
 bool fits(const nnueft_dev::DeviceInfo& d, int B, int K, int R, int L1) {
     Layout L;
     return K <= kSlots && L1 % kTileCols == 0 && L1 >= 512 && (long long)2 * B < (1ll << 26) &&
-           d.max_lds >= kLdsBytes && d.xcds == kXcd && d.cus >= kXcd && layout(B, R, &L);
+           d.max_lds >= kLdsBytes && d.xcds == kXcd && d.cus >= kXcd && layout(B, R, &L) &&
+           L.max_chunks <= kMaxChunks;
 }
 
 __device__ __forceinline__ const int32_t* pair_list(const int32_t* __restrict__ widx,
@@ -168,9 +180,18 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_hist(const int32_t* __restr
     for (int i = tid; i < nbins; i += kSortThreads) hist[(size_t)i * gridDim.x + blockIdx.x] = bins[i];
 }
 
-// Chunks of a block with n pairs: as few as keep each at kChunk pairs or fewer; pair i of the block
-// (longest list first) goes to chunk i % nc, so every chunk gets the same mix of list lengths.
-__device__ __forceinline__ int chunks_of(int n) { return (n + kChunk - 1) / kChunk; }
+// Chunks of a block with n pairs whose lists take e entries (each list padded to a multiple of 8): as few as
+// keep each at kChunk pairs and kListCap entries.  Pair i of the block (longest list first) goes to chunk
+// i % nc, so every chunk gets the same mix of list lengths; of the pairs of one length a chunk can get one more
+// than its even share, kListSlack entries in all, which the entry limit leaves free.
+__device__ __forceinline__ int chunks_of(int n, int e) {
+    if (n == 0) return 0;
+    const int by_pairs = (n + kChunk - 1) / kChunk;
+    const int by_entries = (e + (kListCap - kListSlack) - 1) / (kListCap - kListSlack);
+    return max(1, max(by_pairs, by_entries));
+}
+// how many of the ranks 0 .. x - 1 go to chunk j of nc
+__device__ __forceinline__ int ranks_of_chunk(int x, int j, int nc) { return (x - j + nc - 1) / nc; }
 
 // One wave per bin: the counts of the workgroups become their exclusive prefix, the sum goes to total[bin].
 __global__ __launch_bounds__(kSortThreads) void k_tl_binscan(uint32_t* __restrict__ hist, uint32_t* __restrict__ total,
@@ -200,13 +221,17 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
                                                            const uint32_t* __restrict__ hist,
                                                            const uint32_t* __restrict__ total,
                                                            uint16_t* __restrict__ lists,
-                                                           uint32_t* __restrict__ pidcnt, Chunk* __restrict__ chunks,
+                                                           uint32_t* __restrict__ pidcnt, uint16_t* __restrict__ loff,
+                                                           Chunk* __restrict__ chunks,
                                                            uint32_t* __restrict__ sched, int B, int K, int R,
                                                            int nblocks, int nbins, int vec) {
-    __shared__ uint32_t cursor[kBins];
+    __shared__ uint32_t cursor[kBins];      // next slot of this workgroup in every bin
+    __shared__ uint32_t bin_base[kBins];    // first slot of every bin
+    __shared__ uint32_t chunk_pool8[kMaxChunks];   // where a chunk's lists begin, in units of 8 entries
     __shared__ uint32_t wave_tot[kSortThreads / 64];
-    __shared__ uint32_t blk_start[kMaxBlocks + 1];
-    __shared__ uint32_t blk_base[kMaxBlocks + 1];   // first slot of the block's chunks; [nblocks] = chunks in all
+    __shared__ uint32_t blk_nc[kMaxBlocks], blk_e8[kMaxBlocks];
+    __shared__ uint32_t blk_chunk0[kMaxBlocks + 1];   // chunks before the block; [nblocks] = chunks in all
+    __shared__ uint32_t blk_pool8[kMaxBlocks + 1];    // list entries / 8 before the block
     const int tid = threadIdx.x;
     const int n = blockIdx.x * kSortThreads + tid;
     const int ngroups = gridDim.x;
@@ -236,44 +261,81 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
         for (int u = 0; u < PER; ++u) {
             const int i = tid * PER + u;
             if (i < nbins) {
-                if (i % kLenBins == 0) blk_start[i / kLenBins] = run;
+                bin_base[i] = run;
                 cursor[i] = run + hist[(size_t)i * ngroups + blockIdx.x];
             }
             run += v[u];
         }
     }
     __syncthreads();
-    if (tid == 0) {
-        uint32_t nchunks = 0;
-        for (int b = 0; b < nblocks; ++b) {
-            blk_base[b] = blk_start[b] + nchunks;
-            nchunks += (uint32_t)chunks_of((int)(blk_start[b + 1] - blk_start[b]));
-        }
-        blk_base[nblocks] = nchunks;
+    // bin (b, k) holds the lists of block b with kSlots - k entries; bin_base[nbins - 1] is the end of the last block
+    if (tid < nblocks) {
+        const uint32_t* bb = bin_base + tid * kLenBins;
+        int e = 0;
+        for (int k = 0; k < kLenBins; ++k) e += (int)(bb[k + 1] - bb[k]) * padded(kSlots - k);
+        blk_e8[tid] = (uint32_t)(e >> 3);
+        blk_nc[tid] = (uint32_t)chunks_of((int)(bb[kLenBins] - bb[0]), e);
     }
     __syncthreads();
-    if (blockIdx.x == 0) {
-        // the chunk table, the number of chunks and the unit counters of the gather
-        for (int b = tid; b < nblocks; b += kSortThreads) {
-            const int nb = (int)(blk_start[b + 1] - blk_start[b]);
-            const int nc = chunks_of(nb);
-            const int len = nc ? (nb + nc - 1) / nc : 0;
-            const int first = (int)(blk_base[b] - blk_start[b]);
-            for (int j = 0; j < nc; ++j)
-                chunks[first + j] = Chunk{b, (int)blk_base[b] + j * len, (nb - j + nc - 1) / nc, 0};
+    if (tid == 0) {
+        uint32_t c = 0, p8 = 0;
+        for (int b = 0; b < nblocks; ++b) {
+            blk_chunk0[b] = c;
+            blk_pool8[b] = p8;
+            c += blk_nc[b];
+            p8 += blk_e8[b];
         }
-        if (tid <= kXcd) sched[tid * 32] = tid == kXcd ? blk_base[nblocks] : 0u;
+        blk_chunk0[nblocks] = c;
+        blk_pool8[nblocks] = p8;
     }
+    __syncthreads();
+    // where the lists of every chunk begin (and, by the first workgroup, the chunk table)
+    if (tid < nblocks) {
+        const uint32_t* bb = bin_base + tid * kLenBins;
+        const int nb = (int)(bb[kLenBins] - bb[0]);
+        const int nc = (int)blk_nc[tid];
+        const int len = nc ? (nb + nc - 1) / nc : 0;
+        uint32_t p8 = blk_pool8[tid];
+        for (int j = 0; j < nc; ++j) {
+            int e = 0;
+            for (int k = 0; k < kLenBins; ++k) {
+                const int r0 = (int)(bb[k] - bb[0]), r1 = (int)(bb[k + 1] - bb[0]);
+                e += (ranks_of_chunk(r1, j, nc) - ranks_of_chunk(r0, j, nc)) * padded(kSlots - k);
+            }
+            const uint32_t ci = blk_chunk0[tid] + (uint32_t)j;
+            if (ci < (uint32_t)kMaxChunks) chunk_pool8[ci] = p8;
+            if (blockIdx.x == 0)
+                chunks[ci] = Chunk{tid, (int)(bb[0] + blk_chunk0[tid]) + j * len, ranks_of_chunk(nb, j, nc), (int)p8,
+                                   e >> 3, 0, 0, 0};
+            p8 += (uint32_t)(e >> 3);
+        }
+    }
+    if (blockIdx.x == 0 && tid <= kXcd) sched[tid * 32] = tid == kXcd ? blk_chunk0[nblocks] : 0u;
+    __syncthreads();
     if (n >= 2 * B) return;
     const ListRegs l = load_list(pair_list(widx, bidx, n, B, K), K, vec);
     const ListFacts f = list_facts(l, R);
-    const uint32_t slot = atomicAdd(&cursor[sort_key(f)], 1u);
-    const int nb = (int)(blk_start[f.block + 1] - blk_start[f.block]);
-    const int nc = chunks_of(nb);
+    const int bin = sort_key(f);
+    const uint32_t slot = atomicAdd(&cursor[bin], 1u);
+    const uint32_t* bb = bin_base + f.block * kLenBins;
+    const int nb = (int)(bb[kLenBins] - bb[0]);
+    const int nc = (int)blk_nc[f.block];
     const int len = (nb + nc - 1) / nc;
-    const int i = (int)(slot - blk_start[f.block]);
-    const size_t dst = (size_t)blk_base[f.block] + (size_t)(i % nc) * len + i / nc;
+    const int i = (int)(slot - bb[0]);       // rank inside the block, longest lists first
+    const int j = i % nc;
+    const size_t dst = (size_t)(bb[0] + blk_chunk0[f.block]) + (size_t)j * len + i / nc;
     pidcnt[dst] = (uint32_t)n | ((f.foreign ? kForeign : (uint32_t)f.cnt) << 26);
+    // the list's place among its chunk's lists: behind the chunk's longer lists and its earlier ones of this length
+    int off = 0;
+    const int kbin = bin - f.block * kLenBins;
+    for (int k = 0; k < kbin; ++k) {
+        const int r0 = (int)(bb[k] - bb[0]), r1 = (int)(bb[k + 1] - bb[0]);
+        off += (ranks_of_chunk(r1, j, nc) - ranks_of_chunk(r0, j, nc)) * padded(kSlots - k);
+    }
+    const int pad = padded(f.cnt);
+    off += (i / nc - ranks_of_chunk((int)(bb[kbin] - bb[0]), j, nc)) * pad;
+    loff[dst] = (uint16_t)(off >> 3);
+    const uint32_t ci = blk_chunk0[f.block] + (uint32_t)j;
     // row numbers inside the block, valid entries first in slot order, the rest name the row of zeros
     uint32_t w[kSlots / 2];
     const int base = f.block * kRows;
@@ -306,9 +368,11 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
             }
         }
     }
-    u4* out = reinterpret_cast<u4*>(lists + dst * kSlots);
+    if (ci >= (uint32_t)kMaxChunks) return;   // (the launcher takes this path only when the table is long enough)
+    u4* out = reinterpret_cast<u4*>(lists + ((size_t)chunk_pool8[ci] << 3) + off);
 #pragma unroll
-    for (int q = 0; q < kSlots / 8; ++q) out[q] = u4{w[4 * q], w[4 * q + 1], w[4 * q + 2], w[4 * q + 3]};
+    for (int q = 0; q < kSlots / 8; ++q)
+        if (q * 8 < pad) out[q] = u4{w[4 * q], w[4 * q + 1], w[4 * q + 2], w[4 * q + 3]};
 }
 
 // (16-bit half of w) * bytes per tile row + off: the LDS address of a lane's piece of a row, one instruction.
@@ -355,6 +419,7 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                                                           const int32_t* __restrict__ bidx,
                                                           const uint16_t* __restrict__ lists,
                                                           const uint32_t* __restrict__ pidcnt,
+                                                          const uint16_t* __restrict__ loff,
                                                           const Chunk* __restrict__ chunks,
                                                           uint32_t* __restrict__ sched, const float* __restrict__ W,
                                                           float* __restrict__ acc, int B, int K, int R, int L1,
@@ -362,9 +427,10 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                                                           VirtualTable vt) {
     extern __shared__ float4 lds_raw[];
     char* tb = reinterpret_cast<char*>(lds_raw);
-    u4* moff = reinterpret_cast<u4*>(tb + kTileBytes);                                   // kChunk * 4
-    uint32_t* mpid = reinterpret_cast<uint32_t*>(tb + kTileBytes + kChunk * kSlots * 2);  // kChunk
-    uint32_t* ctr = mpid + kChunk;       // [0] task counter, [1] the unit this workgroup works on next
+    u4* lst = reinterpret_cast<u4*>(tb + kTileBytes);                                         // (kListCap + 32) * 2 bytes
+    uint32_t* mpid = reinterpret_cast<uint32_t*>(tb + kTileBytes + (kListCap + 32) * 2);      // kChunk
+    uint16_t* moff = reinterpret_cast<uint16_t*>(mpid + kChunk);                              // kChunk
+    uint32_t* ctr = reinterpret_cast<uint32_t*>(moff + kChunk);   // [0] task counter, [1] the unit this workgroup works on next
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     constexpr int N4 = kRows * (kRowBytes / 16);
@@ -372,7 +438,9 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
     constexpr int IT = N4 / NT;
     const int x = blockIdx.x % kXcd;
     const int ntiles = L1 / kTileCols;
-    const int groups = (tiles_per_xcd + tile_group - 1) / tile_group;
+    // the column tiles of this XCD, in groups of tile_group; a unit = (chunk, group)
+    const int my_tiles = max(0, min(tiles_per_xcd, ntiles - x * tiles_per_xcd));
+    const int groups = (my_tiles + tile_group - 1) / tile_group;
     const int nunits = (int)sched[kXcd * 32] * groups;
     uint32_t* unit_ctr = sched + x * 32;
     const int g = lane >> 3, j = lane & 7;
@@ -382,43 +450,71 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
 
     f4 v[IT];
     f4 vv[VIRT ? IT : 1];
-    while (true) {
-        __syncthreads();   // the previous unit is done with the lists and the tile; ctr[1] is written
-        const int unit = (int)ctr[1];
-        if (unit >= nunits) break;
-        const int ch = unit / groups;
-        const int tg = unit - ch * groups;
-        const Chunk C = chunks[ch];
-        const int q0 = tg * tile_group;
-        int q1 = min(q0 + tile_group, tiles_per_xcd);
-        q1 = min(q1, ntiles - x * tiles_per_xcd);
-        const int row0 = C.block * kRows;
-        const float* wb = W + (size_t)row0 * out_cols;
-        const int rows_here = min(kRows, R - row0);
-        const int ntasks = (C.count + 7) >> 3;
-        __syncthreads();   // everyone has read ctr[1]
+#define NNUEFT_UNIT(u_, C_, q0_, q1_)                       \
+    {                                                       \
+        const int ch_ = (u_) / groups;                      \
+        C_ = chunks[ch_];                                   \
+        q0_ = ((u_) - ch_ * groups) * tile_group;           \
+        q1_ = min(q0_ + tile_group, my_tiles);              \
+    }
+#define NNUEFT_LOAD_TILE(blk_, c_)                                                                       \
+    {                                                                                                    \
+        const int row0_ = (blk_) * kRows;                                                                \
+        const int rows_here_ = min(kRows, R - row0_);                                                    \
+        const float* src = W + (size_t)row0_ * out_cols + (c_) * kTileCols;                              \
+        _Pragma("unroll") for (int i = 0; i < IT; ++i) {                                                 \
+            const int f = tid + i * NT;                                                                  \
+            const int row = f >> 3;                                                                      \
+            v[i] = row < rows_here_                                                                      \
+                       ? *reinterpret_cast<const f4*>(src + (size_t)row * out_cols + (f & 7) * 4)        \
+                       : f4{0.f, 0.f, 0.f, 0.f};                                                         \
+            if (VIRT)                                                                                    \
+                vv[i] = row < rows_here_ ? *reinterpret_cast<const f4*>(vt.V + (size_t)row * out_cols +  \
+                                                                        (c_) * kTileCols + (f & 7) * 4)  \
+                                         : f4{0.f, 0.f, 0.f, 0.f};                                       \
+        }                                                                                                \
+    }
+    __syncthreads();
+    int unit = __builtin_amdgcn_readfirstlane((int)ctr[1]);
+    Chunk C{};
+    int q0 = 0, q1 = 0;
+    if (unit < nunits) {
+        NNUEFT_UNIT(unit, C, q0, q1)
+        NNUEFT_LOAD_TILE(C.block, x * tiles_per_xcd + q0)
+    }
+    // Entering an iteration the first tile of the unit is on its way into v: the last tile of a unit fetches
+    // the first one of the next.
+    while (unit < nunits) {
+        __syncthreads();   // the previous unit is done with the lists and the tile, and everyone has read ctr[1]
         if (tid == 0) ctr[1] = atomicAdd(unit_ctr, 1u);
         {
-            const u4* ms = reinterpret_cast<const u4*>(lists + (size_t)C.start * kSlots);
-            for (int f = tid; f < C.count * 4; f += NT) moff[f] = ms[f];
-            for (int f = tid; f < C.count; f += NT) mpid[f] = pidcnt[C.start + f];
+            constexpr int LI = ((kListCap + 32) / 8 + NT - 1) / NT;
+            constexpr int PI = (kChunk + NT - 1) / NT;
+            const u4* ms = reinterpret_cast<const u4*>(lists + ((size_t)C.pool8 << 3));
+            u4 t[LI];
+            uint32_t tp[PI];
+            uint16_t to[PI];
+#pragma unroll
+            for (int i = 0; i < LI; ++i) t[i] = tid + i * NT < C.n8 ? ms[tid + i * NT] : u4{0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int i = 0; i < PI; ++i) {
+                tp[i] = tid + i * NT < C.count ? pidcnt[C.start + tid + i * NT] : 0u;
+                to[i] = tid + i * NT < C.count ? loff[C.start + tid + i * NT] : (uint16_t)0;
+            }
+#pragma unroll
+            for (int i = 0; i < LI; ++i)
+                if (tid + i * NT < C.n8) lst[tid + i * NT] = t[i];
+#pragma unroll
+            for (int i = 0; i < PI; ++i)
+                if (tid + i * NT < C.count) {
+                    mpid[tid + i * NT] = tp[i];
+                    moff[tid + i * NT] = to[i];
+                }
         }
-#define NNUEFT_LOAD_TILE(c_)                                                                          \
-    {                                                                                                 \
-        const float* src = wb + (c_) * kTileCols;                                                     \
-        _Pragma("unroll") for (int i = 0; i < IT; ++i) {                                              \
-            const int f = tid + i * NT;                                                               \
-            const int row = f >> 3;                                                                   \
-            v[i] = row < rows_here                                                                    \
-                       ? *reinterpret_cast<const f4*>(src + (size_t)row * out_cols + (f & 7) * 4)     \
-                       : f4{0.f, 0.f, 0.f, 0.f};                                                      \
-            if (VIRT)                                                                                 \
-                vv[i] = row < rows_here ? *reinterpret_cast<const f4*>(vt.V + (size_t)row * out_cols + \
-                                                                       (c_) * kTileCols + (f & 7) * 4) \
-                                        : f4{0.f, 0.f, 0.f, 0.f};                                     \
-        }                                                                                             \
-    }
-        if (q0 < q1) NNUEFT_LOAD_TILE(x * tiles_per_xcd + q0)
+        const int ntasks = (C.count + 7) >> 3;
+        int nunit = nunits;
+        Chunk Cn{};
+        int qn0 = 0, qn1 = 0;
         for (int q = q0; q < q1; ++q) {
             const int c = x * tiles_per_xcd + q;
             if (q != q0) __syncthreads();   // everyone is done reading the previous tile
@@ -429,7 +525,15 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
             }
             if (tid == 0) ctr[0] = 0;
             __syncthreads();
-            if (q + 1 < q1) NNUEFT_LOAD_TILE(c + 1)
+            if (q == q0) {
+                nunit = __builtin_amdgcn_readfirstlane((int)ctr[1]);
+                if (nunit < nunits) NNUEFT_UNIT(nunit, Cn, qn0, qn1)
+            }
+            if (q + 1 < q1) {
+                NNUEFT_LOAD_TILE(C.block, c + 1)
+            } else if (nunit < nunits) {
+                NNUEFT_LOAD_TILE(Cn.block, x * tiles_per_xcd + qn0)
+            }
             int task = 0;
             if (lane == 0) task = (int)atomicAdd(ctr, 1u);
             task = __builtin_amdgcn_readfirstlane(task);
@@ -458,10 +562,15 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                         }
                     }
                 } else {
+                    // the pair's own list is padded to a multiple of 8 entries; what the longest list of the
+                    // task has beyond that names the row of zeros
                     uint32_t oo[kSlots / 2];
+                    const int own = padded((int)field);
+                    const u4* lp = lst + moff[s];
+                    constexpr uint32_t zz = (uint32_t)kRows | ((uint32_t)kRows << 16);
 #pragma unroll
                     for (int i = 0; i < kSlots / 8; ++i) {
-                        const u4 t = moff[s * 4 + i];
+                        const u4 t = i * 8 < own ? lp[i] : u4{zz, zz, zz, zz};
                         oo[4 * i] = t.x; oo[4 * i + 1] = t.y; oo[4 * i + 2] = t.z; oo[4 * i + 3] = t.w;
                     }
                     // blocks of four slots, the next block's reads issued before the current block's adds
@@ -486,7 +595,13 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                 task = __builtin_amdgcn_readfirstlane(nxt);
             }
         }
+        unit = nunit;
+        C = Cn;
+        q0 = qn0;
+        q1 = qn1;
     }
+#undef NNUEFT_UNIT
+#undef NNUEFT_LOAD_TILE
 }
 
 // The gather may ask for most of a CU's LDS; that permission belongs to the loaded kernel on a device
@@ -523,6 +638,7 @@ int double_fwd_tile(const float* us, const float* them, const int32_t* widx, con
     uint32_t* hist = (uint32_t*)(base + L.hist);
     uint16_t* lists = (uint16_t*)(base + L.lists);
     uint32_t* pidcnt = (uint32_t*)(base + L.pidcnt);
+    uint16_t* loff = (uint16_t*)(base + L.loff);
     Chunk* chunks = (Chunk*)(base + L.chunks);
     uint32_t* sched = (uint32_t*)(base + L.sched);
     uint32_t* total = (uint32_t*)(base + L.total);
@@ -533,24 +649,26 @@ int double_fwd_tile(const float* us, const float* them, const int32_t* widx, con
                        total, L.nbins, L.ngroups);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_tl_lists, dim3(L.ngroups), dim3(kSortThreads), 0, st, widx, bidx, hist, total, lists, pidcnt,
-                       chunks, sched, B, K, R, L.nblocks, L.nbins, vec);
+                       loff, chunks, sched, B, K, R, L.nblocks, L.nbins, vec);
     NNUEFT_LAUNCH_CHECK();
     const int out_cols = L1 + n_psqt;
     const int ntiles = L1 / kTileCols;
     const int tiles_per_xcd = (ntiles + kXcd - 1) / kXcd;
-    int tile_group = tiles_per_xcd < 6 ? tiles_per_xcd : 6;
+    // about three tiles per visit of a chunk: its lists are copied into LDS once per visit, and a batch is
+    // cut into enough units for the CUs of an XCD to finish together
+    int tile_group = (tiles_per_xcd + (tiles_per_xcd + 2) / 3 - 1) / ((tiles_per_xcd + 2) / 3);
 #ifdef NNUEFT_TUNE_ENV
     if (const char* e = getenv("NNUEFT_TILE_GROUP")) tile_group = atoi(e) > 0 ? atoi(e) : tile_group;
 #endif
     const int grid = info->cus / kXcd * kXcd;
     if (vt.V)
         hipLaunchKernelGGL((k_acc_tile<kAccThreadsVirtual, true>), dim3(grid), dim3(kAccThreadsVirtual), kLdsBytes, st,
-                           widx, bidx, lists, pidcnt, chunks, sched, W, saved, B, K, R, L1, out_cols, tiles_per_xcd,
+                           widx, bidx, lists, pidcnt, loff, chunks, sched, W, saved, B, K, R, L1, out_cols, tiles_per_xcd,
                            tile_group, vt);
     else
         hipLaunchKernelGGL((k_acc_tile<kAccThreads, false>), dim3(grid), dim3(kAccThreads), kLdsBytes, st, widx, bidx,
-                           lists, pidcnt, chunks, sched, W, saved, B, K, R, L1, out_cols, tiles_per_xcd, tile_group,
-                           vt);
+                           lists, pidcnt, loff, chunks, sched, W, saved, B, K, R, L1, out_cols, tiles_per_xcd,
+                           tile_group, vt);
     NNUEFT_LAUNCH_CHECK();
     return nnueft_blocked::launch_mix(us, them, widx, bidx, psqt_idx, W, bias, saved, max_act, l0, wpsqt, bpsqt, B,
                                       K, R, L1, n_psqt, st, act, vt);
