@@ -227,7 +227,10 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
                                                            int nblocks, int nbins, int vec) {
     __shared__ uint32_t cursor[kBins];      // next slot of this workgroup in every bin
     __shared__ uint32_t bin_base[kBins];    // first slot of every bin
+    __shared__ uint32_t bin_eoff[kBins];    // list entries of its block before the bin's lists
     __shared__ uint32_t chunk_pool8[kMaxChunks];   // where a chunk's lists begin, in units of 8 entries
+    __shared__ uint32_t ck_start[kMaxChunks];      // the chunk table before it is put in order (first workgroup)
+    __shared__ uint16_t ck_block[kMaxChunks], ck_count[kMaxChunks], ck_n8[kMaxChunks];
     __shared__ uint32_t wave_tot[kSortThreads / 64];
     __shared__ uint32_t blk_nc[kMaxBlocks], blk_e8[kMaxBlocks];
     __shared__ uint32_t blk_chunk0[kMaxBlocks + 1];   // chunks before the block; [nblocks] = chunks in all
@@ -272,7 +275,10 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
     if (tid < nblocks) {
         const uint32_t* bb = bin_base + tid * kLenBins;
         int e = 0;
-        for (int k = 0; k < kLenBins; ++k) e += (int)(bb[k + 1] - bb[k]) * padded(kSlots - k);
+        for (int k = 0; k < kLenBins; ++k) {
+            bin_eoff[tid * kLenBins + k] = (uint32_t)e;   // entries of the block's longer lists
+            e += (int)(bb[k + 1] - bb[k]) * padded(kSlots - k);
+        }
         blk_e8[tid] = (uint32_t)(e >> 3);
         blk_nc[tid] = (uint32_t)chunks_of((int)(bb[kLenBins] - bb[0]), e);
     }
@@ -304,14 +310,32 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
             }
             const uint32_t ci = blk_chunk0[tid] + (uint32_t)j;
             if (ci < (uint32_t)kMaxChunks) chunk_pool8[ci] = p8;
-            if (blockIdx.x == 0)
-                chunks[ci] = Chunk{tid, (int)(bb[0] + blk_chunk0[tid]) + j * len, ranks_of_chunk(nb, j, nc), (int)p8,
-                                   e >> 3, 0, 0, 0};
+            if (blockIdx.x == 0 && ci < (uint32_t)kMaxChunks) {
+                ck_block[ci] = (uint16_t)tid;
+                ck_start[ci] = (bb[0] + blk_chunk0[tid]) + (uint32_t)(j * len);
+                ck_count[ci] = (uint16_t)ranks_of_chunk(nb, j, nc);
+                ck_n8[ci] = (uint16_t)(e >> 3);
+            }
             p8 += (uint32_t)(e >> 3);
         }
     }
     if (blockIdx.x == 0 && tid <= kXcd) sched[tid * 32] = tid == kXcd ? blk_chunk0[nblocks] : 0u;
     __syncthreads();
+    // The chunk table, longest lists first: the gather hands units out in table order, and the CUs of an XCD
+    // finish closer together when the small units come last.
+    if (blockIdx.x == 0) {
+        const int nch = min((int)blk_chunk0[nblocks], kMaxChunks);
+        for (int ci = tid; ci < nch; ci += kSortThreads) {
+            const uint32_t mine = ck_n8[ci];
+            int rank = 0;
+            for (int k = 0; k < nch; ++k) {
+                const uint32_t other = ck_n8[k];
+                rank += other > mine || (other == mine && k < ci);
+            }
+            chunks[rank] = Chunk{(int)ck_block[ci], (int)ck_start[ci], (int)ck_count[ci], (int)chunk_pool8[ci],
+                                 (int)ck_n8[ci], 0, 0, 0};
+        }
+    }
     if (n >= 2 * B) return;
     const ListRegs l = load_list(pair_list(widx, bidx, n, B, K), K, vec);
     const ListFacts f = list_facts(l, R);
@@ -328,12 +352,16 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
     // the list's place among its chunk's lists: behind the chunk's longer lists and its earlier ones of this length
     int off = 0;
     const int kbin = bin - f.block * kLenBins;
-    for (int k = 0; k < kbin; ++k) {
-        const int r0 = (int)(bb[k] - bb[0]), r1 = (int)(bb[k + 1] - bb[0]);
-        off += (ranks_of_chunk(r1, j, nc) - ranks_of_chunk(r0, j, nc)) * padded(kSlots - k);
-    }
     const int pad = padded(f.cnt);
-    off += (i / nc - ranks_of_chunk((int)(bb[kbin] - bb[0]), j, nc)) * pad;
+    if (nc == 1) {
+        off = (int)bin_eoff[bin] + (i - (int)(bb[kbin] - bb[0])) * pad;
+    } else {
+        for (int k = 0; k < kbin; ++k) {
+            const int r0 = (int)(bb[k] - bb[0]), r1 = (int)(bb[k + 1] - bb[0]);
+            off += (ranks_of_chunk(r1, j, nc) - ranks_of_chunk(r0, j, nc)) * padded(kSlots - k);
+        }
+        off += (i / nc - ranks_of_chunk((int)(bb[kbin] - bb[0]), j, nc)) * pad;
+    }
     loff[dst] = (uint16_t)(off >> 3);
     const uint32_t ci = blk_chunk0[f.block] + (uint32_t)j;
     // row numbers inside the block, valid entries first in slot order, the rest name the row of zeros
@@ -386,6 +414,10 @@ __device__ __forceinline__ uint32_t row_addr(uint32_t w, uint32_t off) {
         asm("v_mad_u32_u16 %0, %1, %2, %3 op_sel:[0,0,0,0]" : "=v"(r) : "v"(w), "s"(stride), "v"(off));
     return r;
 }
+
+// 16 bytes of LDS at a byte address that already holds the tile's place in LDS (no add of the base per read).
+typedef __attribute__((address_space(3))) const f4 lds_f4;
+__device__ __forceinline__ f4 lds_read16(uint32_t addr) { return *reinterpret_cast<lds_f4*>(addr); }
 
 // round(x * scale) / scale with round-half-to-even, as torch's mul / round / div (the table merge's grid)
 __device__ __forceinline__ float fq(float x, float scale) { return rintf(x * scale) / scale; }
@@ -444,7 +476,8 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
     const int nunits = (int)sched[kXcd * 32] * groups;
     uint32_t* unit_ctr = sched + x * 32;
     const int g = lane >> 3, j = lane & 7;
-    const uint32_t lane_off = j * 16;
+    // low half of a flat LDS address = the byte address inside LDS
+    const uint32_t lane_off = (uint32_t)(uintptr_t)tb + j * 16;
     if (tid < kRowBytes / 16) reinterpret_cast<f4*>(tb)[kRows * (kRowBytes / 16) + tid] = f4{0.f, 0.f, 0.f, 0.f};
     if (tid == 0) ctr[1] = atomicAdd(unit_ctr, 1u);
 
@@ -576,10 +609,10 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                     // blocks of four slots, the next block's reads issued before the current block's adds
                     f4 r[2][4];
 #define NNUEFT_ISSUE(buf_, i_)                                                                   \
-    r[buf_][0] = *reinterpret_cast<const f4*>(tb + row_addr<0>(oo[2 * (i_)], lane_off));          \
-    r[buf_][1] = *reinterpret_cast<const f4*>(tb + row_addr<1>(oo[2 * (i_)], lane_off));          \
-    r[buf_][2] = *reinterpret_cast<const f4*>(tb + row_addr<0>(oo[2 * (i_) + 1], lane_off));      \
-    r[buf_][3] = *reinterpret_cast<const f4*>(tb + row_addr<1>(oo[2 * (i_) + 1], lane_off));
+    r[buf_][0] = lds_read16(row_addr<0>(oo[2 * (i_)], lane_off));          \
+    r[buf_][1] = lds_read16(row_addr<1>(oo[2 * (i_)], lane_off));          \
+    r[buf_][2] = lds_read16(row_addr<0>(oo[2 * (i_) + 1], lane_off));      \
+    r[buf_][3] = lds_read16(row_addr<1>(oo[2 * (i_) + 1], lane_off));
                     NNUEFT_ISSUE(0, 0)
 #pragma unroll
                     for (int i = 0; i < kSlots / 4; ++i) {

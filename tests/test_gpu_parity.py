@@ -133,7 +133,8 @@ DOUBLE_SHAPES = [
     (300, 512, 2000, 32, {}),                  # lists that leave their 768-row block (summed from global memory)
     (700, 544, 24576, 32, dict(halfka=True, weight_scale=0.05, max_act=255 / 256)),   # 17 tiles over 8 XCDs
     (1500, 512, 1000, 20, dict(allow_holes=True)),   # K < 32, holes, a last block of 232 rows
-    (2000, 576, 768, 32, dict(n_psqt=0)),      # one block, eight chunks of lists
+    (2000, 576, 768, 32, dict(n_psqt=0)),      # one block, five chunks (as many as hold its list entries)
+    (3500, 512, 768, 8, dict(n_psqt=0)),       # one block of short lists, five chunks (1536 pairs each at most)
 ]
 
 
