@@ -50,6 +50,13 @@ constexpr int kWavesPerXcd = NNUEFT_SEG_WAVES;  // persistent waves per XCD in t
 #define NNUEFT_LONG_ROW 256
 #endif
 constexpr int kLongRow = NNUEFT_LONG_ROW;  // table rows named by at least this many slots are reduced first
+#ifndef NNUEFT_FILL_U
+#define NNUEFT_FILL_U 8
+#endif
+#ifndef NNUEFT_FILL_THREADS
+#define NNUEFT_FILL_THREADS 1024
+#endif
+constexpr int kFillThreads = NNUEFT_FILL_THREADS;   // all of them load the cursors, one wave hands out the ranks
 #ifndef NNUEFT_RUN_U
 #define NNUEFT_RUN_U 16
 #endif
@@ -269,6 +276,8 @@ __global__ __launch_bounds__(256) void k_chunk_hist(const int32_t* __restrict__ 
                                                     const int32_t* __restrict__ bidx, uint32_t* __restrict__ cnt,
                                                     int B, int K, int R, int cpp, int range) {
     extern __shared__ uint32_t lds_u32[];
+    __shared__ uint32_t idle[64];
+    if (threadIdx.x < 64) idle[threadIdx.x] = 0;
     const int c = blockIdx.x;
     const int r0 = blockIdx.y * range;
     const int nr = min(range, R - r0);
@@ -536,11 +545,13 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
 // Every slot of the chunk writes its position id.  Ranks inside the chunk are handed out position
 // by position (one LDS atomic per position and slot group), so a row's list is in position order.
 // LDS: `range` cursors, then (when they fit) the chunk's index lists staged by all four waves.
-__global__ __launch_bounds__(256) void k_fill(const int32_t* __restrict__ widx, const int32_t* __restrict__ bidx,
+__global__ __launch_bounds__(kFillThreads) void k_fill(const int32_t* __restrict__ widx, const int32_t* __restrict__ bidx,
                                               const uint32_t* __restrict__ cnt,
                                               const uint32_t* __restrict__ seg_off, uint32_t* __restrict__ list,
                                               int B, int K, int R, int cpp, int range, int stage) {
     extern __shared__ uint32_t lds_u32[];
+    __shared__ uint32_t idle[64];
+    if (threadIdx.x < 64) idle[threadIdx.x] = 0;
     const int c = blockIdx.x;
     const int r0 = blockIdx.y * range;
     const int nr = min(range, R - r0);
@@ -551,16 +562,16 @@ __global__ __launch_bounds__(256) void k_fill(const int32_t* __restrict__ widx, 
     // every batch of loads, so the batches are made as large as registers allow: four rows per load
     // where the two arrays are 16-byte aligned, twelve loads of each array in flight per thread.
     if ((R & 3) == 0 && (r0 & 3) == 0 && (nr & 3) == 0) {
-        constexpr int PF = 12;
+        constexpr int PF = 6;
         const uint4* so4 = reinterpret_cast<const uint4*>(seg_off + r0);
         const uint4* co4 = reinterpret_cast<const uint4*>(coff);
         uint4* lds4 = reinterpret_cast<uint4*>(lds_u32);
         const int nr4 = nr >> 2;
-        for (int j0 = threadIdx.x; j0 < nr4; j0 += 256 * PF) {
+        for (int j0 = threadIdx.x; j0 < nr4; j0 += kFillThreads * PF) {
             uint4 a[PF], b[PF];
 #pragma unroll
             for (int u = 0; u < PF; ++u) {
-                const int j = j0 + u * 256;
+                const int j = j0 + u * kFillThreads;
                 if (j < nr4) {
                     a[u] = so4[j];
                     b[u] = co4[j];
@@ -568,34 +579,59 @@ __global__ __launch_bounds__(256) void k_fill(const int32_t* __restrict__ widx, 
             }
 #pragma unroll
             for (int u = 0; u < PF; ++u) {
-                const int j = j0 + u * 256;
+                const int j = j0 + u * kFillThreads;
                 if (j < nr4) lds4[j] = make_uint4(a[u].x + b[u].x, a[u].y + b[u].y, a[u].z + b[u].z, a[u].w + b[u].w);
             }
         }
     } else {
         constexpr int PF = 8;
-        for (int j0 = threadIdx.x; j0 < nr; j0 += 256 * PF) {
+        for (int j0 = threadIdx.x; j0 < nr; j0 += kFillThreads * PF) {
             uint32_t a[PF], b[PF];
 #pragma unroll
             for (int u = 0; u < PF; ++u) {
-                const int j = j0 + u * 256;
+                const int j = j0 + u * kFillThreads;
                 a[u] = j < nr ? seg_off[r0 + j] : 0;
                 b[u] = j < nr ? coff[j] : 0;
             }
 #pragma unroll
             for (int u = 0; u < PF; ++u) {
-                const int j = j0 + u * 256;
+                const int j = j0 + u * kFillThreads;
                 if (j < nr) lds_u32[j] = a[u] + b[u];
             }
         }
     }
     int32_t* staged = reinterpret_cast<int32_t*>(lds_u32 + range);
     if (stage)
-        for (int i = threadIdx.x; i < npos * K; i += 256) staged[i] = ix[i];
+        for (int i = threadIdx.x; i < npos * K; i += kFillThreads) staged[i] = ix[i];
     __syncthreads();
     if (threadIdx.x >= 64) return;
     const int lane = threadIdx.x;
     const uint32_t id0 = (uint32_t)p * (uint32_t)B + (uint32_t)pos0;
+    if (K <= 64) {
+        // One slot group per position.  LDS executes a wave's atomics in the order they were issued, so the ranks
+        // of four positions are asked for before the first is needed; a lane with nothing to add adds 0 to a word
+        // of its own, which keeps the four atomics free of branches.
+        constexpr int U = NNUEFT_FILL_U;
+        for (int i0 = 0; i0 < npos; i0 += U) {
+            uint32_t* at[U];
+            uint32_t one[U], slot[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int i = i0 + u;
+                int r = -1;
+                if (i < npos && lane < K) r = (stage ? staged[i * K + lane] : ix[(size_t)i * K + lane]) - r0;
+                const bool ok = r >= 0 && r < nr;
+                at[u] = ok ? &lds_u32[r] : &idle[lane];
+                one[u] = ok ? 1u : 0u;
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) slot[u] = atomicAdd(at[u], one[u]);
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (one[u]) list[slot[u]] = id0 + (uint32_t)(i0 + u);
+        }
+        return;
+    }
     // all slot groups of a position before the next position
     for (int i = 0; i < npos; ++i) {
         for (int k0 = 0; k0 < K; k0 += 64) {
@@ -951,7 +987,7 @@ int det_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, char
     hipLaunchKernelGGL(k_row_scan, dim3(1), dim3(kScanThreads), (size_t)scan_cap * sizeof(uint32_t), st, seg_off,
                        long_rows, sched, R, scan_cap, (uint32_t)L.row_split);
     NNUEFT_LAUNCH_CHECK();
-    hipLaunchKernelGGL(k_fill, dim3(L.nchunks, nranges), dim3(256), fill_bytes, st, widx, bidx, cnt, seg_off, list,
+    hipLaunchKernelGGL(k_fill, dim3(L.nchunks, nranges), dim3(kFillThreads), fill_bytes, st, widx, bidx, cnt, seg_off, list,
                        B, K, R, L.cpp, range, stage);
     NNUEFT_LAUNCH_CHECK();
     return 0;
