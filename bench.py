@@ -83,8 +83,9 @@ def compulsory_bytes(L1, B, sum_a):
     small = B * 24
     if forward_path(L1) == "tile":
         fwd = {
-            "list sort": 2 * lists + 2 * B * (64 + 4),                    # lists twice, 16-bit lists and pair ids written
-            "k_acc_tile": R_ROWS * oc * 4 + 2 * B * (64 + 4) + saved,     # table once, 16-bit lists, row sums written
+            # 16-bit lists at their own length, pair id and list place per list
+            "list sort": 2 * lists + sum_a * 2 + 2 * B * 6,               # lists twice, packed lists written
+            "k_acc_tile": R_ROWS * oc * 4 + sum_a * 2 + 2 * B * 6 + saved,   # table once, packed lists, row sums written
             "k_mix": saved + B * L1 * 4 + small,                          # row sums read, l0 written
         }
     else:

@@ -1,20 +1,22 @@
 // Forward, LDS-tiled variant: the gather reads the table out of LDS instead of through L2.
 //
 // All indices of one list name rows of a single 768-row block of the table (one king bucket).  A
-// workgroup keeps one tile of the table in LDS, 768 rows x 32 columns (96 KB), and the lists of up to
-// 512 (position, perspective) pairs of that block (32 KB, as 16-bit row numbers inside the block), and
+// workgroup keeps one tile of the table in LDS, 768 rows x 32 columns (96 KB), and the lists of a chunk
+// of that block's (position, perspective) pairs (up to 1536 pairs and 27 648 list entries, 55 KB, as
+// 16-bit row numbers inside the block, every list at its own length rounded up to 8 entries), and
 // sums the tile's columns for every pair: 8 lanes a pair, one 16-byte LDS read per row and lane, the
-// adds in slot order.  Every row of the table then crosses the CU's L1 once per chunk of pairs instead
-// of once per pair naming it (about 24 times in a batch of 16384 positions), which is what bounds the
-// gather through L2: a CU can only keep so many L1 misses pending.
+// adds in slot order.  Every row of the table then crosses the CU's L1 once per chunk of pairs (a whole
+// block at B = 16384) instead of once per pair naming it (about 24 times there), which is what bounds
+// the gather through L2: a CU can only keep so many L1 misses pending.
 //
 //   k_tl_hist     one pair per thread: key (block, list length) counted per workgroup
 //   k_tl_binscan  per key, the counts of the workgroups become their exclusive prefix
 //   k_tl_lists    pairs to their slots, longest lists first inside a block and dealt to the block's
-//                 chunks in turn; writes the 16-bit lists, pair ids and the chunk table
+//                 chunks in turn; writes the packed 16-bit lists, pair ids, list places and the chunk
+//                 table (longest chunks first)
 //   k_acc_tile    persistent workgroups, one per CU: units of (chunk, group of column tiles) handed out
-//                 per XCD; the tile for the next column group is fetched into registers while the
-//                 current one is summed; waves take tasks of 8 pairs from a counter in LDS
+//                 per XCD; the next tile (also the first one of the next unit) is fetched into registers
+//                 while the current one is summed; waves take tasks of 8 pairs from a counter in LDS
 //   k_mix         as in the L2-blocked path
 //
 // A list that names rows of more than one block (the interface allows it) is summed from global
