@@ -288,9 +288,11 @@ def run_int16(args, lib, dev):
     _, ms_chain = time_steps(chain, args.steps, args.warmup)
     gathered = sum_a * L1 * 2
     alg = gathered + B * (2 * K_SLOTS * 4 + L1)
-    # table once, lists by both kernels, white sums written and read, u8 out
-    comp = R * L1 * 2 + R * N_PSQT * 4 + 2 * B * K_SLOTS * 4 * 2 + 2 * B * L1 * 2 + B * L1
-    l2_peak = l2_peak_gbs()
+    # table once, lists read twice by the sort and once for the psqt sums, packed lists written and read, both
+    # lists' sums written and read, u8 out
+    comp = (R * L1 * 2 + R * N_PSQT * 4 + 3 * 2 * B * K_SLOTS * 4 + 2 * (sum_a * 2 + 2 * B * 6) + 2 * (2 * B * L1 * 2)
+            + B * L1)
+    lds_peak = LDS_PEAK_GBS
     gbs = alg / (ms * 1e-3) / 1e9
     print(json.dumps({
         "metric": "quantized FT forward positions/sec (int16 accumulate, L1=3072, B=65536)",
@@ -300,12 +302,14 @@ def run_int16(args, lib, dev):
         "config": {"workload": args.workload, "L1": L1, "batch": B, "table_rows": R,
                    "active_rows_per_position": sum_a / B,
                    "with_int8_layer_stacks_ms": ms_chain, "with_int8_layer_stacks_positions_per_s": B / (ms_chain * 1e-3)},
-        "roofline": {"kernel": "nnueft_ft_int16_fwd: k_acc16_white + k_black_mix16 (+ pair sort)", "bound": "l2",
-                     "achieved": gbs, "peak": l2_peak, "unit": "GB/s", "frac": gbs / l2_peak, "traffic": None,
+        "roofline": {"kernel": "nnueft_ft_int16_fwd: k_acc_tile over the int16 table (the gather out of LDS tiles) + "
+                               "k_mix16 + list sort", "bound": "lds",
+                     "achieved": gbs, "peak": lds_peak, "unit": "GB/s", "frac": gbs / lds_peak, "traffic": None,
                      "algorithmic_bytes_per_launch": alg, "avg_launch_ms": ms,
                      "achieved_over_hbm_peak": gbs / HBM_PEAK_GBS,
-                     "note": "the gathered rows are served from the per-XCD L2s (blocked gather), so the algorithmic "
-                             "rate is held against the L2 line rate; the HBM-side figure is roofline_compulsory"},
+                     "note": "the gathered rows are LDS reads (a tile of 704 rows x 64 int16 columns per workgroup), so "
+                             "the algorithmic rate is held against the LDS read rate; the HBM-side figure is "
+                             "roofline_compulsory"},
         "roofline_compulsory": {"bound": "hbm", "bytes_per_launch": comp, "achieved": comp / (ms * 1e-3) / 1e9,
                                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": comp / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
         "cpu_baseline": None,

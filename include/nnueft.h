@@ -299,10 +299,12 @@ int nnueft_table_virtual_grad(const float* gW, float* gV, int R, int cols, int v
  *   psqt_out[b] = (sum psqt32[idx_P(0), bucket] - sum psqt32[idx_P(1), bucket]) / 2     (C division)
  * stm u8[B]: 0 white to move, 1 black; W16 int16[R,L1]; b16 int16[L1]; psqt32 int32[R,n_psqt];
  * psqt_idx int64[B]; out_u8 u8[B,L1]; psqt_out int32[B].  clip_max*clip_max >> shift must fit 8 bits.
- * workspace: NULL, or nnueft_int16_workspace_bytes() bytes; with it (and L1 % 16 == 0) the gather is
- * blocked for the per-XCD L2 caches like nnueft_double_fwd's.  table_block_rows: rows of one block of
+ * workspace: NULL, or nnueft_int16_workspace_bytes() bytes (two int16 per position and column plus the list
+ * sort's scratch); with it the sums are gathered out of LDS tiles of the table like nnueft_double_fwd's
+ * (L1 % 64 == 0, at least 512 columns, lists of 32 slots at most, table blocks of 768 rows at most), or
+ * else (L1 % 16 == 0) blocked for the per-XCD L2 caches.  table_block_rows: rows of one block of
  * the table whose rows a list stays inside (704 for an exported HalfKAv2_hm net, 0 = 768); only a
- * scheduling hint.  Results do not depend on either.
+ * scheduling hint: a list that leaves its block is summed all the same.  Results do not depend on either.
  */
 size_t nnueft_int16_workspace_bytes(int B, int K, int R, int L1, int table_block_rows);
 int nnueft_ft_int16_fwd(const int32_t* widx, const int32_t* bidx, const uint8_t* stm,

@@ -71,13 +71,15 @@ __host__ __device__ __forceinline__ int padded(int cnt) { return (cnt + 7) & ~7;
 struct Layout {
     size_t hist, total, lists, pidcnt, loff, chunks, sched, end;
     int ngroups, nblocks, nbins, max_chunks, nslots;
+    int block_rows;   // rows of a table block (kRows, or fewer: the tile then keeps rows to spare)
 };
 
 static inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-bool layout(int B, int R, Layout* L) {
-    if (B <= 0 || R <= 0) return false;
-    L->nblocks = (R + kRows - 1) / kRows;
+bool layout(int B, int R, Layout* L, int block_rows = kRows) {
+    if (B <= 0 || R <= 0 || block_rows <= 0 || block_rows > kRows) return false;
+    L->block_rows = block_rows;
+    L->nblocks = (R + block_rows - 1) / block_rows;
     if (L->nblocks > kMaxBlocks) return false;
     L->nbins = L->nblocks * kLenBins + 1;   // + one empty bin: its offset is the end of the last block
     L->ngroups = (2 * B + kSortThreads - 1) / kSortThreads;
@@ -149,16 +151,19 @@ __device__ __forceinline__ ListRegs load_list(const int32_t* __restrict__ ix, in
     return l;
 }
 
-__device__ __forceinline__ ListFacts list_facts(const ListRegs& l, int R) {
+__device__ __forceinline__ ListFacts list_facts(const ListRegs& l, int R, int block_rows) {
     ListFacts f{0, 0, false};
-    int first = -1;
+    int first = -1, base = 0;
 #pragma unroll
     for (int k = 0; k < kSlots; ++k) {
         const int r = l.v[k];
         if (r >= 0 && r < R) {
-            const int b = r / kRows;
-            if (first < 0) first = b;
-            f.foreign |= b != first;
+            if (first < 0) {
+                // r / block_rows for r below 2^32 / block_rows, without the division
+                first = (int)__umulhi((uint32_t)r, 0xffffffffu / (uint32_t)block_rows + 1u);
+                base = first * block_rows;
+            }
+            f.foreign |= r < base || r >= base + block_rows;
             ++f.cnt;
         }
     }
@@ -171,13 +176,13 @@ __device__ __forceinline__ int sort_key(const ListFacts& f) { return f.block * k
 __global__ __launch_bounds__(kSortThreads) void k_tl_hist(const int32_t* __restrict__ widx,
                                                           const int32_t* __restrict__ bidx,
                                                           uint32_t* __restrict__ hist, int B, int K, int R,
-                                                          int nbins, int vec) {
+                                                          int nbins, int vec, int block_rows) {
     __shared__ uint32_t bins[kBins];
     const int tid = threadIdx.x;
     const int n = blockIdx.x * kSortThreads + tid;
     for (int i = tid; i < nbins; i += kSortThreads) bins[i] = 0;
     __syncthreads();
-    if (n < 2 * B) atomicAdd(&bins[sort_key(list_facts(load_list(pair_list(widx, bidx, n, B, K), K, vec), R))], 1u);
+    if (n < 2 * B) atomicAdd(&bins[sort_key(list_facts(load_list(pair_list(widx, bidx, n, B, K), K, vec), R, block_rows))], 1u);
     __syncthreads();
     for (int i = tid; i < nbins; i += kSortThreads) hist[(size_t)i * gridDim.x + blockIdx.x] = bins[i];
 }
@@ -226,7 +231,7 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
                                                            uint32_t* __restrict__ pidcnt, uint16_t* __restrict__ loff,
                                                            Chunk* __restrict__ chunks,
                                                            uint32_t* __restrict__ sched, int B, int K, int R,
-                                                           int nblocks, int nbins, int vec) {
+                                                           int nblocks, int nbins, int vec, int block_rows) {
     __shared__ uint32_t cursor[kBins];      // next slot of this workgroup in every bin
     __shared__ uint32_t bin_base[kBins];    // first slot of every bin
     __shared__ uint32_t bin_eoff[kBins];    // list entries of its block before the bin's lists
@@ -340,7 +345,7 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
     }
     if (n >= 2 * B) return;
     const ListRegs l = load_list(pair_list(widx, bidx, n, B, K), K, vec);
-    const ListFacts f = list_facts(l, R);
+    const ListFacts f = list_facts(l, R, block_rows);
     const int bin = sort_key(f);
     const uint32_t slot = atomicAdd(&cursor[bin], 1u);
     const uint32_t* bb = bin_base + f.block * kLenBins;
@@ -368,7 +373,7 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
     const uint32_t ci = blk_chunk0[f.block] + (uint32_t)j;
     // row numbers inside the block, valid entries first in slot order, the rest name the row of zeros
     uint32_t w[kSlots / 2];
-    const int base = f.block * kRows;
+    const int base = f.block * block_rows;
     bool prefix = true;   // the valid entries are the first cnt slots (what a loader writes)
 #pragma unroll
     for (int k = 0; k < kSlots; ++k) prefix &= (k < f.cnt) == (l.v[k] >= 0 && l.v[k] < R);
@@ -445,10 +450,18 @@ __device__ __forceinline__ f4 merged4(f4 w, f4 v, const VirtualTable& vt) {
     return w;
 }
 
+// a += r: four floats, or (I16) eight 16-bit integers that wrap
+typedef unsigned short us8 __attribute__((ext_vector_type(8)));
+template <bool I16>
+__device__ __forceinline__ void acc_add(f4& a, const f4& r) {
+    if constexpr (I16) a = __builtin_bit_cast(f4, (us8)(__builtin_bit_cast(us8, a) + __builtin_bit_cast(us8, r)));
+    else a += r;
+}
+
 // saved[pair, columns of the tile] = chain from +0 over the pair's list, for every pair of the chunk.
 // VIRT: the table is W + V[row % kRows] (see merged4); the tile is merged on its way into LDS.  That variant
 // runs with 768 threads: the tile of V waits in registers beside the tile of W.
-template <int NT, bool VIRT>
+template <int NT, bool VIRT, bool I16>
 __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ widx,
                                                           const int32_t* __restrict__ bidx,
                                                           const uint16_t* __restrict__ lists,
@@ -458,7 +471,7 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                                                           uint32_t* __restrict__ sched, const float* __restrict__ W,
                                                           float* __restrict__ acc, int B, int K, int R, int L1,
                                                           int out_cols, int tiles_per_xcd, int tile_group,
-                                                          VirtualTable vt) {
+                                                          VirtualTable vt, int block_rows) {
     extern __shared__ float4 lds_raw[];
     char* tb = reinterpret_cast<char*>(lds_raw);
     u4* lst = reinterpret_cast<u4*>(tb + kTileBytes);                                         // (kListCap + 32) * 2 bytes
@@ -471,7 +484,12 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
     static_assert(N4 % NT == 0, "tile load");
     constexpr int IT = N4 / NT;
     const int x = blockIdx.x % kXcd;
-    const int ntiles = L1 / kTileCols;
+    // a tile row is 128 bytes: 32 floats, or 64 of the 16-bit weights of the quantized table (I16: a row of W is
+    // then L1 int16, a row of acc too, the sums wrap like 16-bit adds and their order does not matter)
+    const int ntiles = I16 ? L1 / (2 * kTileCols) : L1 / kTileCols;
+    const size_t w_pitch = I16 ? (size_t)L1 * 2 : (size_t)out_cols * 4;
+    const size_t a_pitch = I16 ? (size_t)L1 * 2 : (size_t)L1 * 4;
+    const char* Wb = reinterpret_cast<const char*>(W);
     // the column tiles of this XCD, in groups of tile_group; a unit = (chunk, group)
     const int my_tiles = max(0, min(tiles_per_xcd, ntiles - x * tiles_per_xcd));
     const int groups = (my_tiles + tile_group - 1) / tile_group;
@@ -494,14 +512,14 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
     }
 #define NNUEFT_LOAD_TILE(blk_, c_)                                                                       \
     {                                                                                                    \
-        const int row0_ = (blk_) * kRows;                                                                \
-        const int rows_here_ = min(kRows, R - row0_);                                                    \
-        const float* src = W + (size_t)row0_ * out_cols + (c_) * kTileCols;                              \
+        const int row0_ = (blk_) * block_rows;                                                           \
+        const int rows_here_ = min(block_rows, R - row0_);                                               \
+        const char* src = Wb + (size_t)row0_ * w_pitch + (c_) * kRowBytes;                               \
         _Pragma("unroll") for (int i = 0; i < IT; ++i) {                                                 \
             const int f = tid + i * NT;                                                                  \
             const int row = f >> 3;                                                                      \
             v[i] = row < rows_here_                                                                      \
-                       ? *reinterpret_cast<const f4*>(src + (size_t)row * out_cols + (f & 7) * 4)        \
+                       ? *reinterpret_cast<const f4*>(src + (size_t)row * w_pitch + (f & 7) * 16)        \
                        : f4{0.f, 0.f, 0.f, 0.f};                                                         \
             if (VIRT)                                                                                    \
                 vv[i] = row < rows_here_ ? *reinterpret_cast<const f4*>(vt.V + (size_t)row * out_cols +  \
@@ -589,11 +607,11 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                     for (int k = 0; k < K; ++k) {
                         const int r = ix[k];
                         if (r >= 0 && r < R) {
-                            f4 w = *reinterpret_cast<const f4*>(W + (size_t)r * out_cols + c * kTileCols + j * 4);
+                            f4 w = *reinterpret_cast<const f4*>(Wb + (size_t)r * w_pitch + c * kRowBytes + j * 16);
                             if (VIRT)
                                 w = merged4(w, *reinterpret_cast<const f4*>(vt.V + (size_t)(r % kRows) * out_cols +
                                                                             c * kTileCols + j * 4), vt);
-                            a += w;
+                            acc_add<I16>(a, w);
                         }
                     }
                 } else {
@@ -621,12 +639,13 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                         if (i * 4 < mx) {
                             if ((i + 1) * 4 < mx) { NNUEFT_ISSUE((i + 1) & 1, (i + 1) & 7) }
 #pragma unroll
-                            for (int h = 0; h < 4; ++h) a += r[i & 1][h];
+                            for (int h = 0; h < 4; ++h) acc_add<I16>(a, r[i & 1][h]);
                         }
                     }
                 }
                 if (valid)
-                    __builtin_nontemporal_store(a, reinterpret_cast<f4*>(acc + (size_t)pair * L1 + c * kTileCols + j * 4));
+                    __builtin_nontemporal_store(a, reinterpret_cast<f4*>(reinterpret_cast<char*>(acc) + (size_t)pair * a_pitch +
+                                                                         c * kRowBytes + j * 16));
                 task = __builtin_amdgcn_readfirstlane(nxt);
             }
         }
@@ -647,22 +666,25 @@ std::atomic<int> g_lds_allowed[kMaxDevices];
 int allow_lds(int device) {
     if (device < 0 || device >= kMaxDevices) return NNUEFT_E_UNSUPPORTED;
     if (g_lds_allowed[device].load(std::memory_order_acquire)) return 0;
-    hipError_t e = hipFuncSetAttribute((const void*)k_acc_tile<kAccThreads, false>,
+    hipError_t e = hipFuncSetAttribute((const void*)k_acc_tile<kAccThreads, false, false>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
     if (e == hipSuccess)
-        e = hipFuncSetAttribute((const void*)k_acc_tile<kAccThreadsVirtual, true>,
+        e = hipFuncSetAttribute((const void*)k_acc_tile<kAccThreadsVirtual, true, false>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute((const void*)k_acc_tile<kAccThreads, false, true>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
     if (e != hipSuccess) return (int)e;
     g_lds_allowed[device].store(1, std::memory_order_release);
     return 0;
 }
 
-int double_fwd_tile(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
-                    const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,
-                    float* wpsqt, float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt, void* ws,
-                    hipStream_t st, ActGrid act, VirtualTable vt) {
+// Sort of the lists and the gather of every pair's row sums into `sums` ([2, B, L1] floats, or with `i16` 16-bit
+// integers over a table W of [R, L1] int16).
+static int gather_tile(const int32_t* widx, const int32_t* bidx, const void* W, void* sums, int B, int K, int R, int L1,
+                       int out_cols, void* ws, hipStream_t st, VirtualTable vt, bool i16, int block_rows = kRows) {
     Layout L;
-    if (!layout(B, R, &L)) return NNUEFT_E_UNSUPPORTED;
+    if (!layout(B, R, &L, block_rows)) return NNUEFT_E_UNSUPPORTED;
     int device = 0;
     const nnueft_dev::DeviceInfo* info = nullptr;
     int rc = nnueft_dev::device_info(&device, &info);
@@ -678,16 +700,15 @@ int double_fwd_tile(const float* us, const float* them, const int32_t* widx, con
     uint32_t* sched = (uint32_t*)(base + L.sched);
     uint32_t* total = (uint32_t*)(base + L.total);
     const int vec = (K % 4 == 0) && aligned16(widx) && aligned16(bidx);
-    hipLaunchKernelGGL(k_tl_hist, dim3(L.ngroups), dim3(kSortThreads), 0, st, widx, bidx, hist, B, K, R, L.nbins, vec);
+    hipLaunchKernelGGL(k_tl_hist, dim3(L.ngroups), dim3(kSortThreads), 0, st, widx, bidx, hist, B, K, R, L.nbins, vec, L.block_rows);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_tl_binscan, dim3((L.nbins + kSortThreads / 64 - 1) / (kSortThreads / 64)), dim3(kSortThreads), 0, st, hist,
                        total, L.nbins, L.ngroups);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_tl_lists, dim3(L.ngroups), dim3(kSortThreads), 0, st, widx, bidx, hist, total, lists, pidcnt,
-                       loff, chunks, sched, B, K, R, L.nblocks, L.nbins, vec);
+                       loff, chunks, sched, B, K, R, L.nblocks, L.nbins, vec, L.block_rows);
     NNUEFT_LAUNCH_CHECK();
-    const int out_cols = L1 + n_psqt;
-    const int ntiles = L1 / kTileCols;
+    const int ntiles = i16 ? L1 / (2 * kTileCols) : L1 / kTileCols;
     const int tiles_per_xcd = (ntiles + kXcd - 1) / kXcd;
     // about three tiles per visit of a chunk: its lists are copied into LDS once per visit, and a batch is
     // cut into enough units for the CUs of an XCD to finish together
@@ -696,17 +717,49 @@ int double_fwd_tile(const float* us, const float* them, const int32_t* widx, con
     if (const char* e = getenv("NNUEFT_TILE_GROUP")) tile_group = atoi(e) > 0 ? atoi(e) : tile_group;
 #endif
     const int grid = info->cus / kXcd * kXcd;
-    if (vt.V)
-        hipLaunchKernelGGL((k_acc_tile<kAccThreadsVirtual, true>), dim3(grid), dim3(kAccThreadsVirtual), kLdsBytes, st,
-                           widx, bidx, lists, pidcnt, loff, chunks, sched, W, saved, B, K, R, L1, out_cols, tiles_per_xcd,
-                           tile_group, vt);
+    const float* Wf = (const float*)W;
+    float* sf = (float*)sums;
+    if (i16)
+        hipLaunchKernelGGL((k_acc_tile<kAccThreads, false, true>), dim3(grid), dim3(kAccThreads), kLdsBytes, st, widx, bidx,
+                           lists, pidcnt, loff, chunks, sched, Wf, sf, B, K, R, L1, out_cols, tiles_per_xcd,
+                           tile_group, vt, L.block_rows);
+    else if (vt.V)
+        hipLaunchKernelGGL((k_acc_tile<kAccThreadsVirtual, true, false>), dim3(grid), dim3(kAccThreadsVirtual), kLdsBytes, st,
+                           widx, bidx, lists, pidcnt, loff, chunks, sched, Wf, sf, B, K, R, L1, out_cols, tiles_per_xcd,
+                           tile_group, vt, L.block_rows);
     else
-        hipLaunchKernelGGL((k_acc_tile<kAccThreads, false>), dim3(grid), dim3(kAccThreads), kLdsBytes, st, widx, bidx,
-                           lists, pidcnt, loff, chunks, sched, W, saved, B, K, R, L1, out_cols, tiles_per_xcd,
-                           tile_group, vt);
+        hipLaunchKernelGGL((k_acc_tile<kAccThreads, false, false>), dim3(grid), dim3(kAccThreads), kLdsBytes, st, widx, bidx,
+                           lists, pidcnt, loff, chunks, sched, Wf, sf, B, K, R, L1, out_cols, tiles_per_xcd,
+                           tile_group, vt, L.block_rows);
     NNUEFT_LAUNCH_CHECK();
+    return 0;
+}
+
+int double_fwd_tile(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+                    const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,
+                    float* wpsqt, float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt, void* ws,
+                    hipStream_t st, ActGrid act, VirtualTable vt) {
+    const int rc = gather_tile(widx, bidx, W, saved, B, K, R, L1, L1 + n_psqt, ws, st, vt, false);
+    if (rc) return rc;
     return nnueft_blocked::launch_mix(us, them, widx, bidx, psqt_idx, W, bias, saved, max_act, l0, wpsqt, bpsqt, B,
                                       K, R, L1, n_psqt, st, act, vt);
+}
+
+bool fits_int16(const nnueft_dev::DeviceInfo& d, int B, int K, int R, int L1, int block_rows) {
+    Layout L;
+    return L1 % (2 * kTileCols) == 0 && fits(d, B, K, R, L1) && layout(B, R, &L, block_rows) &&
+           L.max_chunks <= kMaxChunks;
+}
+
+size_t workspace_int16(int B, int R, int block_rows) {
+    Layout L;
+    return layout(B, R, &L, block_rows) ? L.end : 0;
+}
+
+int int16_sums_tile(const int32_t* widx, const int32_t* bidx, const int16_t* W16, int16_t* sums, int B, int K, int R,
+                    int L1, int block_rows, void* ws, hipStream_t st) {
+    return gather_tile(widx, bidx, W16, sums, B, K, R, L1, L1, ws, st, VirtualTable{nullptr, 1.0f, 1.0f, 0, 0.0f}, true,
+                       block_rows);
 }
 
 }  // namespace nnueft_tile

@@ -10,6 +10,11 @@
 //       k_acc16_white     wave per (white list, slice): b16 + sum of rows -> accW[B, L1] int16
 //       k_black_mix16     wave per (black list, paired slice): black sums in registers, the white ones
 //                         read back, side-to-move order, clip, product, u8 store; psqt sums
+//   LDS-tiled (workspace, table blocks of 768 rows, L1 a multiple of 64, lists of 32 slots at most): the
+//                         forward's gather out of LDS tiles (fwd_tile.hip) over the int16 table
+//       k_acc_tile        sums[2, B, L1] int16 for both lists of every position
+//       k_mix16           wave per (position, paired slice): + b16, side-to-move order, clip, product, u8
+//                         store; psqt sums
 #include "internal.h"
 
 namespace {
@@ -279,8 +284,44 @@ __global__ __launch_bounds__(64) void k_black_mix16(const int32_t* __restrict__ 
     }
 }
 
+// The output bytes of a position from the two lists' row sums (without the bias) that the LDS-tiled gather left.
+__global__ __launch_bounds__(64) void k_mix16(const int32_t* __restrict__ widx, const int32_t* __restrict__ bidx,
+                                              const uint8_t* __restrict__ stm, const int16_t* __restrict__ b16,
+                                              const int16_t* __restrict__ sums, const int32_t* __restrict__ psqt32,
+                                              const int64_t* __restrict__ psqt_idx, uint8_t* __restrict__ out_u8,
+                                              int32_t* __restrict__ psqt_out, int B, int K, int R, int L1, int n_psqt,
+                                              int clip_max, int shift, int nslices) {
+    const int lane = threadIdx.x;
+    const int b = blockIdx.x / nslices;
+    const int s = blockIdx.x - b * nslices;
+    const int h = L1 >> 1;
+    const int first = stm[b] ? 1 : 0;
+    if (s == 0) psqt_diff(widx, bidx, psqt32, psqt_idx[b], first, b, K, R, n_psqt, lane, psqt_out);
+    const int q = s * 64 + lane;
+    if (q >= h / 8) return;
+    const int c0 = q * 8, c1 = c0 + h;
+    const vecs<8> bias0 = ldi<8>(b16 + c0), bias1 = ldi<8>(b16 + c1);
+    vecs<8> w0 = ldi<8>(sums + (size_t)b * L1 + c0), w1 = ldi<8>(sums + (size_t)b * L1 + c1);
+    vecs<8> k0 = ldi<8>(sums + ((size_t)B + b) * L1 + c0), k1 = ldi<8>(sums + ((size_t)B + b) * L1 + c1);
+    iadd<8>(w0, bias0);
+    iadd<8>(w1, bias1);
+    iadd<8>(k0, bias0);
+    iadd<8>(k1, bias1);
+    uint8_t* dst = out_u8 + (size_t)b * L1;
+    // output half 0 shows the side to move, half 1 the other side
+    if (first) {
+        pair_product_store<8>(dst + c0, k0, k1, clip_max, shift);
+        pair_product_store<8>(dst + h + c0, w0, w1, clip_max, shift);
+    } else {
+        pair_product_store<8>(dst + c0, w0, w1, clip_max, shift);
+        pair_product_store<8>(dst + h + c0, k0, k1, clip_max, shift);
+    }
+}
+
 struct Int16Layout {
     size_t accW, sort, end;
+    size_t tile_sums, tile_sort;   // the LDS-tiled path's view of the same bytes
+    bool tile_ok;                  // the table's blocks fit its tiles
 };
 
 inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -293,6 +334,14 @@ bool int16_layout(int B, int R, int L1, int block_rows, Int16Layout* L) {
     L->sort = off;
     off += up256(nnueft_blocked::pair_sort_workspace(B, R, block_rows));
     L->end = off;
+    // the LDS-tiled path keeps both lists' sums and its own sort scratch
+    L->tile_sums = 0;
+    L->tile_sort = up256((size_t)2 * B * L1 * sizeof(int16_t));
+    const int br = block_rows > 0 ? block_rows : nnueft_tile::kBlockRows;
+    const size_t tile_ws = br <= nnueft_tile::kBlockRows ? nnueft_tile::workspace_int16(B, R, br) : 0;
+    L->tile_ok = tile_ws > 0;
+    const size_t tile_end = L->tile_sort + up256(tile_ws);
+    if (L->tile_ok && tile_end > L->end) L->end = tile_end;
     return true;
 }
 
@@ -339,6 +388,19 @@ extern "C" int nnueft_ft_int16_fwd(const int32_t* widx, const int32_t* bidx, con
         const nnueft_dev::DeviceInfo* info = nullptr;
         const int rc_dev = nnueft_dev::device_info(nullptr, &info);
         if (rc_dev) return rc_dev;
+        const int br = table_block_rows > 0 ? table_block_rows : nnueft_tile::kBlockRows;
+        if (vec && L.tile_ok && nnueft_tile::fits_int16(*info, B, K, R, L1, br)) {
+            char* ws = (char*)workspace;
+            int16_t* sums = (int16_t*)(ws + L.tile_sums);
+            const int rc = nnueft_tile::int16_sums_tile(widx, bidx, W16, sums, B, K, R, L1, br, ws + L.tile_sort, st);
+            if (rc) return rc;
+            const int nslices = max(1, (L1 / 16 + 63) / 64);
+            if ((long long)B * nslices > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
+            hipLaunchKernelGGL(k_mix16, dim3((unsigned)(B * nslices)), dim3(64), 0, st, widx, bidx, stm, b16, sums, psqt32,
+                               psqt_idx, out_u8, psqt_out, B, K, R, L1, n_psqt, clip_max, shift, nslices);
+            NNUEFT_LAUNCH_CHECK();
+            return 0;
+        }
         if (vec && (long long)B <= 0x3fffffffLL && nnueft_blocked::blocked_layout_fits(*info)) {
             char* ws = (char*)workspace;
             int16_t* accW = (int16_t*)(ws + L.accW);

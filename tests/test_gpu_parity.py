@@ -363,6 +363,31 @@ def test_deterministic_backward_repeats_bitwise():
     assert np.array_equal(outs[0][1], outs[1][1])
 
 
+@pytest.mark.parametrize("B,L1", [(700, 1024), (3000, 512), (64, 3072)])
+def test_int16_forward_on_exported_lists(oracle_cpu, B, L1):
+    """Lists as the loader makes them for an exported net (22528 rows, king buckets of 704 rows, every list inside
+    one bucket): with a workspace the sums come out of LDS tiles of the int16 table (3000 positions: several
+    chunks of lists per bucket)."""
+    from nnueft import halfka_v2_hm as hk
+    from nnueft.quantized import ft_int16_forward
+
+    rng = np.random.default_rng(640 + B)
+    R = hk.NUM_INPUTS_EXPORT
+    us, _, widx, bidx, _ = hk.synthetic_batch(B, 77 + B, fold_kings=True)
+    stm = (1 - us[:, 0]).astype(np.uint8)
+    W16 = rng.integers(-3000, 3000, size=(R, L1)).astype(np.int16)
+    W16[:, : L1 // 3] = rng.integers(-40, 60, size=(R, L1 // 3)).astype(np.int16)
+    b16 = rng.integers(-200, 400, size=L1).astype(np.int16)
+    psqt32 = rng.integers(-100000, 100000, size=(R, 8)).astype(np.int32)
+    psqt_idx = rng.integers(0, 8, size=B).astype(np.int64)
+    r_out, r_ps = oracle_cpu.ft_int16_fwd(widx, bidx, stm, W16, b16, psqt32, psqt_idx, 255, 9)
+    for use_workspace in (True, False):
+        out, ps = ft_int16_forward(_t(widx), _t(bidx), _t(stm), _t(W16), _t(b16), _t(psqt32), _t(psqt_idx), 255, 9,
+                                   use_workspace=use_workspace)
+        assert np.array_equal(out.cpu().numpy(), r_out)
+        assert np.array_equal(ps.cpu().numpy(), r_ps)
+
+
 INT16_SHAPES = [(5, 32, 50, 32), (33, 1024, 22528, 32), (17, 3072, 22528, 32), (9, 38, 40, 70)]
 
 
