@@ -600,7 +600,9 @@ def run_ft(args, lib, dev):
             ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
             sbytes = lib.nnueft_det_sort_bytes(B, K_, R_ROWS, oc, 2)
             lists = torch.empty(sbytes, dtype=torch.uint8, device=dev)
-            G = torch.randn(2, B, oc, device=dev)
+            # upstream rows at the pitch the backward gives its own (whole 128-byte lines)
+            g_pitch = lib.nnueft_det_upstream_pitch(oc)
+            G = torch.randn(2, B, g_pitch, device=dev)
 
             def whole(stream=stream, aux_stream=aux_stream):
                 rc = lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT,
@@ -634,8 +636,8 @@ def run_ft(args, lib, dev):
             def reduce_only():
                 # the segmented reduction alone: k_seg_reduce, then the window sums of split rows (k_split_combine)
                 # and the rewind of the task counters, a few microseconds together
-                rc = lib.nnueft_det_reduce_rows(G.data_ptr(), gW.data_ptr(), B, K_, R_ROWS, oc, 2, row_split,
-                                                ws.data_ptr(), nbytes, lists.data_ptr(), stream)
+                rc = lib.nnueft_det_reduce_rows_pitched(G.data_ptr(), g_pitch, gW.data_ptr(), B, K_, R_ROWS, oc, 2,
+                                                        row_split, ws.data_ptr(), nbytes, lists.data_ptr(), stream)
                 assert rc == 0
 
             out = {}
@@ -712,7 +714,7 @@ def run_ft(args, lib, dev):
         alg, gathered, comp = seg_reduce_bytes(L1, B, sum_a)
         seg_traffic = sum_traffic(traffic, ("k_seg_reduce", "k_split_combine"))
         out["roofline"], out["roofline_compulsory"] = bound_block(
-            "k_seg_reduce<4,3> (timed through nnueft_det_reduce_rows, which launches it with k_split_combine, which also "
+            "k_seg_reduce<4,3> (timed through nnueft_det_reduce_rows_pitched, which launches it with k_split_combine, which also "
             "rewinds the task counters, a few microseconds, behind it)", det["reduce"], alg, gathered, comp,
             seg_traffic, l2_peak,
             note="dominant kernel of the step; it gathers one upstream row per slot through L2 (blocked by king bucket "

@@ -267,6 +267,17 @@ int nnueft_det_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int 
 int nnueft_det_reduce_rows(const float* G, float* gW, int B, int K, int R, int out_cols, int n_persp,
                            int row_split, void* workspace, size_t workspace_bytes, void* sorted_lists,
                            void* stream);
+/*
+ * The same with g_pitch >= out_cols floats from one row of G to the next (G f32[n_persp, B, g_pitch]).
+ * nnueft_det_upstream_pitch(out_cols) is the pitch nnueft_double_bwd_det gives its own upstream rows: whole
+ * 128-byte lines, so that the 1 KB a wave gathers of a row lies in 8 cache lines and not in 9 (3080 -> 3104
+ * floats: the reduction 452 -> 438 us and the kernel that writes the rows 182 -> 170 us at L1 = 3072,
+ * B = 16384).  Results do not depend on the pitch.  No counterpart in the reference.
+ */
+int nnueft_det_upstream_pitch(int out_cols);
+int nnueft_det_reduce_rows_pitched(const float* G, int g_pitch, float* gW, int B, int K, int R, int out_cols,
+                                   int n_persp, int row_split, void* workspace, size_t workspace_bytes,
+                                   void* sorted_lists, void* stream);
 
 /*
  * merged[r, c] = q(W[r, c] + V[r % vrows, c]): the table the gather reads, from the real weights

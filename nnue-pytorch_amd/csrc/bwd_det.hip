@@ -95,6 +95,13 @@ struct DetLayout {
 inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 // row_split: a table row named by more slots than this is summed window by window; 0 = no row is.
+// Floats from one upstream row of G to the next where the library lays G out itself (the two-perspective backward):
+// whole 128-byte lines, so that a wave's 1 KB load touches 8 lines, not 9.
+#ifndef NNUEFT_G_PAD
+#define NNUEFT_G_PAD 1
+#endif
+inline int g_pitch_of(int out_cols) { return NNUEFT_G_PAD ? (out_cols + 31) / 32 * 32 : out_cols; }
+
 bool det_layout(int B, int K, int R, int out_cols, int n_persp, int row_split, DetLayout* L) {
     if (B <= 0 || K <= 0 || R <= 0 || out_cols <= 0 || (n_persp != 1 && n_persp != 2) || row_split < 0) return false;
     L->row_split = row_split;
@@ -103,7 +110,7 @@ bool det_layout(int B, int K, int R, int out_cols, int n_persp, int row_split, D
     L->ntiles = (B + NNUEFT_BIAS_TILE - 1) / NNUEFT_BIAS_TILE;
     size_t off = 0;
     L->G = off;
-    off += up256(n_persp == 2 ? (size_t)2 * B * out_cols * sizeof(float) : 0);
+    off += up256(n_persp == 2 ? (size_t)2 * B * g_pitch_of(out_cols) * sizeof(float) : 0);
     L->partial = off;
     off += up256((size_t)L->ntiles * out_cols * sizeof(float));
     L->sort_begin = off;
@@ -152,7 +159,7 @@ __global__ __launch_bounds__(64) void k_bwd_rows(const float* __restrict__ us, c
                                                  const float* __restrict__ grad_bpsqt,
                                                  const float* __restrict__ saved, float* __restrict__ G,
                                                  float* __restrict__ partial, int B, int L1, int n_psqt, int group,
-                                                 int ntiles, int nslices) {
+                                                 int ntiles, int nslices, int g_pitch) {
     // `group` lanes share a tile (64 for wide rows; narrow rows put 64 / group tiles into one wave)
     const int lane = threadIdx.x;
     const int s = blockIdx.x % nslices;          // launched 1-D: the slices of a tile are neighbours
@@ -165,7 +172,7 @@ __global__ __launch_bounds__(64) void k_bwd_rows(const float* __restrict__ us, c
     const int b0 = tile * NNUEFT_BIAS_TILE;
     const int b1 = min(b0 + NNUEFT_BIAS_TILE, B);
     float* Gw = G;
-    float* Gb = G + (size_t)B * out_cols;
+    float* Gb = G + (size_t)B * g_pitch;
 
     const int q = s * group + ql;
     if (q < hv) {
@@ -190,10 +197,10 @@ __global__ __launch_bounds__(64) void k_bwd_rows(const float* __restrict__ us, c
                 part0.v[i] = part0.v[i] + (gw0.v[i] + gb0.v[i]);
                 part1.v[i] = part1.v[i] + (gw1.v[i] + gb1.v[i]);
             }
-            stv<VW>(Gw + (size_t)b * out_cols + c, gw0);
-            stv<VW>(Gw + (size_t)b * out_cols + h + c, gw1);
-            stv<VW>(Gb + (size_t)b * out_cols + c, gb0);
-            stv<VW>(Gb + (size_t)b * out_cols + h + c, gb1);
+            stv<VW>(Gw + (size_t)b * g_pitch + c, gw0);
+            stv<VW>(Gw + (size_t)b * g_pitch + h + c, gw1);
+            stv<VW>(Gb + (size_t)b * g_pitch + c, gb0);
+            stv<VW>(Gb + (size_t)b * g_pitch + h + c, gb1);
         }
         stv<VW>(partial + (size_t)tile * out_cols + c, part0);
         stv<VW>(partial + (size_t)tile * out_cols + h + c, part1);
@@ -205,8 +212,8 @@ __global__ __launch_bounds__(64) void k_bwd_rows(const float* __restrict__ us, c
                 const bool hit = psqt_idx[b] == (int64_t)j;
                 const float gw = hit ? grad_wpsqt[b] : 0.0f;
                 const float gb = hit ? grad_bpsqt[b] : 0.0f;
-                Gw[(size_t)b * out_cols + L1 + j] = gw;
-                Gb[(size_t)b * out_cols + L1 + j] = gb;
+                Gw[(size_t)b * g_pitch + L1 + j] = gw;
+                Gb[(size_t)b * g_pitch + L1 + j] = gb;
                 part = part + (gw + gb);
             }
             partial[(size_t)tile * out_cols + L1 + j] = part;
@@ -652,7 +659,7 @@ __global__ __launch_bounds__(kFillThreads) void k_fill(const int32_t* __restrict
 template <int VW, int NQ, int U>
 __device__ __forceinline__ void seg_reduce_task(const float* __restrict__ G, const uint32_t* __restrict__ list,
                                                 uint32_t beg, uint32_t mid, uint32_t end, float* __restrict__ dst,
-                                                int s, int lane, int out_cols, int slice_v, int two_persp,
+                                                int s, int lane, int out_cols, int g_pitch, int slice_v, int two_persp,
                                                 bool pre = false, int pre_my = 0) {
     const int nv = out_cols / VW;
     int col[NQ];
@@ -674,8 +681,8 @@ __device__ __forceinline__ void seg_reduce_task(const float* __restrict__ G, con
         const uint32_t nw = mid - beg, n = end - beg;
         const u64 all = n >= 64 ? ~0ull : ((1ull << n) - 1ull);
         const u64 white = nw >= 64 ? ~0ull : ((1ull << nw) - 1ull);
-        chain_rows<VW, NQ, U>(acc[0], G, (size_t)out_cols, col, pre_my, white);
-        chain_rows<VW, NQ, U>(acc[1], G, (size_t)out_cols, col, pre_my, all & ~white);
+        chain_rows<VW, NQ, U>(acc[0], G, (size_t)g_pitch, col, pre_my, white);
+        chain_rows<VW, NQ, U>(acc[1], G, (size_t)g_pitch, col, pre_my, all & ~white);
     } else {
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
@@ -684,7 +691,7 @@ __device__ __forceinline__ void seg_reduce_task(const float* __restrict__ G, con
                 const uint32_t n = min(64u, e_end - e0);
                 const int my = lane < (int)n ? (int)list[e0 + lane] : 0;
                 const u64 mask = n >= 64 ? ~0ull : ((1ull << n) - 1ull);
-                chain_rows<VW, NQ, U>(acc[p], G, (size_t)out_cols, col, my, mask);
+                chain_rows<VW, NQ, U>(acc[p], G, (size_t)g_pitch, col, my, mask);
             }
         }
     }
@@ -704,8 +711,8 @@ template <int VW, int U>
 __device__ __forceinline__ void tail_rows_task(const float* __restrict__ G, const uint32_t* __restrict__ list,
                                                const uint32_t* __restrict__ seg_off,
                                                const uint32_t* __restrict__ wcount, float* __restrict__ gW,
-                                               uint32_t r0, uint32_t r1, int lane, int out_cols, int tail_v, int g,
-                                               int two_persp, uint32_t row_split) {
+                                               uint32_t r0, uint32_t r1, int lane, int out_cols, int g_pitch, int tail_v,
+                                               int g, int two_persp, uint32_t row_split) {
     const int sub = lane % g;
     const uint32_t row = r0 + (uint32_t)(lane / g);
     bool on = row < r1 && sub < tail_v;
@@ -733,7 +740,7 @@ __device__ __forceinline__ void tail_rows_task(const float* __restrict__ G, cons
         while (__any(e < e_end)) {
             vecf<VW> v[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u) v[u] = e + u < e_end ? ldv<VW>(src + (size_t)nid[u] * out_cols) : vzero<VW>();
+            for (int u = 0; u < U; ++u) v[u] = e + u < e_end ? ldv<VW>(src + (size_t)nid[u] * g_pitch) : vzero<VW>();
 #pragma unroll
             for (int u = 0; u < U; ++u) nid[u] = e + U + u < e_end ? list[e + U + u] : 0u;
             // a chain that started at +0 never holds -0, so adding the +0 of a lane that has run out changes no bit
@@ -768,6 +775,7 @@ struct RunPlan {
     int R, cpp, nchunks, wch, nwin, n_persp;
     int nslices, slice_v;  // 64-lane slices
     int tail_v, tail_g;    // trailing vectors of a row that tail_rows_task reduces (0: none), lanes per row there
+    int g_pitch;           // floats from one row of G to the next
     uint32_t row_split;    // rows named by more slots than this are the split ones (0: none)
 };
 
@@ -831,7 +839,7 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
             const uint32_t beg = seg + rp.cnt[(size_t)c0 * rp.R + r];
             const uint32_t end = c1 == (uint32_t)rp.nchunks ? seg_off[r + 1] : seg + rp.cnt[(size_t)c1 * rp.R + r];
             float* dst = rp.runs + ((size_t)(j * (uint32_t)rp.n_persp + p) * rp.nwin + w) * out_cols;
-            seg_reduce_task<VW, 1, kRunUnroll>(G, list, beg, end, end, dst, (int)s, lane, out_cols, rp.slice_v, 0);
+            seg_reduce_task<VW, 1, kRunUnroll>(G, list, beg, end, end, dst, (int)s, lane, out_cols, rp.g_pitch, rp.slice_v, 0);
             continue;
         }
         if (t < long_end) {
@@ -841,13 +849,13 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
             const uint32_t r = long_rows[xcd + i * kXcd];
             const uint32_t beg = seg_off[r], end = seg_off[r + 1];
             seg_reduce_task<VW, 1, kRunUnroll>(G, list, beg, beg + wcount[r], end, gW + (size_t)r * out_cols, s, lane,
-                                               out_cols, rp.slice_v, two_persp);
+                                               out_cols, rp.g_pitch, rp.slice_v, two_persp);
             continue;
         }
         uint32_t u = t - long_end;
         if (u < tail_tasks) {   // first: they are few and each is a long chain of short steps
             const uint32_t r0 = lo + u * tail_rows;
-            tail_rows_task<VW, kTailUnroll>(G, list, seg_off, wcount, gW, r0, hi, lane, out_cols, rp.tail_v, rp.tail_g,
+            tail_rows_task<VW, kTailUnroll>(G, list, seg_off, wcount, gW, r0, hi, lane, out_cols, rp.g_pitch, rp.tail_v, rp.tail_g,
                                             two_persp, rp.row_split);
             continue;
         }
@@ -863,11 +871,11 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
         const int my = (pre && (uint32_t)lane < len) ? (int)list[beg + lane] : 0;
         float* dst = gW + (size_t)r * out_cols;
         if (narrow)
-            seg_reduce_task<VW, 1, kRunUnroll>(G, list, beg, beg + wcount[r], end, dst, s, lane, out_cols, rp.slice_v,
-                                               two_persp, pre, my);
+            seg_reduce_task<VW, 1, kRunUnroll>(G, list, beg, beg + wcount[r], end, dst, s, lane, out_cols, rp.g_pitch,
+                                               rp.slice_v, two_persp, pre, my);
         else
-            seg_reduce_task<VW, NQ, kRowsUnroll>(G, list, beg, beg + wcount[r], end, dst, s, lane, out_cols, slice_v,
-                                                 two_persp, pre, my);
+            seg_reduce_task<VW, NQ, kRowsUnroll>(G, list, beg, beg + wcount[r], end, dst, s, lane, out_cols, rp.g_pitch,
+                                                 slice_v, two_persp, pre, my);
     }
   }
 }
@@ -994,7 +1002,7 @@ int det_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, char
 }
 
 // The reduction over the sorted lists, and the last step of the bias gradient.
-int det_reduce(const float* G, float* gW, float* gbias, int B, int R, int out_cols, int n_persp, char* ws,
+int det_reduce(const float* G, int g_pitch, float* gW, float* gbias, int B, int R, int out_cols, int n_persp, char* ws,
                char* sorted, const DetLayout& L, hipStream_t st) {
     char* sw = sorted - L.sort_begin;
     uint32_t* cnt = (uint32_t*)(sw + L.cnt);
@@ -1005,7 +1013,7 @@ int det_reduce(const float* G, float* gW, float* gbias, int B, int R, int out_co
     uint32_t* list = (uint32_t*)(sw + L.list);
     float* partial = (float*)(ws + L.partial);
 
-    const bool vec = (out_cols % 4 == 0) && aligned16(G) && aligned16(gW);
+    const bool vec = (out_cols % 4 == 0) && (g_pitch % 4 == 0) && aligned16(G) && aligned16(gW);
     const int VWr = vec ? 4 : 1;
     const int nv = out_cols / VWr;
     const int NQ = nv > 64 ? NNUEFT_SEG_NQ : 1;
@@ -1037,6 +1045,7 @@ int det_reduce(const float* G, float* gW, float* gbias, int B, int R, int out_co
     rp.slice_v = tail_v ? 64 : ((nv + rp.nslices - 1) / rp.nslices + line_v - 1) / line_v * line_v;
     rp.tail_v = tail_v;
     rp.tail_g = tail_g;
+    rp.g_pitch = g_pitch;
     rp.row_split = (uint32_t)L.row_split;
     if ((long long)L.max_split * rp.nslices * NNUEFT_ROW_WINDOWS > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
 #define SEG_LAUNCH(VW_, NQ_)                                                                                      \
@@ -1073,10 +1082,10 @@ constexpr long long kRowsScalarBelow = 2048;   // waves of 16-byte lanes below w
 
 int launch_bwd_rows(const float* us, const float* them, const int64_t* psqt_idx, const float* bias, float max_act,
                     const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt, const float* saved,
-                    float* G, float* partial, int B, int L1, int n_psqt, hipStream_t st) {
+                    float* G, int g_pitch, float* partial, int B, int L1, int n_psqt, hipStream_t st) {
     const int out_cols = L1 + n_psqt;
     const int ntiles = (B + NNUEFT_BIAS_TILE - 1) / NNUEFT_BIAS_TILE;
-    bool vec = (L1 % 8 == 0) && (out_cols % 4 == 0) && aligned16(grad_l0) && aligned16(saved) &&
+    bool vec = (L1 % 8 == 0) && (out_cols % 4 == 0) && (g_pitch % 4 == 0) && aligned16(grad_l0) && aligned16(saved) &&
                aligned16(bias) && aligned16(G) && aligned16(partial);
     // a tile is one chain over its positions: with few tiles and narrow rows, 16-byte lanes leave most of the
     // chip without a wave; 4-byte lanes give four times the waves (config 2: 128 -> 512 waves, 44 -> 30 us)
@@ -1090,10 +1099,10 @@ int launch_bwd_rows(const float* us, const float* them, const int64_t* psqt_idx,
     const dim3 grid((unsigned)((ntiles + tiles_per_wave - 1) / tiles_per_wave) * nslices);
     if (vec)
         hipLaunchKernelGGL(k_bwd_rows<4>, grid, dim3(64), 0, st, us, them, psqt_idx, bias, max_act, grad_l0,
-                           grad_wpsqt, grad_bpsqt, saved, G, partial, B, L1, n_psqt, group, ntiles, nslices);
+                           grad_wpsqt, grad_bpsqt, saved, G, partial, B, L1, n_psqt, group, ntiles, nslices, g_pitch);
     else
         hipLaunchKernelGGL(k_bwd_rows<1>, grid, dim3(64), 0, st, us, them, psqt_idx, bias, max_act, grad_l0,
-                           grad_wpsqt, grad_bpsqt, saved, G, partial, B, L1, n_psqt, group, ntiles, nslices);
+                           grad_wpsqt, grad_bpsqt, saved, G, partial, B, L1, n_psqt, group, ntiles, nslices, g_pitch);
     NNUEFT_LAUNCH_CHECK();
     return 0;
 }
@@ -1131,17 +1140,26 @@ extern "C" int nnueft_det_sort(const int32_t* widx, const int32_t* bidx, int B, 
     return det_sort(widx, n_persp == 2 ? bidx : widx, B, K, R, (char*)sorted_lists, L, (hipStream_t)stream);
 }
 
-extern "C" int nnueft_det_reduce_rows(const float* G, float* gW, int B, int K, int R, int out_cols, int n_persp,
-                                      int row_split, void* workspace, size_t workspace_bytes, void* sorted_lists,
-                                      void* stream) {
-    if (!G || !gW) return NNUEFT_E_ARG;
+extern "C" int nnueft_det_upstream_pitch(int out_cols) { return out_cols > 0 ? g_pitch_of(out_cols) : 0; }
+
+extern "C" int nnueft_det_reduce_rows_pitched(const float* G, int g_pitch, float* gW, int B, int K, int R, int out_cols,
+                                              int n_persp, int row_split, void* workspace, size_t workspace_bytes,
+                                              void* sorted_lists, void* stream) {
+    if (!G || !gW || g_pitch < out_cols) return NNUEFT_E_ARG;
     if ((long long)B * K > 0x3fffffffLL || (long long)B > 0x3fffffffLL) return NNUEFT_E_UNSUPPORTED;
     DetLayout L;
     if (!det_layout(B, K, R, out_cols, n_persp, row_split, &L)) return NNUEFT_E_ARG;
     if (!workspace || !aligned256(workspace) || workspace_bytes < L.end) return NNUEFT_E_WORKSPACE;
     if (!sorted_lists || !aligned256(sorted_lists)) return NNUEFT_E_WORKSPACE;
-    return det_reduce(G, gW, nullptr, B, R, out_cols, n_persp, (char*)workspace, (char*)sorted_lists, L,
+    return det_reduce(G, g_pitch, gW, nullptr, B, R, out_cols, n_persp, (char*)workspace, (char*)sorted_lists, L,
                       (hipStream_t)stream);
+}
+
+extern "C" int nnueft_det_reduce_rows(const float* G, float* gW, int B, int K, int R, int out_cols, int n_persp,
+                                      int row_split, void* workspace, size_t workspace_bytes, void* sorted_lists,
+                                      void* stream) {
+    return nnueft_det_reduce_rows_pitched(G, out_cols, gW, B, K, R, out_cols, n_persp, row_split, workspace,
+                                          workspace_bytes, sorted_lists, stream);
 }
 
 extern "C" int nnueft_sparse_bwd_det(const int32_t* idx, const float* gout, float* gW, float* gbias, int B, int K,
@@ -1160,7 +1178,7 @@ extern "C" int nnueft_sparse_bwd_det(const int32_t* idx, const float* gout, floa
     NNUEFT_LAUNCH_CHECK();
     const int rc = det_sort(idx, idx, B, K, R, ws + L.sort_begin, L, st);
     if (rc) return rc;
-    return det_reduce(gout, gW, gbias, B, R, out_cols, 1, ws, ws + L.sort_begin, L, st);
+    return det_reduce(gout, out_cols, gW, gbias, B, R, out_cols, 1, ws, ws + L.sort_begin, L, st);
 }
 
 extern "C" int nnueft_double_bwd_det(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
@@ -1200,14 +1218,14 @@ extern "C" int nnueft_double_bwd_det(const float* us, const float* them, const i
         // the caller ran nnueft_det_sort on these lists already; if on aux_stream, it may still be
         // running there: only the reduction has to wait for it, the upstream rows do not
         const int rc = nnueft_det::launch_bwd_rows(us, them, psqt_idx, bias, max_act, grad_l0, grad_wpsqt, grad_bpsqt,
-                                                   saved, G, partial, B, L1, n_psqt, st);
+                                                   saved, G, g_pitch_of(out_cols), partial, B, L1, n_psqt, st);
         if (rc) return rc;
         if (two_streams) {
             hipError_t e = hipEventRecord(joined, aux);
             if (e == hipSuccess) e = hipStreamWaitEvent(st, joined, 0);
             if (e != hipSuccess) return (int)e;
         }
-        return det_reduce(G, gW, gbias, B, R, out_cols, 2, ws, (char*)sorted_lists, L, st);
+        return det_reduce(G, g_pitch_of(out_cols), gW, gbias, B, R, out_cols, 2, ws, (char*)sorted_lists, L, st);
     }
     if (two_streams) {
         hipError_t e = hipEventRecord(forked, st);
@@ -1220,12 +1238,12 @@ extern "C" int nnueft_double_bwd_det(const float* us, const float* them, const i
     // the upstream rows go onto the caller's stream before it is made to wait for the sort
     if (rc == 0)
         rc = nnueft_det::launch_bwd_rows(us, them, psqt_idx, bias, max_act, grad_l0, grad_wpsqt, grad_bpsqt, saved, G,
-                                         partial, B, L1, n_psqt, st);
+                                         g_pitch_of(out_cols), partial, B, L1, n_psqt, st);
     if (two_streams) {
         // always rejoin, also after a failed launch: the caller's stream must not run ahead of the other one
         if (sorted == hipSuccess) sorted = hipStreamWaitEvent(st, joined, 0);
         if (rc == 0 && sorted != hipSuccess) rc = (int)sorted;
     }
     if (rc) return rc;
-    return det_reduce(G, gW, gbias, B, R, out_cols, 2, ws, ws + L.sort_begin, L, st);
+    return det_reduce(G, g_pitch_of(out_cols), gW, gbias, B, R, out_cols, 2, ws, ws + L.sort_begin, L, st);
 }

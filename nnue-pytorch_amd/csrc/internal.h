@@ -89,11 +89,11 @@ int int16_sums_tile(const int32_t* widx, const int32_t* bidx, const int16_t* W16
 
 namespace nnueft_det {
 
-// Upstream rows G[2, B, L1 + n_psqt] of the two sparse-linear outputs and the bias partial sums
-// partial[ceil(B / NNUEFT_BIAS_TILE), L1 + n_psqt]; then the chain over the partial sums.
+// Upstream rows G[2, B, g_pitch] (L1 + n_psqt floats of a row used) of the two sparse-linear outputs and the
+// bias partial sums partial[ceil(B / NNUEFT_BIAS_TILE), L1 + n_psqt]; then the chain over the partial sums.
 int launch_bwd_rows(const float* us, const float* them, const int64_t* psqt_idx, const float* bias, float max_act,
                     const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt, const float* saved,
-                    float* G, float* partial, int B, int L1, int n_psqt, hipStream_t st);
+                    float* G, int g_pitch, float* partial, int B, int L1, int n_psqt, hipStream_t st);
 int launch_bias_final(const float* partial, float* gbias, int B, int out_cols, uint32_t* sched, hipStream_t st);
 
 }  // namespace nnueft_det

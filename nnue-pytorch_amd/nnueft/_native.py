@@ -59,6 +59,9 @@ PROTOTYPES = {
     "nnueft_det_sort_bytes": (c_size_t, [c_int] * 5),
     "nnueft_det_sort": (c_int, [c_void_p] * 2 + [c_int] * 6 + [c_void_p, c_size_t, c_void_p]),
     "nnueft_det_reduce_rows": (c_int, [c_void_p] * 2 + [c_int] * 6 + [c_void_p, c_size_t, c_void_p, c_void_p]),
+    "nnueft_det_upstream_pitch": (c_int, [c_int]),
+    "nnueft_det_reduce_rows_pitched": (c_int, [c_void_p, c_int, c_void_p] + [c_int] * 6
+                                       + [c_void_p, c_size_t, c_void_p, c_void_p]),
     "nnueft_table_merge": (c_int, [c_void_p] * 3 + [c_int] * 4 + [c_float] * 2 + [c_int, c_void_p]),
     "nnueft_table_virtual_grad": (c_int, [c_void_p] * 2 + [c_int] * 3 + [c_void_p]),
     "nnueft_int16_workspace_bytes": (c_size_t, [c_int] * 5),

@@ -215,6 +215,17 @@ def test_reduce_rows_stage_equals_the_sparse_backward(oracle_cpu):
                                                      nbytes, lists.data_ptr(), st), "reduce_rows")
             rW, _ = oracle_cpu.sparse_bwd(c["idx"], c["g"], R, row_split=rs)
             assert np.array_equal(gW.cpu().numpy(), rW)
+        # the same rows at the pitch the two-perspective backward gives its own upstream rows
+        pitch = lib.nnueft_det_upstream_pitch(oc)
+        assert pitch >= oc and pitch % 32 == 0
+        gp = torch.full((B, pitch), float("nan"), device=DEV)
+        gp[:, :oc] = g
+        gW.fill_(float("nan"))
+        _native.check(lib.nnueft_det_reduce_rows_pitched(gp.data_ptr(), pitch, gW.data_ptr(), B, K, R, oc, 1, rs,
+                                                         ws.data_ptr(), nbytes, lists.data_ptr(), st), "reduce_rows_pitched")
+        assert np.array_equal(gW.cpu().numpy(), rW)
+        assert lib.nnueft_det_reduce_rows_pitched(gp.data_ptr(), oc - 1, gW.data_ptr(), B, K, R, oc, 1, rs, ws.data_ptr(),
+                                                  nbytes, lists.data_ptr(), st) == -1
 
 
 @pytest.mark.parametrize("L1", [256, 1024], ids=["l2_blocked_forward", "lds_tiled_forward"])
