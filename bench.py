@@ -719,7 +719,9 @@ def run_ft(args, lib, dev):
             seg_traffic, l2_peak,
             note="dominant kernel of the step; it gathers one upstream row per slot through L2 (blocked by king bucket "
                  "and column slice), so `achieved` (algorithmic bytes) is held against the L2 line rate; against HBM "
-                 "see roofline_compulsory (bytes that must cross HBM once) and `traffic` (counter-measured)")
+                 "see roofline_compulsory (bytes that must cross HBM once) and `traffic` (counter-measured); the L2's "
+                 "channels are busy 95 % of this kernel's time (TCC_BUSY in "
+                 "profiles/ft_fwd_bwd_L1_3072_B16384_utilisation_pmc.txt)")
     elif "atomic" in bwd_ms:
         _, bwd_bytes = algorithmic_bytes(L1, B, sum_a, "atomic")
         gbs = bwd_bytes / (bwd_ms["atomic"]["entry"] * 1e-3) / 1e9
