@@ -219,6 +219,32 @@ int nnueft_double_bwd_atomic(const float* us, const float* them, const int32_t* 
                              int B, int K, int R, int L1, int n_psqt, void* stream);
 
 /*
+ * The same gradient as nnueft_double_bwd_atomic (sums in no fixed order, so their last bits vary from run
+ * to run), with the atomic adds made in LDS: a workgroup keeps a tile of one 768-row table block of gW
+ * (768 rows x 16 columns, as doubles) in LDS, adds the upstream rows of every position whose list names rows of
+ * that block, and writes the tile out once, rounded to float.  gW and gbias are fully written and need not be zero on entry.
+ * workspace: nnueft_atomic_lds_workspace_bytes(B, K, R, L1 + n_psqt, 2) bytes of device memory, 256-byte
+ * aligned; a return of 0 from that function, or NNUEFT_E_UNSUPPORTED from this one, says that the
+ * shape or the device cannot take this path (K > 32, a row that is not whole 16-byte vectors, more than
+ * 62 table blocks, a device that does not present 8 XCDs): call nnueft_double_bwd_atomic then.
+ * The bias gradient is the deterministic one (tiles of nnueft_bias_tile() positions).  B >= 1.
+ * Replaces `fused_double_ft_backward`, fused_ft_functions.py:94-120 (kernel: fused_ft_kernel.py:147-272,
+ * whose shared-memory partial sums, :172-176, are what the LDS tile generalises).
+ */
+size_t nnueft_atomic_lds_workspace_bytes(int B, int K, int R, int out_cols, int n_persp);
+/* The one-list form (n_persp = 1 for the workspace): gradient of nnueft_sparse_fwd, as nnueft_sparse_bwd_atomic.
+ * Replaces `sparse_input_linear_backward`, sparse_linear_functions.py:118-134 (kernel: sparse_linear_kernel.py:237-288). */
+int nnueft_sparse_bwd_atomic_lds(const int32_t* idx, const float* gout, float* gW, float* gbias,
+                                 int B, int K, int R, int out_cols,
+                                 void* workspace, size_t workspace_bytes, void* stream);
+int nnueft_double_bwd_atomic_lds(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
+                                 const int64_t* psqt_idx, const float* bias, float max_act,
+                                 const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt,
+                                 const float* saved, float* gW, float* gbias,
+                                 int B, int K, int R, int L1, int n_psqt,
+                                 void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Same gradient in the fixed order stated at the top; gW and gbias are fully written.
  * No counterpart in the reference's GPU code; the order is that of autograd through the
  * reference's CPU composition (double_ft_functions.py:62-80).

@@ -1107,6 +1107,13 @@ int launch_bwd_rows(const float* us, const float* them, const int64_t* psqt_idx,
     return 0;
 }
 
+int launch_tile_colsum(const float* gout, float* partial, int B, int out_cols, hipStream_t st) {
+    const int ntiles = (B + NNUEFT_BIAS_TILE - 1) / NNUEFT_BIAS_TILE;
+    hipLaunchKernelGGL(k_tile_colsum, dim3(ntiles, (out_cols + 255) / 256), dim3(256), 0, st, gout, partial, B, out_cols);
+    NNUEFT_LAUNCH_CHECK();
+    return 0;
+}
+
 int launch_bias_final(const float* partial, float* gbias, int B, int out_cols, uint32_t* sched, hipStream_t st) {
     const int ntiles = (B + NNUEFT_BIAS_TILE - 1) / NNUEFT_BIAS_TILE;
     hipLaunchKernelGGL(k_bias_final, dim3((out_cols + 63) / 64), dim3(64), 0, st, partial, gbias, ntiles, out_cols,

@@ -25,73 +25,27 @@
 #include <cstdlib>
 
 #include "gather.h"
-#include "internal.h"
+#include "tile_sort.h"
 
 namespace nnueft_tile {
 
-using nnueft_blocked::kXcd;
-
-constexpr int kRows = 768;                         // rows of a table block = rows of a tile
-constexpr int kTileCols = 32;                      // floats per tile row
-constexpr int kRowBytes = kTileCols * 4;
-constexpr int kTileBytes = (kRows + 1) * kRowBytes;   // + one row of zeros for the padding slots
-constexpr int kSlots = 32;                         // list slots the 16-bit lists hold
-constexpr int kLenBins = kSlots + 1;
-constexpr int kLenBins8 = kLenBins * kSlots;       // entries a chunk can get beyond its even share of a block
-constexpr int kChunk = 1536;                       // most pairs whose lists a workgroup holds
-constexpr int kListCap = 27648;                    // most list entries (padded, 16 bits each) it holds
-constexpr int kListSlack = kLenBins8;              // see chunks_of()
-constexpr int kMaxBlocks = 62;
-constexpr int kMaxChunks = 1024;                   // chunks whose places a workgroup of the sort keeps in LDS
-constexpr int kBins = 2048;                        // LDS counters of the sort (kMaxBlocks * kLenBins + 1 used at most)
-static_assert(kMaxBlocks * kLenBins + 1 <= kBins, "sort bins");
-static_assert(kRows == kBlockRows, "rows of a table block");
-constexpr uint32_t kForeign = 63;                  // count field of a list that leaves its block
-#ifndef NNUEFT_TILE_NT
-#define NNUEFT_TILE_NT 1024
-#endif
-constexpr int kAccThreads = NNUEFT_TILE_NT;
-constexpr int kAccThreadsVirtual = 768;
-constexpr int kSortThreads = 256;
-constexpr int kLdsBytes = kTileBytes + (kListCap + 32) * 2 + kChunk * 4 + kChunk * 2 + 16;
-
-typedef float f4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u4 __attribute__((ext_vector_type(4)));
-
-// A chunk of a block's pairs: pairs [start, start + count) of pidcnt / loff, their lists in
-// lists[pool8 * 8 .. + n8 * 8) (every list padded to a multiple of 8 entries).
-struct Chunk {
-    int block, start, count, pool8, n8, pad0, pad1, pad2;
-};
-
-// entries of a list of `cnt` slots in the pool
-__host__ __device__ __forceinline__ int padded(int cnt) { return (cnt + 7) & ~7; }
-
-// What the sort and the gather share in the workspace.
-struct Layout {
-    size_t hist, total, lists, pidcnt, loff, chunks, sched, end;
-    int ngroups, nblocks, nbins, max_chunks, nslots;
-    int block_rows;   // rows of a table block (kRows, or fewer: the tile then keeps rows to spare)
-};
-
-static inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
-
-bool layout(int B, int R, Layout* L, int block_rows = kRows) {
-    if (B <= 0 || R <= 0 || block_rows <= 0 || block_rows > kRows) return false;
+bool layout(int npairs, int R, Layout* L, int block_rows) {
+    if (npairs <= 0 || R <= 0 || block_rows <= 0 || block_rows > kRows) return false;
+    L->npairs = npairs;
     L->block_rows = block_rows;
     L->nblocks = (R + block_rows - 1) / block_rows;
     if (L->nblocks > kMaxBlocks) return false;
     L->nbins = L->nblocks * kLenBins + 1;   // + one empty bin: its offset is the end of the last block
-    L->ngroups = (2 * B + kSortThreads - 1) / kSortThreads;
-    L->max_chunks = (2 * B + 511) / 512 + 2 * L->nblocks + 2;
-    L->nslots = 2 * B + L->max_chunks;     // a block's chunks are equally long, the last ones one pair short
+    L->ngroups = (npairs + kSortThreads - 1) / kSortThreads;
+    L->max_chunks = (npairs + 511) / 512 + 2 * L->nblocks + 2;
+    L->nslots = npairs + L->max_chunks;     // a block's chunks are equally long, the last ones one pair short
     size_t off = 0;
     L->hist = off;
     off += up256((size_t)L->ngroups * L->nbins * sizeof(uint32_t));
     L->total = off;
     off += up256((size_t)kBins * sizeof(uint32_t));
     L->lists = off;
-    off += up256(((size_t)2 * B * kSlots + 64) * sizeof(uint16_t));
+    off += up256(((size_t)npairs * kSlots + 64) * sizeof(uint16_t));
     L->pidcnt = off;
     off += up256((size_t)L->nslots * sizeof(uint32_t));
     L->loff = off;
@@ -100,6 +54,12 @@ bool layout(int B, int R, Layout* L, int block_rows = kRows) {
     off += up256((size_t)L->max_chunks * sizeof(Chunk));
     L->sched = off;
     off += up256((size_t)(kXcd + 1) * 32 * sizeof(uint32_t));
+    L->brec = off;
+    off += up256((size_t)kMaxBlocks * sizeof(BlockRec));
+    L->cpool8 = off;
+    off += up256((size_t)kMaxChunks * sizeof(uint32_t));
+    L->border = off;
+    off += up256((size_t)kMaxBlocks * sizeof(uint32_t));
     L->end = off;
     return true;
 }
@@ -107,14 +67,14 @@ bool layout(int B, int R, Layout* L, int block_rows = kRows) {
 size_t workspace(int B, int R) {
     Layout L;
     const size_t blocked = nnueft_blocked::pair_sort_workspace(B, R, 0);
-    if (!layout(B, R, &L)) return blocked;
+    if (B >= (1 << 25) || !layout(2 * B, R, &L)) return blocked;
     return L.end > blocked ? L.end : blocked;
 }
 
 bool fits(const nnueft_dev::DeviceInfo& d, int B, int K, int R, int L1) {
     Layout L;
     return K <= kSlots && L1 % kTileCols == 0 && L1 >= 512 && (long long)2 * B < (1ll << 26) &&
-           d.max_lds >= kLdsBytes && d.xcds == kXcd && d.cus >= kXcd && layout(B, R, &L) &&
+           d.max_lds >= kLdsBytes && d.xcds == kXcd && d.cus >= kXcd && layout(2 * B, R, &L) &&
            L.max_chunks <= kMaxChunks;
 }
 
@@ -175,14 +135,14 @@ __device__ __forceinline__ int sort_key(const ListFacts& f) { return f.block * k
 
 __global__ __launch_bounds__(kSortThreads) void k_tl_hist(const int32_t* __restrict__ widx,
                                                           const int32_t* __restrict__ bidx,
-                                                          uint32_t* __restrict__ hist, int B, int K, int R,
-                                                          int nbins, int vec, int block_rows) {
+                                                          uint32_t* __restrict__ hist, int npairs, int B, int K,
+                                                          int R, int nbins, int vec, int block_rows) {
     __shared__ uint32_t bins[kBins];
     const int tid = threadIdx.x;
     const int n = blockIdx.x * kSortThreads + tid;
     for (int i = tid; i < nbins; i += kSortThreads) bins[i] = 0;
     __syncthreads();
-    if (n < 2 * B) atomicAdd(&bins[sort_key(list_facts(load_list(pair_list(widx, bidx, n, B, K), K, vec), R, block_rows))], 1u);
+    if (n < npairs) atomicAdd(&bins[sort_key(list_facts(load_list(pair_list(widx, bidx, n, B, K), K, vec), R, block_rows))], 1u);
     __syncthreads();
     for (int i = tid; i < nbins; i += kSortThreads) hist[(size_t)i * gridDim.x + blockIdx.x] = bins[i];
 }
@@ -197,8 +157,6 @@ __device__ __forceinline__ int chunks_of(int n, int e) {
     const int by_entries = (e + (kListCap - kListSlack) - 1) / (kListCap - kListSlack);
     return max(1, max(by_pairs, by_entries));
 }
-// how many of the ranks 0 .. x - 1 go to chunk j of nc
-__device__ __forceinline__ int ranks_of_chunk(int x, int j, int nc) { return (x - j + nc - 1) / nc; }
 
 // One wave per bin: the counts of the workgroups become their exclusive prefix, the sum goes to total[bin].
 __global__ __launch_bounds__(kSortThreads) void k_tl_binscan(uint32_t* __restrict__ hist, uint32_t* __restrict__ total,
@@ -230,8 +188,10 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
                                                            uint16_t* __restrict__ lists,
                                                            uint32_t* __restrict__ pidcnt, uint16_t* __restrict__ loff,
                                                            Chunk* __restrict__ chunks,
-                                                           uint32_t* __restrict__ sched, int B, int K, int R,
-                                                           int nblocks, int nbins, int vec, int block_rows) {
+                                                           uint32_t* __restrict__ sched,
+                                                           BlockRec* __restrict__ brec, uint32_t* __restrict__ cpool8,
+                                                           uint32_t* __restrict__ border, int npairs, int B, int K,
+                                                           int R, int nblocks, int nbins, int vec, int block_rows) {
     __shared__ uint32_t cursor[kBins];      // next slot of this workgroup in every bin
     __shared__ uint32_t bin_base[kBins];    // first slot of every bin
     __shared__ uint32_t bin_eoff[kBins];    // list entries of its block before the bin's lists
@@ -318,6 +278,7 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
             const uint32_t ci = blk_chunk0[tid] + (uint32_t)j;
             if (ci < (uint32_t)kMaxChunks) chunk_pool8[ci] = p8;
             if (blockIdx.x == 0 && ci < (uint32_t)kMaxChunks) {
+                cpool8[ci] = p8;
                 ck_block[ci] = (uint16_t)tid;
                 ck_start[ci] = (bb[0] + blk_chunk0[tid]) + (uint32_t)(j * len);
                 ck_count[ci] = (uint16_t)ranks_of_chunk(nb, j, nc);
@@ -327,6 +288,19 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
         }
     }
     if (blockIdx.x == 0 && tid <= kXcd) sched[tid * 32] = tid == kXcd ? blk_chunk0[nblocks] : 0u;
+    // the blocks as the backward scatter walks them, and their order by population (most pairs first)
+    if (blockIdx.x == 0 && tid < nblocks) {
+        const uint32_t* bb = bin_base + tid * kLenBins;
+        const int nb = (int)(bb[kLenBins] - bb[0]);
+        const int nc = (int)blk_nc[tid];
+        brec[tid] = BlockRec{(int)(bb[0] + blk_chunk0[tid]), nb, nc, nc ? (nb + nc - 1) / nc : 0, (int)blk_chunk0[tid], 0, 0, 0};
+        int rank = 0;
+        for (int k = 0; k < nblocks; ++k) {
+            const int other = (int)(bin_base[(k + 1) * kLenBins] - bin_base[k * kLenBins]);
+            rank += other > nb || (other == nb && k < tid);
+        }
+        border[rank] = (uint32_t)tid;
+    }
     __syncthreads();
     // The chunk table, longest lists first: the gather hands units out in table order, and the CUs of an XCD
     // finish closer together when the small units come last.
@@ -343,7 +317,7 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
                                  (int)ck_n8[ci], 0, 0, 0};
         }
     }
-    if (n >= 2 * B) return;
+    if (n >= npairs) return;
     const ListRegs l = load_list(pair_list(widx, bidx, n, B, K), K, vec);
     const ListFacts f = list_facts(l, R, block_rows);
     const int bin = sort_key(f);
@@ -679,18 +653,8 @@ int allow_lds(int device) {
     return 0;
 }
 
-// Sort of the lists and the gather of every pair's row sums into `sums` ([2, B, L1] floats, or with `i16` 16-bit
-// integers over a table W of [R, L1] int16).
-static int gather_tile(const int32_t* widx, const int32_t* bidx, const void* W, void* sums, int B, int K, int R, int L1,
-                       int out_cols, void* ws, hipStream_t st, VirtualTable vt, bool i16, int block_rows = kRows) {
-    Layout L;
-    if (!layout(B, R, &L, block_rows)) return NNUEFT_E_UNSUPPORTED;
-    int device = 0;
-    const nnueft_dev::DeviceInfo* info = nullptr;
-    int rc = nnueft_dev::device_info(&device, &info);
-    if (rc) return rc;
-    rc = allow_lds(device);
-    if (rc) return rc;
+int launch_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, const Layout& L, void* ws, hipStream_t st,
+                Sorted* out) {
     char* base = (char*)ws;
     uint32_t* hist = (uint32_t*)(base + L.hist);
     uint16_t* lists = (uint16_t*)(base + L.lists);
@@ -699,15 +663,43 @@ static int gather_tile(const int32_t* widx, const int32_t* bidx, const void* W, 
     Chunk* chunks = (Chunk*)(base + L.chunks);
     uint32_t* sched = (uint32_t*)(base + L.sched);
     uint32_t* total = (uint32_t*)(base + L.total);
+    BlockRec* brec = (BlockRec*)(base + L.brec);
+    uint32_t* cpool8 = (uint32_t*)(base + L.cpool8);
+    uint32_t* border = (uint32_t*)(base + L.border);
     const int vec = (K % 4 == 0) && aligned16(widx) && aligned16(bidx);
-    hipLaunchKernelGGL(k_tl_hist, dim3(L.ngroups), dim3(kSortThreads), 0, st, widx, bidx, hist, B, K, R, L.nbins, vec, L.block_rows);
+    hipLaunchKernelGGL(k_tl_hist, dim3(L.ngroups), dim3(kSortThreads), 0, st, widx, bidx, hist, L.npairs, B, K, R, L.nbins, vec,
+                       L.block_rows);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_tl_binscan, dim3((L.nbins + kSortThreads / 64 - 1) / (kSortThreads / 64)), dim3(kSortThreads), 0, st, hist,
                        total, L.nbins, L.ngroups);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_tl_lists, dim3(L.ngroups), dim3(kSortThreads), 0, st, widx, bidx, hist, total, lists, pidcnt,
-                       loff, chunks, sched, B, K, R, L.nblocks, L.nbins, vec, L.block_rows);
+                       loff, chunks, sched, brec, cpool8, border, L.npairs, B, K, R, L.nblocks, L.nbins, vec, L.block_rows);
     NNUEFT_LAUNCH_CHECK();
+    *out = Sorted{lists, pidcnt, loff, chunks, brec, cpool8, border, sched};
+    return 0;
+}
+
+// Sort of the lists and the gather of every pair's row sums into `sums` ([2, B, L1] floats, or with `i16` 16-bit
+// integers over a table W of [R, L1] int16).
+static int gather_tile(const int32_t* widx, const int32_t* bidx, const void* W, void* sums, int B, int K, int R, int L1,
+                       int out_cols, void* ws, hipStream_t st, VirtualTable vt, bool i16, int block_rows = kRows) {
+    Layout L;
+    if (!layout(2 * B, R, &L, block_rows)) return NNUEFT_E_UNSUPPORTED;
+    int device = 0;
+    const nnueft_dev::DeviceInfo* info = nullptr;
+    int rc = nnueft_dev::device_info(&device, &info);
+    if (rc) return rc;
+    rc = allow_lds(device);
+    if (rc) return rc;
+    Sorted S;
+    rc = launch_sort(widx, bidx, B, K, R, L, ws, st, &S);
+    if (rc) return rc;
+    const uint16_t* lists = S.lists;
+    const uint32_t* pidcnt = S.pidcnt;
+    const uint16_t* loff = S.loff;
+    const Chunk* chunks = S.chunks;
+    uint32_t* sched = S.sched;
     const int ntiles = i16 ? L1 / (2 * kTileCols) : L1 / kTileCols;
     const int tiles_per_xcd = (ntiles + kXcd - 1) / kXcd;
     // about three tiles per visit of a chunk: its lists are copied into LDS once per visit, and a batch is
@@ -747,13 +739,13 @@ int double_fwd_tile(const float* us, const float* them, const int32_t* widx, con
 
 bool fits_int16(const nnueft_dev::DeviceInfo& d, int B, int K, int R, int L1, int block_rows) {
     Layout L;
-    return L1 % (2 * kTileCols) == 0 && fits(d, B, K, R, L1) && layout(B, R, &L, block_rows) &&
+    return L1 % (2 * kTileCols) == 0 && fits(d, B, K, R, L1) && layout(2 * B, R, &L, block_rows) &&
            L.max_chunks <= kMaxChunks;
 }
 
 size_t workspace_int16(int B, int R, int block_rows) {
     Layout L;
-    return layout(B, R, &L, block_rows) ? L.end : 0;
+    return B < (1 << 25) && layout(2 * B, R, &L, block_rows) ? L.end : 0;
 }
 
 int int16_sums_tile(const int32_t* widx, const int32_t* bidx, const int16_t* W16, int16_t* sums, int B, int K, int R,

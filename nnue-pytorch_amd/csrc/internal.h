@@ -94,6 +94,8 @@ namespace nnueft_det {
 int launch_bwd_rows(const float* us, const float* them, const int64_t* psqt_idx, const float* bias, float max_act,
                     const float* grad_l0, const float* grad_wpsqt, const float* grad_bpsqt, const float* saved,
                     float* G, int g_pitch, float* partial, int B, int L1, int n_psqt, hipStream_t st);
+// partial[tile, c] = chain over the tile's positions of gout[b, c] (the bias partial sums of the one-list backward)
+int launch_tile_colsum(const float* gout, float* partial, int B, int out_cols, hipStream_t st);
 int launch_bias_final(const float* partial, float* gbias, int B, int out_cols, uint32_t* sched, hipStream_t st);
 
 }  // namespace nnueft_det

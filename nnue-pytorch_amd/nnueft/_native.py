@@ -52,6 +52,11 @@ PROTOTYPES = {
     ),
     "nnueft_double_fwd_noalloc": (c_int, [c_void_p] * 7 + [c_float] + [c_void_p] * 4 + [c_int] * 5 + [c_void_p]),
     "nnueft_double_bwd_atomic": (c_int, [c_void_p] * 6 + [c_float] + [c_void_p] * 6 + [c_int] * 5 + [c_void_p]),
+    "nnueft_atomic_lds_workspace_bytes": (c_size_t, [c_int] * 5),
+    "nnueft_sparse_bwd_atomic_lds": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
+    "nnueft_double_bwd_atomic_lds": (
+        c_int, [c_void_p] * 6 + [c_float] + [c_void_p] * 6 + [c_int] * 5 + [c_void_p, c_size_t, c_void_p],
+    ),
     "nnueft_double_bwd_det": (
         c_int,
         [c_void_p] * 6 + [c_float] + [c_void_p] * 6 + [c_int] * 6 + [c_void_p, c_size_t, c_void_p, c_void_p, c_void_p],
@@ -90,6 +95,8 @@ PROTOTYPES = {
     "nnueft_ranger_lite_update_variance": (c_int, [c_void_p] * 2 + [c_longlong] + [c_float] * 2 + [c_void_p]),
     "nnueft_ranger_lite_lookahead_merge": (c_int, [c_void_p] * 2 + [c_longlong, c_float, c_void_p]),
 }
+
+E_UNSUPPORTED = -3   # NNUEFT_E_UNSUPPORTED of the header
 
 _lib = None
 _load_error = None

@@ -72,6 +72,17 @@ def _warn_once_about_xcds(lib, device) -> None:
                       "not used (results are the same, the gathers run two to three times slower)")
 
 
+# Rows from which the atomic backward adds in LDS tiles (narrower rows give an XCD too few column tiles to share).
+ATOMIC_LDS_MIN_COLS = 512
+
+
+def _atomic_lds_bytes(lib, B: int, K: int, num_rows: int, out_cols: int, n_persp: int, device) -> int:
+    """Workspace of the LDS-tiled atomic backward for this shape, 0 when it is not to be taken."""
+    if B <= 0 or out_cols < ATOMIC_LDS_MIN_COLS or lib.nnueft_device_xcds() != 8:
+        return 0
+    return int(lib.nnueft_atomic_lds_workspace_bytes(B, K, num_rows, out_cols, n_persp))
+
+
 # ------------------------------------------------------------------------------------------ sparse linear
 
 def sparse_fwd_impl(feature_indices: Tensor, weight: Tensor, bias: Tensor) -> Tensor:
@@ -114,13 +125,28 @@ def sparse_bwd_impl(feature_indices: Tensor, grad_output: Tensor, num_rows: int,
             )
             _native.check(rc, "nnueft_sparse_bwd_det")
         else:
+            # atomic adds in LDS tiles where the shape and the device can take them (rows of 512 columns and
+            # more; the gradient is then written, not accumulated), else atomics on the zeroed gradient
+            nbytes = _atomic_lds_bytes(lib, B, K, num_rows, out_cols, 1, device)
+            if nbytes:
+                weight_grad = torch.empty(num_rows, out_cols, dtype=torch.float32, device=device)
+                bias_grad = torch.empty(out_cols, dtype=torch.float32, device=device)
+                ws = workspace(nbytes, device)
+                rc = lib.nnueft_sparse_bwd_atomic_lds(
+                    feature_indices.data_ptr(), grad_output.data_ptr(), weight_grad.data_ptr(), bias_grad.data_ptr(),
+                    B, K, num_rows, out_cols, ws.data_ptr(), nbytes, stream_ptr(device),
+                )
+                if rc != _native.E_UNSUPPORTED:
+                    _native.check(rc, "nnueft_sparse_bwd_atomic_lds")
+                    return weight_grad, bias_grad
             weight_grad = torch.zeros(num_rows, out_cols, dtype=torch.float32, device=device)
             bias_grad = torch.zeros(out_cols, dtype=torch.float32, device=device)
-            rc = lib.nnueft_sparse_bwd_atomic(
-                feature_indices.data_ptr(), grad_output.data_ptr(), weight_grad.data_ptr(), bias_grad.data_ptr(),
-                B, K, num_rows, out_cols, stream_ptr(device),
-            )
-            _native.check(rc, "nnueft_sparse_bwd_atomic")
+            if B > 0:
+                rc = lib.nnueft_sparse_bwd_atomic(
+                    feature_indices.data_ptr(), grad_output.data_ptr(), weight_grad.data_ptr(), bias_grad.data_ptr(),
+                    B, K, num_rows, out_cols, stream_ptr(device),
+                )
+                _native.check(rc, "nnueft_sparse_bwd_atomic")
     return weight_grad, bias_grad
 
 
@@ -241,6 +267,18 @@ def double_bwd_impl(us: Tensor, them: Tensor, white_indices: Tensor, black_indic
             )
             _native.check(rc, "nnueft_double_bwd_det")
         else:
+            nbytes = _atomic_lds_bytes(lib, B, K, num_rows, output_size, 2, device)
+            if nbytes:
+                grad_weight = torch.empty(num_rows, output_size, dtype=torch.float32, device=device)
+                grad_bias = torch.empty(output_size, dtype=torch.float32, device=device)
+                ws = workspace(nbytes, device)
+                rc = lib.nnueft_double_bwd_atomic_lds(
+                    *head, grad_weight.data_ptr(), grad_bias.data_ptr(), B, K, num_rows, l1_size, n_psqt,
+                    ws.data_ptr(), nbytes, stream_ptr(device),
+                )
+                if rc != _native.E_UNSUPPORTED:
+                    _native.check(rc, "nnueft_double_bwd_atomic_lds")
+                    return grad_weight, grad_bias
             grad_weight = torch.zeros(num_rows, output_size, dtype=torch.float32, device=device)
             grad_bias = torch.zeros(output_size, dtype=torch.float32, device=device)
             if B > 0:

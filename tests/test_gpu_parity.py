@@ -100,6 +100,30 @@ def test_sparse_backward_atomic(oracle_cpu, B, out_cols, R, K):
     assert _rel_err(gb.cpu().numpy(), rb) <= 1e-4
 
 
+@pytest.mark.parametrize("B,out_cols,R,K", SPARSE_SHAPES + [(3000, 520, 1800, 32), (700, 1032, 768, 12)])
+def test_sparse_backward_atomic_in_lds_tiles(oracle_cpu, B, out_cols, R, K):
+    """nnueft_sparse_bwd_atomic_lds: the gradient is written (not accumulated), to the atomic bar; the bias
+    gradient is the deterministic one.  Shapes it does not take answer with 0 bytes and NNUEFT_E_UNSUPPORTED."""
+    c = sparse_case(250 + B, B, out_cols, R, K, allow_holes=True)
+    nat, lib = _native()
+    idx, g = _t(c["idx"]), _t(c["g"])
+    gW = torch.full((R, out_cols), float("nan"), device=_dev())
+    gb = torch.full((out_cols,), float("nan"), device=_dev())
+    nbytes = lib.nnueft_atomic_lds_workspace_bytes(B, K, R, out_cols, 1)
+    ws = torch.full((max(nbytes, 256),), 0xA5, dtype=torch.uint8, device=_dev())
+    rc = lib.nnueft_sparse_bwd_atomic_lds(idx.data_ptr(), g.data_ptr(), gW.data_ptr(), gb.data_ptr(), B, K, R, out_cols,
+                                          ws.data_ptr(), ws.numel(), _stream())
+    if nbytes == 0:
+        assert rc == nat.E_UNSUPPORTED and (K > 32 or out_cols % 4)
+        return
+    nat.check(rc, "sparse_bwd_atomic_lds")
+    rW, rb = oracle_cpu.sparse_bwd(c["idx"], c["g"], R, row_split=0)
+    assert _rel_err(gW.cpu().numpy(), rW) <= 1e-4
+    assert np.array_equal(gb.cpu().numpy(), rb)
+    assert lib.nnueft_sparse_bwd_atomic_lds(idx.data_ptr(), g.data_ptr(), gW.data_ptr(), gb.data_ptr(), B, K, R, out_cols,
+                                            ws.data_ptr(), nbytes - 1, _stream()) == -2
+
+
 @pytest.mark.parametrize("B,out_cols,R,K", SPARSE_SHAPES)
 def test_sparse_backward_deterministic(oracle_cpu, B, out_cols, R, K):
     c = sparse_case(300 + B, B, out_cols, R, K, allow_holes=True)
@@ -199,7 +223,7 @@ def test_double_forward(oracle_cpu, B, L1, R, K, kw, with_workspace):
         assert np.array_equal(got, ref)
 
 
-@pytest.mark.parametrize("mode", ["atomic", "deterministic"])
+@pytest.mark.parametrize("mode", ["atomic", "atomic_lds", "deterministic"])
 @pytest.mark.parametrize("B,L1,R,K,kw", DOUBLE_SHAPES)
 def test_double_backward(oracle_cpu, B, L1, R, K, kw, mode):
     c = double_case(500 + B, B, L1, R, K, **kw)
@@ -216,6 +240,20 @@ def test_double_backward(oracle_cpu, B, L1, R, K, kw, mode):
         gb = torch.zeros(out_cols, device=_dev())
         nat.check(lib.nnueft_double_bwd_atomic(*head, gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt, _stream()),
                   "double_bwd_atomic")
+    elif mode == "atomic_lds":
+        # the atomic adds in LDS tiles: every element written, twice on one workspace; shapes it does not
+        # take (lists longer than 32 slots, rows that are not whole 16-byte vectors) say so
+        nbytes = lib.nnueft_atomic_lds_workspace_bytes(B, K, R, out_cols, 2)
+        ws = torch.full((max(nbytes, 256),), 0xA5, dtype=torch.uint8, device=_dev())
+        for _ in range(2):
+            gW = torch.full((R, out_cols), float("nan"), device=_dev())
+            gb = torch.full((out_cols,), float("nan"), device=_dev())
+            rc = lib.nnueft_double_bwd_atomic_lds(*head, gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt, ws.data_ptr(),
+                                                  ws.numel(), _stream())
+            if nbytes == 0:
+                assert rc == nat.E_UNSUPPORTED and (K > 32 or out_cols % 4)
+                return
+            nat.check(rc, "double_bwd_atomic_lds")
     else:
         nbytes = lib.nnueft_det_workspace_bytes(B, K, R, out_cols, 2, RS(lib))
         ws = torch.empty(nbytes, dtype=torch.uint8, device=_dev())
@@ -250,6 +288,9 @@ def test_double_backward(oracle_cpu, B, L1, R, K, kw, mode):
     if mode == "atomic":
         assert _rel_err(gW, rW) <= 1e-4
         assert _rel_err(gb, rb) <= 1e-4
+    elif mode == "atomic_lds":
+        assert _rel_err(gW, rW) <= 1e-4
+        assert np.array_equal(gb, rb)   # its bias gradient is the deterministic one
     else:
         assert np.array_equal(gW, rW)
         assert np.array_equal(gb, rb)
