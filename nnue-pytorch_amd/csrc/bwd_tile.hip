@@ -66,14 +66,18 @@ struct Meta {
 };
 
 constexpr int kTaskPairs = 16;   // pairs a wave adds side by side: 4 lanes a pair
-constexpr int kBatchTasks = 64 / kTaskPairs;
+#ifndef NNUEFT_SCATTER_BATCH
+#define NNUEFT_SCATTER_BATCH 1
+#endif
+constexpr int kBatchTasks = NNUEFT_SCATTER_BATCH;   // tasks a wave takes per ticket (their pairs' facts are loaded a lane each)
+static_assert(kBatchTasks * kTaskPairs <= 64, "a lane per pair of a batch");
 
 __device__ __forceinline__ Meta load_meta(const BlockRec& rec, int tpc, int ntasks, int batch, int lane,
                                           const uint32_t* __restrict__ pidcnt, const uint16_t* __restrict__ loff,
                                           const uint32_t* __restrict__ cpool8) {
     Meta m{0u, 0u};
     const int t = batch * kBatchTasks + lane / kTaskPairs;
-    if (t < ntasks) {
+    if (t < ntasks && lane < kBatchTasks * kTaskPairs) {
         const int jc = t / tpc;
         const int local = (t - jc * tpc) * kTaskPairs + lane % kTaskPairs;
         if (local < ranks_of_chunk(rec.nb, jc, rec.nc)) {

@@ -435,7 +435,26 @@ __device__ __forceinline__ void acc_add(f4& a, const f4& r) {
 // saved[pair, columns of the tile] = chain from +0 over the pair's list, for every pair of the chunk.
 // VIRT: the table is W + V[row % kRows] (see merged4); the tile is merged on its way into LDS.  That variant
 // runs with 768 threads: the tile of V waits in registers beside the tile of W.
-template <int NT, bool VIRT, bool I16>
+// What the quantized forward does with a pair's sums when the gather finishes them itself (FUSE): + bias, clip,
+// product of column j with column j + L1/2, >> shift, one byte per column pair, written to the half of the
+// position's output row that the side to move selects.
+struct Fuse16 {
+    const uint8_t* stm;
+    const int16_t* b16;
+    uint8_t* out;
+    int clip_max, shift;
+};
+
+typedef unsigned int u2 __attribute__((ext_vector_type(2)));
+
+// 16 bytes of a row in the FUSE layout: four 16-bit columns at `lo` and the four that pair with them, L1/2 further on
+__device__ __forceinline__ f4 load_pair8(const char* lo, size_t half_bytes) {
+    const u2 a = *reinterpret_cast<const u2*>(lo);
+    const u2 b = *reinterpret_cast<const u2*>(lo + half_bytes);
+    return __builtin_bit_cast(f4, u4{a.x, a.y, b.x, b.y});
+}
+
+template <int NT, bool VIRT, bool I16, bool FUSE = false>
 __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ widx,
                                                           const int32_t* __restrict__ bidx,
                                                           const uint16_t* __restrict__ lists,
@@ -445,7 +464,8 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                                                           uint32_t* __restrict__ sched, const float* __restrict__ W,
                                                           float* __restrict__ acc, int B, int K, int R, int L1,
                                                           int out_cols, int tiles_per_xcd, int tile_group,
-                                                          VirtualTable vt, int block_rows) {
+                                                          VirtualTable vt, int block_rows, Fuse16 fz) {
+    static_assert(!FUSE || I16, "the fused epilogue belongs to the quantized table");
     extern __shared__ float4 lds_raw[];
     char* tb = reinterpret_cast<char*>(lds_raw);
     u4* lst = reinterpret_cast<u4*>(tb + kTileBytes);                                         // (kListCap + 32) * 2 bytes
@@ -464,9 +484,16 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
     const size_t w_pitch = I16 ? (size_t)L1 * 2 : (size_t)out_cols * 4;
     const size_t a_pitch = I16 ? (size_t)L1 * 2 : (size_t)L1 * 4;
     const char* Wb = reinterpret_cast<const char*>(W);
+    // FUSE: a tile row is 32 column pairs (j, j + L1/2): lane piece q holds columns 4q .. 4q+3 of the tile's 32 and
+    // their four partners, so the product needs no other lane
+    const size_t half_bytes = (size_t)L1;   // L1/2 columns of 2 bytes
     // the column tiles of this XCD, in groups of tile_group; a unit = (chunk, group)
     const int my_tiles = max(0, min(tiles_per_xcd, ntiles - x * tiles_per_xcd));
     const int groups = (my_tiles + tile_group - 1) / tile_group;
+    // FUSE: a unit's tiles are `groups` apart, so that the units (chunk, g), (chunk, g + 1), handed to two CUs one
+    // after the other, fetch the two halves of the same cache lines at about the same time (a tile row is two half
+    // lines there, and its neighbour tile holds the other halves)
+    const int qs = FUSE ? groups : 1;
     const int nunits = (int)sched[kXcd * 32] * groups;
     uint32_t* unit_ctr = sched + x * 32;
     const int g = lane >> 3, j = lane & 7;
@@ -481,8 +508,13 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
     {                                                       \
         const int ch_ = (u_) / groups;                      \
         C_ = chunks[ch_];                                   \
-        q0_ = ((u_) - ch_ * groups) * tile_group;           \
-        q1_ = min(q0_ + tile_group, my_tiles);              \
+        if (FUSE) {                                         \
+            q0_ = (u_) - ch_ * groups;                      \
+            q1_ = my_tiles;                                 \
+        } else {                                            \
+            q0_ = ((u_) - ch_ * groups) * tile_group;       \
+            q1_ = min(q0_ + tile_group, my_tiles);          \
+        }                                                   \
     }
 #define NNUEFT_LOAD_TILE(blk_, c_)                                                                       \
     {                                                                                                    \
@@ -492,6 +524,11 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
         _Pragma("unroll") for (int i = 0; i < IT; ++i) {                                                 \
             const int f = tid + i * NT;                                                                  \
             const int row = f >> 3;                                                                      \
+            if (FUSE)                                                                                    \
+                v[i] = row < rows_here_ ? load_pair8(Wb + (size_t)(row0_ + row) * w_pitch + (c_) * 64 +  \
+                                                     (f & 7) * 8, half_bytes)                            \
+                                        : f4{0.f, 0.f, 0.f, 0.f};                                        \
+            else                                                                                         \
             v[i] = row < rows_here_                                                                      \
                        ? *reinterpret_cast<const f4*>(src + (size_t)row * w_pitch + (f & 7) * 16)        \
                        : f4{0.f, 0.f, 0.f, 0.f};                                                         \
@@ -542,7 +579,7 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
         int nunit = nunits;
         Chunk Cn{};
         int qn0 = 0, qn1 = 0;
-        for (int q = q0; q < q1; ++q) {
+        for (int q = q0; q < q1; q += qs) {
             const int c = x * tiles_per_xcd + q;
             if (q != q0) __syncthreads();   // everyone is done reading the previous tile
 #pragma unroll
@@ -551,13 +588,15 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                 reinterpret_cast<f4*>(tb)[f] = VIRT ? merged4(v[i], vv[i], vt) : v[i];
             }
             if (tid == 0) ctr[0] = 0;
+            f4 bias8 = {0.f, 0.f, 0.f, 0.f};
+            if (FUSE) bias8 = load_pair8(reinterpret_cast<const char*>(fz.b16) + c * 64 + j * 8, half_bytes);
             __syncthreads();
             if (q == q0) {
                 nunit = __builtin_amdgcn_readfirstlane((int)ctr[1]);
                 if (nunit < nunits) NNUEFT_UNIT(nunit, Cn, qn0, qn1)
             }
-            if (q + 1 < q1) {
-                NNUEFT_LOAD_TILE(C.block, c + 1)
+            if (q + qs < q1) {
+                NNUEFT_LOAD_TILE(C.block, c + qs)
             } else if (nunit < nunits) {
                 NNUEFT_LOAD_TILE(Cn.block, x * tiles_per_xcd + qn0)
             }
@@ -574,6 +613,12 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                 const uint32_t field = pc >> 26;
                 const int pair = (int)(pc & 0x3ffffffu);
                 const int mx = __builtin_amdgcn_readfirstlane((int)field);   // lists are sorted longest first
+                // FUSE: which half of the output row the pair's bytes go to (asked for here, used after the sums)
+                int half = 0;
+                if (FUSE) {
+                    const int persp = pair >= B;
+                    half = persp == (fz.stm[pair - persp * B] ? 1 : 0) ? 0 : 1;   // half 0 shows the side to move
+                }
                 f4 a = {0.f, 0.f, 0.f, 0.f};
                 if (__ballot(field == kForeign) != 0) {
                     // some list of the task leaves its block: the wave's 8 pairs from global memory
@@ -581,7 +626,8 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                     for (int k = 0; k < K; ++k) {
                         const int r = ix[k];
                         if (r >= 0 && r < R) {
-                            f4 w = *reinterpret_cast<const f4*>(Wb + (size_t)r * w_pitch + c * kRowBytes + j * 16);
+                            f4 w = FUSE ? load_pair8(Wb + (size_t)r * w_pitch + c * 64 + j * 8, half_bytes)
+                                        : *reinterpret_cast<const f4*>(Wb + (size_t)r * w_pitch + c * kRowBytes + j * 16);
                             if (VIRT)
                                 w = merged4(w, *reinterpret_cast<const f4*>(vt.V + (size_t)(r % kRows) * out_cols +
                                                                             c * kTileCols + j * 4), vt);
@@ -617,7 +663,24 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                         }
                     }
                 }
-                if (valid)
+                if (FUSE) {
+                    acc_add<true>(a, bias8);
+                    const us8 s8 = __builtin_bit_cast(us8, a);
+                    uint32_t o4 = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int c0 = min(max((int)(short)s8[e], 0), fz.clip_max);
+                        const int c1 = min(max((int)(short)s8[e + 4], 0), fz.clip_max);
+                        o4 |= ((uint32_t)((c0 * c1) >> fz.shift) & 0xffu) << (8 * e);
+                    }
+                    if (valid) {
+                        const int pos = pair >= B ? pair - B : pair;
+                        // streaming store: 32 bytes a pair and tile, written once (measured 0.43 against 0.455 ms
+                        // for the whole forward at B = 65536 with a plain store)
+                        __builtin_nontemporal_store(o4, reinterpret_cast<uint32_t*>(fz.out + (size_t)pos * L1 + (size_t)half * (L1 >> 1) +
+                                                                                 c * 32 + j * 4));
+                    }
+                } else if (valid)
                     __builtin_nontemporal_store(a, reinterpret_cast<f4*>(reinterpret_cast<char*>(acc) + (size_t)pair * a_pitch +
                                                                          c * kRowBytes + j * 16));
                 task = __builtin_amdgcn_readfirstlane(nxt);
@@ -646,7 +709,7 @@ int allow_lds(int device) {
         e = hipFuncSetAttribute((const void*)k_acc_tile<kAccThreadsVirtual, true, false>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
     if (e == hipSuccess)
-        e = hipFuncSetAttribute((const void*)k_acc_tile<kAccThreads, false, true>,
+        e = hipFuncSetAttribute((const void*)k_acc_tile<kAccThreads, false, true, true>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
     if (e != hipSuccess) return (int)e;
     g_lds_allowed[device].store(1, std::memory_order_release);
@@ -683,7 +746,8 @@ int launch_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, c
 // Sort of the lists and the gather of every pair's row sums into `sums` ([2, B, L1] floats, or with `i16` 16-bit
 // integers over a table W of [R, L1] int16).
 static int gather_tile(const int32_t* widx, const int32_t* bidx, const void* W, void* sums, int B, int K, int R, int L1,
-                       int out_cols, void* ws, hipStream_t st, VirtualTable vt, bool i16, int block_rows = kRows) {
+                       int out_cols, void* ws, hipStream_t st, VirtualTable vt, bool i16, int block_rows = kRows,
+                       Fuse16 fz = Fuse16{nullptr, nullptr, nullptr, 0, 0}) {
     Layout L;
     if (!layout(2 * B, R, &L, block_rows)) return NNUEFT_E_UNSUPPORTED;
     int device = 0;
@@ -711,18 +775,20 @@ static int gather_tile(const int32_t* widx, const int32_t* bidx, const void* W, 
     const int grid = info->cus / kXcd * kXcd;
     const float* Wf = (const float*)W;
     float* sf = (float*)sums;
-    if (i16)
-        hipLaunchKernelGGL((k_acc_tile<kAccThreads, false, true>), dim3(grid), dim3(kAccThreads), kLdsBytes, st, widx, bidx,
-                           lists, pidcnt, loff, chunks, sched, Wf, sf, B, K, R, L1, out_cols, tiles_per_xcd,
-                           tile_group, vt, L.block_rows);
+    if (i16 && fz.out)
+        hipLaunchKernelGGL((k_acc_tile<kAccThreads, false, true, true>), dim3(grid), dim3(kAccThreads), kLdsBytes, st, widx,
+                           bidx, lists, pidcnt, loff, chunks, sched, Wf, sf, B, K, R, L1, out_cols, tiles_per_xcd,
+                           tile_group, vt, L.block_rows, fz);
+    else if (i16)
+        return NNUEFT_E_ARG;   // the quantized table is only gathered with the fused epilogue
     else if (vt.V)
         hipLaunchKernelGGL((k_acc_tile<kAccThreadsVirtual, true, false>), dim3(grid), dim3(kAccThreadsVirtual), kLdsBytes, st,
                            widx, bidx, lists, pidcnt, loff, chunks, sched, Wf, sf, B, K, R, L1, out_cols, tiles_per_xcd,
-                           tile_group, vt, L.block_rows);
+                           tile_group, vt, L.block_rows, fz);
     else
         hipLaunchKernelGGL((k_acc_tile<kAccThreads, false, false>), dim3(grid), dim3(kAccThreads), kLdsBytes, st, widx, bidx,
                            lists, pidcnt, loff, chunks, sched, Wf, sf, B, K, R, L1, out_cols, tiles_per_xcd,
-                           tile_group, vt, L.block_rows);
+                           tile_group, vt, L.block_rows, fz);
     NNUEFT_LAUNCH_CHECK();
     return 0;
 }
@@ -748,10 +814,11 @@ size_t workspace_int16(int B, int R, int block_rows) {
     return B < (1 << 25) && layout(2 * B, R, &L, block_rows) ? L.end : 0;
 }
 
-int int16_sums_tile(const int32_t* widx, const int32_t* bidx, const int16_t* W16, int16_t* sums, int B, int K, int R,
-                    int L1, int block_rows, void* ws, hipStream_t st) {
-    return gather_tile(widx, bidx, W16, sums, B, K, R, L1, L1, ws, st, VirtualTable{nullptr, 1.0f, 1.0f, 0, 0.0f}, true,
-                       block_rows);
+int int16_fused_tile(const int32_t* widx, const int32_t* bidx, const uint8_t* stm, const int16_t* W16, const int16_t* b16,
+                     uint8_t* out_u8, int B, int K, int R, int L1, int clip_max, int shift, int block_rows, void* ws,
+                     hipStream_t st) {
+    return gather_tile(widx, bidx, W16, nullptr, B, K, R, L1, L1, ws, st, VirtualTable{nullptr, 1.0f, 1.0f, 0, 0.0f}, true,
+                       block_rows, Fuse16{stm, b16, out_u8, clip_max, shift});
 }
 
 }  // namespace nnueft_tile

@@ -12,9 +12,9 @@
 //                         read back, side-to-move order, clip, product, u8 store; psqt sums
 //   LDS-tiled (workspace, table blocks of 768 rows, L1 a multiple of 64, lists of 32 slots at most): the
 //                         forward's gather out of LDS tiles (fwd_tile.hip) over the int16 table
-//       k_acc_tile        sums[2, B, L1] int16 for both lists of every position
-//       k_mix16           wave per (position, paired slice): + b16, side-to-move order, clip, product, u8
-//                         store; psqt sums
+//       k_acc_tile        a tile is 32 column pairs (j, j + L1/2): the sums of a pair and tile stay in registers and
+//                         leave as 32 output bytes (+ b16, clip, product >> shift) in the half the side to move selects
+//       k_psqt16          the psqt difference of every position
 #include "internal.h"
 
 namespace {
@@ -284,43 +284,35 @@ __global__ __launch_bounds__(64) void k_black_mix16(const int32_t* __restrict__ 
     }
 }
 
-// The output bytes of a position from the two lists' row sums (without the bias) that the LDS-tiled gather left.
-__global__ __launch_bounds__(64) void k_mix16(const int32_t* __restrict__ widx, const int32_t* __restrict__ bidx,
-                                              const uint8_t* __restrict__ stm, const int16_t* __restrict__ b16,
-                                              const int16_t* __restrict__ sums, const int32_t* __restrict__ psqt32,
-                                              const int64_t* __restrict__ psqt_idx, uint8_t* __restrict__ out_u8,
-                                              int32_t* __restrict__ psqt_out, int B, int K, int R, int L1, int n_psqt,
-                                              int clip_max, int shift, int nslices) {
-    const int lane = threadIdx.x;
-    const int b = blockIdx.x / nslices;
-    const int s = blockIdx.x - b * nslices;
-    const int h = L1 >> 1;
-    const int first = stm[b] ? 1 : 0;
-    if (s == 0) psqt_diff(widx, bidx, psqt32, psqt_idx[b], first, b, K, R, n_psqt, lane, psqt_out);
-    const int q = s * 64 + lane;
-    if (q >= h / 8) return;
-    const int c0 = q * 8, c1 = c0 + h;
-    const vecs<8> bias0 = ldi<8>(b16 + c0), bias1 = ldi<8>(b16 + c1);
-    vecs<8> w0 = ldi<8>(sums + (size_t)b * L1 + c0), w1 = ldi<8>(sums + (size_t)b * L1 + c1);
-    vecs<8> k0 = ldi<8>(sums + ((size_t)B + b) * L1 + c0), k1 = ldi<8>(sums + ((size_t)B + b) * L1 + c1);
-    iadd<8>(w0, bias0);
-    iadd<8>(w1, bias1);
-    iadd<8>(k0, bias0);
-    iadd<8>(k1, bias1);
-    uint8_t* dst = out_u8 + (size_t)b * L1;
-    // output half 0 shows the side to move, half 1 the other side
-    if (first) {
-        pair_product_store<8>(dst + c0, k0, k1, clip_max, shift);
-        pair_product_store<8>(dst + h + c0, w0, w1, clip_max, shift);
-    } else {
-        pair_product_store<8>(dst + c0, w0, w1, clip_max, shift);
-        pair_product_store<8>(dst + h + c0, k0, k1, clip_max, shift);
+// psqt_out of a position on its own (the LDS-tiled path finishes the output bytes inside its gather): four
+// positions a workgroup, a wave each, the white list on lanes 0 .. 31 and the black one on lanes 32 .. 63.
+__global__ __launch_bounds__(256) void k_psqt16(const int32_t* __restrict__ widx, const int32_t* __restrict__ bidx,
+                                                const uint8_t* __restrict__ stm, const int32_t* __restrict__ psqt32,
+                                                const int64_t* __restrict__ psqt_idx, int32_t* __restrict__ psqt_out,
+                                                int B, int K, int R, int n_psqt) {
+    const int lane = threadIdx.x & 63;
+    const int b = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (b >= B) return;
+    const int64_t pi = psqt_idx[b];
+    const int p = lane >> 5;
+    uint32_t ps = 0u;
+    if (pi >= 0 && pi < n_psqt) {
+        const int32_t* ix = (p ? bidx : widx) + (size_t)b * K;
+        for (int k = lane & 31; k < K; k += 32) {
+            const int r = ix[k];
+            if (r >= 0 && r < R) ps += (uint32_t)psqt32[(size_t)r * n_psqt + pi];
+        }
     }
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) ps += (uint32_t)__shfl_xor((int)ps, off);
+    const uint32_t white = (uint32_t)__shfl((int)ps, 0), black = (uint32_t)__shfl((int)ps, 32);
+    // (sum over the mover's list - sum over the other list) / 2
+    if (lane == 0) psqt_out[b] = (int32_t)(stm[b] ? black - white : white - black) / 2;
 }
 
 struct Int16Layout {
     size_t accW, sort, end;
-    size_t tile_sums, tile_sort;   // the LDS-tiled path's view of the same bytes
+    size_t tile_sort;              // the LDS-tiled path's view of the same bytes: its sort scratch
     bool tile_ok;                  // the table's blocks fit its tiles
 };
 
@@ -334,9 +326,8 @@ bool int16_layout(int B, int R, int L1, int block_rows, Int16Layout* L) {
     L->sort = off;
     off += up256(nnueft_blocked::pair_sort_workspace(B, R, block_rows));
     L->end = off;
-    // the LDS-tiled path keeps both lists' sums and its own sort scratch
-    L->tile_sums = 0;
-    L->tile_sort = up256((size_t)2 * B * L1 * sizeof(int16_t));
+    // the LDS-tiled path needs its sort scratch only: the sums never leave the gather
+    L->tile_sort = 0;
     const int br = block_rows > 0 ? block_rows : nnueft_tile::kBlockRows;
     const size_t tile_ws = br <= nnueft_tile::kBlockRows ? nnueft_tile::workspace_int16(B, R, br) : 0;
     L->tile_ok = tile_ws > 0;
@@ -391,15 +382,13 @@ extern "C" int nnueft_ft_int16_fwd(const int32_t* widx, const int32_t* bidx, con
         const int br = table_block_rows > 0 ? table_block_rows : nnueft_tile::kBlockRows;
         if (vec && L.tile_ok && nnueft_tile::fits_int16(*info, B, K, R, L1, br)) {
             char* ws = (char*)workspace;
-            int16_t* sums = (int16_t*)(ws + L.tile_sums);
-            const int rc = nnueft_tile::int16_sums_tile(widx, bidx, W16, sums, B, K, R, L1, br, ws + L.tile_sort, st);
-            if (rc) return rc;
-            const int nslices = max(1, (L1 / 16 + 63) / 64);
-            if ((long long)B * nslices > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
-            hipLaunchKernelGGL(k_mix16, dim3((unsigned)(B * nslices)), dim3(64), 0, st, widx, bidx, stm, b16, sums, psqt32,
-                               psqt_idx, out_u8, psqt_out, B, K, R, L1, n_psqt, clip_max, shift, nslices);
+            // an output half depends on one list's sums only, so the gather finishes the bytes itself (32 column
+            // pairs a tile) and no sums pass through memory; the psqt difference is a kernel of its own
+            hipLaunchKernelGGL(k_psqt16, dim3((unsigned)((B + 3) / 4)), dim3(256), 0, st, widx, bidx, stm, psqt32, psqt_idx,
+                               psqt_out, B, K, R, n_psqt);
             NNUEFT_LAUNCH_CHECK();
-            return 0;
+            return nnueft_tile::int16_fused_tile(widx, bidx, stm, W16, b16, out_u8, B, K, R, L1, clip_max, shift, br,
+                                                 ws + L.tile_sort, st);
         }
         if (vec && (long long)B <= 0x3fffffffLL && nnueft_blocked::blocked_layout_fits(*info)) {
             char* ws = (char*)workspace;
