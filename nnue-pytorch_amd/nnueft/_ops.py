@@ -12,7 +12,14 @@ of a step at the reference's micro-benchmark shape).
   nnueft::sparse_fwd   nnueft_sparse_fwd
   nnueft::sparse_bwd   nnueft_sparse_bwd_{atomic,det}
   nnueft::double_fwd   nnueft_double_fwd / nnueft_double_fwd_act
-  nnueft::double_bwd   nnueft_double_bwd_{atomic,det}
+  nnueft::double_bwd   nnueft_double_bwd_{atomic,atomic_lds,det}
+
+and what ComposedFeatureTransformer launches around the operator, so that the module compiles as one graph too:
+
+  nnueft::double_fwd_virtual   nnueft_double_fwd_virtual (real + virtual weights merged inside the gather)
+  nnueft::table_merge          nnueft_table_merge
+  nnueft::table_virtual_grad   nnueft_table_virtual_grad
+  nnueft::act_fake_quantize    nnueft_act_fake_quantize
 """
 from typing import Optional, Tuple
 
@@ -299,13 +306,120 @@ def _(us, them, white_indices, black_indices, psqt_indices, bias, max_ft_activat
     return grad_l0.new_empty(num_rows, output_size), grad_l0.new_empty(output_size)
 
 
+# ------------------------------------------------------------------------------------------ module layer
+
+def double_fwd_virtual_impl(us: Tensor, them: Tensor, white_indices: Tensor, black_indices: Tensor, psqt_indices: Tensor,
+                            weight: Tensor, virtual: Tensor, bias: Tensor, max_ft_activation: float, l1_size: int,
+                            scale_ft: float, scale_psqt: float, quantize: bool, act_on: bool, act_scale: float,
+                            act_eps: float, act_post_mul: float) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+    """double_fwd over the table q(weight + virtual[row % virtual rows]) without that table being written."""
+    lib = _native.load()
+    device = weight.device
+    B, K = white_indices.shape
+    R, cols = weight.shape
+    l0_ = torch.empty(B, l1_size, dtype=torch.float32, device=device)
+    wpsqt = torch.empty(B, 1, dtype=torch.float32, device=device)
+    bpsqt = torch.empty(B, 1, dtype=torch.float32, device=device)
+    row_sums = torch.empty(2, B, l1_size, dtype=torch.float32, device=device)
+    with torch.cuda.device(device):
+        nbytes = lib.nnueft_fwd_workspace_bytes(B, K, R, l1_size, cols - l1_size)
+        ws = workspace(nbytes, device)
+        rc = lib.nnueft_double_fwd_virtual(
+            us.data_ptr(), them.data_ptr(), white_indices.data_ptr(), black_indices.data_ptr(),
+            psqt_indices.data_ptr(), weight.data_ptr(), virtual.data_ptr(), bias.data_ptr(), float(max_ft_activation),
+            l0_.data_ptr(), wpsqt.data_ptr(), bpsqt.data_ptr(), row_sums.data_ptr(), B, K, R, l1_size,
+            cols - l1_size, virtual.shape[0], float(scale_ft), float(scale_psqt), int(bool(quantize)),
+            ws.data_ptr(), nbytes, int(bool(act_on)), float(act_scale), float(act_eps), float(act_post_mul),
+            stream_ptr(device))
+    _native.check(rc, "nnueft_double_fwd_virtual")
+    return l0_, wpsqt, bpsqt, row_sums
+
+
+double_fwd_virtual = torch.library.custom_op("nnueft::double_fwd_virtual", double_fwd_virtual_impl, mutates_args=(),
+                                             device_types="cuda")
+
+
+@double_fwd_virtual.register_fake
+def _(us, them, white_indices, black_indices, psqt_indices, weight, virtual, bias, max_ft_activation, l1_size, scale_ft,
+      scale_psqt, quantize, act_on, act_scale, act_eps, act_post_mul):
+    B = white_indices.shape[0]
+    return (weight.new_empty(B, l1_size), weight.new_empty(B, 1), weight.new_empty(B, 1),
+            weight.new_empty(2, B, l1_size))
+
+
+def table_merge_impl(weight: Tensor, virtual: Optional[Tensor], l1_size: int, scale_ft: float, scale_psqt: float,
+                     quantize: bool) -> Tensor:
+    """q(weight + virtual[row % virtual rows]) in one pass (virtual None: the grid alone)."""
+    lib = _native.load()
+    R, cols = weight.shape
+    merged = torch.empty_like(weight)
+    with torch.cuda.device(weight.device):
+        rc = lib.nnueft_table_merge(weight.data_ptr(), None if virtual is None else virtual.data_ptr(),
+                                    merged.data_ptr(), R, cols, l1_size, 1 if virtual is None else virtual.shape[0],
+                                    float(scale_ft), float(scale_psqt), int(bool(quantize)), stream_ptr(weight.device))
+    _native.check(rc, "nnueft_table_merge")
+    return merged
+
+
+table_merge = torch.library.custom_op("nnueft::table_merge", table_merge_impl, mutates_args=(), device_types="cuda")
+
+
+@table_merge.register_fake
+def _(weight, virtual, l1_size, scale_ft, scale_psqt, quantize):
+    return torch.empty_like(weight)
+
+
+def table_virtual_grad_impl(grad: Tensor, vrows: int) -> Tensor:
+    """The gradient of the virtual rows: the sum of the table's blocks of `vrows` rows."""
+    lib = _native.load()
+    R, cols = grad.shape
+    gv = torch.empty(vrows, cols, dtype=grad.dtype, device=grad.device)
+    with torch.cuda.device(grad.device):
+        rc = lib.nnueft_table_virtual_grad(grad.data_ptr(), gv.data_ptr(), R, cols, vrows, stream_ptr(grad.device))
+    _native.check(rc, "nnueft_table_virtual_grad")
+    return gv
+
+
+table_virtual_grad = torch.library.custom_op("nnueft::table_virtual_grad", table_virtual_grad_impl, mutates_args=(),
+                                             device_types="cuda")
+
+
+@table_virtual_grad.register_fake
+def _(grad, vrows):
+    return grad.new_empty(vrows, grad.shape[1])
+
+
+def act_fake_quantize_impl(x: Tensor, scale: float, eps: float, post_mul: float) -> Tensor:
+    """(floor(x * scale + eps) / scale) * post_mul in one pass."""
+    lib = _native.load()
+    out = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        rc = lib.nnueft_act_fake_quantize(x.data_ptr(), out.data_ptr(), x.numel(), float(scale), float(eps),
+                                          float(post_mul), stream_ptr(x.device))
+    _native.check(rc, "nnueft_act_fake_quantize")
+    return out
+
+
+act_fake_quantize = torch.library.custom_op("nnueft::act_fake_quantize", act_fake_quantize_impl, mutates_args=(),
+                                            device_types="cuda")
+
+
+@act_fake_quantize.register_fake
+def _(x, scale, eps, post_mul):
+    return torch.empty_like(x)
+
+
 _IMPLS = {"sparse_fwd": sparse_fwd_impl, "sparse_bwd": sparse_bwd_impl, "double_fwd": double_fwd_impl,
-          "det_sort": det_sort_impl, "double_bwd": double_bwd_impl}
+          "det_sort": det_sort_impl, "double_bwd": double_bwd_impl, "double_fwd_virtual": double_fwd_virtual_impl,
+          "table_merge": table_merge_impl, "table_virtual_grad": table_virtual_grad_impl,
+          "act_fake_quantize": act_fake_quantize_impl}
 
 
 _OPS = {"sparse_fwd": torch.ops.nnueft.sparse_fwd, "sparse_bwd": torch.ops.nnueft.sparse_bwd,
         "double_fwd": torch.ops.nnueft.double_fwd, "det_sort": torch.ops.nnueft.det_sort,
-        "double_bwd": torch.ops.nnueft.double_bwd}
+        "double_bwd": torch.ops.nnueft.double_bwd, "double_fwd_virtual": torch.ops.nnueft.double_fwd_virtual,
+        "table_merge": torch.ops.nnueft.table_merge, "table_virtual_grad": torch.ops.nnueft.table_virtual_grad,
+        "act_fake_quantize": torch.ops.nnueft.act_fake_quantize}
 
 
 def launch(name: str, *args):

@@ -24,7 +24,7 @@ import torch
 import torch.nn.functional as F
 from torch import nn
 
-from . import _native
+from . import _native, _ops
 from . import halfka_v2_hm as hk
 from .double_ft_functions import double_feature_transform
 from .fused_ft_functions import FusedDoubleFtFunction
@@ -207,35 +207,18 @@ def get_feature_cls(name: str):
 
 # ------------------------------------------------------------------------------------------ FT module
 
-@torch.compiler.disable(recursive=False)
 def _launch_table_merge(weight, virtual, l1_size, scale_ft, scale_psqt, quantize):
-    lib = _native.load()
-    R, cols = weight.shape
-    merged = torch.empty_like(weight)
-    with torch.cuda.device(weight.device):
-        rc = lib.nnueft_table_merge(weight.data_ptr(), None if virtual is None else virtual.data_ptr(),
-                                    merged.data_ptr(), R, cols, l1_size, 1 if virtual is None else virtual.shape[0],
-                                    float(scale_ft), float(scale_psqt), int(bool(quantize)),
-                                    _stream_ptr(weight.device))
-    _native.check(rc, "nnueft_table_merge")
-    return merged
+    return _ops.launch("table_merge", weight, virtual, int(l1_size), float(scale_ft), float(scale_psqt), bool(quantize))
 
 
-@torch.compiler.disable(recursive=False)
 def _launch_table_virtual_grad(grad, vrows):
-    lib = _native.load()
-    R, cols = grad.shape
-    gv = torch.empty(vrows, cols, dtype=grad.dtype, device=grad.device)
-    with torch.cuda.device(grad.device):
-        rc = lib.nnueft_table_virtual_grad(grad.data_ptr(), gv.data_ptr(), R, cols, vrows, _stream_ptr(grad.device))
-    _native.check(rc, "nnueft_table_virtual_grad")
-    return gv
+    return _ops.launch("table_virtual_grad", grad, int(vrows))
 
 
 class _TableMerge(torch.autograd.Function):
     """merged = q(weight + virtual[row % 768]) in one pass; STE gradient: weight gets the incoming
-    gradient itself, virtual its sum over the table blocks.  The launches sit in functions dynamo
-    does not trace (it would choke on data_ptr() and the raw stream handle)."""
+    gradient itself, virtual its sum over the table blocks.  The launches are torch custom ops
+    (nnueft/_ops.py), so a compiled graph keeps them inside."""
 
     @staticmethod
     def forward(ctx, weight, virtual, l1_size, scale_ft, scale_psqt, quantize):
@@ -261,41 +244,31 @@ def _table_merge(weight, virtual, l1_size, scale_ft, scale_psqt, quantize):
 FOLD_TABLE_MERGE = True
 
 
-@torch.compiler.disable(recursive=False)
-def _virtual_forward_fits(white_indices, weight, virtual, l1_size) -> bool:
-    if not (FOLD_TABLE_MERGE and weight.is_cuda and _native.available()):
+@torch.compiler.assume_constant_result
+def _virtual_fits(B: int, K: int, R: int, l1_size: int, n_psqt: int, vrows: int, device_index: int) -> bool:
+    """Whether the library can merge the virtual weights inside its forward for these sizes on that device: a
+    host-side question about shapes and the device, so a traced graph takes the answer as a constant."""
+    if not (FOLD_TABLE_MERGE and _native.available()) or B <= 0:
         return False
-    lib = _native.load()
+    with torch.cuda.device(device_index):
+        return _native.load().nnueft_double_fwd_virtual_fits(B, K, R, l1_size, n_psqt, vrows) == 1
+
+
+def _virtual_forward_fits(white_indices, weight, virtual, l1_size) -> bool:
+    if not weight.is_cuda:
+        return False
     B, K = white_indices.shape
     R, cols = weight.shape
-    with torch.cuda.device(weight.device):
-        return B > 0 and lib.nnueft_double_fwd_virtual_fits(B, K, R, l1_size, cols - l1_size, virtual.shape[0]) == 1
+    index = weight.device.index if weight.device.index is not None else torch.cuda.current_device()
+    return _virtual_fits(int(B), int(K), int(R), int(l1_size), int(cols - l1_size), int(virtual.shape[0]), int(index))
 
 
-@torch.compiler.disable(recursive=False)
 def _launch_double_fwd_virtual(us, them, white_indices, black_indices, psqt_indices, weight, virtual, bias,
                                max_ft_activation, l1_size, scale_ft, scale_psqt, quantize, act_grid):
-    lib = _native.load()
-    device = weight.device
-    B, K = white_indices.shape
-    R, cols = weight.shape
-    l0_ = torch.empty(B, l1_size, dtype=torch.float32, device=device)
-    wpsqt = torch.empty(B, 1, dtype=torch.float32, device=device)
-    bpsqt = torch.empty(B, 1, dtype=torch.float32, device=device)
-    row_sums = torch.empty(2, B, l1_size, dtype=torch.float32, device=device)
     act = act_grid if act_grid is not None else (1.0, 0.0, 1.0)
-    with torch.cuda.device(device):
-        nbytes = lib.nnueft_fwd_workspace_bytes(B, K, R, l1_size, cols - l1_size)
-        ws = torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
-        rc = lib.nnueft_double_fwd_virtual(
-            us.data_ptr(), them.data_ptr(), white_indices.data_ptr(), black_indices.data_ptr(),
-            psqt_indices.data_ptr(), weight.data_ptr(), virtual.data_ptr(), bias.data_ptr(), float(max_ft_activation),
-            l0_.data_ptr(), wpsqt.data_ptr(), bpsqt.data_ptr(), row_sums.data_ptr(), B, K, R, l1_size,
-            cols - l1_size, virtual.shape[0], float(scale_ft), float(scale_psqt), int(bool(quantize)),
-            ws.data_ptr(), nbytes, int(act_grid is not None), float(act[0]), float(act[1]), float(act[2]),
-            _stream_ptr(device))
-    _native.check(rc, "nnueft_double_fwd_virtual")
-    return l0_, wpsqt, bpsqt, row_sums
+    return _ops.launch("double_fwd_virtual", us, them, white_indices, black_indices, psqt_indices, weight, virtual, bias,
+                       float(max_ft_activation), int(l1_size), float(scale_ft), float(scale_psqt), bool(quantize),
+                       act_grid is not None, float(act[0]), float(act[1]), float(act[2]))
 
 
 class _FusedDoubleFtVirtual(torch.autograd.Function):
@@ -328,7 +301,6 @@ class _FusedDoubleFtVirtual(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_l0, grad_wpsqt, grad_bpsqt):
-        from . import _ops
 
         us, them, white_indices, black_indices, psqt_indices, bias, row_sums = ctx.saved_tensors
         if ctx.act_grid is not None and ctx.act_grid[2] != 1.0:
@@ -342,15 +314,8 @@ class _FusedDoubleFtVirtual(torch.autograd.Function):
         return (None, None, None, None, None, grad_weight, grad_virtual, grad_bias, None, None, None, None, None, None)
 
 
-@torch.compiler.disable(recursive=False)
 def _launch_act_fake_quantize(x, scale, post_mul):
-    lib = _native.load()
-    out = torch.empty_like(x)
-    with torch.cuda.device(x.device):
-        rc = lib.nnueft_act_fake_quantize(x.data_ptr(), out.data_ptr(), x.numel(), float(scale),
-                                          float(FAKE_QUANTIZE_EPS), float(post_mul), _stream_ptr(x.device))
-    _native.check(rc, "nnueft_act_fake_quantize")
-    return out
+    return _ops.launch("act_fake_quantize", x, float(scale), float(FAKE_QUANTIZE_EPS), float(post_mul))
 
 
 class _ActFakeQuantize(torch.autograd.Function):

@@ -392,7 +392,8 @@ FULL = [(1024, 8192), (128, 16384), (3072, 16384)]   # BASELINE.json configs 1-3
 
 @pytest.mark.parametrize("L1,B", FULL)
 def test_baseline_configs_full_size_against_oracle(oracle_cpu, L1, B):
-    """fwd bit-exact, deterministic backward bit-exact, atomic backward 1e-4 relative, at full size."""
+    """fwd bit-exact, both deterministic orders bit-exact (the strict one is the reference CPU path's), atomic
+    backward 1e-4 relative, at full size."""
     n_psqt, R = 8, hk.NUM_INPUTS
     us, them, white, black, pc = hk.synthetic_batch(B, 1234 + L1)
     psqt_idx = (pc - 1) // 4
@@ -405,10 +406,13 @@ def test_baseline_configs_full_size_against_oracle(oracle_cpu, L1, B):
     r_l0, r_wp, r_bp, r_saved = oracle_cpu.double_fwd(us, them, white, black, psqt_idx, Wn, bn, max_act, L1)
     r_gW, r_gb = oracle_cpu.double_bwd(us, them, white, black, psqt_idx, bn, max_act, grads[0], grads[1], grads[2],
                                        r_saved, R, n_psqt)
+    s_gW, s_gb = oracle_cpu.double_bwd(us, them, white, black, psqt_idx, bn, max_act, grads[0], grads[1], grads[2],
+                                       r_saved, R, n_psqt, row_split=0)
+    assert not np.array_equal(s_gW, r_gW)   # the two orders differ on the rows named beyond the split threshold
     t = lambda a: torch.from_numpy(a).to(DEV)
     args = [t(us), t(them), t(white), t(black), t(psqt_idx)]
     det = None
-    for mode in ("deterministic", "atomic", "deterministic"):
+    for mode in ("deterministic", "atomic", "deterministic_strict", "deterministic"):
         nnueft.set_backward_mode(mode)
         W = t(Wn).requires_grad_()
         bias = t(bn).requires_grad_()
@@ -424,6 +428,9 @@ def test_baseline_configs_full_size_against_oracle(oracle_cpu, L1, B):
             if det is not None:          # run to run
                 assert np.array_equal(gW, det[0]) and np.array_equal(gb, det[1])
             det = (gW, gb)
+        elif mode == "deterministic_strict":
+            assert np.array_equal(gW, s_gW)
+            assert np.array_equal(gb, s_gb)
         else:
             assert np.abs(gW - r_gW).max() <= 1e-4 * np.abs(r_gW).max()
             assert np.abs(gb - r_gb).max() <= 1e-4 * np.abs(r_gb).max()

@@ -159,6 +159,8 @@ DOUBLE_SHAPES = [
     (1500, 512, 1000, 20, dict(allow_holes=True)),   # K < 32, holes, a last block of 232 rows
     (2000, 576, 768, 32, dict(n_psqt=0)),      # one block, five chunks (as many as hold its list entries)
     (3500, 512, 768, 8, dict(n_psqt=0)),       # one block of short lists, five chunks (1536 pairs each at most)
+    (500, 512, 2000, 30, {}),                  # K not a multiple of 4: the sort reads the lists entry by entry
+    (300, 512, 50000, 32, {}),                 # 66 table blocks, more than the LDS-tiled kernels index: L2-blocked path
 ]
 
 
@@ -223,6 +225,68 @@ def test_double_forward(oracle_cpu, B, L1, R, K, kw, with_workspace):
         assert np.array_equal(got, ref)
 
 
+def test_double_forward_from_index_lists_that_are_not_16_byte_aligned(oracle_cpu):
+    """Index tensors that begin 4 bytes past a 16-byte boundary (a view into a larger buffer): the sort of the
+    LDS-tiled forward then reads the lists entry by entry; same bits."""
+    B, L1, R, K = 600, 512, 24576, 32
+    c = double_case(77, B, L1, R, K, halfka=True, weight_scale=0.05, max_act=255 / 256)
+    nat, lib = _native()
+    d = {k: _t(c[k]) for k in ("us", "them", "psqt_idx", "W", "bias")}
+    bufs = []
+    for name in ("widx", "bidx"):
+        buf = torch.empty(B * K + 1, dtype=torch.int32, device=_dev())
+        buf[1:] = _t(c[name]).reshape(-1)
+        assert buf[1:].data_ptr() % 16 == 4
+        bufs.append(buf)
+    n_psqt = c["n_psqt"]
+    l0 = torch.full((B, L1), float("nan"), device=_dev())
+    wp = torch.empty(B, 1, device=_dev())
+    bp = torch.empty(B, 1, device=_dev())
+    saved = torch.full((2, B, L1), float("nan"), device=_dev())
+    nbytes = lib.nnueft_fwd_workspace_bytes(B, K, R, L1, n_psqt)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=_dev())
+    nat.check(lib.nnueft_double_fwd(d["us"].data_ptr(), d["them"].data_ptr(), bufs[0][1:].data_ptr(), bufs[1][1:].data_ptr(),
+                                    d["psqt_idx"].data_ptr(), d["W"].data_ptr(), d["bias"].data_ptr(), c["max_act"],
+                                    l0.data_ptr(), wp.data_ptr(), bp.data_ptr(), saved.data_ptr(), B, K, R, L1, n_psqt,
+                                    ws.data_ptr(), nbytes, _stream()), "double_fwd")
+    r_l0, r_wp, r_bp, r_saved = oracle_cpu.double_fwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["W"], c["bias"],
+                                                      c["max_act"], L1)
+    for got, ref in ((l0, r_l0), (wp, r_wp), (bp, r_bp), (saved, r_saved)):
+        assert np.array_equal(got.cpu().numpy(), ref)
+
+
+def test_double_forward_with_more_chunks_than_the_tiled_sort_indexes(oracle_cpu):
+    """2 B / 512 beyond 1024: the sort of the LDS-tiled forward cannot keep the chunk table in LDS, the entry point
+    takes the L2-blocked kernels; same bits."""
+    B, L1, R, K = 262144, 512, 768, 8
+    rng = np.random.default_rng(5)
+    c = double_case(78, 8, L1, R, K, n_psqt=0, binary_side=True, weight_scale=0.05, max_act=0.9)
+    widx = rng.integers(0, R, size=(B, K)).astype(np.int32)
+    bidx = rng.integers(0, R, size=(B, K)).astype(np.int32)
+    widx[:, 6:] = -1
+    us = rng.integers(0, 2, size=(B, 1)).astype(np.float32)
+    them = (1.0 - us).astype(np.float32)
+    psqt_idx = np.zeros(B, np.int64)
+    nat, lib = _native()
+    l0 = torch.empty(B, L1, device=_dev())
+    wp = torch.empty(B, 1, device=_dev())
+    bp = torch.empty(B, 1, device=_dev())
+    saved = torch.empty(2, B, L1, device=_dev())
+    nbytes = lib.nnueft_fwd_workspace_bytes(B, K, R, L1, 0)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=_dev())
+    W, bias = _t(c["W"]), _t(c["bias"])
+    d_us, d_them, d_w, d_b, d_p = _t(us), _t(them), _t(widx), _t(bidx), _t(psqt_idx)
+    nat.check(lib.nnueft_double_fwd(d_us.data_ptr(), d_them.data_ptr(), d_w.data_ptr(), d_b.data_ptr(),
+                                    d_p.data_ptr(), W.data_ptr(), bias.data_ptr(), c["max_act"], l0.data_ptr(),
+                                    wp.data_ptr(), bp.data_ptr(), saved.data_ptr(), B, K, R, L1, 0, ws.data_ptr(), nbytes,
+                                    _stream()), "double_fwd")
+    r_l0, r_wp, r_bp, r_saved = oracle_cpu.double_fwd(us, them, widx, bidx, psqt_idx, c["W"], c["bias"], c["max_act"], L1)
+    assert np.array_equal(l0.cpu().numpy(), r_l0)
+    assert np.array_equal(saved.cpu().numpy(), r_saved)
+    # the atomic adds in LDS tiles walk the same tables: this batch is beyond them too
+    assert lib.nnueft_atomic_lds_workspace_bytes(B, K, R, L1, 2) == 0
+
+
 @pytest.mark.parametrize("mode", ["atomic", "atomic_lds", "deterministic"])
 @pytest.mark.parametrize("B,L1,R,K,kw", DOUBLE_SHAPES)
 def test_double_backward(oracle_cpu, B, L1, R, K, kw, mode):
@@ -251,7 +315,7 @@ def test_double_backward(oracle_cpu, B, L1, R, K, kw, mode):
             rc = lib.nnueft_double_bwd_atomic_lds(*head, gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt, ws.data_ptr(),
                                                   ws.numel(), _stream())
             if nbytes == 0:
-                assert rc == nat.E_UNSUPPORTED and (K > 32 or out_cols % 4)
+                assert rc == nat.E_UNSUPPORTED and (K > 32 or out_cols % 4 or R > 62 * 768)
                 return
             nat.check(rc, "double_bwd_atomic_lds")
     else:
