@@ -37,6 +37,84 @@ def test_leb128_known_encodings():
     assert S.encode_leb_128_array(np.array([v for v, _ in known])) == b"".join(e for _, e in known)
 
 
+def test_leb128_edge_values_as_the_reference_encoder_loop_gives_them():
+    """The reference's encoder (model/utils/serialize.py:64-75) takes 7 bits at a time and stops when what is left is
+    0 with bit 6 clear or -1 with bit 6 set.  Worked by hand for the edges of one byte and of int16:
+      63: byte 0x3f, rest 0, bit 6 clear -> 3f.            64: byte 0x40, rest 0 but bit 6 set -> c0, then 00.
+     -64: byte 0x40, rest -1, bit 6 set -> 40.            -65: byte 0x3f, rest -1 but bit 6 clear -> bf, then 7f.
+    32767: 7f|80, 7f|80, then 01 (rest 0, bit 6 clear).  -32768: 00|80, 00|80, then 7e (rest -1, bit 6 set)."""
+    hand = [(63, "3f"), (64, "c000"), (-64, "40"), (-65, "bf7f"), (32767, "ffff01"), (-32768, "80807e"),
+            (8191, "ff3f"), (8192, "80c000"), (-8192, "8040"), (-8193, "ffbf7f")]
+    for v, hexbytes in hand:
+        assert S.encode_leb_128_array(np.array([v], np.int16)).hex() == hexbytes, v
+        assert S.decode_leb_128_array(bytes.fromhex(hexbytes), 1).tolist() == [v]
+    # a tensor in the file: the 17 bytes of the tag, the byte count as u32, the values
+    w = S.NNUEWriter.__new__(S.NNUEWriter)
+    w.buf = bytearray()
+    w.write_tensor(torch.tensor([63, 64, -64, -65, 32767, -32768], dtype=torch.int16), "leb128")
+    assert bytes(w.buf) == b"COMPRESSED_LEB128" + bytes.fromhex("0c000000" "3f" "c000" "40" "bf7f" "ffff01" "80807e")
+
+
+# What model/utils/serialize.py:102-160 and composed_feature_transformer.py:41-52 fix for a HalfKAv2_hm^ net, worked out
+# by hand from those lines (nothing below calls this build's own hash functions):
+#   feature hash 0x7F234CB8 (one feature block: rotate-left of 0, xor HASH); version 0x6A448AFA;
+#   fc_hash: prev = 0xEC42E90D ^ 2 L1; per layer of out = L2, L3, 1 outputs: h = 0xCC03DAE4 + out, h ^= prev >> 1,
+#   h ^= (prev << 31) mod 2^32, and + 0x538D24C7 mod 2^32 unless out == 1.
+#     L1 = 1024: 0xEC42E10D -> 0x8DAFD049 -> 0x5E6157E7 -> 0x63337116       (L2 = 32, L3 = 32: the reference's defaults,
+#     L1 = 3072: 0xEC42F10D -> 0x8DAFC739 -> 0x5E615D5F -> 0x6333744A        modules/config.py:10-15; L2 = 16: 15 + 1)
+#   network hash = fc_hash ^ feature hash ^ 2 L1; feature transformer hash = feature hash ^ 2 L1.
+#   Sections, uncompressed, behind the 84-byte default description (12 + 84 = 96): FT hash, int16 bias[L1],
+#   int16 weight[22528, L1], int32 psqt[22528, 8], then per bucket: hash, int32 bias[L2], int8 [L2, L1], int32 bias[L3],
+#   int8 [L3, 2 L2 padded to 32], int32 bias[1], int8 [1, 2 L2 + 2 L3 padded to 32].
+LAYOUTS = [
+    dict(L1=1024, L2=32, L3=32, header="fa8a446a" "ae35101c" "54000000", ft_hash=0x7F2344B8, fc_hash=0x63337116,
+         ft_bias=100, ft_weight=2148, psqt=46139492, bucket0=46860388, bucket_bytes=35208,
+         in_bucket=dict(l1_bias=4, l1_weight=132, l2_bias=32900, l2_weight=33028, out_bias=35076, out_weight=35080),
+         size=47142052),
+    dict(L1=3072, L2=16, L3=32, header="fa8a446a" "f220101c" "54000000", ft_hash=0x7F2354B8, fc_hash=0x6333744A,
+         ft_bias=100, ft_weight=6244, psqt=138418276, bucket0=139139172, bucket_bytes=50472,
+         in_bucket=dict(l1_bias=4, l1_weight=68, l2_bias=49220, l2_weight=49348, out_bias=50372, out_weight=50376),
+         size=139542948),
+]
+
+
+@pytest.mark.parametrize("lay", LAYOUTS, ids=["default_1024_32_32", "config4_3072_16_32"])
+def test_file_layout_against_literals_worked_out_from_the_reference(lay):
+    L1, L2, L3 = lay["L1"], lay["L2"], lay["L3"]
+    torch.manual_seed(L1)
+    m = M.NNUEModel("HalfKAv2_hm^", M.ModelConfig(L1=L1, L2=L2, L3=L3))
+    buf = bytes(S.NNUEWriter(m).buf)          # default description, no compression
+    assert buf[:12].hex() == lay["header"]
+    assert buf[12:96].decode() == "Network trained with the https://github.com/official-stockfish/nnue-pytorch trainer."
+    assert struct.unpack_from("<I", buf, 96)[0] == lay["ft_hash"]
+    assert len(buf) == lay["size"]
+    for b in range(8):
+        assert struct.unpack_from("<I", buf, lay["bucket0"] + b * lay["bucket_bytes"])[0] == lay["fc_hash"], b
+    # every section at its literal offset holds the quantized tensor it is meant to
+    export = m.input.get_export_weights()
+    w16, b16, p32 = quantized.quantize_feature_transformer(export, m.input.bias.data, L1)
+    assert np.array_equal(np.frombuffer(buf, "<i2", L1, lay["ft_bias"]), b16.numpy())
+    for row in (0, 1, 22527):     # whole-table comparisons are the other test's; here the place of the rows
+        assert np.array_equal(np.frombuffer(buf, "<i2", L1, lay["ft_weight"] + row * L1 * 2), w16[row].numpy())
+        assert np.array_equal(np.frombuffer(buf, "<i4", 8, lay["psqt"] + row * 32), p32[row].numpy())
+    w1, b1, w2, b2, wo, bo = [t.numpy() for t in quantized.quantize_layer_stacks(m.layer_stacks)]
+    pad = lambda n: (n + 31) // 32 * 32
+    for b in (0, 7):
+        at = lay["bucket0"] + b * lay["bucket_bytes"]
+        o = lay["in_bucket"]
+        assert np.array_equal(np.frombuffer(buf, "<i4", L2, at + o["l1_bias"]), b1[b * L2:(b + 1) * L2])
+        assert np.array_equal(np.frombuffer(buf, "i1", L2 * L1, at + o["l1_weight"]).reshape(L2, L1), w1[b * L2:(b + 1) * L2])
+        assert np.array_equal(np.frombuffer(buf, "<i4", L3, at + o["l2_bias"]), b2[b * L3:(b + 1) * L3])
+        l2w = np.frombuffer(buf, "i1", L3 * pad(2 * L2), at + o["l2_weight"]).reshape(L3, pad(2 * L2))
+        assert np.array_equal(l2w[:, :2 * L2], w2[b * L3:(b + 1) * L3]) and not l2w[:, 2 * L2:].any()
+        assert np.array_equal(np.frombuffer(buf, "<i4", 1, at + o["out_bias"]), bo[b:b + 1])
+        ow = np.frombuffer(buf, "i1", pad(2 * L2 + 2 * L3), at + o["out_weight"])
+        assert np.array_equal(ow[:2 * L2 + 2 * L3], wo[b]) and not ow[2 * L2 + 2 * L3:].any()
+    # and the reader takes the file for exactly this architecture
+    r = S.NNUEReader(io.BytesIO(buf), "HalfKAv2_hm^", M.ModelConfig(L1=L1, L2=L2, L3=L3))
+    assert r.description.startswith("Network trained with")
+
+
 def test_leb128_round_trip_and_truncation():
     rng = np.random.default_rng(0)
     a = np.concatenate([rng.integers(-2 ** 31, 2 ** 31, size=5000), rng.integers(-300, 300, size=5000),
