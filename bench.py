@@ -246,6 +246,42 @@ def l2_peak_gbs():
     return L2_CHANNELS * L2_LINE_BYTES * ENGINE_CLOCK_GHZ
 
 
+def measured_peaks(lib, dev):
+    """What the two memory paths of the gathers deliver on this device, from the library's probe kernels (HIP events,
+    one warm-up launch and one timed): random pieces of an L2-resident set (2.5 MB per XCD) and 16-byte reads out of
+    a 96 KB LDS tile.  GB/s, whole chip."""
+    import ctypes
+    import torch
+
+    out = {}
+    stream = torch.cuda.current_stream().cuda_stream
+    sink = torch.zeros(1, device=dev)
+    set_bytes = 2560 * 1024
+    src = torch.zeros(8 * set_bytes // 4, device=dev)
+    n = ctypes.c_longlong(0)
+
+    def timed(launch):
+        assert launch() == 0
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        assert launch() == 0
+        e1.record()
+        torch.cuda.synchronize()
+        return n.value / (e0.elapsed_time(e1) * 1e-3) / 1e9
+
+    for span, depth, key in ((1024, 8, "l2_gather_1KiB_pieces_GBs"), (128, 8, "l2_gather_128B_lines_GBs"),
+                             (1024, 16, "l2_gather_1KiB_pieces_depth16_GBs")):
+        out[key] = timed(lambda: lib.nnueft_probe_l2_gather(src.data_ptr(), src.numel() * 4, sink.data_ptr(), set_bytes, span,
+                                                            depth, 400, ctypes.byref(n), stream))
+    for pattern, key in ((0, "lds_read_1KiB_in_a_row_GBs"), (1, "lds_read_random_128B_rows_GBs")):
+        out[key] = timed(lambda: lib.nnueft_probe_lds_read(sink.data_ptr(), pattern, 4000, ctypes.byref(n), stream))
+    out["l2_gather_measured_GBs"] = max(out["l2_gather_1KiB_pieces_GBs"], out["l2_gather_1KiB_pieces_depth16_GBs"])
+    out["how"] = ("nnueft_probe_l2_gather: all CUs, 32 waves each, random pieces of a 2.5 MB set per XCD, 8 (16) loads of 16 "
+                  "bytes in flight per lane; nnueft_probe_lds_read: all CUs, 16 waves each, 8 reads of 16 bytes in flight per lane")
+    return out
+
+
 # ------------------------------------------------------------------------------------------------
 # other workloads
 
@@ -506,14 +542,18 @@ def run_handoff(args, dev):
 # ------------------------------------------------------------------------------------------------
 # the feature-transformer workloads (configs 1-3)
 
-def bound_block(kernel, ms, alg_bytes, gathered_bytes, comp_bytes, traffic_bytes, l2_peak, note=None):
-    """One launch against its three yardsticks."""
+def bound_block(kernel, ms, alg_bytes, gathered_bytes, comp_bytes, traffic_bytes, l2_peak, note=None, measured_peak=None):
+    """One launch against its three yardsticks.  measured_peak: what the probe kernel of this run reached on the path
+    that serves the algorithmic bytes; `frac` is then against that, `frac_of_nominal_peak` against the nominal rate."""
     s = ms * 1e-3
     alg_gbs = alg_bytes / s / 1e9
+    peak = measured_peak if measured_peak else l2_peak
     out = {
         "kernel": kernel, "avg_launch_ms": ms,
         # the algorithmic bytes are served by L2 (the gathers are blocked for it), so that is the bound they are held to
-        "bound": "l2", "achieved": alg_gbs, "peak": l2_peak, "unit": "GB/s", "frac": alg_gbs / l2_peak,
+        "bound": "l2", "achieved": alg_gbs, "peak": peak, "unit": "GB/s", "frac": alg_gbs / peak,
+        "peak_is": "measured in this run (probe kernel)" if measured_peak else "nominal",
+        "nominal_peak": l2_peak, "frac_of_nominal_peak": alg_gbs / l2_peak,
         "algorithmic_bytes_per_launch": alg_bytes, "achieved_over_hbm_peak": alg_gbs / HBM_PEAK_GBS,
         "l2_lines_per_clock_per_channel": gathered_bytes / s / 1e9 / l2_peak if gathered_bytes else None,
         "traffic": traffic_bytes,
@@ -540,6 +580,7 @@ def run_ft(args, lib, dev):
     W = t["W"].requires_grad_()
     bias = t["bias"].requires_grad_()
     l2_peak = l2_peak_gbs()
+    probes = measured_peaks(lib, dev)
 
     def step(mode, t=t):
         nnueft.set_backward_mode(mode)
@@ -651,17 +692,30 @@ def run_ft(args, lib, dev):
             _, out["reduce"] = time_steps(reduce_only, n_entry, args.warmup)
             return out
 
+        # the atomic mode as the operator runs it: adds in LDS tiles where the shape takes them (the gradient is
+        # written, no zero fill), else global atomics on the zeroed gradient
+        from nnueft._ops import ATOMIC_LDS_MIN_COLS
+
+        lds_bytes = lib.nnueft_atomic_lds_workspace_bytes(B, K_, R_ROWS, oc, 2) if oc >= ATOMIC_LDS_MIN_COLS else 0
+        lds_ws = torch.empty(max(lds_bytes, 1), dtype=torch.uint8, device=dev)
+
         def bwd_atomic():
-            gW.zero_()
-            gb.zero_()
-            rc = lib.nnueft_double_bwd_atomic(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT, stream)
+            if lds_bytes:
+                rc = lib.nnueft_double_bwd_atomic_lds(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT,
+                                                      lds_ws.data_ptr(), lds_bytes, stream)
+            else:
+                gW.zero_()
+                gb.zero_()
+                rc = lib.nnueft_double_bwd_atomic(*head, gW.data_ptr(), gb.data_ptr(), B, K_, R_ROWS, L1, N_PSQT, stream)
             assert rc == 0
 
         fwd_only()   # `saved` holds this batch's row sums
         for mode in (["deterministic"] if args.only == "reduce" else modes):
             if mode == "atomic":
                 _, ms = time_steps(bwd_atomic, n_entry, args.warmup)
-                bwd_ms[mode] = {"entry": ms}
+                bwd_ms[mode] = {"entry": ms, "kernel": "k_scatter_tile (atomic adds into LDS tiles of doubles) behind "
+                                                       "k_bwd_rows and the list sort" if lds_bytes else
+                                "k_double_bwd_atomic (global atomics, + the zero fill of the dense gradient)"}
             else:
                 bwd_ms[mode] = det_entry(row_split_of(mode))
 
@@ -688,28 +742,41 @@ def run_ft(args, lib, dev):
         "config": {
             "workload": args.workload, "L1": L1, "batch": B, "table_rows": R_ROWS, "psqt_columns": N_PSQT,
             "slots": K_SLOTS, "active_rows_per_position": sum_a / B, "backward": head_mode,
+            "summation_order": {
+                "deterministic_strict": "the reference CPU path's: per table row one chain over its slots in (position, slot) "
+                                        "order, white + black; bit-equal to torch CPU autograd",
+                "deterministic": "this build's default: as strict, except that a row named by more than 512 slots is summed "
+                                 "window by window (bit-equal to the oracle and from run to run, to rounding against torch)",
+                "atomic": "none (atomic adds into LDS tiles of doubles); 1e-4 relative against the oracle",
+            }[head_mode],
             "index_scheme": "HalfKAv2_hm, seeded random positions", "positions": args.positions,
             "sort_placement": args.sort_placement,
         },
-        "peaks": {"hbm_GBs": HBM_PEAK_GBS, "l2_GBs": l2_peak,
-                  "l2": f"{L2_CHANNELS} channels x {L2_LINE_BYTES} B per clock at {ENGINE_CLOCK_GHZ} GHz",
-                  "traffic_source": traffic_file},
+        "peaks": {"hbm_GBs": HBM_PEAK_GBS, "l2_nominal_GBs": l2_peak,
+                  "l2_nominal": f"{L2_CHANNELS} channels x {L2_LINE_BYTES} B per clock at {ENGINE_CLOCK_GHZ} GHz",
+                  "lds_nominal_GBs": LDS_PEAK_GBS, "lds_nominal": f"256 CUs x 256 B per clock at {ENGINE_CLOCK_GHZ} GHz",
+                  "measured": probes, "traffic_source": traffic_file},
     }
     if forward_path(L1) == "tile":
         # the gather reads the table out of LDS tiles: its algorithmic bytes are LDS reads
         fwd_block, fwd_comp = bound_block(
             "nnueft_double_fwd: k_acc_tile (the gather out of LDS tiles, ~2/3 of the time) + k_mix + list sort", fwd_ms,
             fwd_bytes, None, sum(comp_fwd.values()), sum_traffic(traffic, fwd_kernels(L1)), LDS_PEAK_GBS,
-            note="peak: 256 CUs x 256 B of LDS reads per clock at 2.4 GHz; 16-byte reads of whole 128-byte rows at "
-                 "random rows reach 69 TB/s, consecutive ones 124 TB/s (measured on this part)")
+            note="the gathered rows are LDS reads: peak = what 16-byte reads of whole 128-byte rows at random rows of a "
+                 "96 KB tile reach on this device (probe kernel, this run); the kernel is bound by its memory side "
+                 "(tile fetches and stores of the sums), see roofline_forward_compulsory",
+            measured_peak=probes["lds_read_random_128B_rows_GBs"])
         fwd_block["bound"] = "lds"
     else:
         fwd_block, fwd_comp = bound_block(
             "nnueft_double_fwd: k_acc_blocked (the gather, ~3/4 of the time) + k_mix + pair sort", fwd_ms, fwd_bytes,
-            sum_a * oc * 4, sum(comp_fwd.values()), sum_traffic(traffic, fwd_kernels(L1)), l2_peak)
+            sum_a * oc * 4, sum(comp_fwd.values()), sum_traffic(traffic, fwd_kernels(L1)), l2_peak,
+            measured_peak=probes["l2_gather_measured_GBs"])
     out["roofline_forward"] = fwd_block
     out["roofline_forward_compulsory"] = fwd_comp
-    det = bwd_ms.get("deterministic") or bwd_ms.get("deterministic_strict")
+    # the dominant kernel as the headline's order launches it
+    det = (bwd_ms.get(head_mode) if head_mode != "atomic" else None) or bwd_ms.get("deterministic") or \
+        bwd_ms.get("deterministic_strict")
     if det:
         alg, gathered, comp = seg_reduce_bytes(L1, B, sum_a)
         seg_traffic = sum_traffic(traffic, ("k_seg_reduce", "k_split_combine"))
@@ -718,14 +785,16 @@ def run_ft(args, lib, dev):
             "rewinds the task counters, a few microseconds, behind it)", det["reduce"], alg, gathered, comp,
             seg_traffic, l2_peak,
             note="dominant kernel of the step; it gathers one upstream row per slot through L2 (blocked by king bucket "
-                 "and column slice), so `achieved` (algorithmic bytes) is held against the L2 line rate; against HBM "
-                 "see roofline_compulsory (bytes that must cross HBM once) and `traffic` (counter-measured); the L2's "
-                 "channels are busy 95 % of this kernel's time (TCC_BUSY in "
-                 "profiles/ft_fwd_bwd_L1_3072_B16384_utilisation_pmc.txt)")
+                 "and column slice), so `achieved` (algorithmic bytes) is held against what a gather of random 1 KiB "
+                 "pieces out of an L2-resident set reaches on this device (probe kernel, this run; the nominal L2 line "
+                 "rate is in nominal_peak); against HBM see roofline_compulsory (bytes that must cross HBM once) and "
+                 "`traffic` (counter-measured); the L2's channels are busy 95 % of this kernel's time (TCC_BUSY in "
+                 "profiles/ft_fwd_bwd_L1_3072_B16384_utilisation_pmc.txt)",
+            measured_peak=probes["l2_gather_measured_GBs"])
     elif "atomic" in bwd_ms:
         _, bwd_bytes = algorithmic_bytes(L1, B, sum_a, "atomic")
         gbs = bwd_bytes / (bwd_ms["atomic"]["entry"] * 1e-3) / 1e9
-        out["roofline"] = {"kernel": "k_double_bwd_atomic<4> (+ the zero fill of the dense gradient)", "bound": "hbm",
+        out["roofline"] = {"kernel": "nnueft_double_bwd_atomic*: " + bwd_ms["atomic"]["kernel"], "bound": "hbm",
                            "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
                            "traffic": None, "algorithmic_bytes_per_launch": bwd_bytes,
                            "avg_launch_ms": bwd_ms["atomic"]["entry"]}
@@ -746,7 +815,16 @@ def run_ft(args, lib, dev):
             st["traffic_bytes"] = tr
             st["traffic_frac_of_hbm_peak"] = tr / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS if tr else None
         else:
+            # algorithmic: the formula of the atomic scheme (8 bytes of read-modify-write per gathered float and the
+            # zero fill), a ratio since the adds moved into LDS; compulsory: what this decomposition moves through HBM
+            # (upstream rows written and read once, lists, the dense gradient written once)
             st["algorithmic_frac_of_hbm_peak"] = st["algorithmic_GBs"] / HBM_PEAK_GBS
+            if oc >= 512:
+                comp_atomic = (comp_bwd["k_bwd_rows"] + 2 * 2 * B * K_SLOTS * 4 + sum_a * 2 + 2 * B * 6
+                               + 2 * B * oc * 4 + sum_a * 2 + R_ROWS * oc * 4 + comp_bwd["bias"])
+                comp_step = sum(comp_fwd.values()) + comp_atomic
+                st["compulsory_bytes"] = comp_step
+                st["compulsory_frac_of_hbm_peak"] = comp_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS
         if mode in bwd_ms:
             e = bwd_ms[mode]
             st["backward_entry_ms"] = e.get("entry")
@@ -761,7 +839,7 @@ def run_ft(args, lib, dev):
         # the same step on game-like index lists (not the headline: what real training data looks like)
         tg, sum_g = make_inputs(L1, B, seed, dev, "game")
         game = {"active_rows_per_position": sum_g / B}
-        for mode in ("deterministic", "deterministic_strict"):
+        for mode in ("deterministic", "deterministic_strict", "atomic"):
             ms_g, _ = time_steps(lambda: step(mode, tg), args.steps, args.warmup)
             game[mode] = {"ms_per_step": ms_g, "positions_per_s": B / (ms_g * 1e-3)}
         out["game_like_positions"] = game
@@ -780,7 +858,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="ft_fwd_bwd_L1_3072_B16384", choices=sorted(WORKLOADS))
-    ap.add_argument("--backward", default="deterministic", choices=["deterministic", "deterministic_strict", "atomic"],
+    ap.add_argument("--backward", default="deterministic_strict", choices=["deterministic", "deterministic_strict", "atomic"],
                     help="backward mode the headline value is measured with (the others are reported beside it)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--optimizer", default="rangerlite", choices=["rangerlite", "adam"],

@@ -525,6 +525,20 @@ int nnueft_sf_loss_bwd(const float* terms, const float* sums, const float* grad_
 int nnueft_batch_unpack(const float* us, const int32_t* piece_count32, float* them, int64_t* piece_count,
                         int B, void* stream);
 
+/*
+ * Measurement aids (no counterpart in the reference; nothing in the library's own paths calls them): what the
+ * memory paths of the gathers deliver on the device at hand, for the roofline figures of a benchmark.
+ * nnueft_probe_l2_gather: every CU gathers pieces of `span` (128 or 1024) contiguous bytes at random places of a
+ * set of set_bytes that is resident in its XCD's L2 (src: 8 * set_bytes of device memory, one set per XCD),
+ * `depth` (4, 8 or 16) loads of 16 bytes in flight per lane, `iters` rounds; *bytes_read (host) = bytes the launch
+ * reads.  nnueft_probe_lds_read: every CU reads 16 bytes per lane out of a 96 KB LDS tile, pattern 0 a wave
+ * 1 KB in a row, pattern 1 each 8-lane group a whole 128-byte row at a random row.  sink: 4 bytes of device
+ * memory (never written in practice).  Time the launches with events on `stream`.
+ */
+int nnueft_probe_l2_gather(const void* src, size_t src_bytes, float* sink, int set_bytes, int span, int depth,
+                           int iters, long long* bytes_read, void* stream);
+int nnueft_probe_lds_read(float* sink, int pattern, int iters, long long* bytes_read, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

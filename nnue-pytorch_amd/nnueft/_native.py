@@ -94,6 +94,8 @@ PROTOTYPES = {
     "nnueft_ranger_lite_update_multi": (c_int, [ctypes.POINTER(RangerArgs), c_int, c_void_p]),
     "nnueft_ranger_lite_update_variance": (c_int, [c_void_p] * 2 + [c_longlong] + [c_float] * 2 + [c_void_p]),
     "nnueft_ranger_lite_lookahead_merge": (c_int, [c_void_p] * 2 + [c_longlong, c_float, c_void_p]),
+    "nnueft_probe_l2_gather": (c_int, [c_void_p, c_size_t, c_void_p] + [c_int] * 4 + [ctypes.POINTER(c_longlong), c_void_p]),
+    "nnueft_probe_lds_read": (c_int, [c_void_p, c_int, c_int, ctypes.POINTER(c_longlong), c_void_p]),
 }
 
 E_UNSUPPORTED = -3   # NNUEFT_E_UNSUPPORTED of the header
