@@ -25,6 +25,8 @@
 //   k_bias_final    the same chain as a launch of its own where no row can be split (strict order)
 #include <atomic>
 
+#include <algorithm>
+
 #include "gather.h"
 #include "internal.h"
 
@@ -76,12 +78,28 @@ constexpr uint32_t kSplitFlag = 0x80000000u;   // on a row's slot count between 
 constexpr int kSchedCtr = 0;       // kXcd * kSchedQueues task counters, 32 words (128 bytes) apart
 constexpr int kSchedQueues = 16;   // room for that many counters per XCD
 constexpr int kSchedNLong = kXcd * kSchedQueues * 32;         // long_rows[0 .. n_long): long rows that are not split
-constexpr int kSchedNSplit = kSchedNLong + 1;  // long_rows[R - n_split .. R), from the back: split rows
-constexpr int kSchedRowLo = kSchedNSplit + 1;  // kXcd + 1 range bounds
-constexpr int kSchedWords = kSchedRowLo + kXcd + 1;
+constexpr int kSchedNSplit = kSchedNLong + 1;  // long_rows[R - n_split .. R), from the back: split rows, in three classes:
+constexpr int kSchedNRemote = kSchedNSplit + 1;   // the first n_remote: window sums by (perspective, window) pair, any XCD
+constexpr int kSchedNLocal = kSchedNRemote + 1;   // the next n_local: window sums inside their XCD's walk of its row range
+                                                  // (the rest: more rows than there is room for window sums; reduced whole)
+constexpr int kSchedRowSplit = kSchedNLocal + 1;  // the threshold the lists were sorted for
+constexpr int kSchedRowLo = kSchedRowSplit + 1;   // kXcd + 1 range bounds
+constexpr int kSchedLocalCnt = kSchedRowLo + kXcd + 1;   // kXcd counts: the local split rows of each XCD's range
+constexpr int kSchedWords = kSchedLocalCnt + kXcd;
+// Window sums are kept for this many split rows at most (uniform positions split 32 rows, game-like ones a few hundred);
+// further ones are reduced by one wave per 64-lane slice, window by window in the same order, so the bits are the same.
+#ifndef NNUEFT_SPLIT_CAP
+#define NNUEFT_SPLIT_CAP 384
+#endif
+constexpr int kSplitCap = NNUEFT_SPLIT_CAP;
+constexpr int kLocalMax = 64;        // most local split rows per XCD (a wave keeps them one per lane)
+#ifndef NNUEFT_LOCAL_LEN
+#define NNUEFT_LOCAL_LEN 4096
+#endif
+constexpr uint32_t kLocalLen = NNUEFT_LOCAL_LEN;   // a split row named by more slots than this is never local
 
 struct DetLayout {
-    size_t G, partial, cnt, wcount, seg_off, long_rows, sched, list, runs, end;
+    size_t G, partial, cnt, wcount, seg_off, long_rows, split_local, sched, list, runs, end;
     size_t sort_begin, sort_end;   // cnt .. list: what the sort writes and the reduction reads (one block)
     int cpp;     // chunks per perspective
     int nchunks; // n_persp * cpp
@@ -122,6 +140,8 @@ bool det_layout(int B, int K, int R, int out_cols, int n_persp, int row_split, D
     off += up256(((size_t)R + 1) * sizeof(uint32_t));
     L->long_rows = off;
     off += up256((size_t)R * sizeof(uint32_t));
+    L->split_local = off;
+    off += up256((size_t)kXcd * kLocalMax * sizeof(uint32_t));
     L->sched = off;
     off += up256((size_t)kSchedWords * sizeof(uint32_t));
     L->list = off;
@@ -133,7 +153,8 @@ bool det_layout(int B, int K, int R, int out_cols, int n_persp, int row_split, D
     L->nwin = (B + wpos - 1) / wpos;
     const long long most = row_split > 0 ? ((long long)n_persp * B * K) / ((long long)row_split + 1) : 0;
     if (most > 0x3fffffffLL) return false;
-    L->max_split = (int)most;
+    // window sums are kept for kSplitCap rows at most (and no table has more split rows than rows)
+    L->max_split = (int)std::min<long long>(std::min<long long>(most, R), kSplitCap);
     L->runs = off;
     off += up256((size_t)L->max_split * n_persp * L->nwin * out_cols * sizeof(float));
     L->end = off;
@@ -389,8 +410,9 @@ __device__ __forceinline__ int long_class(uint32_t len) {
 }
 __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict__ seg_off,
                                                            uint32_t* __restrict__ long_rows,
+                                                           uint32_t* __restrict__ split_local,
                                                            uint32_t* __restrict__ sched, int R, int cap,
-                                                           uint32_t row_split) {
+                                                           uint32_t row_split, uint32_t split_cap) {
     extern __shared__ uint32_t stage[];   // `cap` row lengths, turned into offsets in place
     // two running sums: all slots, and what slots_elsewhere() takes off the weight of the row ranges
     __shared__ uint32_t wave_tot[2][kScanThreads / 64];
@@ -547,6 +569,85 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
             long_rows[atomicAdd(&long_cnt[long_class(len)], 1u)] = (uint32_t)i;
     }
     if (tid <= kXcd) sched[kSchedRowLo + tid] = lo_s[tid];
+    // The split rows in three classes (see kSchedNRemote).  A split row is local when its XCD's row range is
+    // sparse (few slots per row: the range is walked in wide slices and the upstream rows its rows name stay in
+    // that XCD's L2 meanwhile, the split row's among them), it is not too long, and the XCD has room for it.
+    __shared__ uint32_t sparse_s[kXcd], loc_cnt_s[kXcd], n_remote_s, n_local_s, slot_s[2];
+    if (tid < kXcd) {
+        const uint32_t lo = lo_s[tid], hi = lo_s[tid + 1];
+        const uint32_t a = lo >= (uint32_t)R ? total : one_pass ? stage[lo] : seg_off[lo];
+        const uint32_t b = hi >= (uint32_t)R ? total : one_pass ? stage[hi] : seg_off[hi];
+        sparse_s[tid] = hi > lo && (b - a) / (hi - lo) <= (uint32_t)kNarrowAvg;
+        loc_cnt_s[tid] = 0;
+    }
+    if (tid == 0) {
+        n_remote_s = 0;
+        n_local_s = 0;
+        slot_s[0] = 0;
+        slot_s[1] = 0;
+    }
+    __syncthreads();
+    const uint32_t n_split = n_split_s;
+    constexpr int SPT = 4;   // split rows a thread classifies; beyond kScanThreads * SPT of them none is local
+    uint32_t row_of[SPT];
+    int cls[SPT];            // 0 remote, 1 local, 2 reduced whole
+    int xcd_of_row[SPT];
+    const bool classify = n_split <= (uint32_t)(kScanThreads * SPT);
+#pragma unroll
+    for (int u = 0; u < SPT; ++u) {
+        const uint32_t k = (uint32_t)(tid + u * kScanThreads);
+        cls[u] = -1;
+        row_of[u] = 0;
+        xcd_of_row[u] = 0;
+        if (classify && k < n_split) {
+            const uint32_t r = long_rows[R - 1 - (int)k];
+            row_of[u] = r;
+            int x = 0;
+            for (int q = 1; q < kXcd; ++q) x += r >= lo_s[q] ? 1 : 0;
+            xcd_of_row[u] = x;
+            const uint32_t a = one_pass ? stage[r] : seg_off[r];
+            const uint32_t b = r + 1 == (uint32_t)R ? total : one_pass ? stage[r + 1] : seg_off[r + 1];
+            cls[u] = 0;
+            if (sparse_s[x] && b - a <= kLocalLen) {
+                // room among the window sums and in the XCD's list (first come, first served: which rows are
+                // local only moves work, never a bit of the result)
+                if (atomicAdd(&n_local_s, 1u) < split_cap) {
+                    if (atomicAdd(&loc_cnt_s[x], 1u) < (uint32_t)kLocalMax) cls[u] = 1;
+                    else atomicSub(&n_local_s, 1u);
+                } else {
+                    atomicSub(&n_local_s, 1u);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    const uint32_t n_local = min(n_local_s, split_cap);
+    const uint32_t n_remote = classify ? min(n_split - n_local, split_cap - n_local) : min(n_split, split_cap);
+    if (tid < kXcd) loc_cnt_s[tid] = 0;
+    __syncthreads();
+    if (classify) {
+        // the list again, class by class: remote, local, whole
+#pragma unroll
+        for (int u = 0; u < SPT; ++u) {
+            if (cls[u] < 0) continue;
+            uint32_t slot;
+            if (cls[u] == 1) {
+                slot = n_remote + atomicAdd(&slot_s[1], 1u);
+                split_local[xcd_of_row[u] * kLocalMax + (int)atomicAdd(&loc_cnt_s[xcd_of_row[u]], 1u)] = slot;
+            } else {
+                const uint32_t i = atomicAdd(&slot_s[0], 1u);
+                slot = i < n_remote ? i : n_local + i;
+            }
+            long_rows[R - 1 - (int)slot] = row_of[u];
+        }
+    }
+    __syncthreads();
+    if (tid < kXcd) sched[kSchedLocalCnt + tid] = classify ? min(loc_cnt_s[tid], (uint32_t)kLocalMax) : 0u;
+    if (tid == 0) {
+        sched[kSchedNRemote] = n_remote;
+        sched[kSchedNLocal] = classify ? n_local : 0u;
+        sched[kSchedRowSplit] = row_split;
+    }
 }
 
 // Every slot of the chunk writes its position id.  Ranks inside the chunk are handed out position
@@ -656,14 +757,10 @@ __global__ __launch_bounds__(kFillThreads) void k_fill(const int32_t* __restrict
 // Segmented reduction.  list[seg_off[r] .. +wcount[r]) are the white-perspective rows of G naming
 // table row r, the rest of the segment the black ones.  gW[r] = white chain (+ black chain).
 // `pre`: the caller already holds list[beg + lane] of a segment of at most 64 slots in `pre_my`.
-template <int VW, int NQ, int U>
-__device__ __forceinline__ void seg_reduce_task(const float* __restrict__ G, const uint32_t* __restrict__ list,
-                                                uint32_t beg, uint32_t mid, uint32_t end, float* __restrict__ dst,
-                                                int s, int lane, int out_cols, int g_pitch, int slice_v, int two_persp,
-                                                bool pre = false, int pre_my = 0) {
+// The columns of a lane in slice s of slice_v vectors.
+template <int VW, int NQ>
+__device__ __forceinline__ void seg_cols(int (&col)[NQ], bool (&act)[NQ], int s, int lane, int out_cols, int slice_v) {
     const int nv = out_cols / VW;
-    int col[NQ];
-    bool act[NQ];
 #pragma unroll
     for (int m = 0; m < NQ; ++m) {
         const int w = m * 64 + lane;
@@ -671,7 +768,13 @@ __device__ __forceinline__ void seg_reduce_task(const float* __restrict__ G, con
         act[m] = w < slice_v && q < nv;
         col[m] = act[m] ? q * VW : 0;
     }
-    vecf<VW> acc[2][NQ];
+}
+
+// acc[0] = chain from +0 over list[beg .. mid), acc[1] = the same over list[mid .. end).
+template <int VW, int NQ, int U>
+__device__ __forceinline__ void seg_chains(vecf<VW> (&acc)[2][NQ], const float* __restrict__ G,
+                                           const uint32_t* __restrict__ list, uint32_t beg, uint32_t mid, uint32_t end,
+                                           const int (&col)[NQ], int lane, int g_pitch, bool pre = false, int pre_my = 0) {
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
 #pragma unroll
@@ -695,6 +798,18 @@ __device__ __forceinline__ void seg_reduce_task(const float* __restrict__ G, con
             }
         }
     }
+}
+
+template <int VW, int NQ, int U>
+__device__ __forceinline__ void seg_reduce_task(const float* __restrict__ G, const uint32_t* __restrict__ list,
+                                                uint32_t beg, uint32_t mid, uint32_t end, float* __restrict__ dst,
+                                                int s, int lane, int out_cols, int g_pitch, int slice_v, int two_persp,
+                                                bool pre = false, int pre_my = 0) {
+    int col[NQ];
+    bool act[NQ];
+    seg_cols<VW, NQ>(col, act, s, lane, out_cols, slice_v);
+    vecf<VW> acc[2][NQ];
+    seg_chains<VW, NQ, U>(acc, G, list, beg, mid, end, col, lane, g_pitch, pre, pre_my);
 #pragma unroll
     for (int m = 0; m < NQ; ++m) {
         if (!act[m]) continue;
@@ -777,7 +892,44 @@ struct RunPlan {
     int tail_v, tail_g;    // trailing vectors of a row that tail_rows_task reduces (0: none), lanes per row there
     int g_pitch;           // floats from one row of G to the next
     uint32_t row_split;    // rows named by more slots than this are the split ones (0: none)
+    const uint32_t* split_local;   // [kXcd, kLocalMax] the local split rows of each XCD, as places in the split list
 };
+
+// The window (perspective p, window w) of split row r: its part [beg, end) of the sorted list.
+__device__ __forceinline__ void window_bounds(const RunPlan& rp, const uint32_t* __restrict__ seg_off, uint32_t r, uint32_t p,
+                                              uint32_t w, uint32_t* beg, uint32_t* end) {
+    const uint32_t c0 = p * (uint32_t)rp.cpp + w * (uint32_t)rp.wch;
+    const uint32_t c1 = min(c0 + (uint32_t)rp.wch, (p + 1u) * (uint32_t)rp.cpp);
+    const uint32_t seg = seg_off[r];
+    *beg = seg + rp.cnt[(size_t)c0 * rp.R + r];
+    *end = c1 == (uint32_t)rp.nchunks ? seg_off[r + 1] : seg + rp.cnt[(size_t)c1 * rp.R + r];
+}
+
+// A split row reduced whole by one wave per 64-lane slice: per perspective the chain over its windows of the window
+// sums (each a chain from +0 over the window's slots), white + black: the order k_split_combine gives the rows whose
+// window sums are kept, so the same bits.
+template <int VW, int U>
+__device__ __forceinline__ void split_row_whole(const RunPlan& rp, const float* __restrict__ G,
+                                                const uint32_t* __restrict__ list, const uint32_t* __restrict__ seg_off,
+                                                uint32_t r, float* __restrict__ dst, int s, int lane, int out_cols) {
+    int col[1];
+    bool act[1];
+    seg_cols<VW, 1>(col, act, s, lane, out_cols, rp.slice_v);
+    vecf<VW> tot = vzero<VW>();
+    for (uint32_t p = 0; p < (uint32_t)rp.n_persp; ++p) {
+        vecf<VW> run = vzero<VW>();
+        for (uint32_t w = 0; w < (uint32_t)rp.nwin; ++w) {
+            uint32_t beg, end;
+            window_bounds(rp, seg_off, r, p, w, &beg, &end);
+            vecf<VW> acc[2][1];
+            seg_chains<VW, 1, U>(acc, G, list, beg, end, end, col, lane, rp.g_pitch);
+            vadd<VW>(run, acc[0][0]);
+        }
+        if (p == 0) tot = run;
+        else vadd<VW>(tot, run);
+    }
+    if (act[0]) stv_stream<VW>(dst + col[0], tot);
+}
 
 // Persistent waves.  A wave takes tasks from its home queue of its XCD, then from the XCD's other
 // queues, until none is left (a counter only grows, so every wave leaves every loop).  Task order per XCD: the
@@ -793,18 +945,23 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
                                                    RunPlan rp) {
     const int lane = threadIdx.x;
     const int xcd = blockIdx.x % kXcd;
+    if (sched[kSchedRowSplit] != rp.row_split) return;   // the lists were sorted for another threshold
     const uint32_t n_long = sched[kSchedNLong], n_split = sched[kSchedNSplit];
+    const uint32_t n_remote = sched[kSchedNRemote], n_stored = n_remote + sched[kSchedNLocal];
+    const uint32_t n_whole = n_split - n_stored;
     const uint32_t npairs = (uint32_t)(rp.n_persp * rp.nwin);
     const uint32_t my_pairs = npairs > (uint32_t)xcd ? (npairs - xcd + kXcd - 1) / kXcd : 0;
-    const uint32_t pair_tasks = (uint32_t)rp.nslices * n_split;
+    const uint32_t pair_tasks = (uint32_t)rp.nslices * n_remote;
     const uint32_t run_tasks = my_pairs * pair_tasks;
     const uint32_t my_long = n_long > (uint32_t)xcd ? (n_long - xcd + kXcd - 1) / kXcd : 0;
+    const uint32_t my_whole = n_whole > (uint32_t)xcd ? (n_whole - xcd + kXcd - 1) / kXcd : 0;
     const uint32_t lo = sched[kSchedRowLo + xcd], hi = sched[kSchedRowLo + xcd + 1];
     const uint32_t nreg = hi - lo;
     // long rows: 64-lane slices with kRunUnroll rows in flight (a chain of hundreds of slots is bound by how
     // many of its loads are in flight; three times as many waves share the row)
     const uint32_t long_slices = (uint32_t)rp.nslices;
-    const uint32_t long_end = run_tasks + my_long * long_slices;
+    const uint32_t whole_end = run_tasks + my_whole * long_slices;
+    const uint32_t long_end = whole_end + my_long * long_slices;
     // A range whose rows are named by many slots each belongs to a table block that a large part of
     // the batch sits in: one wide slice of all those positions' upstream rows would not fit the L2,
     // so such a range is walked in 64-lane slices (the results do not depend on the slicing).
@@ -813,7 +970,34 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
     const uint32_t walk_slices = narrow ? narrow_slices : (uint32_t)nslices;
     const uint32_t tail_rows = rp.tail_v ? 64u / (uint32_t)rp.tail_g : 1u;
     const uint32_t tail_tasks = rp.tail_v ? (nreg + tail_rows - 1) / tail_rows : 0u;
-    const uint32_t ntasks = long_end + tail_tasks + nreg * walk_slices;
+    // The local split rows of this range, one per lane in row order: in the walk of a slice such a row stands for
+    // npairs tasks, one per (perspective, window), at the row's place among the others (whose upstream rows are
+    // those of the same positions, in this XCD's L2 at that time).
+    const uint32_t nloc = min(sched[kSchedLocalCnt + xcd], (uint32_t)kLocalMax);
+    uint32_t loc_r = 0xffffffffu, loc_j = 0, loc_pos = 0xffffffffu;
+    if (nloc) {
+        uint32_t my_j = 0, my_r = 0xffffffffu;
+        if ((uint32_t)lane < nloc) {
+            my_j = rp.split_local[xcd * kLocalMax + lane];
+            my_r = long_rows[(uint32_t)rp.R - 1u - my_j];
+        }
+        uint32_t rank = 0;
+        for (uint32_t k = 0; k < nloc; ++k) rank += (uint32_t)__builtin_amdgcn_readlane((int)my_r, (int)k) < my_r ? 1u : 0u;
+        for (uint32_t q = 0; q < nloc; ++q) {
+            const int src = __ffsll((long long)__ballot((uint32_t)lane < nloc && rank == q)) - 1;
+            const uint32_t r = (uint32_t)__builtin_amdgcn_readlane((int)my_r, src);
+            const uint32_t j = (uint32_t)__builtin_amdgcn_readlane((int)my_j, src);
+            if ((uint32_t)lane == q) {
+                loc_r = r;
+                loc_j = j;
+            }
+        }
+        if ((uint32_t)lane < nloc) loc_pos = (loc_r - lo) + (uint32_t)lane * (npairs - 1u);
+    }
+    const uint32_t nexp = nreg + nloc * (npairs - 1u);          // tasks of a slice of the walk
+    const uint32_t walk_end = long_end + tail_tasks + nexp * walk_slices;
+    const uint32_t loc_tail = rp.tail_v ? nloc * npairs : 0u;   // the trailing columns of the local rows' windows
+    const uint32_t ntasks = walk_end + loc_tail;
     static_assert(kQueues <= kSchedQueues, "counters per XCD");
     const int home = (blockIdx.x / kXcd) % kQueues;
 
@@ -828,22 +1012,27 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
         if (t < run_tasks) {
             const uint32_t pl = t / pair_tasks;
             const uint32_t rem = t - pl * pair_tasks;
-            const uint32_t s = rem / n_split;
-            const uint32_t j = rem - s * n_split;
+            const uint32_t s = rem / n_remote;
+            const uint32_t j = rem - s * n_remote;
             const uint32_t pair = (uint32_t)xcd + pl * kXcd;
             const uint32_t p = pair / (uint32_t)rp.nwin, w = pair - p * (uint32_t)rp.nwin;
             const uint32_t r = long_rows[(uint32_t)rp.R - 1u - j];
-            const uint32_t c0 = p * (uint32_t)rp.cpp + w * (uint32_t)rp.wch;
-            const uint32_t c1 = min(c0 + (uint32_t)rp.wch, (p + 1u) * (uint32_t)rp.cpp);
-            const uint32_t seg = seg_off[r];
-            const uint32_t beg = seg + rp.cnt[(size_t)c0 * rp.R + r];
-            const uint32_t end = c1 == (uint32_t)rp.nchunks ? seg_off[r + 1] : seg + rp.cnt[(size_t)c1 * rp.R + r];
+            uint32_t beg, end;
+            window_bounds(rp, seg_off, r, p, w, &beg, &end);
             float* dst = rp.runs + ((size_t)(j * (uint32_t)rp.n_persp + p) * rp.nwin + w) * out_cols;
             seg_reduce_task<VW, 1, kRunUnroll>(G, list, beg, end, end, dst, (int)s, lane, out_cols, rp.g_pitch, rp.slice_v, 0);
             continue;
         }
-        if (t < long_end) {
+        if (t < whole_end) {
             const uint32_t u = t - run_tasks;
+            const uint32_t i = u / long_slices;
+            const int s = (int)(u - i * long_slices);
+            const uint32_t r = long_rows[(uint32_t)rp.R - 1u - (n_stored + (uint32_t)xcd + i * kXcd)];
+            split_row_whole<VW, kRunUnroll>(rp, G, list, seg_off, r, gW + (size_t)r * out_cols, s, lane, out_cols);
+            continue;
+        }
+        if (t < long_end) {
+            const uint32_t u = t - whole_end;
             const uint32_t i = u / long_slices;
             const int s = (int)(u - i * long_slices);
             const uint32_t r = long_rows[xcd + i * kXcd];
@@ -859,9 +1048,45 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
                                             two_persp, rp.row_split);
             continue;
         }
+        if (t >= walk_end) {
+            // trailing columns of a local split row's window: the last 64-lane slice
+            const uint32_t v = t - walk_end;
+            const uint32_t i = v / npairs, pw = v - i * npairs;
+            const uint32_t r = (uint32_t)__builtin_amdgcn_readlane((int)loc_r, (int)i);
+            const uint32_t j = (uint32_t)__builtin_amdgcn_readlane((int)loc_j, (int)i);
+            const uint32_t p = pw / (uint32_t)rp.nwin, w = pw - p * (uint32_t)rp.nwin;
+            uint32_t beg, end;
+            window_bounds(rp, seg_off, r, p, w, &beg, &end);
+            float* dst = rp.runs + ((size_t)(j * (uint32_t)rp.n_persp + p) * rp.nwin + w) * out_cols;
+            seg_reduce_task<VW, 1, kRunUnroll>(G, list, beg, end, end, dst, rp.nslices - 1, lane, out_cols, rp.g_pitch, rp.slice_v, 0);
+            continue;
+        }
         u -= tail_tasks;
-        const int s = (int)(u / nreg);
-        const uint32_t r = lo + (u - (uint32_t)s * nreg);
+        const int s = (int)(u / nexp);
+        uint32_t v = u - (uint32_t)s * nexp;
+        if (nloc) {
+            // local rows that begin at or before place v of the slice
+            const uint32_t k = (uint32_t)__popcll(__ballot(loc_pos <= v));
+            if (k) {
+                const uint32_t pos = (uint32_t)__builtin_amdgcn_readlane((int)loc_pos, (int)k - 1);
+                if (v < pos + npairs) {
+                    const uint32_t pw = v - pos;
+                    const uint32_t r = (uint32_t)__builtin_amdgcn_readlane((int)loc_r, (int)k - 1);
+                    const uint32_t j = (uint32_t)__builtin_amdgcn_readlane((int)loc_j, (int)k - 1);
+                    const uint32_t p = pw / (uint32_t)rp.nwin, w = pw - p * (uint32_t)rp.nwin;
+                    uint32_t beg, end;
+                    window_bounds(rp, seg_off, r, p, w, &beg, &end);
+                    float* dst = rp.runs + ((size_t)(j * (uint32_t)rp.n_persp + p) * rp.nwin + w) * out_cols;
+                    if (narrow)
+                        seg_reduce_task<VW, 1, kRunUnroll>(G, list, beg, end, end, dst, s, lane, out_cols, rp.g_pitch, rp.slice_v, 0);
+                    else
+                        seg_reduce_task<VW, NQ, kRowsUnroll>(G, list, beg, end, end, dst, s, lane, out_cols, rp.g_pitch, slice_v, 0);
+                    continue;
+                }
+                v -= k * (npairs - 1u);
+            }
+        }
+        const uint32_t r = lo + v;
         const uint32_t beg = seg_off[r], end = seg_off[r + 1];
         const uint32_t len = end - beg;
         // long or split: done elsewhere
@@ -896,7 +1121,8 @@ __global__ __launch_bounds__(64) void k_split_combine(const uint32_t* __restrict
         if (blockIdx.y == 0) bias_final_block(partial, gbias, ntiles, out_cols, sched, (int)blockIdx.x);
         return;
     }
-    const uint32_t n_split = sched[kSchedNSplit];
+    if (sched[kSchedRowSplit] != rp.row_split) return;   // the lists were sorted for another threshold
+    const uint32_t n_split = sched[kSchedNRemote] + sched[kSchedNLocal];   // the rows whose window sums were kept
     const int q = blockIdx.y * 64 + lane;
     if (q >= out_cols / VW) return;
     const int col = q * VW;
@@ -971,6 +1197,7 @@ int det_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, char
     uint32_t* wcount = (uint32_t*)(ws + L.wcount);
     uint32_t* seg_off = (uint32_t*)(ws + L.seg_off);
     uint32_t* long_rows = (uint32_t*)(ws + L.long_rows);
+    uint32_t* split_local = (uint32_t*)(ws + L.split_local);
     uint32_t* sched = (uint32_t*)(ws + L.sched);
     uint32_t* list = (uint32_t*)(ws + L.list);
 
@@ -993,7 +1220,7 @@ int det_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, char
                        L.nchunks, (uint32_t)L.row_split);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_row_scan, dim3(1), dim3(kScanThreads), (size_t)scan_cap * sizeof(uint32_t), st, seg_off,
-                       long_rows, sched, R, scan_cap, (uint32_t)L.row_split);
+                       long_rows, split_local, sched, R, scan_cap, (uint32_t)L.row_split, (uint32_t)L.max_split);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_fill, dim3(L.nchunks, nranges), dim3(kFillThreads), fill_bytes, st, widx, bidx, cnt, seg_off, list,
                        B, K, R, L.cpp, range, stage);
@@ -1047,6 +1274,7 @@ int det_reduce(const float* G, int g_pitch, float* gW, float* gbias, int B, int 
     rp.tail_g = tail_g;
     rp.g_pitch = g_pitch;
     rp.row_split = (uint32_t)L.row_split;
+    rp.split_local = (const uint32_t*)(sw + L.split_local);
     if ((long long)L.max_split * rp.nslices * NNUEFT_ROW_WINDOWS > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
 #define SEG_LAUNCH(VW_, NQ_)                                                                                      \
     hipLaunchKernelGGL((k_seg_reduce<VW_, NQ_>), dim3(kXcd * kWavesPerXcd), dim3(64), 0, st, G, list, seg_off,      \

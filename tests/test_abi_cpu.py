@@ -58,7 +58,13 @@ def test_host_only_entry_points():
     strict = lib.nnueft_det_workspace_bytes(16384, 32, 24576, 3080, 2, 0)
     assert a > b > 0 and a % 256 == 0 and b % 256 == 0
     assert a > strict >= 2 * 16384 * 3080 * 4   # holds the two upstream rows of every position; no window sums
-    assert lib.nnueft_det_workspace_bytes(16384, 32, 24576, 3080, 2, 256) > a      # more rows can be split
+    # window sums are kept for 384 split rows at most, however many rows a lower threshold could split
+    assert lib.nnueft_det_workspace_bytes(16384, 32, 24576, 3080, 2, 256) == a
+    assert lib.nnueft_det_workspace_bytes(16384, 32, 24576, 3080, 2, 1) == a
+    assert a - strict <= 384 * 2 * 16 * 3080 * 4 + 4096 and a <= 600 * 1000 * 1000
+    # a small batch cannot split that many rows: 2 * 64 * 32 slots over a threshold of 512 make 7 rows at most
+    small = lib.nnueft_det_workspace_bytes(64, 32, 24576, 3080, 2, 512) - lib.nnueft_det_workspace_bytes(64, 32, 24576, 3080, 2, 0)
+    assert 0 < small <= 7 * 2 * 1 * 3080 * 4 + 4096
     assert lib.nnueft_det_workspace_bytes(0, 32, 10, 8, 1, 512) == 0
     assert lib.nnueft_det_workspace_bytes(4, 32, 10, 8, 3, 512) == 0
     assert lib.nnueft_det_workspace_bytes(4, 32, 10, 8, 1, -1) == 0

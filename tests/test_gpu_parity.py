@@ -124,6 +124,48 @@ def test_sparse_backward_atomic_in_lds_tiles(oracle_cpu, B, out_cols, R, K):
                                             ws.data_ptr(), nbytes - 1, _stream()) == -2
 
 
+@pytest.mark.parametrize("n_persp", [1, 2])
+def test_deterministic_backward_with_more_split_rows_than_window_sums_are_kept_for(oracle_cpu, n_persp):
+    """Every one of 700 table rows is named by more slots than the threshold (50): window sums are kept for 384 rows,
+    the others are reduced whole, window by window in the same order; all of them bit-equal to the oracle.  The
+    workspace does not grow with the number of rows that could be split."""
+    nat, lib = _native()
+    B, K, R, rs = 3000, 32, 700, 50
+    if n_persp == 1:
+        out_cols = 520
+        c = sparse_case(41, B, out_cols, R, K)
+        idx, g = _t(c["idx"]), _t(c["g"])
+        nbytes = lib.nnueft_det_workspace_bytes(B, K, R, out_cols, 1, rs)
+        assert nbytes < B * out_cols * 4 + 384 * 3 * out_cols * 4 + 16 * B * K + (4 << 20)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=_dev())
+        gW = torch.full((R, out_cols), float("nan"), device=_dev())
+        gb = torch.full((out_cols,), float("nan"), device=_dev())
+        nat.check(lib.nnueft_sparse_bwd_det(idx.data_ptr(), g.data_ptr(), gW.data_ptr(), gb.data_ptr(), B, K, R, out_cols, rs,
+                                            ws.data_ptr(), nbytes, _stream()), "sparse_bwd_det")
+        rW, rb = oracle_cpu.sparse_bwd(c["idx"], c["g"], R, row_split=rs)
+        counts = np.bincount(c["idx"][c["idx"] >= 0], minlength=R)
+    else:
+        L1, n_psqt = 512, 8
+        out_cols = L1 + n_psqt
+        c = double_case(42, B, L1, R, K, weight_scale=0.05, max_act=0.9)
+        d, l0, wp, bp, saved = _run_double_fwd(c)
+        g_l0, g_wp, g_bp = _t(c["g_l0"]), _t(c["g_wp"]), _t(c["g_bp"])
+        nbytes = lib.nnueft_det_workspace_bytes(B, K, R, out_cols, 2, rs)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=_dev())
+        gW = torch.full((R, out_cols), float("nan"), device=_dev())
+        gb = torch.full((out_cols,), float("nan"), device=_dev())
+        nat.check(lib.nnueft_double_bwd_det(d["us"].data_ptr(), d["them"].data_ptr(), d["widx"].data_ptr(), d["bidx"].data_ptr(),
+                                            d["psqt_idx"].data_ptr(), d["bias"].data_ptr(), c["max_act"], g_l0.data_ptr(),
+                                            g_wp.data_ptr(), g_bp.data_ptr(), saved.data_ptr(), gW.data_ptr(), gb.data_ptr(), B, K, R,
+                                            L1, n_psqt, rs, ws.data_ptr(), nbytes, None, _stream(), None), "double_bwd_det")
+        rW, rb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["bias"], c["max_act"],
+                                       c["g_l0"], c["g_wp"], c["g_bp"], saved.cpu().numpy(), R, n_psqt, row_split=rs)
+        counts = np.bincount(np.concatenate([c["widx"][c["widx"] >= 0], c["bidx"][c["bidx"] >= 0]]), minlength=R)
+    assert (counts > rs).sum() > 600      # far more split rows than the 384 whose window sums are kept
+    assert np.array_equal(gW.cpu().numpy(), rW)
+    assert np.array_equal(gb.cpu().numpy(), rb)
+
+
 @pytest.mark.parametrize("B,out_cols,R,K", SPARSE_SHAPES)
 def test_sparse_backward_deterministic(oracle_cpu, B, out_cols, R, K):
     c = sparse_case(300 + B, B, out_cols, R, K, allow_holes=True)
