@@ -304,8 +304,6 @@ __global__ __launch_bounds__(256) void k_chunk_hist(const int32_t* __restrict__ 
                                                     const int32_t* __restrict__ bidx, uint32_t* __restrict__ cnt,
                                                     int B, int K, int R, int cpp, int range) {
     extern __shared__ uint32_t lds_u32[];
-    __shared__ uint32_t idle[64];
-    if (threadIdx.x < 64) idle[threadIdx.x] = 0;
     const int c = blockIdx.x;
     const int r0 = blockIdx.y * range;
     const int nr = min(range, R - r0);
@@ -1150,6 +1148,10 @@ __global__ __launch_bounds__(64) void k_split_combine(const uint32_t* __restrict
 // Table rows per sort pass and whether the chunk's index lists are staged in LDS by k_fill.
 bool lds_plan(int max_lds, int R, int K, int* range_out, int* stage_out, size_t* hist_bytes, size_t* fill_bytes) {
     if (max_lds < 16 * 1024) return false;
+    // what the sort kernels declare statically (scan sums, counters, the spare words of k_fill) comes out of the
+    // same budget as the dynamic part planned here
+    constexpr int kStaticLds = 1024;
+    max_lds -= kStaticLds;
     const size_t stage_bytes = (size_t)kChunk * K * sizeof(int32_t);
     const int stage = stage_bytes <= (size_t)max_lds / 4;
     const size_t avail = (size_t)max_lds - (stage ? stage_bytes : 0);

@@ -69,6 +69,9 @@ SPARSE_SHAPES = [
     (257, 70, 90, 16),      # scalar path, 6 over, every row named several times
     (120, 260, 1000, 32),   # 16-byte path, 1 vector over
     (90, 284, 333, 24),     # 16-byte path, 7 vectors over, range ends inside a group of rows
+    # long lists over a long table: the sort's staged lists and its row counters together want all of a workgroup's LDS
+    (40, 72, 40000, 64),
+    (40, 72, 40000, 80),
 ]
 
 
@@ -122,6 +125,34 @@ def test_sparse_backward_atomic_in_lds_tiles(oracle_cpu, B, out_cols, R, K):
     assert np.array_equal(gb.cpu().numpy(), rb)
     assert lib.nnueft_sparse_bwd_atomic_lds(idx.data_ptr(), g.data_ptr(), gW.data_ptr(), gb.data_ptr(), B, K, R, out_cols,
                                             ws.data_ptr(), nbytes - 1, _stream()) == -2
+
+
+def test_reduction_refuses_lists_sorted_for_another_threshold():
+    """The sorted lists carry the threshold they were made for; a reduction asked for another one leaves the gradient
+    unwritten instead of reading window sums that are not there (the call itself cannot report it: it does not wait
+    for the device)."""
+    nat, lib = _native()
+    B, L1, R, K, n_psqt = 2000, 512, 768, 32, 8
+    out_cols = L1 + n_psqt
+    c = double_case(43, B, L1, R, K, weight_scale=0.05, max_act=0.9)
+    d, l0, wp, bp, saved = _run_double_fwd(c)
+    g_l0, g_wp, g_bp = _t(c["g_l0"]), _t(c["g_wp"]), _t(c["g_bp"])
+    sbytes = lib.nnueft_det_sort_bytes(B, K, R, out_cols, 2)
+    lists = torch.empty(sbytes, dtype=torch.uint8, device=_dev())
+    nat.check(lib.nnueft_det_sort(d["widx"].data_ptr(), d["bidx"].data_ptr(), B, K, R, out_cols, 2, 100, lists.data_ptr(),
+                                  sbytes, _stream()), "det_sort")
+    for rs, written in ((100, True), (512, False), (0, False)):
+        nbytes = lib.nnueft_det_workspace_bytes(B, K, R, out_cols, 2, rs)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=_dev())
+        gW = torch.full((R, out_cols), float("nan"), device=_dev())
+        gb = torch.full((out_cols,), float("nan"), device=_dev())
+        nat.check(lib.nnueft_double_bwd_det(d["us"].data_ptr(), d["them"].data_ptr(), d["widx"].data_ptr(), d["bidx"].data_ptr(),
+                                            d["psqt_idx"].data_ptr(), d["bias"].data_ptr(), c["max_act"], g_l0.data_ptr(),
+                                            g_wp.data_ptr(), g_bp.data_ptr(), saved.data_ptr(), gW.data_ptr(), gb.data_ptr(), B, K, R,
+                                            L1, n_psqt, rs, ws.data_ptr(), nbytes, lists.data_ptr(), _stream(), None), "double_bwd_det")
+        torch.cuda.synchronize()
+        assert bool(torch.isnan(gW).any()) != written
+        assert not bool(torch.isnan(gb).any())   # the bias gradient does not depend on the lists
 
 
 @pytest.mark.parametrize("n_persp", [1, 2])
