@@ -104,10 +104,15 @@ def compulsory_bytes(L1, B, sum_a):
     return fwd, bwd
 
 
-def read_profile_traffic(workload, positions):
+# the summaries under profiles/ of one workload by backward mode: no suffix = the headline's (strict) order
+PROFILE_SUFFIX = {"deterministic_strict": "", "deterministic": "_windowed", "atomic": "_atomic"}
+
+
+def read_profile_traffic(workload, positions, mode="deterministic_strict"):
     """Counter-measured bytes per dispatch (FETCH_SIZE, WRITE_SIZE scaled by a copy kernel of known size) from the
-    tracked summary profiles/<workload>[_game_like]_pmc.txt: lines `traffic <kernel> fetched_bytes=N written_bytes=N`."""
-    name = workload + ("_game_like" if positions == "game" else "") + "_pmc.txt"
+    tracked summary profiles/<workload>[_game_like][_windowed|_atomic]_pmc.txt: lines
+    `traffic <kernel> fetched_bytes=N written_bytes=N`."""
+    name = workload + ("_game_like" if positions == "game" else "") + PROFILE_SUFFIX[mode] + "_pmc.txt"
     path = os.path.join(ROOT, "profiles", name)
     out = {}
     if not os.path.exists(path):
@@ -141,8 +146,12 @@ def fwd_kernels(L1):
     return ("k_pair_hist", "k_pair_scan", "k_pair_scatter", "k_acc_blocked", "k_mix")
 
 
-# (the default order has no k_bias_final launch: the bias gradient's last step rides in k_split_combine)
-BWD_KERNELS = ("k_bwd_rows", "k_chunk_hist", "k_col_scan", "k_row_scan", "k_fill", "k_seg_reduce", "k_split_combine")
+# (the windowed order has no k_bias_final launch: the bias gradient's last step rides in k_split_combine)
+BWD_KERNELS = {
+    "deterministic": ("k_bwd_rows", "k_chunk_hist", "k_col_scan", "k_row_scan", "k_fill", "k_seg_reduce", "k_split_combine"),
+    "deterministic_strict": ("k_bwd_rows", "k_chunk_hist", "k_col_scan", "k_row_scan", "k_fill", "k_seg_reduce", "k_bias_final"),
+    "atomic": ("k_bwd_rows", "k_tl_hist", "k_tl_binscan", "k_tl_lists", "k_scatter_tile", "k_scatter_foreign", "k_bias_final"),
+}
 
 
 # ------------------------------------------------------------------------------------------------
@@ -720,7 +729,7 @@ def run_ft(args, lib, dev):
                 bwd_ms[mode] = det_entry(row_split_of(mode))
 
     # ---- report
-    traffic, traffic_file = read_profile_traffic(args.workload, args.positions)
+    traffic, traffic_file = read_profile_traffic(args.workload, args.positions, modes[0])
     fwd_bytes, _ = algorithmic_bytes(L1, B, sum_a, "atomic")
     comp_fwd, comp_bwd = compulsory_bytes(L1, B, sum_a)
     head_mode = modes[0]
@@ -779,10 +788,11 @@ def run_ft(args, lib, dev):
         bwd_ms.get("deterministic_strict")
     if det:
         alg, gathered, comp = seg_reduce_bytes(L1, B, sum_a)
-        seg_traffic = sum_traffic(traffic, ("k_seg_reduce", "k_split_combine"))
+        seg_traffic = sum_traffic(traffic, ("k_seg_reduce",) + (("k_split_combine",) if head_mode == "deterministic" else ()))
         out["roofline"], out["roofline_compulsory"] = bound_block(
-            "k_seg_reduce<4,3> (timed through nnueft_det_reduce_rows_pitched, which launches it with k_split_combine, which also "
-            "rewinds the task counters, a few microseconds, behind it)", det["reduce"], alg, gathered, comp,
+            "k_seg_reduce<4,3> (timed through nnueft_det_reduce_rows_pitched, which launches it with "
+            + ("k_split_combine" if head_mode == "deterministic" else "k_bias_final")
+            + ", which rewinds the task counters, a few microseconds, behind it)", det["reduce"], alg, gathered, comp,
             seg_traffic, l2_peak,
             note="dominant kernel of the step; it gathers one upstream row per slot through L2 (blocked by king bucket "
                  "and column slice), so `achieved` (algorithmic bytes) is held against what a gather of random 1 KiB "
@@ -811,7 +821,7 @@ def run_ft(args, lib, dev):
             comp_step = sum(comp_fwd.values()) + sum(comp_bwd.values())
             st["compulsory_bytes"] = comp_step
             st["compulsory_frac_of_hbm_peak"] = comp_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS
-            tr = sum_traffic(traffic, fwd_kernels(L1) + BWD_KERNELS) if mode == "deterministic" else None
+            tr = sum_traffic(read_profile_traffic(args.workload, args.positions, mode)[0], fwd_kernels(L1) + BWD_KERNELS[mode])
             st["traffic_bytes"] = tr
             st["traffic_frac_of_hbm_peak"] = tr / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS if tr else None
         else:
@@ -825,6 +835,9 @@ def run_ft(args, lib, dev):
                 comp_step = sum(comp_fwd.values()) + comp_atomic
                 st["compulsory_bytes"] = comp_step
                 st["compulsory_frac_of_hbm_peak"] = comp_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS
+                tr = sum_traffic(read_profile_traffic(args.workload, args.positions, mode)[0], fwd_kernels(L1) + BWD_KERNELS[mode])
+                st["traffic_bytes"] = tr
+                st["traffic_frac_of_hbm_peak"] = tr / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS if tr else None
         if mode in bwd_ms:
             e = bwd_ms[mode]
             st["backward_entry_ms"] = e.get("entry")
