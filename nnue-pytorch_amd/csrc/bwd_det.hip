@@ -60,8 +60,11 @@ constexpr int kLongRow = NNUEFT_LONG_ROW;  // table rows named by at least this 
 #endif
 constexpr int kFillThreads = NNUEFT_FILL_THREADS;   // all of them load the cursors, one wave hands out the ranks
 #ifndef NNUEFT_RUN_U
-#define NNUEFT_RUN_U 16
+#define NNUEFT_RUN_U 32
 #endif
+// rows in flight per lane in the 64-lane-slice chains (window sums of split rows, long rows): a chain of thousands of
+// slots is as many dependent steps as its slots over this number (16 -> 32: the strict order's reduction on game-like
+// lists 1.02 -> 0.94 ms at L1 = 3072, 75 -> 67 us at L1 = 128; nothing elsewhere)
 constexpr int kRunUnroll = NNUEFT_RUN_U;
 #ifndef NNUEFT_TAIL_U
 #define NNUEFT_TAIL_U 8
