@@ -194,6 +194,47 @@ def test_strict_deterministic_backward_bits_equal_the_reference_cpu_path_on_game
     torch.testing.assert_close(windowed, g_cpu, atol=1e-4, rtol=1e-3)
 
 
+def test_backward_modes_agree_on_game_like_lists_at_the_metric_size():
+    """L1=3072, B=16384 with the bucket statistics of game positions (the crowded table blocks hold thousands of pairs:
+    several chunks of lists a block for the LDS tiles, hundreds of split rows for the reduction): the windowed order
+    against the strict one (same bits on the rows it leaves whole, rounding apart on the others) and the atomic adds
+    in LDS tiles against the strict order to the atomic bar; the strict order is pinned against torch CPU autograd
+    and the oracle by the tests above."""
+    L1, B, n_psqt, R = 3072, 16384, 8, hk.NUM_INPUTS
+    us, them, white, black, pc = hk.synthetic_batch(B, 1240, game_like=True)
+    counts = np.bincount(np.concatenate([white[white >= 0], black[black >= 0]]), minlength=R)
+    assert (counts > 512).sum() > 100 and counts.max() > 4000
+    block_pairs = np.bincount(np.concatenate([white[:, 0], black[:, 0]]) // 768, minlength=32)
+    assert block_pairs.max() > 2 * 1536      # more pairs in a block than two chunks of lists hold
+    g = torch.Generator().manual_seed(1240)
+    W0 = (torch.randn(R, L1 + n_psqt, generator=g) * 0.01).to(DEV)
+    b0 = (torch.randn(L1 + n_psqt, generator=g) * 0.01).to(DEV)
+    grads = [torch.randn(B, L1, generator=g).to(DEV), torch.randn(B, 1, generator=g).to(DEV),
+             torch.randn(B, 1, generator=g).to(DEV)]
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    args = [t(us), t(them), t(white), t(black), t((pc - 1) // 4)]
+    got = {}
+    old = nnueft.get_backward_mode()
+    try:
+        for mode in ("deterministic_strict", "deterministic", "atomic"):
+            nnueft.set_backward_mode(mode)
+            W, bias = W0.clone().requires_grad_(), b0.clone().requires_grad_()
+            out = double_feature_transform(*args, W, bias, 255.0 / 256.0, L1, "fused")
+            torch.autograd.backward(list(out), grads)
+            got[mode] = (W.grad, bias.grad)
+    finally:
+        nnueft.set_backward_mode(old)
+    strict_W, strict_b = got["deterministic_strict"]
+    whole = torch.from_numpy(counts <= 512).to(DEV)
+    assert torch.equal(got["deterministic"][0][whole], strict_W[whole])
+    assert not torch.equal(got["deterministic"][0], strict_W)
+    assert torch.equal(got["deterministic"][1], strict_b)
+    scale = strict_W.abs().max()
+    assert (got["deterministic"][0] - strict_W).abs().max() <= 1e-5 * scale
+    assert (got["atomic"][0] - strict_W).abs().max() <= 1e-4 * scale
+    assert torch.equal(got["atomic"][1], strict_b)
+
+
 def test_reduce_rows_stage_equals_the_sparse_backward(oracle_cpu):
     """nnueft_det_sort + nnueft_det_reduce_rows on G = gout is the weight gradient of nnueft_sparse_bwd_det."""
     lib = _native.load()
