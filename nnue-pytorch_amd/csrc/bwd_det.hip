@@ -26,6 +26,7 @@
 #include <atomic>
 
 #include <algorithm>
+#include <cstdlib>
 
 #include "gather.h"
 #include "internal.h"
@@ -106,7 +107,8 @@ constexpr int kLocalMax = 64;        // most local split rows per XCD (a wave ke
 constexpr uint32_t kLocalPerWindow = NNUEFT_LOCAL_PER_WINDOW;
 
 struct DetLayout {
-    size_t G, partial, cnt, wcount, seg_off, long_rows, split_local, sched, list, runs, end;
+    size_t G, partial, cnt, wcount, seg_off, long_rows, split_local, sched, list, chain, runs, end;
+    bool chain_shape;   // the shape can take the strict-order reduction out of LDS tiles (its tables are in the sort block)
     size_t sort_begin, sort_end;   // cnt .. list: what the sort writes and the reduction reads (one block)
     int cpp;     // chunks per perspective
     int nchunks; // n_persp * cpp
@@ -153,6 +155,13 @@ bool det_layout(int B, int K, int R, int out_cols, int n_persp, int row_split, D
     off += up256((size_t)kSchedWords * sizeof(uint32_t));
     L->list = off;
     off += up256((size_t)n_persp * B * K * sizeof(uint32_t));
+    // the two-perspective backward in the strict order takes wide rows out of LDS tiles (bwd_chain.hip) where the
+    // device allows; the tables of that path are part of what the sort writes (last, so that the other tables lie
+    // at the same places whatever the threshold)
+    L->chain = off;
+    const size_t chain_bytes = n_persp == 2 && row_split == 0 ? nnueft_chain::shape_workspace(B, K, R, out_cols, n_persp) : 0;
+    L->chain_shape = chain_bytes != 0;
+    off += chain_bytes;
     L->sort_end = off;
     static_assert(NNUEFT_ROW_WINDOW_MIN % kChunk == 0, "windows are whole sort chunks");
     const int wpos = nnueft_window_positions(B);
@@ -309,7 +318,8 @@ __device__ __forceinline__ const int32_t* chunk_indices(const int32_t* widx, con
 
 __global__ __launch_bounds__(256) void k_chunk_hist(const int32_t* __restrict__ widx,
                                                     const int32_t* __restrict__ bidx, uint32_t* __restrict__ cnt,
-                                                    int B, int K, int R, int cpp, int range) {
+                                                    int B, int K, int R, int cpp, int range, const uint32_t* __restrict__ only_if) {
+    if (only_if && *only_if == 0) return;   // the batch went to the reduction out of LDS tiles
     extern __shared__ uint32_t lds_u32[];
     const int c = blockIdx.x;
     const int r0 = blockIdx.y * range;
@@ -342,7 +352,8 @@ __global__ __launch_bounds__(256) void k_chunk_hist(const int32_t* __restrict__ 
 // Per table row: chunk counts -> exclusive offsets; total and white share.
 __global__ __launch_bounds__(64) void k_col_scan(uint32_t* __restrict__ cnt, uint32_t* __restrict__ wcount,
                                                  uint32_t* __restrict__ seg_off, int R, int cpp, int nchunks,
-                                                 uint32_t row_split) {
+                                                 uint32_t row_split, const uint32_t* __restrict__ only_if) {
+    if (only_if && *only_if == 0) return;   // the batch went to the reduction out of LDS tiles
     const int r = blockIdx.x * 64 + threadIdx.x;
     if (r >= R) return;
     constexpr int PF = 16;
@@ -417,7 +428,8 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
                                                            uint32_t* __restrict__ long_rows,
                                                            uint32_t* __restrict__ split_local,
                                                            uint32_t* __restrict__ sched, int R, int cap,
-                                                           uint32_t row_split, uint32_t split_cap, uint32_t local_len) {
+                                                           uint32_t row_split, uint32_t split_cap, uint32_t local_len, const uint32_t* __restrict__ only_if) {
+    if (only_if && *only_if == 0) return;   // the batch went to the reduction out of LDS tiles
     extern __shared__ uint32_t stage[];   // `cap` row lengths, turned into offsets in place
     // two running sums: all slots, and what slots_elsewhere() takes off the weight of the row ranges
     __shared__ uint32_t wave_tot[2][kScanThreads / 64];
@@ -661,7 +673,8 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
 __global__ __launch_bounds__(kFillThreads) void k_fill(const int32_t* __restrict__ widx, const int32_t* __restrict__ bidx,
                                               const uint32_t* __restrict__ cnt,
                                               const uint32_t* __restrict__ seg_off, uint32_t* __restrict__ list,
-                                              int B, int K, int R, int cpp, int range, int stage) {
+                                              int B, int K, int R, int cpp, int range, int stage, const uint32_t* __restrict__ only_if) {
+    if (only_if && *only_if == 0) return;   // the batch went to the reduction out of LDS tiles
     extern __shared__ uint32_t lds_u32[];
     __shared__ uint32_t idle[64];
     if (threadIdx.x < 64) idle[threadIdx.x] = 0;
@@ -947,7 +960,8 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
                                                    const uint32_t* __restrict__ long_rows,
                                                    uint32_t* __restrict__ sched, float* __restrict__ gW,
                                                    int out_cols, int nslices, int slice_v, int two_persp,
-                                                   RunPlan rp) {
+                                                   RunPlan rp, const uint32_t* __restrict__ only_if) {
+    if (only_if && *only_if == 0) return;   // the batch went to the reduction out of LDS tiles
     const int lane = threadIdx.x;
     const int xcd = blockIdx.x % kXcd;
     if (sched[kSchedRowSplit] != rp.row_split) return;   // the lists were sorted for another threshold
@@ -1199,8 +1213,19 @@ int allow_full_lds(int device, int max_lds) {
 
 // The sort: everything the reduction needs to know about the index lists (it reads no gradient).
 // `sorted` is the block [L.sort_begin, L.sort_end) of the layout, wherever the caller keeps it.
-int det_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, char* sorted, const DetLayout& L,
-             hipStream_t st) {
+// Whether this call takes the strict-order reduction out of LDS tiles: the shape and the threshold say so (the
+// layout), and the device.
+bool chain_in_use(const DetLayout& L, const nnueft_dev::DeviceInfo& d) {
+    // NNUEFT_STRICT_LDS=0 in the environment keeps every batch on the segmented reduction (for comparing the two)
+    static const bool enabled = [] {
+        const char* e = getenv("NNUEFT_STRICT_LDS");
+        return !(e && e[0] == '0');
+    }();
+    return enabled && L.chain_shape && L.row_split == 0 && nnueft_chain::device_ok(d);
+}
+
+int det_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, int n_persp, char* sorted,
+             const DetLayout& L, hipStream_t st) {
     char* ws = sorted - L.sort_begin;
     uint32_t* cnt = (uint32_t*)(ws + L.cnt);
     uint32_t* wcount = (uint32_t*)(ws + L.wcount);
@@ -1222,18 +1247,25 @@ int det_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, char
     const int scan_cap = max(kScanThreads, min(range, (R + kScanThreads - 1) / kScanThreads * kScanThreads));
     rc = allow_full_lds(device, info->max_lds);
     if (rc) return rc;
+    // with the tables of the LDS-tiled reduction made first, the kernels below run only for a batch it cannot take
+    const uint32_t* only_if = nullptr;
+    if (chain_in_use(L, *info)) {
+        rc = nnueft_chain::sort(widx, bidx, B, K, R, n_persp, ws + L.chain, st);
+        if (rc) return rc;
+        only_if = nnueft_chain::fallback_flag(ws + L.chain, B, R, n_persp);
+    }
     hipLaunchKernelGGL(k_chunk_hist, dim3(L.nchunks, nranges), dim3(256), hist_bytes, st, widx, bidx, cnt, B, K, R,
-                       L.cpp, range);
+                       L.cpp, range, only_if);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_col_scan, dim3((R + 63) / 64), dim3(64), 0, st, cnt, wcount, seg_off, R, L.cpp,
-                       L.nchunks, (uint32_t)L.row_split);
+                       L.nchunks, (uint32_t)L.row_split, only_if);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_row_scan, dim3(1), dim3(kScanThreads), (size_t)scan_cap * sizeof(uint32_t), st, seg_off,
                        long_rows, split_local, sched, R, scan_cap, (uint32_t)L.row_split, (uint32_t)L.max_split,
-                       kLocalPerWindow * (uint32_t)(L.nchunks / L.cpp) * (uint32_t)L.nwin);
+                       kLocalPerWindow * (uint32_t)(L.nchunks / L.cpp) * (uint32_t)L.nwin, only_if);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_fill, dim3(L.nchunks, nranges), dim3(kFillThreads), fill_bytes, st, widx, bidx, cnt, seg_off, list,
-                       B, K, R, L.cpp, range, stage);
+                       B, K, R, L.cpp, range, stage, only_if);
     NNUEFT_LAUNCH_CHECK();
     return 0;
 }
@@ -1250,6 +1282,22 @@ int det_reduce(const float* G, int g_pitch, float* gW, float* gbias, int B, int 
     uint32_t* list = (uint32_t*)(sw + L.list);
     float* partial = (float*)(ws + L.partial);
 
+    // the strict order out of LDS tiles where the sort made its tables; the kernels below then run only for a
+    // batch that path could not take
+    const uint32_t* only_if = nullptr;
+    {
+        int device = 0;
+        const nnueft_dev::DeviceInfo* info = nullptr;
+        int rc = nnueft_dev::device_info(&device, &info);
+        if (rc) return rc;
+        if (chain_in_use(L, *info) && g_pitch % 4 == 0 && aligned16(G)) {
+            rc = nnueft_chain::reduce(G, g_pitch, gW, B, R, out_cols, n_persp, sw + L.chain, st);
+            if (rc) return rc;
+            only_if = nnueft_chain::fallback_flag(sw + L.chain, B, R, n_persp);
+        } else if (chain_in_use(L, *info)) {
+            return NNUEFT_E_UNSUPPORTED;   // the sort left the lists to the other path, which needs 16-byte rows
+        }
+    }
     const bool vec = (out_cols % 4 == 0) && (g_pitch % 4 == 0) && aligned16(G) && aligned16(gW);
     const int VWr = vec ? 4 : 1;
     const int nv = out_cols / VWr;
@@ -1288,7 +1336,7 @@ int det_reduce(const float* G, int g_pitch, float* gW, float* gbias, int B, int 
     if ((long long)L.max_split * rp.nslices * NNUEFT_ROW_WINDOWS > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
 #define SEG_LAUNCH(VW_, NQ_)                                                                                      \
     hipLaunchKernelGGL((k_seg_reduce<VW_, NQ_>), dim3(kXcd * kWavesPerXcd), dim3(64), 0, st, G, list, seg_off,      \
-                       wcount, long_rows, sched, gW, out_cols, nslices, slice_v, two, rp)
+                       wcount, long_rows, sched, gW, out_cols, nslices, slice_v, two, rp, only_if)
     if (vec && NQ > 1) SEG_LAUNCH(4, NNUEFT_SEG_NQ);
     else if (vec) SEG_LAUNCH(4, 1);
     else if (NQ > 1) SEG_LAUNCH(1, NNUEFT_SEG_NQ);
@@ -1382,7 +1430,7 @@ extern "C" int nnueft_det_sort(const int32_t* widx, const int32_t* bidx, int B, 
     if (!det_layout(B, K, R, out_cols, n_persp, row_split, &L)) return NNUEFT_E_ARG;
     if (!sorted_lists || !aligned256(sorted_lists) || sorted_bytes < L.sort_end - L.sort_begin)
         return NNUEFT_E_WORKSPACE;
-    return det_sort(widx, n_persp == 2 ? bidx : widx, B, K, R, (char*)sorted_lists, L, (hipStream_t)stream);
+    return det_sort(widx, n_persp == 2 ? bidx : widx, B, K, R, n_persp, (char*)sorted_lists, L, (hipStream_t)stream);
 }
 
 extern "C" int nnueft_det_upstream_pitch(int out_cols) { return out_cols > 0 ? g_pitch_of(out_cols) : 0; }
@@ -1421,7 +1469,7 @@ extern "C" int nnueft_sparse_bwd_det(const int32_t* idx, const float* gout, floa
     hipLaunchKernelGGL(k_tile_colsum, dim3(L.ntiles, (out_cols + 255) / 256), dim3(256), 0, st, gout,
                        (float*)(ws + L.partial), B, out_cols);
     NNUEFT_LAUNCH_CHECK();
-    const int rc = det_sort(idx, idx, B, K, R, ws + L.sort_begin, L, st);
+    const int rc = det_sort(idx, idx, B, K, R, 1, ws + L.sort_begin, L, st);
     if (rc) return rc;
     return det_reduce(gout, out_cols, gW, gbias, B, R, out_cols, 1, ws, ws + L.sort_begin, L, st);
 }
@@ -1477,7 +1525,7 @@ extern "C" int nnueft_double_bwd_det(const float* us, const float* them, const i
         if (e == hipSuccess) e = hipStreamWaitEvent(aux, forked, 0);
         if (e != hipSuccess) return (int)e;
     }
-    int rc = det_sort(widx, bidx, B, K, R, ws + L.sort_begin, L, two_streams ? aux : st);
+    int rc = det_sort(widx, bidx, B, K, R, 2, ws + L.sort_begin, L, two_streams ? aux : st);
     hipError_t sorted = hipSuccess;
     if (two_streams) sorted = hipEventRecord(joined, aux);
     // the upstream rows go onto the caller's stream before it is made to wait for the sort

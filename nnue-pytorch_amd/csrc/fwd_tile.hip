@@ -713,6 +713,13 @@ int allow_lds(int device) {
     return 0;
 }
 
+int launch_binscan(uint32_t* hist, uint32_t* total, int nbins, int ngroups, hipStream_t st) {
+    hipLaunchKernelGGL(k_tl_binscan, dim3((nbins + kSortThreads / 64 - 1) / (kSortThreads / 64)), dim3(kSortThreads), 0, st, hist,
+                       total, nbins, ngroups);
+    NNUEFT_LAUNCH_CHECK();
+    return 0;
+}
+
 int launch_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, const Layout& L, void* ws, hipStream_t st,
                 Sorted* out) {
     char* base = (char*)ws;

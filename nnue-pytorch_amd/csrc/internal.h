@@ -90,6 +90,21 @@ int int16_fused_tile(const int32_t* widx, const int32_t* bidx, const uint8_t* st
                      hipStream_t st);
 }  // namespace nnueft_tile
 
+namespace nnueft_chain {
+
+// The strict-order backward out of LDS tiles (bwd_chain.hip).  shape_workspace(): bytes of its tables, 0 where the
+// shape cannot take it; device_ok(): whether the device can; sort(): the tables of a batch's index lists; reduce():
+// the weight gradient from the upstream rows G[n_persp * B, g_pitch] (every element of gW written).  A batch whose
+// lists it cannot take (rows of two blocks, or a row twice, in one list) sets *fallback_flag(): reduce() then does
+// nothing, and the caller's other path has to run; the flag is valid once sort() has run on the stream.
+size_t shape_workspace(int B, int K, int R, int out_cols, int n_persp);
+bool device_ok(const nnueft_dev::DeviceInfo& d);
+const uint32_t* fallback_flag(const void* ws, int B, int R, int n_persp);
+int sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, int n_persp, void* ws, hipStream_t st);
+int reduce(const float* G, int g_pitch, float* gW, int B, int R, int out_cols, int n_persp, void* ws, hipStream_t st);
+
+}  // namespace nnueft_chain
+
 namespace nnueft_det {
 
 // Upstream rows G[2, B, g_pitch] (L1 + n_psqt floats of a row used) of the two sparse-linear outputs and the

@@ -82,6 +82,9 @@ struct Sorted {
 int launch_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, const Layout& L, void* ws, hipStream_t st,
                 Sorted* out);
 
+// One wave per bin: hist[bin][0 .. ngroups) becomes its exclusive prefix, total[bin] the sum.
+int launch_binscan(uint32_t* hist, uint32_t* total, int nbins, int ngroups, hipStream_t st);
+
 static inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 }  // namespace nnueft_tile

@@ -63,8 +63,13 @@ def test_host_only_entry_points():
     assert lib.nnueft_det_workspace_bytes(16384, 32, 24576, 3080, 2, 1) == a
     assert a - strict <= 384 * 2 * 16 * 3080 * 4 + 4096 and a <= 600 * 1000 * 1000
     # a small batch cannot split that many rows: 2 * 64 * 32 slots over a threshold of 512 make 7 rows at most
-    small = lib.nnueft_det_workspace_bytes(64, 32, 24576, 3080, 2, 512) - lib.nnueft_det_workspace_bytes(64, 32, 24576, 3080, 2, 0)
+    # (against a threshold that no row can reach: no window sums at all)
+    small = lib.nnueft_det_workspace_bytes(64, 32, 24576, 3080, 2, 512) - lib.nnueft_det_workspace_bytes(64, 32, 24576, 3080, 2, 2 * 64 * 32)
     assert 0 < small <= 7 * 2 * 1 * 3080 * 4 + 4096
+    # the strict order keeps the tables of its reduction out of LDS tiles beside the sorted lists: a chunk table, and
+    # per chunk of 624 pairs its inverted lists (65 KB at most) and the facts of its chains
+    tables = strict - lib.nnueft_det_workspace_bytes(16384, 32, 24576, 3080, 2, 2 * 16384 * 32)
+    assert 0 < tables <= 13 * 1000 * 1000
     assert lib.nnueft_det_workspace_bytes(0, 32, 10, 8, 1, 512) == 0
     assert lib.nnueft_det_workspace_bytes(4, 32, 10, 8, 3, 512) == 0
     assert lib.nnueft_det_workspace_bytes(4, 32, 10, 8, 1, -1) == 0

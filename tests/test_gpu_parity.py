@@ -517,6 +517,90 @@ def test_sparse_backward_deterministic_with_split_rows(oracle_cpu, row_split, B,
     assert np.array_equal(gb.cpu().numpy(), rb)
 
 
+def _strict_tile_lists(kind, B, R, K, rng):
+    """Index lists for the strict order's reduction out of LDS tiles (every list inside one 768-row block)."""
+    nblocks = (R + 767) // 768
+
+    def lists(blocks, n_valid):
+        out = np.full((B, K), -1, np.int32)
+        for b in range(B):
+            rows_here = min(768, R - blocks[b] * 768)
+            out[b, :n_valid[b]] = blocks[b] * 768 + rng.choice(rows_here, size=n_valid[b], replace=False)
+        return out
+
+    n_valid = rng.integers(1, K + 1, size=B)
+    if kind == "one_block":
+        # several chunks of 624 pairs for either perspective: the chains go from chunk to chunk through LDS, the
+        # white sums wait in the gradient while the black ones are made
+        w, b = lists(np.full(B, 1), n_valid), lists(np.full(B, 1), n_valid[::-1])
+        w[:, 0] = 768 + 5     # a row that every white list names (summed without a list)
+        for ix in (w, b):     # ... entered once only
+            for r in range(B):
+                dup = np.flatnonzero(ix[r, 1:] == ix[r, 0]) + 1
+                ix[r, dup] = -1
+    elif kind == "white_heavy":
+        # one block with many white chunks and a single black one; other blocks with black pairs only
+        w, b = lists(np.full(B, 0), n_valid), lists(rng.integers(0, nblocks, size=B), n_valid)
+    elif kind == "last_block":
+        # a table whose last block is short, blocks without any pair, an empty list
+        blocks = rng.choice([0, nblocks - 1], size=B)
+        w, b = lists(blocks, n_valid), lists(blocks[::-1], n_valid)
+        w[3] = -1
+    elif kind == "two_blocks_in_a_list":
+        w, b = lists(rng.integers(0, nblocks, size=B), n_valid), lists(rng.integers(0, nblocks, size=B), n_valid)
+        w[B // 2, :2] = (5, 768 * (nblocks - 1) + 1)     # left to the segmented reduction, all of the batch
+    elif kind == "a_row_twice":
+        w, b = lists(rng.integers(0, nblocks, size=B), n_valid), lists(rng.integers(0, nblocks, size=B), n_valid)
+        b[B // 3, :2] = b[B // 3, 0]
+    else:
+        raise ValueError(kind)
+    return w, b
+
+
+@pytest.mark.parametrize("kind,B,L1,R", [("one_block", 2100, 256, 2000), ("white_heavy", 1500, 512, 3000),
+                                         ("last_block", 700, 264, 768 * 3 + 100), ("two_blocks_in_a_list", 900, 256, 2400),
+                                         ("a_row_twice", 900, 256, 2400)])
+def test_double_backward_strict_order_out_of_lds_tiles(oracle_cpu, kind, B, L1, R):
+    """Rows of 256 columns and more, lists of up to 32 slots, strict order: the chains are summed out of LDS tiles."""
+    K, n_psqt = 32, 8
+    rng = np.random.default_rng(len(kind) * 1000 + B)
+    c = double_case(1300 + B, B, L1, R, K, binary_side=True)
+    c["widx"], c["bidx"] = _strict_tile_lists(kind, B, R, K, rng)
+    nat, lib = _native()
+    out_cols = L1 + n_psqt
+    d, l0, wp, bp, saved = _run_double_fwd(c)
+    g_l0, g_wp, g_bp = _t(c["g_l0"]), _t(c["g_wp"]), _t(c["g_bp"])
+    head = (d["us"].data_ptr(), d["them"].data_ptr(), d["widx"].data_ptr(), d["bidx"].data_ptr(),
+            d["psqt_idx"].data_ptr(), d["bias"].data_ptr(), c["max_act"], g_l0.data_ptr(), g_wp.data_ptr(),
+            g_bp.data_ptr(), saved.data_ptr())
+    nbytes = lib.nnueft_det_workspace_bytes(B, K, R, out_cols, 2, 0)
+    ws = torch.full((nbytes,), 0x3C, dtype=torch.uint8, device=_dev())
+    rW, rb = oracle_cpu.double_bwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], c["bias"], c["max_act"],
+                                   c["g_l0"], c["g_wp"], c["g_bp"], saved.cpu().numpy(), R, n_psqt, row_split=0)
+    # a gradient at a 16-byte boundary, and one 4 bytes past it (stored a float at a time)
+    flat = torch.full((R * out_cols + 1,), float("nan"), device=_dev())
+    for gW in (flat[:R * out_cols].view(R, out_cols), flat[1:].view(R, out_cols)):
+        gb = torch.full((out_cols,), float("nan"), device=_dev())
+        nat.check(lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt, 0, ws.data_ptr(),
+                                            nbytes, None, _stream(), None), "double_bwd_det")
+        assert np.array_equal(gW.cpu().numpy(), rW)
+        assert np.array_equal(gb.cpu().numpy(), rb)
+        flat.fill_(float("nan"))
+    # lists sorted beforehand, used twice (the reduction leaves its counters as it found them)
+    sbytes = lib.nnueft_det_sort_bytes(B, K, R, out_cols, 2)
+    lists = torch.full((sbytes,), 0x5A, dtype=torch.uint8, device=_dev())
+    nat.check(lib.nnueft_det_sort(d["widx"].data_ptr(), d["bidx"].data_ptr(), B, K, R, out_cols, 2, 0,
+                                  lists.data_ptr(), sbytes, _stream()), "det_sort")
+    gW = torch.empty(R, out_cols, device=_dev())
+    for _ in range(2):
+        gW.fill_(float("nan"))
+        gb = torch.full((out_cols,), float("nan"), device=_dev())
+        nat.check(lib.nnueft_double_bwd_det(*head, gW.data_ptr(), gb.data_ptr(), B, K, R, L1, n_psqt, 0, ws.data_ptr(),
+                                            nbytes, lists.data_ptr(), _stream(), None), "double_bwd_det")
+        assert np.array_equal(gW.cpu().numpy(), rW)
+        assert np.array_equal(gb.cpu().numpy(), rb)
+
+
 def test_deterministic_backward_repeats_bitwise():
     """Two runs of the deterministic backward give the same bits (the atomic one need not)."""
     c = double_case(77, 300, 256, 600, 32, binary_side=True)
