@@ -141,15 +141,39 @@ bool chain_layout(int B, int n_persp, int R, ChainLayout* L) {
 // a value every lane holds alike, moved to a scalar register
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
+// A pair's list in registers: kSlots entries, -1 beyond K; 16-byte loads when `vec` (K a multiple of 4, the lists at
+// 16-byte boundaries), so that the list is one or two trips to memory and not K.
+struct ListRegs {
+    int v[kSlots];
+};
+
+__device__ __forceinline__ ListRegs load_list(const int32_t* __restrict__ ix, int K, bool vec) {
+    ListRegs l;
+    if (vec) {
+        const int4* p = reinterpret_cast<const int4*>(ix);
+#pragma unroll
+        for (int q = 0; q < kSlots / 4; ++q) {
+            const int4 t = 4 * q < K ? p[q] : make_int4(-1, -1, -1, -1);
+            l.v[4 * q] = t.x; l.v[4 * q + 1] = t.y; l.v[4 * q + 2] = t.z; l.v[4 * q + 3] = t.w;
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < kSlots; ++k) l.v[k] = k < K ? ix[k] : -1;
+    }
+    return l;
+}
+
 // The key of a pair's list: (block of its first valid entry) * 2 + perspective; nkeys for a list that names rows of
 // more than one block.  A list without a valid entry belongs to block 0 (it adds nothing anywhere).
-__device__ __forceinline__ int list_key(const int32_t* __restrict__ ix, int K, int R, int persp, int nkeys) {
+__device__ __forceinline__ int list_key(const ListRegs& l, int R, int persp, int nkeys) {
     int block = -1;
     bool foreign = false;
-    for (int k = 0; k < K; ++k) {
-        const int r = ix[k];
+#pragma unroll
+    for (int k = 0; k < kSlots; ++k) {
+        const int r = l.v[k];
         if (r >= 0 && r < R) {
-            const int b = r / kRows;
+            // r / 768 for r below 2^32 / 768, without the division
+            const int b = (int)__umulhi((uint32_t)r, 0xffffffffu / (uint32_t)kRows + 1u);
             if (block < 0) block = b;
             foreign |= b != block;
         }
@@ -168,7 +192,7 @@ __device__ __forceinline__ const int32_t* pair_list(const int32_t* __restrict__ 
 __global__ __launch_bounds__(kSortThreads) void k_cs_hist(const int32_t* __restrict__ widx,
                                                           const int32_t* __restrict__ bidx,
                                                           uint32_t* __restrict__ hist, int npairs, int B, int K, int R,
-                                                          int nkeys) {
+                                                          int nkeys, int vec) {
     __shared__ uint32_t bins[kMaxKeys + 1];
     const int tid = threadIdx.x;
     const int n = blockIdx.x * kSortThreads + tid;
@@ -177,7 +201,7 @@ __global__ __launch_bounds__(kSortThreads) void k_cs_hist(const int32_t* __restr
     if (n < npairs) {
         int persp;
         const int32_t* ix = pair_list(widx, bidx, n, B, K, &persp);
-        atomicAdd(&bins[list_key(ix, K, R, persp, nkeys)], 1u);
+        atomicAdd(&bins[list_key(load_list(ix, K, vec), R, persp, nkeys)], 1u);
     }
     __syncthreads();
     for (int i = tid; i <= nkeys; i += kSortThreads) hist[(size_t)i * gridDim.x + blockIdx.x] = bins[i];
@@ -193,7 +217,7 @@ __global__ __launch_bounds__(kSortThreads) void k_cs_place(const int32_t* __rest
                                                            uint32_t* __restrict__ bpairs, RChunk* __restrict__ chunks,
                                                            BlockChunks* __restrict__ ublocks,
                                                            uint32_t* __restrict__ sched, int npairs, int n_persp, int B,
-                                                           int K, int R, int nkeys, int nblocks) {
+                                                           int K, int R, int nkeys, int nblocks, int vec) {
     __shared__ uint32_t keybase[kMaxKeys + 1];
     __shared__ uint32_t wcnt[kSortThreads / 64][kMaxKeys];
     __shared__ uint32_t chunk0[kMaxKeys + 1];
@@ -202,14 +226,17 @@ __global__ __launch_bounds__(kSortThreads) void k_cs_place(const int32_t* __rest
     const int ngroups = gridDim.x;
     for (int i = tid; i < (kSortThreads / 64) * kMaxKeys; i += kSortThreads) (&wcnt[0][0])[i] = 0;
     if (blockIdx.x == 0 && tid < 64) bpairs[npairs + tid] = 0;   // a chunk without pairs reads one id at its start
+    __shared__ uint32_t tot[kMaxKeys + 1];
+    for (int i = tid; i <= nkeys; i += kSortThreads) tot[i] = total[i];
+    __syncthreads();
     if (tid == 0) {
         uint32_t run = 0, cr = 0;
         for (int k = 0; k < nkeys; ++k) {
             keybase[k] = run;
             chunk0[k] = cr;
-            run += total[k];
+            run += tot[k];
             // a single list of the batch (n_persp == 1) has no black chunks at all
-            cr += (n_persp == 1 && (k & 1)) ? 0 : chunks_of((int)total[k]);
+            cr += (n_persp == 1 && (k & 1)) ? 0 : chunks_of((int)tot[k]);
         }
         keybase[nkeys] = run;
         chunk0[nkeys] = cr;
@@ -219,7 +246,7 @@ __global__ __launch_bounds__(kSortThreads) void k_cs_place(const int32_t* __rest
     if (n < npairs) {
         int persp;
         const int32_t* ix = pair_list(widx, bidx, n, B, K, &persp);
-        key = list_key(ix, K, R, persp, nkeys);
+        key = list_key(load_list(ix, K, vec), R, persp, nkeys);
     }
     // a pair's place among the pairs of its key in this workgroup: those of the waves in front, then those of the
     // lanes in front
@@ -243,10 +270,10 @@ __global__ __launch_bounds__(kSortThreads) void k_cs_place(const int32_t* __rest
     if (blockIdx.x != 0) return;
     // the first workgroup also writes the tables of the batch
     for (int i = tid; i < kSchedWords; i += kSortThreads)
-        sched[i] = i == kFlagWord ? (total[nkeys] != 0 ? 1u : 0u) : i == kChunksWord ? chunk0[nkeys] : 0u;
+        sched[i] = i == kFlagWord ? (tot[nkeys] != 0 ? 1u : 0u) : i == kChunksWord ? chunk0[nkeys] : 0u;
     for (int k = tid; k < nkeys; k += kSortThreads) {
         if (n_persp == 1 && (k & 1)) continue;
-        const int nk = (int)total[k];
+        const int nk = (int)tot[k];
         const int nc = chunks_of(nk);
         const int ln = (nk + nc - 1) / nc;
         for (int j = 0; j < nc; ++j) {
@@ -264,14 +291,14 @@ __global__ __launch_bounds__(kSortThreads) void k_cs_place(const int32_t* __rest
         }
     }
     for (int b = tid; b < nblocks; b += kSortThreads) {
-        const uint32_t mine = total[2 * b] + total[2 * b + 1];
+        const uint32_t mine = tot[2 * b] + tot[2 * b + 1];
         int r = 0;
         for (int o = 0; o < nblocks; ++o) {
-            const uint32_t other = total[2 * o] + total[2 * o + 1];
+            const uint32_t other = tot[2 * o] + tot[2 * o + 1];
             r += other > mine || (other == mine && o < b);
         }
-        ublocks[r] = BlockChunks{(int)chunk0[2 * b], chunks_of((int)total[2 * b]),
-                                 n_persp == 1 ? 0 : chunks_of((int)total[2 * b + 1]), b};
+        ublocks[r] = BlockChunks{(int)chunk0[2 * b], chunks_of((int)tot[2 * b]),
+                                 n_persp == 1 ? 0 : chunks_of((int)tot[2 * b + 1]), b};
     }
 }
 
@@ -280,7 +307,7 @@ __global__ __launch_bounds__(kThreads) void k_cs_expand(const int32_t* __restric
                                                         const int32_t* __restrict__ bidx,
                                                         const uint32_t* __restrict__ bpairs, RChunk* __restrict__ chunks,
                                                         uint32_t* __restrict__ md, uint16_t* __restrict__ ent,
-                                                        uint32_t* __restrict__ sched, int B, int K, int R) {
+                                                        uint32_t* __restrict__ sched, int B, int K, int R, int vec) {
     extern __shared__ float4 lds_raw[];
     uint32_t* mask = reinterpret_cast<uint32_t*>(lds_raw);             // [kRows][kMaskWords]
     uint32_t* keys = mask + kRows * kMaskWords;                        // [1024] sort keys, then the rows in slot order
@@ -299,11 +326,12 @@ __global__ __launch_bounds__(kThreads) void k_cs_expand(const int32_t* __restric
     if (tid < C.count) {
         const int pair = (int)bpairs[C.start + tid];
         int persp;
-        const int32_t* ix = pair_list(widx, bidx, pair, B, K, &persp);
+        const ListRegs l = load_list(pair_list(widx, bidx, pair, B, K, &persp), K, vec);
         const int row0 = C.block * kRows;
         bool twice = false;
-        for (int k = 0; k < K; ++k) {
-            const int r = ix[k];
+#pragma unroll
+        for (int k = 0; k < kSlots; ++k) {
+            const int r = l.v[k];
             if (r >= 0 && r < R) {
                 const uint32_t bit = 1u << (tid & 31);
                 twice |= (atomicOr(&mask[(r - row0) * kMaskWords + (tid >> 5)], bit) & bit) != 0;
@@ -517,8 +545,16 @@ __global__ __launch_bounds__(kThreads) void k_chain_tile(const float* __restrict
     // the loads.
     f4 v[IT];
     u4 t[LI];
-    u4 tm;
+    u4 tm = u4{0u, 0u, 0u, 0u};
     uint32_t pr[IT];   // the pair ids of the rows a thread loads, read a step earlier
+#pragma unroll
+    for (int i = 0; i < IT; ++i) {
+        v[i] = f4{0.f, 0.f, 0.f, 0.f};
+        pr[i] = 0;
+    }
+#pragma unroll
+    for (int i = 0; i < LI; ++i) t[i] = u4{0u, 0u, 0u, 0u};
+    const int wave0 = uni(tid & ~63);   // the wave's first thread
 #define NNUEFT_PREFETCH(C_, ci_, c_, cols_)                                                               \
     {                                                                                                     \
         const int col0_ = (c_) * kCols;                                                                   \
@@ -526,18 +562,20 @@ __global__ __launch_bounds__(kThreads) void k_chain_tile(const float* __restrict
         const int n16_ = (C_).n4 >> 1;                                                                    \
         _Pragma("unroll") for (int i_ = 0; i_ < IT; ++i_) {                                               \
             const int p4_ = (tid + i_ * NT) & 3;                                                          \
-            v[i_] = *reinterpret_cast<const f4*>(G + (size_t)pr[i_] * g_pitch + col0_ +                   \
-                                                 (p4_ * 4 < (cols_) ? p4_ * 4 : 0));                      \
+            /* a wave whose rows all lie beyond the chunk's pairs loads nothing */                         \
+            if ((wave0 + i_ * NT) >> 2 < (C_).count)                                                      \
+                v[i_] = *reinterpret_cast<const f4*>(G + (size_t)pr[i_] * g_pitch + col0_ +               \
+                                                     (p4_ * 4 < (cols_) ? p4_ * 4 : 0));                  \
         }                                                                                                 \
         _Pragma("unroll") for (int i_ = 0; i_ < LI; ++i_)                                                 \
-            t[i_] = src_[min(tid + i_ * NT, max(n16_ - 1, 0))];                                           \
-        tm = reinterpret_cast<const u4*>(md + (size_t)(ci_) * kMdWords)[min(tid, MD16 - 1)];              \
+            if (wave0 + i_ * NT < n16_) t[i_] = src_[min(tid + i_ * NT, n16_ - 1)];                       \
+        if (wave0 < MD16) tm = reinterpret_cast<const u4*>(md + (size_t)(ci_) * kMdWords)[min(tid, MD16 - 1)]; \
     }
 #define NNUEFT_PAIR_IDS(C_)                                                                               \
     {                                                                                                     \
         _Pragma("unroll") for (int i_ = 0; i_ < IT; ++i_) {                                               \
             const int row_ = (tid + i_ * NT) >> 2;                                                        \
-            pr[i_] = bpairs[(C_).start + max(min(row_, (C_).count - 1), 0)];                              \
+            if ((wave0 + i_ * NT) >> 2 < (C_).count) pr[i_] = bpairs[(C_).start + min(row_, (C_).count - 1)]; \
         }                                                                                                 \
     }
 
@@ -560,30 +598,50 @@ __global__ __launch_bounds__(kThreads) void k_chain_tile(const float* __restrict
                 const uint32_t off = (uint32_t)(uintptr_t)tb + col * 4;
                 float* sp = reinterpret_cast<float*>(lsum) + row * kCols + col;
                 float a = 0.f;
-                if (!first) a = *sp;
+                if (!first) asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(a) : "v"((uint32_t)(uintptr_t)sp));
                 // a long chain is what the step waits for: its wave goes first on its SIMD
                 __builtin_amdgcn_s_setprio(3);
                 if (tmd & 0x80000000u) {
                     // a chain that every pair of the chunk is part of: the tile's rows from the first to the last, no
                     // list; nb blocks of 16 rows (rows past the chunk's pairs are zero)
+                    // Written instruction by instruction: two blocks of 16 rows are in flight, and a wait lets the
+                    // older one land while the younger one stays out (the compiler's own placement of the waits
+                    // drains the queue once per block, which is what this chain, the longest of the step, waits for).
+                    // The waits are tied to the registers they make valid, so that no add moves in front of them.
+                    typedef float f2 __attribute__((ext_vector_type(2)));
+                    f2 qa[8], qb[8];
+#define NNUEFT_RD2(dst_, addr_, o0_, o1_) \
+    asm volatile("ds_read2_b32 %0, %1 offset0:" #o0_ " offset1:" #o1_ : "=v"(dst_) : "v"(addr_))
+#define NNUEFT_ISSUE16(q_, addr_)                                                                          \
+    NNUEFT_RD2(q_[0], addr_, 0, 16); NNUEFT_RD2(q_[1], addr_, 32, 48); NNUEFT_RD2(q_[2], addr_, 64, 80);    \
+    NNUEFT_RD2(q_[3], addr_, 96, 112); NNUEFT_RD2(q_[4], addr_, 128, 144); NNUEFT_RD2(q_[5], addr_, 160, 176); \
+    NNUEFT_RD2(q_[6], addr_, 192, 208); NNUEFT_RD2(q_[7], addr_, 224, 240);
+#define NNUEFT_LANDED(n_, q_)                                                                              \
+    asm volatile("s_waitcnt lgkmcnt(" #n_ ")"                                                             \
+                 : "+v"(q_[0]), "+v"(q_[1]), "+v"(q_[2]), "+v"(q_[3]), "+v"(q_[4]), "+v"(q_[5]), "+v"(q_[6]), "+v"(q_[7]))
+#define NNUEFT_ADD16(q_)                                                                                   \
+    _Pragma("unroll") for (int h = 0; h < 8; ++h) {                                                        \
+        a += q_[h].x;                                                                                      \
+        a += q_[h].y;                                                                                      \
+    }
+                    static_assert(kRowB == 64, "offsets of the reads: 16 dwords a row");
                     uint32_t pa = off;
-                    constexpr int DU = 16;
-                    float r0[DU], r1[DU];
-#pragma unroll
-                    for (int h = 0; h < DU; ++h) r0[h] = *reinterpret_cast<lds_f*>(pa + h * kRowB);
+                    NNUEFT_ISSUE16(qa, pa)
                     for (int k = 0; k < nb; k += 2) {
-#pragma unroll
-                        for (int h = 0; h < DU; ++h) r1[h] = *reinterpret_cast<lds_f*>(pa + (DU + h) * kRowB);
-#pragma unroll
-                        for (int h = 0; h < DU; ++h) a += r0[h];
-#pragma unroll
-                        for (int h = 0; h < DU; ++h) r0[h] = *reinterpret_cast<lds_f*>(pa + (2 * DU + h) * kRowB);
-                        if (k + 1 < nb) {
-#pragma unroll
-                            for (int h = 0; h < DU; ++h) a += r1[h];
-                        }
-                        pa += 2 * DU * kRowB;
+                        const uint32_t pb = pa + 16 * kRowB;
+                        NNUEFT_ISSUE16(qb, pb)
+                        NNUEFT_LANDED(8, qa);
+                        NNUEFT_ADD16(qa)
+                        pa += 32 * kRowB;
+                        NNUEFT_ISSUE16(qa, pa)   // past the last block: inside LDS, never added
+                        NNUEFT_LANDED(8, qb);
+                        if (k + 1 < nb) { NNUEFT_ADD16(qb) }
                     }
+                    NNUEFT_LANDED(0, qa);
+#undef NNUEFT_RD2
+#undef NNUEFT_ISSUE16
+#undef NNUEFT_LANDED
+#undef NNUEFT_ADD16
                 } else {
                     // 4 chains: block j of the task's lists is 4 chains x 8 entries
                     const u4* lp = reinterpret_cast<const u4*>(lent + (tmd & 0xfffffu)) + g16;
@@ -618,6 +676,9 @@ __global__ __launch_bounds__(kThreads) void k_chain_tile(const float* __restrict
             } else {
                 // 16 chains, 4 lanes each: block j of the task's lists is 16 chains x 4 entries
                 const int row = lrows[nlong * 4 + (task - nlong) * kTaskChains + g];
+                // (left to the compiler: it issues the four reads of a block and adds as they land, which keeps
+                // fewer reads of these chains in the queue in front of the long chain's; hand-written loops with
+                // two and with four reads ahead made the step slower, 0.380 -> 0.394 and 0.427 ms)
                 const uint2* lp = lent + (tmd & 0xfffffu) + g;
                 f4* sp = lsum + row * (kRowB / 16) + li;
                 f4 a = {0.f, 0.f, 0.f, 0.f};
@@ -828,15 +889,16 @@ int sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, int n_pe
     uint32_t* md = (uint32_t*)(base + L.md);
     uint16_t* ent = (uint16_t*)(base + L.ent);
     uint32_t* sched = (uint32_t*)(base + L.sched);
-    hipLaunchKernelGGL(k_cs_hist, dim3(L.ngroups), dim3(kSortThreads), 0, st, widx, bidx, hist, L.npairs, B, K, R, L.nkeys);
+    const int vec = (K % 4 == 0) && aligned16(widx) && aligned16(bidx);
+    hipLaunchKernelGGL(k_cs_hist, dim3(L.ngroups), dim3(kSortThreads), 0, st, widx, bidx, hist, L.npairs, B, K, R, L.nkeys, vec);
     NNUEFT_LAUNCH_CHECK();
     rc = nnueft_tile::launch_binscan(hist, total, L.nkeys + 1, L.ngroups, st);
     if (rc) return rc;
     hipLaunchKernelGGL(k_cs_place, dim3(L.ngroups), dim3(kSortThreads), 0, st, widx, bidx, hist, total, bpairs, chunks,
-                       ublocks, sched, L.npairs, n_persp, B, K, R, L.nkeys, L.nblocks);
+                       ublocks, sched, L.npairs, n_persp, B, K, R, L.nkeys, L.nblocks, vec);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_cs_expand, dim3(L.max_chunks), dim3(kThreads), kExpandLds, st, widx, bidx, bpairs, chunks, md,
-                       ent, sched, B, K, R);
+                       ent, sched, B, K, R, vec);
     NNUEFT_LAUNCH_CHECK();
     return 0;
 }
