@@ -579,16 +579,12 @@ __global__ __launch_bounds__(kThreads) void k_chain_tile(const float* __restrict
         }                                                                                                 \
     }
 
-    auto run_tasks = [&](auto mode_c, int c, bool first, int row0, int rows_here, int cols) {
-        constexpr int MODE = decltype(mode_c)::value;
-        const uint32_t head = ltask[0];
-        const int nlong = uni((int)(head & 0xffffu)), ntasks = uni((int)(head >> 16));
-        int task = 0;
-        if (lane == 0) task = (int)atomicAdd(ctr, 1u);
-        task = uni(task);
-        while (task < ntasks) {
-            int nxt = 0;
-            if (lane == 0) nxt = (int)atomicAdd(ctr, 1u);
+    // One task: the chains of `task` summed, their sums kept or written out (MODE).  Returns the task to do next
+    // (drawn at the start, so that the counter's answer is there at the end).
+    auto do_task = [&](const int task, const int nlong, const int MODE, int c, bool first, int row0, int rows_here, int cols) {
+        int nxt = 0;
+        if (lane == 0) nxt = (int)atomicAdd(ctr, 1u);
+        {
             const uint32_t tmd = ltask[1 + task];
             const int nb = uni((int)((tmd >> 20) & 0x7ffu));
             if (task < nlong) {
@@ -718,8 +714,13 @@ __global__ __launch_bounds__(kThreads) void k_chain_tile(const float* __restrict
                     }
                 }
             }
-            task = uni(nxt);
         }
+        return uni(nxt);
+    };
+    auto draw = [&]() {
+        int t = 0;
+        if (lane == 0) t = (int)atomicAdd(ctr, 1u);
+        return uni(t);
     };
 
     // The step after S; a new unit's ticket was drawn two units ago, and the one for two units on is drawn into the
@@ -797,24 +798,29 @@ __global__ __launch_bounds__(kThreads) void k_chain_tile(const float* __restrict
         if (tid == 0) ctr[0] = 0;
         __syncthreads();
         // everything one step on
-        D1 = D2;
-        C1 = C2;
-        if (D1.unit < nunits) NNUEFT_PREFETCH(C1, D1.chunk0 + D1.ci, D1.c, D1.cols)
-        D2 = D3;
-        if (D2.unit < nunits) {
-            C2 = uni_chunk(c3raw);
-            NNUEFT_PAIR_IDS(C2)
-        }
-        D3 = next_step(D2, tix);
-        if (D3.unit < nunits) c3raw = chunks[D3.chunk0 + D3.ci];
+        auto advance = [&]() {
+            D1 = D2;
+            C1 = C2;
+            if (D1.unit < nunits) NNUEFT_PREFETCH(C1, D1.chunk0 + D1.ci, D1.c, D1.cols)
+            D2 = D3;
+            if (D2.unit < nunits) {
+                C2 = uni_chunk(c3raw);
+                NNUEFT_PAIR_IDS(C2)
+            }
+            D3 = next_step(D2, tix);
+            if (D3.unit < nunits) c3raw = chunks[D3.chunk0 + D3.ci];
+        };
         const bool first = C.flags & 1;
         const bool last_of_unit = cur.ci + 1 == cur.nw + cur.nb;
-        if (last_of_unit && cur.nb == 1)
-            run_tasks(std::integral_constant<int, kOutAdd>{}, cur.c, first, row0, rows_here, cur.cols);
-        else if (last_of_unit && cur.nb == 0)
-            run_tasks(std::integral_constant<int, kOut>{}, cur.c, first, row0, rows_here, cur.cols);
-        else
-            run_tasks(std::integral_constant<int, kKeep>{}, cur.c, first, row0, rows_here, cur.cols);
+        const int mode = last_of_unit && cur.nb == 1 ? kOutAdd : last_of_unit && cur.nb == 0 ? kOut : kKeep;
+        const uint32_t head = ltask[0];
+        const int nlong = uni((int)(head & 0xffffu)), ntasks = uni((int)(head >> 16));
+        // A wave that draws a long chain starts on it at once, since the step waits for that chain, and asks for the
+        // data of the steps to come after it; every other wave asks first (one place in the code, see above).
+        int task = draw();
+        if (task < nlong) task = do_task(task, nlong, mode, cur.c, first, row0, rows_here, cur.cols);
+        advance();
+        while (task < ntasks) task = do_task(task, nlong, mode, cur.c, first, row0, rows_here, cur.cols);
         if (last_of_unit && cur.nb > 1) {
             // several black chunks: the gradient holds the white sums, LDS the black ones
             __syncthreads();
