@@ -6,10 +6,11 @@ A step is one pass of the hot path over one synthetic batch: the fused two-persp
 function the trainer calls.  Inputs are resident in HBM before the timed region.
 
 Prints ONE JSON line: positions/s for the workload BASELINE.json's metric is quoted on (L1=3072,
-B=16384, HalfKAv2_hm lists, 24576-row table); the roofline of the dominant kernel (k_seg_reduce, the
-segmented reduction of the deterministic backward) from HIP event timings of the entry point that
-launches it alone, against three bounds (algorithmic bytes against the L2 line rate that serves them,
-the bytes that must cross HBM, and the counter-measured traffic read from profiles/); the same for the
+B=16384, HalfKAv2_hm lists, 24576-row table); the roofline of the dominant kernel (k_chain_tile, the
+strict order's reduction of the deterministic backward out of LDS tiles; k_seg_reduce, the segmented
+reduction through L2, for the windowed order and narrow rows) from HIP event timings of the entry point
+that launches it alone, against three bounds (algorithmic bytes against the rate of the path that serves
+them, the bytes that must cross HBM, and the counter-measured traffic read from profiles/); the same for the
 two entry points and the step; and the reference's CPU path (torch embedding_bag composition) timed on
 the host cores on the same workload.
 """
@@ -95,13 +96,22 @@ def compulsory_bytes(L1, B, sum_a):
             "k_mix": saved + B * L1 * 4 + small,                          # row sums read, l0 written
         }
     nchunks = 2 * ((B + 127) // 128)
+    tiles16 = (oc + 15) // 16
+    bwd_chain = {
+        "k_bwd_rows": saved + B * L1 * 4 + 2 * B * oc * 4 + small,    # row sums + grad_l0 read, upstream rows written
+        # lists three times (key, place, bit map), pair order written, inverted lists (2 bytes an entry) written
+        "sort": 3 * lists + 2 * B * 4 + sum_a * 2,
+        # upstream rows once, dense gradient once, the inverted lists once per 16-column tile (out of L2 after the first)
+        "k_chain_tile": 2 * B * oc * 4 + R_ROWS * oc * 4 + sum_a * 2,
+        "bias": 2 * (B // 32) * oc * 4,
+    }
     bwd = {
         "k_bwd_rows": saved + B * L1 * 4 + 2 * B * oc * 4 + small,    # row sums + grad_l0 read, upstream rows written
         "sort": 2 * lists + 3 * nchunks * R_ROWS * 4 + sum_a * 4,     # lists twice, chunk counts w/r/w, sorted list
         "k_seg_reduce": seg_reduce_bytes(L1, B, sum_a)[2],
         "bias": 2 * (B // 32) * oc * 4,
     }
-    return fwd, bwd
+    return fwd, bwd, bwd_chain
 
 
 # the summaries under profiles/ of one workload by backward mode: no suffix = the headline's (strict) order
@@ -138,6 +148,21 @@ def sum_traffic(traffic, kernels):
 def forward_path(L1):
     """Which gather nnueft_double_fwd takes with a workspace: out of LDS tiles for wide rows, else blocked for L2."""
     return "tile" if L1 >= 512 and L1 % 32 == 0 else "blocked"
+
+
+def strict_path(L1):
+    """Which reduction the strict order takes: chains summed out of LDS tiles for rows of 256 columns and more (lists of
+    up to 32 slots, as all workloads here have), else the segmented reduction through L2."""
+    return "chain" if L1 + N_PSQT >= 256 else "segmented"
+
+
+def bwd_kernels(L1, mode):
+    """Kernels of the backward entry point by mode (for summing their counter-measured traffic)."""
+    if mode == "deterministic_strict" and strict_path(L1) == "chain":
+        # (the sort and the reduction of the other path are launched too and return at once: a batch whose lists
+        # the tiles cannot take would run them)
+        return ("k_bwd_rows", "k_cs_hist", "k_tl_binscan", "k_cs_place", "k_cs_expand", "k_chain_tile", "k_bias_final")
+    return BWD_KERNELS[mode]
 
 
 def fwd_kernels(L1):
@@ -731,7 +756,7 @@ def run_ft(args, lib, dev):
     # ---- report
     traffic, traffic_file = read_profile_traffic(args.workload, args.positions, modes[0])
     fwd_bytes, _ = algorithmic_bytes(L1, B, sum_a, "atomic")
-    comp_fwd, comp_bwd = compulsory_bytes(L1, B, sum_a)
+    comp_fwd, comp_bwd, comp_bwd_chain = compulsory_bytes(L1, B, sum_a)
     head_mode = modes[0]
     ms_step = results.get(head_mode, float("nan"))
     out = {
@@ -786,7 +811,23 @@ def run_ft(args, lib, dev):
     # the dominant kernel as the headline's order launches it
     det = (bwd_ms.get(head_mode) if head_mode != "atomic" else None) or bwd_ms.get("deterministic") or \
         bwd_ms.get("deterministic_strict")
-    if det:
+    if det and head_mode == "deterministic_strict" and strict_path(L1) == "chain":
+        # the strict order's reduction out of LDS tiles: the gathered upstream rows are LDS reads
+        alg, gathered, _ = seg_reduce_bytes(L1, B, sum_a)
+        blk, comp_blk = bound_block(
+            "k_chain_tile (timed through nnueft_det_reduce_rows_pitched, which launches it with k_bias_final behind it "
+            "and the segmented reduction of the other path, which returns at once)", det["reduce"], alg, None,
+            comp_bwd_chain["k_chain_tile"], sum_traffic(traffic, ("k_chain_tile",)), LDS_PEAK_GBS,
+            note="dominant kernel of the step; every table row's chain is summed out of a tile of upstream rows in LDS, "
+                 "so `achieved` (algorithmic bytes: one 16-column piece of an upstream row per slot) is held against "
+                 "what 16-byte LDS reads at random rows reach on this device (probe kernel, this run).  The kernel does "
+                 "not run at that bound: a step (one chunk of ~500 pairs x 16 columns) lasts as long as its longest "
+                 "chain, the row of the own king, which every pair of the chunk names: ~500 dependent adds fed by LDS "
+                 "reads that queue behind those of the other 15 waves.  Against HBM see roofline_compulsory and `traffic`.",
+            measured_peak=probes["lds_read_random_128B_rows_GBs"])
+        blk["bound"] = "lds"
+        out["roofline"], out["roofline_compulsory"] = blk, comp_blk
+    elif det:
         alg, gathered, comp = seg_reduce_bytes(L1, B, sum_a)
         seg_traffic = sum_traffic(traffic, ("k_seg_reduce",) + (("k_split_combine",) if head_mode == "deterministic" else ()))
         out["roofline"], out["roofline_compulsory"] = bound_block(
@@ -818,10 +859,11 @@ def run_ft(args, lib, dev):
         ms = results[mode]
         st = {"ms_per_step": ms, "positions_per_s": B / (ms * 1e-3), "algorithmic_GBs": (fb + bb) / (ms * 1e-3) / 1e9}
         if mode != "atomic":
-            comp_step = sum(comp_fwd.values()) + sum(comp_bwd.values())
+            comp_step = sum(comp_fwd.values()) + sum(
+                (comp_bwd_chain if mode == "deterministic_strict" and strict_path(L1) == "chain" else comp_bwd).values())
             st["compulsory_bytes"] = comp_step
             st["compulsory_frac_of_hbm_peak"] = comp_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS
-            tr = sum_traffic(read_profile_traffic(args.workload, args.positions, mode)[0], fwd_kernels(L1) + BWD_KERNELS[mode])
+            tr = sum_traffic(read_profile_traffic(args.workload, args.positions, mode)[0], fwd_kernels(L1) + bwd_kernels(L1, mode))
             st["traffic_bytes"] = tr
             st["traffic_frac_of_hbm_peak"] = tr / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS if tr else None
         else:
@@ -835,7 +877,7 @@ def run_ft(args, lib, dev):
                 comp_step = sum(comp_fwd.values()) + comp_atomic
                 st["compulsory_bytes"] = comp_step
                 st["compulsory_frac_of_hbm_peak"] = comp_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS
-                tr = sum_traffic(read_profile_traffic(args.workload, args.positions, mode)[0], fwd_kernels(L1) + BWD_KERNELS[mode])
+                tr = sum_traffic(read_profile_traffic(args.workload, args.positions, mode)[0], fwd_kernels(L1) + bwd_kernels(L1, mode))
                 st["traffic_bytes"] = tr
                 st["traffic_frac_of_hbm_peak"] = tr / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS if tr else None
         if mode in bwd_ms:
