@@ -26,10 +26,13 @@
 //                 pairs, the counters
 //   k_cs_expand   one workgroup per chunk: a bit per (row, pair) set with LDS atomics (ascending order for free),
 //                 rows sorted by chain length, tasks formed, lists written
-//   k_chain_tile  persistent workgroups, one per CU: units of (table block, column tile) handed out per XCD; a
-//                 step is one chunk of a unit; while a step runs, the tile, the lists and the facts of the next
-//                 step are on their way into registers, the pair ids of the one after it and the chunk record of
-//                 the one after that are being read
+//   k_chain_tile  persistent workgroups, one per CU: units of (table block, column tile) dealt to the workgroups of
+//                 an XCD round by round; a step is one chunk of a unit; while a step runs, the tile, the lists and
+//                 the facts of the next step are on their way into registers, the pair ids of the one after it and
+//                 the chunk record of the one after that are being read.  A step lasts as long as its longest
+//                 chain (the own king's row: as many dependent adds as the chunk has pairs), so the waves that sum
+//                 the long chains are fixed (wave i takes long task i), ask for the next step's data first, while
+//                 the address units are idle, and run at raised priority; the other waves do a task before they ask
 //
 // A batch with a list that names rows of more than one block, or the same row twice (the interface allows both),
 // is left to the sort and the segmented reduction of bwd_det.hip: the kernels here then do nothing, and a flag in
@@ -74,7 +77,7 @@ constexpr int kLdsSum = kTileB;
 constexpr int kLdsEnt = kLdsSum + (kRows + 1) * kRowB;
 constexpr int kLdsMd = kLdsEnt + kEntCap * 2 + kEntGuard;
 constexpr int kLdsCtr = kLdsMd + kMdB;
-constexpr int kLdsUb = kLdsCtr + 16;
+constexpr int kLdsUb = kLdsCtr + 32;
 constexpr int kLds = kLdsUb + nnueft_tile::kMaxBlocks * 16;
 constexpr int kThreads = 1024;
 constexpr int kSortThreads = 256;
@@ -85,11 +88,10 @@ static_assert(kEntCap * 2 / 16 <= 4 * kThreads, "lists: four 16-byte pieces a th
 static_assert(kLds <= 160 * 1024, "LDS of a CU");
 static_assert(kLongTasks + (kRows + kTaskChains - 1) / kTaskChains <= kMaxTasks, "tasks of a chunk");
 
-// Words of the scheduling block: kXcd unit counters 32 words apart, then these.
-constexpr int kFlagWord = kXcd * 32;       // not zero: the batch is left to the sort and reduction of bwd_det.hip
-constexpr int kChunksWord = kFlagWord + 1; // chunks in all
-constexpr int kDoneWord = kFlagWord + 2;   // workgroups of the reduction that are through
-constexpr int kSchedWords = kFlagWord + 32;
+// Words of the block the sort leaves for the kernels behind it.
+constexpr int kFlagWord = 0;               // not zero: the batch is left to the sort and reduction of bwd_det.hip
+constexpr int kChunksWord = 1;             // chunks in all
+constexpr int kSchedWords = 32;
 
 // A chunk of a block's pairs of one perspective: pairs bpairs[start .. start + count), its lists
 // ent[ent4 * 4 .. + n4 * 4), its facts md[chunk].
@@ -136,6 +138,13 @@ bool chain_layout(int B, int n_persp, int R, ChainLayout* L) {
     off += up256((size_t)kSchedWords * sizeof(uint32_t));
     L->end = off;
     return true;
+}
+
+// What tables were made for: the sizes that lay them out (never 0).
+static inline uint32_t table_tag(int B, int R, int n_persp) {
+    uint32_t h = 0x9e3779b9u;
+    for (uint32_t v : {(uint32_t)B, (uint32_t)R, (uint32_t)n_persp}) h = (h ^ v) * 0x85ebca6bu + 0xc2b2ae35u;
+    return h | 1u;
 }
 
 // a value every lane holds alike, moved to a scalar register
@@ -216,8 +225,10 @@ __global__ __launch_bounds__(kSortThreads) void k_cs_place(const int32_t* __rest
                                                            const uint32_t* __restrict__ total,
                                                            uint32_t* __restrict__ bpairs, RChunk* __restrict__ chunks,
                                                            BlockChunks* __restrict__ ublocks,
-                                                           uint32_t* __restrict__ sched, int npairs, int n_persp, int B,
-                                                           int K, int R, int nkeys, int nblocks, int vec) {
+                                                           uint32_t* __restrict__ sched, uint32_t* __restrict__ split_word,
+                                                           uint32_t* __restrict__ tag_word, uint32_t tag, int npairs,
+                                                           int n_persp, int B, int K, int R, int nkeys, int nblocks,
+                                                           int vec) {
     __shared__ uint32_t keybase[kMaxKeys + 1];
     __shared__ uint32_t wcnt[kSortThreads / 64][kMaxKeys];
     __shared__ uint32_t chunk0[kMaxKeys + 1];
@@ -268,7 +279,11 @@ __global__ __launch_bounds__(kSortThreads) void k_cs_place(const int32_t* __rest
         bpairs[keybase[key] + hist[(size_t)key * ngroups + blockIdx.x] + before + rank] = (uint32_t)n;
     }
     if (blockIdx.x != 0) return;
-    // the first workgroup also writes the tables of the batch
+    // the first workgroup also writes the tables of the batch, and what they were made for
+    if (tid == 0) {
+        *split_word = 0;   // the strict order
+        *tag_word = tag;
+    }
     for (int i = tid; i < kSchedWords; i += kSortThreads)
         sched[i] = i == kFlagWord ? (tot[nkeys] != 0 ? 1u : 0u) : i == kChunksWord ? chunk0[nkeys] : 0u;
     for (int k = tid; k < nkeys; k += kSortThreads) {
@@ -475,7 +490,7 @@ __device__ __forceinline__ RChunk uni_chunk(const RChunk& c) {
 
 // A step of a workgroup's walk: one chunk of one unit (table block x column tile).
 struct Step {
-    int unit, blk, c, cols, chunk0, nw, nb, ci;
+    int unit, blk, c, cols, chunk0, nw, nb, ci, round;
 };
 
 // What a task does with its chains' sums.
@@ -491,16 +506,19 @@ __global__ __launch_bounds__(kThreads) void k_chain_tile(const float* __restrict
                                                          const uint16_t* __restrict__ ent,
                                                          uint32_t* __restrict__ sched, float* __restrict__ gW,
                                                          int R, int out_cols, int main_tiles, int tpx, int tail_cols,
-                                                         int nblocks, int gw_vec) {
+                                                         int nblocks, int gw_vec, const uint32_t* __restrict__ tag_word,
+                                                         uint32_t tag) {
     extern __shared__ float4 lds_raw[];
     char* tb = reinterpret_cast<char*>(lds_raw);
     f4* lsum = reinterpret_cast<f4*>(tb + kLdsSum);
     uint2* lent = reinterpret_cast<uint2*>(tb + kLdsEnt);
     uint32_t* ltask = reinterpret_cast<uint32_t*>(tb + kLdsMd);
     uint16_t* lrows = reinterpret_cast<uint16_t*>(tb + kLdsMd + 256);
-    uint32_t* ctr = reinterpret_cast<uint32_t*>(tb + kLdsCtr);   // [0] task counter, [1 .. 3] the next units' tickets in turns
+    uint32_t* ctr = reinterpret_cast<uint32_t*>(tb + kLdsCtr);   // [0] task counter
     int4* lub = reinterpret_cast<int4*>(tb + kLdsUb);
-    if (sched[kFlagWord] != 0) return;
+    // tables that were not made for these lists (sorted for another threshold) are not even there: nothing is read
+    // before the tag says they are
+    if (*tag_word != tag || sched[kFlagWord] != 0) return;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     constexpr int NT = kThreads;
@@ -514,12 +532,11 @@ __global__ __launch_bounds__(kThreads) void k_chain_tile(const float* __restrict
     const int nmain = nblocks * my_tiles;
     const int ntail = tail_cols && nblocks > x ? (nblocks - x + kXcd - 1) / kXcd : 0;
     const int nunits = nmain + ntail;
-    uint32_t* unit_ctr = sched + x * 32;
     const int g = lane >> 2, li = lane & 3;
     const uint32_t lane_off = (uint32_t)(uintptr_t)tb + li * 16;
 
     auto decode = [&](int u) {
-        Step S{u, 0, 0, 0, 0, 1, 1, 0};
+        Step S{u, 0, 0, 0, 0, 1, 1, 0, 0};
         if (u >= nunits) return S;
         int r;
         if (u < nmain) {
@@ -723,16 +740,21 @@ __global__ __launch_bounds__(kThreads) void k_chain_tile(const float* __restrict
         return uni(t);
     };
 
-    // The step after S; a new unit's ticket was drawn two units ago, and the one for two units on is drawn into the
-    // slot of the ticket in front of it, which everyone has read.
-    auto next_step = [&](const Step& S, int& tix) {
+    // The step after S.  The units of an XCD are dealt to its workgroups round by round, forth and back (blocks with
+    // the most pairs come first, so every workgroup gets about the same mix and the cheapest units come last): no
+    // counter in memory, whose answer a wave has to wait for behind the loads it has just issued (with one, and with
+    // a ticket drawn ahead and read a step later, the reduction at L1 = 3072, B = 16384 took 0.353 and 0.332 ms
+    // against 0.321; on game-like lists 0.550 and 0.559 against 0.526; only at L1 = 1024, B = 8192 on game-like
+    // lists, where a workgroup gets 8 units of very unequal blocks, the counter was ahead: 0.159 against 0.186 ms).
+    const int wg = blockIdx.x / kXcd, nwg = gridDim.x / kXcd;
+    auto unit_of = [&](int round) { return round * nwg + ((round & 1) ? nwg - 1 - wg : wg); };
+    auto next_step = [&](const Step& S) {
         if (S.unit >= nunits) return S;
         Step N = S;
         N.ci = S.ci + 1;
         if (N.ci == S.nw + S.nb) {
-            ++tix;
-            N = decode(uni((int)ctr[1 + tix % 3]));
-            if (tid == 0) ctr[1 + (tix + 2) % 3] = atomicAdd(unit_ctr, 1u);
+            N = decode(unit_of(S.round + 1));
+            N.round = S.round + 1;
         }
         return N;
     };
@@ -743,21 +765,13 @@ __global__ __launch_bounds__(kThreads) void k_chain_tile(const float* __restrict
         constexpr uint32_t zz = (uint32_t)kCP | ((uint32_t)kCP << 16);
         for (int i = tid; i < (kEntCap * 2 + kEntGuard) / 16; i += NT) reinterpret_cast<u4*>(lent)[i] = u4{zz, zz, zz, zz};
     }
-    if (tid == 0) {
-        ctr[1] = atomicAdd(unit_ctr, 1u);
-        ctr[2] = atomicAdd(unit_ctr, 1u);
-        ctr[3] = atomicAdd(unit_ctr, 1u);
-    }
     __syncthreads();
     // D1: the step whose data is in (or on its way into) the registers; D2: its successor, whose pair ids are being
     // read; D3: the one after, whose chunk record is being read
-    int tix = 0;
-    Step D1 = decode(uni((int)ctr[1]));
-    __syncthreads();   // ticket 0 is read: its slot may be drawn into
+    Step D1 = decode(unit_of(0));
     RChunk C1{}, C2{}, c3raw{};
-    Step D2 = next_step(D1, tix);
-    __syncthreads();
-    Step D3 = next_step(D2, tix);
+    Step D2 = next_step(D1);
+    Step D3 = next_step(D2);
     if (D1.unit < nunits) {
         C1 = uni_chunk(chunks[D1.chunk0 + D1.ci]);
         NNUEFT_PAIR_IDS(C1)
@@ -795,7 +809,7 @@ __global__ __launch_bounds__(kThreads) void k_chain_tile(const float* __restrict
                 if (f < NP) reinterpret_cast<f4*>(tb)[f] = live ? v[i] : f4{0.f, 0.f, 0.f, 0.f};
             }
         }
-        if (tid == 0) ctr[0] = 0;
+        if (tid == 0) ctr[0] = tm.x & 0xffffu;   // the tasks the counter hands out begin behind the long ones
         __syncthreads();
         // everything one step on
         auto advance = [&]() {
@@ -807,7 +821,7 @@ __global__ __launch_bounds__(kThreads) void k_chain_tile(const float* __restrict
                 C2 = uni_chunk(c3raw);
                 NNUEFT_PAIR_IDS(C2)
             }
-            D3 = next_step(D2, tix);
+            D3 = next_step(D2);
             if (D3.unit < nunits) c3raw = chunks[D3.chunk0 + D3.ci];
         };
         const bool first = C.flags & 1;
@@ -815,11 +829,18 @@ __global__ __launch_bounds__(kThreads) void k_chain_tile(const float* __restrict
         const int mode = last_of_unit && cur.nb == 1 ? kOutAdd : last_of_unit && cur.nb == 0 ? kOut : kKeep;
         const uint32_t head = ltask[0];
         const int nlong = uni((int)(head & 0xffffu)), ntasks = uni((int)(head >> 16));
-        // A wave that draws a long chain starts on it at once, since the step waits for that chain, and asks for the
-        // data of the steps to come after it; every other wave asks first (one place in the code, see above).
-        int task = draw();
-        if (task < nlong) task = do_task(task, nlong, mode, cur.c, first, row0, rows_here, cur.cols);
+        // The step waits for its long chains.  Long task i belongs to wave i (the counter hands out the others): that
+        // wave asks for the data of the steps to come at once, while the address units are idle, and starts on its
+        // chain; every other wave does a task first and asks then (one place in the code for the asking, see above),
+        // so that the long chain's wave neither queues behind their loads nor waits for its own at the next step.
+        const int wave = wave0 >> 6;
+        int task = ntasks;
+        if (wave >= nlong) {
+            task = draw();
+            if (task < ntasks) task = do_task(task, nlong, mode, cur.c, first, row0, rows_here, cur.cols);
+        }
         advance();
+        if (wave < nlong) task = do_task(wave, nlong, mode, cur.c, first, row0, rows_here, cur.cols);
         while (task < ntasks) task = do_task(task, nlong, mode, cur.c, first, row0, rows_here, cur.cols);
         if (last_of_unit && cur.nb > 1) {
             // several black chunks: the gradient holds the white sums, LDS the black ones
@@ -835,16 +856,6 @@ __global__ __launch_bounds__(kThreads) void k_chain_tile(const float* __restrict
     }
 #undef NNUEFT_PREFETCH
 #undef NNUEFT_PAIR_IDS
-    // the last workgroup through rewinds the unit counters: the same tables serve another launch
-    __syncthreads();
-    if (tid == 0) {
-        __threadfence();
-        if (atomicAdd(&sched[kDoneWord], 1u) == gridDim.x - 1) {
-            for (int i = 0; i < kXcd; ++i) sched[i * 32] = 0;
-            sched[kDoneWord] = 0;
-            __threadfence();
-        }
-    }
 }
 
 constexpr int kMaxDevices = 64;
@@ -877,7 +888,8 @@ const uint32_t* fallback_flag(const void* ws, int B, int R, int n_persp) {
     return (const uint32_t*)((const char*)ws + L.sched) + kFlagWord;
 }
 
-int sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, int n_persp, void* ws, hipStream_t st) {
+int sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, int n_persp, void* ws, uint32_t* split_word,
+         uint32_t* tag_word, hipStream_t st) {
     ChainLayout L;
     if (!chain_layout(B, n_persp, R, &L)) return NNUEFT_E_UNSUPPORTED;
     int device = 0;
@@ -901,7 +913,8 @@ int sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, int n_pe
     rc = nnueft_tile::launch_binscan(hist, total, L.nkeys + 1, L.ngroups, st);
     if (rc) return rc;
     hipLaunchKernelGGL(k_cs_place, dim3(L.ngroups), dim3(kSortThreads), 0, st, widx, bidx, hist, total, bpairs, chunks,
-                       ublocks, sched, L.npairs, n_persp, B, K, R, L.nkeys, L.nblocks, vec);
+                       ublocks, sched, split_word, tag_word, table_tag(B, R, n_persp), L.npairs, n_persp, B, K, R, L.nkeys,
+                       L.nblocks, vec);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_cs_expand, dim3(L.max_chunks), dim3(kThreads), kExpandLds, st, widx, bidx, bpairs, chunks, md,
                        ent, sched, B, K, R, vec);
@@ -909,7 +922,8 @@ int sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, int n_pe
     return 0;
 }
 
-int reduce(const float* G, int g_pitch, float* gW, int B, int R, int out_cols, int n_persp, void* ws, hipStream_t st) {
+int reduce(const float* G, int g_pitch, float* gW, int B, int R, int out_cols, int n_persp, void* ws,
+           const uint32_t* tag_word, hipStream_t st) {
     ChainLayout L;
     if (!chain_layout(B, n_persp, R, &L)) return NNUEFT_E_UNSUPPORTED;
     if (!aligned16(G) || g_pitch % 4) return NNUEFT_E_UNSUPPORTED;
@@ -927,7 +941,7 @@ int reduce(const float* G, int g_pitch, float* gW, int B, int R, int out_cols, i
     hipLaunchKernelGGL(k_chain_tile, dim3(grid), dim3(kThreads), kLds, st, G, g_pitch, (const uint32_t*)(base + L.bpairs),
                        (const RChunk*)(base + L.chunks), (const BlockChunks*)(base + L.ublocks),
                        (const uint32_t*)(base + L.md), (const uint16_t*)(base + L.ent), (uint32_t*)(base + L.sched), gW, R,
-                       out_cols, main_tiles, tpx, tail_cols, L.nblocks, aligned16(gW) ? 1 : 0);
+                       out_cols, main_tiles, tpx, tail_cols, L.nblocks, aligned16(gW) ? 1 : 0, tag_word, table_tag(B, R, n_persp));
     NNUEFT_LAUNCH_CHECK();
     return 0;
 }

@@ -89,7 +89,10 @@ constexpr int kSchedNLocal = kSchedNRemote + 1;   // the next n_local: window su
 constexpr int kSchedRowSplit = kSchedNLocal + 1;  // the threshold the lists were sorted for
 constexpr int kSchedRowLo = kSchedRowSplit + 1;   // kXcd + 1 range bounds
 constexpr int kSchedLocalCnt = kSchedRowLo + kXcd + 1;   // kXcd counts: the local split rows of each XCD's range
-constexpr int kSchedWords = kSchedLocalCnt + kXcd;
+// What the tables of the reduction out of LDS tiles were made for (0: they were not made, or not for these lists): set
+// by that path's sort, cleared by k_row_scan, so that a reduction never reads tables that are not there.
+constexpr int kSchedChainTag = kSchedLocalCnt + kXcd;
+constexpr int kSchedWords = kSchedChainTag + 1;
 // Window sums are kept for this many split rows at most (uniform positions split 32 rows, game-like ones a few hundred);
 // further ones are reduced by one wave per 64-lane slice, window by window in the same order, so the bits are the same.
 #ifndef NNUEFT_SPLIT_CAP
@@ -664,6 +667,7 @@ __global__ __launch_bounds__(kScanThreads) void k_row_scan(uint32_t* __restrict_
         sched[kSchedNRemote] = n_remote;
         sched[kSchedNLocal] = classify ? n_local : 0u;
         sched[kSchedRowSplit] = row_split;
+        sched[kSchedChainTag] = 0;
     }
 }
 
@@ -961,10 +965,11 @@ __global__ __launch_bounds__(64) void k_seg_reduce(const float* __restrict__ G, 
                                                    uint32_t* __restrict__ sched, float* __restrict__ gW,
                                                    int out_cols, int nslices, int slice_v, int two_persp,
                                                    RunPlan rp, const uint32_t* __restrict__ only_if) {
-    if (only_if && *only_if == 0) return;   // the batch went to the reduction out of LDS tiles
     const int lane = threadIdx.x;
     const int xcd = blockIdx.x % kXcd;
     if (sched[kSchedRowSplit] != rp.row_split) return;   // the lists were sorted for another threshold
+    // (asked behind the threshold: the flag lies in tables that only a sort for the strict order makes)
+    if (only_if && *only_if == 0) return;   // the batch went to the reduction out of LDS tiles
     const uint32_t n_long = sched[kSchedNLong], n_split = sched[kSchedNSplit];
     const uint32_t n_remote = sched[kSchedNRemote], n_stored = n_remote + sched[kSchedNLocal];
     const uint32_t n_whole = n_split - n_stored;
@@ -1250,7 +1255,7 @@ int det_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, int 
     // with the tables of the LDS-tiled reduction made first, the kernels below run only for a batch it cannot take
     const uint32_t* only_if = nullptr;
     if (chain_in_use(L, *info)) {
-        rc = nnueft_chain::sort(widx, bidx, B, K, R, n_persp, ws + L.chain, st);
+        rc = nnueft_chain::sort(widx, bidx, B, K, R, n_persp, ws + L.chain, sched + kSchedRowSplit, sched + kSchedChainTag, st);
         if (rc) return rc;
         only_if = nnueft_chain::fallback_flag(ws + L.chain, B, R, n_persp);
     }
@@ -1291,7 +1296,7 @@ int det_reduce(const float* G, int g_pitch, float* gW, float* gbias, int B, int 
         int rc = nnueft_dev::device_info(&device, &info);
         if (rc) return rc;
         if (chain_in_use(L, *info) && g_pitch % 4 == 0 && aligned16(G)) {
-            rc = nnueft_chain::reduce(G, g_pitch, gW, B, R, out_cols, n_persp, sw + L.chain, st);
+            rc = nnueft_chain::reduce(G, g_pitch, gW, B, R, out_cols, n_persp, sw + L.chain, sched + kSchedChainTag, st);
             if (rc) return rc;
             only_if = nnueft_chain::fallback_flag(sw + L.chain, B, R, n_persp);
         } else if (chain_in_use(L, *info)) {

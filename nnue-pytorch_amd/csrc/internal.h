@@ -100,8 +100,14 @@ namespace nnueft_chain {
 size_t shape_workspace(int B, int K, int R, int out_cols, int n_persp);
 bool device_ok(const nnueft_dev::DeviceInfo& d);
 const uint32_t* fallback_flag(const void* ws, int B, int R, int n_persp);
-int sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, int n_persp, void* ws, hipStream_t st);
-int reduce(const float* G, int g_pitch, float* gW, int B, int R, int out_cols, int n_persp, void* ws, hipStream_t st);
+// split_word / tag_word: two words outside `ws` that every sort of these lists writes (the threshold the lists were
+// sorted for, and what the tables in `ws` were made for): sort() sets them, reduce() does nothing unless the tag is
+// the one of its own arguments, so that it never reads tables that were not made (lists sorted for another
+// threshold, whose block may not even hold room for `ws`).
+int sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, int n_persp, void* ws, uint32_t* split_word,
+         uint32_t* tag_word, hipStream_t st);
+int reduce(const float* G, int g_pitch, float* gW, int B, int R, int out_cols, int n_persp, void* ws,
+           const uint32_t* tag_word, hipStream_t st);
 
 }  // namespace nnueft_chain
 
