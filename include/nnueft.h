@@ -253,6 +253,11 @@ int nnueft_double_bwd_atomic_lds(const float* us, const float* them, const int32
  * its own sort.  The block stays valid for further calls, one at a time: it holds the task counters
  * of the reduction, which the call's last kernel rewinds, so two reductions that overlap on one
  * block (two streams, two threads) race on them.
+ * row_split = 0 (the strict order) with rows of 256 columns and more, lists of up to 32 slots and a
+ * device of 8 XCDs: the chains of the table rows are summed out of LDS tiles of the upstream rows
+ * (a second set of tables in the sorted block).  A batch in which a list names rows of two 768-row
+ * table blocks, or one row twice, is noticed on the device and summed by the segmented reduction
+ * in the same call; the bits are the same either way.
  * aux_stream: NULL, or a second stream of the same device.
  *   With sorted_lists NULL: sorting the index lists and computing the upstream rows are independent;
  *   given a second stream the call runs the sort there, beside the other work on `stream`, and
