@@ -127,6 +127,13 @@ __device__ __forceinline__ void mix4(float u, float t, float sw0, float sw1, flo
     xb1 = u * k1 + t * w1;
 }
 
+// Whether a position's output row is one perspective's sums on each half: with (us, them) = (1, 0) the mixed
+// values are w and k themselves, with (0, 1) they change places (u * w + t * k = w bit for bit when u = 1, t = 0
+// and k is finite: a sum of a chain from +0 plus a bias is never -0).
+__device__ __forceinline__ bool one_sided(float u, float t) {
+    return (u == 1.0f && t == 0.0f) || (u == 0.0f && t == 1.0f);
+}
+
 // The four upstream values of that column pair for the two perspectives' sparse-linear outputs.
 __device__ __forceinline__ void grad4(float u, float t, float xw0, float xw1, float xb0, float xb1, float g0,
                                       float g1, float max_act, float& gw0, float& gw1, float& gb0, float& gb1) {

@@ -162,23 +162,14 @@ __global__ __launch_bounds__(64) void k_acc_blocked(const int32_t* __restrict__ 
         if (act[m]) stv_stream<VW>(dst + col[m], a[m]);
 }
 
-// Per position: bias, mix, clamp, product; slice 0 also does the two psqt chains.
+// One 64-lane slice of a position's output row: bias, mix, clamp, product (lane = threadIdx.x, s = the slice).
 template <int VW>
-__global__ __launch_bounds__(64) void k_mix(const float* __restrict__ us, const float* __restrict__ them,
-                                            const int32_t* __restrict__ widx, const int32_t* __restrict__ bidx,
-                                            const int64_t* __restrict__ psqt_idx, const float* __restrict__ W,
-                                            const float* __restrict__ bias, const float* __restrict__ saved,
-                                            float max_act, float* __restrict__ l0, float* __restrict__ wpsqt,
-                                            float* __restrict__ bpsqt, int B, int K, int R, int L1, int n_psqt,
-                                            int nslices, ActGrid act, VirtualTable vt) {
-    const int lane = threadIdx.x;
-    // 1-D launch, the slices of a position next to each other: its rows are then read and written
-    // at about the same time (a few per cent faster than position-fastest)
-    const int s = blockIdx.x % nslices;
-    const int b = blockIdx.x / nslices;
+__device__ __forceinline__ void mix_slice(int s, int b, int lane, const float* __restrict__ us,
+                                          const float* __restrict__ them, const float* __restrict__ bias,
+                                          const float* __restrict__ saved, float max_act, float* __restrict__ l0, int B,
+                                          int L1, const ActGrid& act) {
     const int h = L1 >> 1;
     const int hv = h / VW;
-    const size_t out_cols = (size_t)L1 + n_psqt;
     const int q = s * 64 + lane;
     if (q < hv) {
         const int c = q * VW;
@@ -204,34 +195,80 @@ __global__ __launch_bounds__(64) void k_mix(const float* __restrict__ us, const 
         stv<VW>(o + c, o0);
         stv<VW>(o + h + c, o1);
     }
-    if (s == 0) {
-        const int64_t pi = psqt_idx[b];
-        const bool do_psqt = pi >= 0 && pi < n_psqt;
-        float ps[2] = {0.0f, 0.0f};
-        if (do_psqt) {
+}
+
+// The two psqt chains of a position, one wave: wpsqt[b], bpsqt[b] = chain over the list's valid slots + bias.
+__device__ __forceinline__ void psqt_chains(int b, int lane, const int32_t* __restrict__ widx,
+                                            const int32_t* __restrict__ bidx, const int64_t* __restrict__ psqt_idx,
+                                            const float* __restrict__ W, const float* __restrict__ bias,
+                                            float* __restrict__ wpsqt, float* __restrict__ bpsqt, int K, int R, int L1,
+                                            int n_psqt, const VirtualTable& vt) {
+    const size_t out_cols = (size_t)L1 + n_psqt;
+    const int64_t pi = psqt_idx[b];
+    const bool do_psqt = pi >= 0 && pi < n_psqt;
+    float ps[2] = {0.0f, 0.0f};
+    if (do_psqt) {
 #pragma unroll
-            for (int p = 0; p < 2; ++p) {
-                const int32_t* ix = (p ? bidx : widx) + (size_t)b * K;
-                for (int k0 = 0; k0 < K; k0 += 64) {
-                    const int my = (k0 + lane < K) ? ix[k0 + lane] : -1;
-                    const bool ok = my >= 0 && my < R;
-                    u64 mask = __ballot(ok);
-                    float myps = ok ? W[(size_t)my * out_cols + L1 + pi] : 0.0f;
-                    if (ok && vt.V) {
-                        // the merged table's entry: W + V[row % 768], on the psqt grid when asked for
-                        myps = myps + vt.V[(size_t)(my % nnueft_tile::kBlockRows) * out_cols + L1 + pi];
-                        if (vt.quantize) myps = rintf(myps * vt.scale_psqt) / vt.scale_psqt;
-                    }
-                    while (mask) ps[p] = ps[p] + bcast_f(myps, pop_lane(mask));
+        for (int p = 0; p < 2; ++p) {
+            const int32_t* ix = (p ? bidx : widx) + (size_t)b * K;
+            for (int k0 = 0; k0 < K; k0 += 64) {
+                const int my = (k0 + lane < K) ? ix[k0 + lane] : -1;
+                const bool ok = my >= 0 && my < R;
+                u64 mask = __ballot(ok);
+                float myps = ok ? W[(size_t)my * out_cols + L1 + pi] : 0.0f;
+                if (ok && vt.V) {
+                    // the merged table's entry: W + V[row % 768], on the psqt grid when asked for
+                    myps = myps + vt.V[(size_t)(my % nnueft_tile::kBlockRows) * out_cols + L1 + pi];
+                    if (vt.quantize) myps = rintf(myps * vt.scale_psqt) / vt.scale_psqt;
                 }
+                while (mask) ps[p] = ps[p] + bcast_f(myps, pop_lane(mask));
             }
         }
-        if (lane == 0) {
-            const float pb = do_psqt ? bias[L1 + pi] : 0.0f;
-            wpsqt[b] = ps[0] + pb;
-            bpsqt[b] = ps[1] + pb;
-        }
     }
+    if (lane == 0) {
+        const float pb = do_psqt ? bias[L1 + pi] : 0.0f;
+        wpsqt[b] = ps[0] + pb;
+        bpsqt[b] = ps[1] + pb;
+    }
+}
+
+// Per position: bias, mix, clamp, product; slice 0 also does the two psqt chains.
+template <int VW>
+__global__ __launch_bounds__(64) void k_mix(const float* __restrict__ us, const float* __restrict__ them,
+                                            const int32_t* __restrict__ widx, const int32_t* __restrict__ bidx,
+                                            const int64_t* __restrict__ psqt_idx, const float* __restrict__ W,
+                                            const float* __restrict__ bias, const float* __restrict__ saved,
+                                            float max_act, float* __restrict__ l0, float* __restrict__ wpsqt,
+                                            float* __restrict__ bpsqt, int B, int K, int R, int L1, int n_psqt,
+                                            int nslices, ActGrid act, VirtualTable vt) {
+    const int lane = threadIdx.x;
+    // 1-D launch, the slices of a position next to each other: its rows are then read and written
+    // at about the same time (a few per cent faster than position-fastest)
+    const int s = blockIdx.x % nslices;
+    const int b = blockIdx.x / nslices;
+    mix_slice<VW>(s, b, lane, us, them, bias, saved, max_act, l0, B, L1, act);
+    if (s == 0) psqt_chains(b, lane, widx, bidx, psqt_idx, W, bias, wpsqt, bpsqt, K, R, L1, n_psqt, vt);
+}
+
+// What is left per position when the gather has written the output rows itself (it does for a position whose
+// (us, them) is (1, 0) or (0, 1): such a row is one perspective's sums on each half): the two psqt chains, and
+// the whole row of a position with any other (us, them), which needs both perspectives' sums at once; every row
+// when the gather met a sum that is not finite (*nonfinite != 0: 0 * inf of the other perspective's sum is NaN
+// in the mix, which the gather's row does not show).
+template <int VW>
+__global__ __launch_bounds__(64) void k_mix_rest(const float* __restrict__ us, const float* __restrict__ them,
+                                                 const int32_t* __restrict__ widx, const int32_t* __restrict__ bidx,
+                                                 const int64_t* __restrict__ psqt_idx, const float* __restrict__ W,
+                                                 const float* __restrict__ bias, const float* __restrict__ saved,
+                                                 float max_act, float* __restrict__ l0, float* __restrict__ wpsqt,
+                                                 float* __restrict__ bpsqt, int B, int K, int R, int L1, int n_psqt,
+                                                 int nslices, ActGrid act, VirtualTable vt,
+                                                 const uint32_t* __restrict__ nonfinite) {
+    const int lane = threadIdx.x;
+    const int b = blockIdx.x;
+    if (!one_sided(us[b], them[b]) || *nonfinite != 0u)
+        for (int s = 0; s < nslices; ++s) mix_slice<VW>(s, b, lane, us, them, bias, saved, max_act, l0, B, L1, act);
+    psqt_chains(b, lane, widx, bidx, psqt_idx, W, bias, wpsqt, bpsqt, K, R, L1, n_psqt, vt);
 }
 
 static inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -247,10 +284,16 @@ int launch_scan(uint32_t* data, int n, hipStream_t st) {
 int launch_mix(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                const int64_t* psqt_idx, const float* W, const float* bias, const float* saved, float max_act,
                float* l0, float* wpsqt, float* bpsqt, int B, int K, int R, int L1, int n_psqt, hipStream_t st,
-               ActGrid act, VirtualTable vt) {
+               ActGrid act, VirtualTable vt, const uint32_t* nonfinite) {
     const int hv = (L1 / 2) / 4;
     const int mix_slices = (hv + 63) / 64;
     if ((long long)B * mix_slices > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
+    if (nonfinite) {
+        hipLaunchKernelGGL(k_mix_rest<4>, dim3((unsigned)B), dim3(64), 0, st, us, them, widx, bidx, psqt_idx, W, bias, saved,
+                           max_act, l0, wpsqt, bpsqt, B, K, R, L1, n_psqt, mix_slices, act, vt, nonfinite);
+        NNUEFT_LAUNCH_CHECK();
+        return 0;
+    }
     const dim3 mix_grid((unsigned)B * mix_slices);
     hipLaunchKernelGGL(k_mix<4>, mix_grid, dim3(64), 0, st, us, them, widx, bidx, psqt_idx, W, bias, saved, max_act,
                        l0, wpsqt, bpsqt, B, K, R, L1, n_psqt, mix_slices, act, vt);
@@ -337,7 +380,7 @@ int double_fwd_blocked(const float* us, const float* them, const int32_t* widx, 
     }
     NNUEFT_LAUNCH_CHECK();
     return launch_mix(us, them, widx, bidx, psqt_idx, W, bias, saved, max_act, l0, wpsqt, bpsqt, B, K, R, L1, n_psqt,
-                      st, act, VirtualTable{nullptr, 1.0f, 1.0f, 0, 0.0f});
+                      st, act, VirtualTable{nullptr, 1.0f, 1.0f, 0, 0.0f}, nullptr);
 }
 
 }  // namespace nnueft_blocked

@@ -191,7 +191,9 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
                                                            uint32_t* __restrict__ sched,
                                                            BlockRec* __restrict__ brec, uint32_t* __restrict__ cpool8,
                                                            uint32_t* __restrict__ border, int npairs, int B, int K,
-                                                           int R, int nblocks, int nbins, int vec, int block_rows) {
+                                                           int R, int nblocks, int nbins, int vec, int block_rows,
+                                                           const float* __restrict__ us,
+                                                           const float* __restrict__ them) {
     __shared__ uint32_t cursor[kBins];      // next slot of this workgroup in every bin
     __shared__ uint32_t bin_base[kBins];    // first slot of every bin
     __shared__ uint32_t bin_eoff[kBins];    // list entries of its block before the bin's lists
@@ -288,6 +290,7 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
         }
     }
     if (blockIdx.x == 0 && tid <= kXcd) sched[tid * 32] = tid == kXcd ? blk_chunk0[nblocks] : 0u;
+    if (blockIdx.x == 0 && tid == 0) sched[kSchedNonFinite] = 0u;
     // the blocks as the backward scatter walks them, and their order by population (most pairs first)
     if (blockIdx.x == 0 && tid < nblocks) {
         const uint32_t* bb = bin_base + tid * kLenBins;
@@ -343,7 +346,15 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
         }
         off += (i / nc - ranks_of_chunk((int)(bb[kbin] - bb[0]), j, nc)) * pad;
     }
-    loff[dst] = (uint16_t)(off >> 3);
+    // with the sides to move at hand (both perspectives' lists, n = perspective * B + position): whether the pair's
+    // sums alone make a half of the position's output row, and which half
+    uint32_t side = 0;
+    if (us) {
+        const int p = n >= B;
+        const float u = us[n - p * B], t = them[n - p * B];
+        side = (one_sided(u, t) ? kLoffOwnRow : 0u) | ((p == 0) == (u == 1.0f) ? 0u : kLoffSecondHalf);
+    }
+    loff[dst] = (uint16_t)((uint32_t)(off >> 3) | side);
     const uint32_t ci = blk_chunk0[f.block] + (uint32_t)j;
     // row numbers inside the block, valid entries first in slot order, the rest name the row of zeros
     uint32_t w[kSlots / 2];
@@ -445,6 +456,30 @@ struct Fuse16 {
     int clip_max, shift;
 };
 
+// What the float forward does with a pair's sums when the gather finishes them itself (FUSE == kFuseF).  A unit then
+// visits the column tiles two by two, tile c and its partner c + ntiles / 2 (columns j and j + L1/2): after the
+// second the wave that holds a pair's sums of the partner tile reads the pair's sums of the first back (they went to
+// `saved` a moment ago, from the same CU) and has both factors of the product.  For a position whose (us, them) is
+// (1, 0) or (0, 1) the pair's half of the output row is + bias, clamp, product, the activation grid when asked for:
+// exactly what the mix of both perspectives gives there, as long as the other perspective's sums are finite (0 * inf
+// is NaN in the mix).  A sum that is not finite therefore raises sched[kSchedNonFinite], and the pass that follows
+// (k_mix_rest) then redoes every row from the saved sums; it always does the rows of positions with any other
+// (us, them), which this kernel leaves alone.
+struct FuseF {
+    const float* us;
+    const float* them;
+    const float* bias;
+    float* l0;
+    float max_act;
+    ActGrid act;
+};
+constexpr int kFuse16 = 1, kFuseF = 2;
+
+__device__ __forceinline__ bool finite4(const f4& x) {
+    return fabsf(x.x) <= 3.402823466e+38f && fabsf(x.y) <= 3.402823466e+38f && fabsf(x.z) <= 3.402823466e+38f &&
+           fabsf(x.w) <= 3.402823466e+38f;
+}
+
 typedef unsigned int u2 __attribute__((ext_vector_type(2)));
 
 // 16 bytes of a row in the FUSE layout: four 16-bit columns at `lo` and the four that pair with them, L1/2 further on
@@ -454,7 +489,7 @@ __device__ __forceinline__ f4 load_pair8(const char* lo, size_t half_bytes) {
     return __builtin_bit_cast(f4, u4{a.x, a.y, b.x, b.y});
 }
 
-template <int NT, bool VIRT, bool I16, bool FUSE = false>
+template <int NT, bool VIRT, bool I16, int FUSE = 0>
 __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ widx,
                                                           const int32_t* __restrict__ bidx,
                                                           const uint16_t* __restrict__ lists,
@@ -464,14 +499,18 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                                                           uint32_t* __restrict__ sched, const float* __restrict__ W,
                                                           float* __restrict__ acc, int B, int K, int R, int L1,
                                                           int out_cols, int tiles_per_xcd, int tile_group,
-                                                          VirtualTable vt, int block_rows, Fuse16 fz) {
-    static_assert(!FUSE || I16, "the fused epilogue belongs to the quantized table");
+                                                          VirtualTable vt, int block_rows, Fuse16 fz, FuseF ff) {
+    static_assert((FUSE == kFuse16) == I16, "the quantized table is gathered with its own epilogue, and only it");
+    static_assert(FUSE == 0 || FUSE == kFuse16 || FUSE == kFuseF, "epilogue");
+    constexpr bool F16 = FUSE == kFuse16;   // the tile's rows are column pairs (j, j + L1/2) of the quantized table
+    constexpr bool FF = FUSE == kFuseF;     // the tiles come in pairs (c, c + ntiles / 2) of the float table
     extern __shared__ float4 lds_raw[];
     char* tb = reinterpret_cast<char*>(lds_raw);
     u4* lst = reinterpret_cast<u4*>(tb + kTileBytes);                                         // (kListCap + 32) * 2 bytes
     uint32_t* mpid = reinterpret_cast<uint32_t*>(tb + kTileBytes + (kListCap + 32) * 2);      // kChunk
     uint16_t* moff = reinterpret_cast<uint16_t*>(mpid + kChunk);                              // kChunk
     uint32_t* ctr = reinterpret_cast<uint32_t*>(moff + kChunk);   // [0] task counter, [1] the unit this workgroup works on next
+    f4* lbias = reinterpret_cast<f4*>(ctr + 4);                   // FF: the bias of the pair of tiles at work, 2 x 32 floats
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     constexpr int N4 = kRows * (kRowBytes / 16);
@@ -480,7 +519,9 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
     const int x = blockIdx.x % kXcd;
     // a tile row is 128 bytes: 32 floats, or 64 of the 16-bit weights of the quantized table (I16: a row of W is
     // then L1 int16, a row of acc too, the sums wrap like 16-bit adds and their order does not matter)
-    const int ntiles = I16 ? L1 / (2 * kTileCols) : L1 / kTileCols;
+    // FF: what the XCDs share out and the units visit are the pairs of tiles, ntiles / 2 of them
+    const int ntiles = I16 ? L1 / (2 * kTileCols) : (FF ? L1 / (2 * kTileCols) : L1 / kTileCols);
+    const int partner = ntiles;   // FF: tile c + partner holds the columns L1/2 beyond tile c's
     const size_t w_pitch = I16 ? (size_t)L1 * 2 : (size_t)out_cols * 4;
     const size_t a_pitch = I16 ? (size_t)L1 * 2 : (size_t)L1 * 4;
     const char* Wb = reinterpret_cast<const char*>(W);
@@ -521,7 +562,7 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
         _Pragma("unroll") for (int i = 0; i < IT; ++i) {                                                 \
             const int f = tid + i * NT;                                                                  \
             const int row = f >> 3;                                                                      \
-            if (FUSE)                                                                                    \
+            if (F16)                                                                                     \
                 v[i] = row < rows_here_ ? load_pair8(Wb + (size_t)(row0_ + row) * w_pitch + (c_) * 64 +  \
                                                      (f & 7) * 8, half_bytes)                            \
                                         : f4{0.f, 0.f, 0.f, 0.f};                                        \
@@ -576,9 +617,16 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
         int nunit = nunits;
         Chunk Cn{};
         int qn0 = 0, qn1 = 0;
-        for (int q = q0; q < q1; q += qs) {
-            const int c = x * tiles_per_xcd + q;
-            if (q != q0) __syncthreads();   // everyone is done reading the previous tile
+        // FF: a visit is two tiles, c and then its partner (second == 1)
+        for (int qq = FF ? 2 * q0 : q0; qq < (FF ? 2 * q1 : q1); qq += FF ? (qq & 1 ? 2 * qs - 1 : 1) : qs) {
+            const int q = FF ? qq >> 1 : qq;
+            const int second = FF ? qq & 1 : 0;
+            const int c = x * tiles_per_xcd + q + second * partner;
+            // everyone is done reading the previous tile.  (FF: the sums of the first tile of the visit are on their
+            // way to memory, and the waves that read them back after the second are others than those that wrote them,
+            // but of this workgroup: the barrier orders the two, and a fence of wider scope would write the XCD's L2
+            // back, 0.7 ms a forward.)
+            if (q != q0 || second) __syncthreads();
 #pragma unroll
             for (int i = 0; i < IT; ++i) {
                 const int f = tid + i * NT;
@@ -586,14 +634,18 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
             }
             if (tid == 0) ctr[0] = 0;
             f4 bias8 = {0.f, 0.f, 0.f, 0.f};
-            if (FUSE) bias8 = load_pair8(reinterpret_cast<const char*>(fz.b16) + c * 64 + j * 8, half_bytes);
+            if (F16) bias8 = load_pair8(reinterpret_cast<const char*>(fz.b16) + c * 64 + j * 8, half_bytes);
+            if (FF && tid < kTileCols / 4)
+                lbias[second * (kTileCols / 4) + tid] = *reinterpret_cast<const f4*>(ff.bias + c * kTileCols + tid * 4);
             __syncthreads();
-            if (q == q0) {
+            if (q == q0 && !second) {
                 nunit = __builtin_amdgcn_readfirstlane((int)ctr[1]);
                 if (nunit < nunits) NNUEFT_UNIT(nunit, Cn, qn0, qn1)
             }
-            if (q + qs < q1) {
-                NNUEFT_LOAD_TILE(C.block, c + qs)
+            if (FF && !second) {
+                NNUEFT_LOAD_TILE(C.block, c + partner)
+            } else if (q + qs < q1) {
+                NNUEFT_LOAD_TILE(C.block, x * tiles_per_xcd + q + qs)
             } else if (nunit < nunits) {
                 NNUEFT_LOAD_TILE(Cn.block, x * tiles_per_xcd + qn0)
             }
@@ -612,9 +664,20 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                 const int mx = __builtin_amdgcn_readfirstlane((int)field);   // lists are sorted longest first
                 // FUSE: which half of the output row the pair's bytes go to (asked for here, used after the sums)
                 int half = 0;
-                if (FUSE) {
+                if (F16) {
                     const int persp = pair >= B;
                     half = persp == (fz.stm[pair - persp * B] ? 1 : 0) ? 0 : 1;   // half 0 shows the side to move
+                }
+                // FF, second tile of a visit: the pair's sums of the first tile, back from `saved`, and whether the
+                // pair's half of the output row is written here (asked for now, used after the sums)
+                bool own_row = false;
+                f4 first = {0.f, 0.f, 0.f, 0.f};
+                if (FF && second) {
+                    const uint32_t mo = moff[s];
+                    own_row = (mo & kLoffOwnRow) != 0;
+                    half = (mo & kLoffSecondHalf) ? 1 : 0;
+                    first = *reinterpret_cast<const f4*>(reinterpret_cast<const char*>(acc) + (size_t)pair * a_pitch +
+                                                         (c - partner) * kRowBytes + j * 16);
                 }
                 f4 a = {0.f, 0.f, 0.f, 0.f};
                 if (__ballot(field == kForeign) != 0) {
@@ -623,7 +686,7 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                     for (int k = 0; k < K; ++k) {
                         const int r = ix[k];
                         if (r >= 0 && r < R) {
-                            f4 w = FUSE ? load_pair8(Wb + (size_t)r * w_pitch + c * 64 + j * 8, half_bytes)
+                            f4 w = F16 ? load_pair8(Wb + (size_t)r * w_pitch + c * 64 + j * 8, half_bytes)
                                         : *reinterpret_cast<const f4*>(Wb + (size_t)r * w_pitch + c * kRowBytes + j * 16);
                             if (VIRT)
                                 w = merged4(w, *reinterpret_cast<const f4*>(vt.V + (size_t)(r % kRows) * out_cols +
@@ -636,7 +699,7 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                     // task has beyond that names the row of zeros
                     uint32_t oo[kSlots / 2];
                     const int own = padded((int)field);
-                    const u4* lp = lst + moff[s];
+                    const u4* lp = lst + (moff[s] & kLoffMask);
                     constexpr uint32_t zz = (uint32_t)kRows | ((uint32_t)kRows << 16);
 #pragma unroll
                     for (int i = 0; i < kSlots / 8; ++i) {
@@ -660,7 +723,34 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                         }
                     }
                 }
-                if (FUSE) {
+                if (FF && second) {
+                    const f4 x0 = first + lbias[j], x1 = a + lbias[kTileCols / 4 + j];
+                    if (!finite4(x0) || !finite4(x1)) sched[kSchedNonFinite] = 1u;
+                    f4 o;
+                    o.x = clamp_act(x0.x, ff.max_act) * clamp_act(x1.x, ff.max_act);
+                    o.y = clamp_act(x0.y, ff.max_act) * clamp_act(x1.y, ff.max_act);
+                    o.z = clamp_act(x0.z, ff.max_act) * clamp_act(x1.z, ff.max_act);
+                    o.w = clamp_act(x0.w, ff.max_act) * clamp_act(x1.w, ff.max_act);
+                    if (ff.act.on) {
+                        o.x = (floorf(o.x * ff.act.scale + ff.act.eps) / ff.act.scale) * ff.act.post_mul;
+                        o.y = (floorf(o.y * ff.act.scale + ff.act.eps) / ff.act.scale) * ff.act.post_mul;
+                        o.z = (floorf(o.z * ff.act.scale + ff.act.eps) / ff.act.scale) * ff.act.post_mul;
+                        o.w = (floorf(o.w * ff.act.scale + ff.act.eps) / ff.act.scale) * ff.act.post_mul;
+                    }
+                    if (valid) {
+                        const int pos = pair >= B ? pair - B : pair;
+                        __builtin_nontemporal_store(a, reinterpret_cast<f4*>(reinterpret_cast<char*>(acc) + (size_t)pair * a_pitch +
+                                                                             c * kRowBytes + j * 16));
+                        if (own_row)
+                            __builtin_nontemporal_store(o, reinterpret_cast<f4*>(reinterpret_cast<char*>(ff.l0) + (size_t)pos * a_pitch +
+                                                                                 (size_t)half * (a_pitch >> 1) +
+                                                                                 (c - partner) * kRowBytes + j * 16));
+                    }
+                } else if (FF) {
+                    // first tile of a visit: a plain store, the sums are read back after the second
+                    if (valid)
+                        *reinterpret_cast<f4*>(reinterpret_cast<char*>(acc) + (size_t)pair * a_pitch + c * kRowBytes + j * 16) = a;
+                } else if (F16) {
                     acc_add<true>(a, bias8);
                     const us8 s8 = __builtin_bit_cast(us8, a);
                     uint32_t o4 = 0;
@@ -706,7 +796,10 @@ int allow_lds(int device) {
         e = hipFuncSetAttribute((const void*)k_acc_tile<kAccThreadsVirtual, true, false>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
     if (e == hipSuccess)
-        e = hipFuncSetAttribute((const void*)k_acc_tile<kAccThreads, false, true, true>,
+        e = hipFuncSetAttribute((const void*)k_acc_tile<kAccThreads, false, true, kFuse16>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute((const void*)k_acc_tile<kAccThreads, false, false, kFuseF>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
     if (e != hipSuccess) return (int)e;
     g_lds_allowed[device].store(1, std::memory_order_release);
@@ -721,7 +814,8 @@ int launch_binscan(uint32_t* hist, uint32_t* total, int nbins, int ngroups, hipS
 }
 
 int launch_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, const Layout& L, void* ws, hipStream_t st,
-                Sorted* out) {
+                Sorted* out, const float* us, const float* them) {
+    if ((us != nullptr) != (them != nullptr) || (us && L.npairs != 2 * B)) return NNUEFT_E_ARG;
     char* base = (char*)ws;
     uint32_t* hist = (uint32_t*)(base + L.hist);
     uint16_t* lists = (uint16_t*)(base + L.lists);
@@ -741,7 +835,8 @@ int launch_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, c
                        total, L.nbins, L.ngroups);
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_tl_lists, dim3(L.ngroups), dim3(kSortThreads), 0, st, widx, bidx, hist, total, lists, pidcnt,
-                       loff, chunks, sched, brec, cpool8, border, L.npairs, B, K, R, L.nblocks, L.nbins, vec, L.block_rows);
+                       loff, chunks, sched, brec, cpool8, border, L.npairs, B, K, R, L.nblocks, L.nbins, vec, L.block_rows,
+                       us, them);
     NNUEFT_LAUNCH_CHECK();
     *out = Sorted{lists, pidcnt, loff, chunks, brec, cpool8, border, sched};
     return 0;
@@ -751,7 +846,10 @@ int launch_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, c
 // integers over a table W of [R, L1] int16).
 static int gather_tile(const int32_t* widx, const int32_t* bidx, const void* W, void* sums, int B, int K, int R, int L1,
                        int out_cols, void* ws, hipStream_t st, VirtualTable vt, bool i16, int block_rows = kRows,
-                       Fuse16 fz = Fuse16{nullptr, nullptr, nullptr, 0, 0}) {
+                       Fuse16 fz = Fuse16{nullptr, nullptr, nullptr, 0, 0},
+                       FuseF ff = FuseF{nullptr, nullptr, nullptr, nullptr, 0.0f, ActGrid{1.0f, 0.0f, 1.0f, 0}},
+                       const uint32_t** nonfinite = nullptr) {
+    if (ff.l0 && (i16 || vt.V || L1 % (2 * kTileCols) != 0)) return NNUEFT_E_ARG;   // the tiles must come in pairs
     Layout L;
     if (!layout(2 * B, R, &L, block_rows)) return NNUEFT_E_UNSUPPORTED;
     int device = 0;
@@ -761,18 +859,20 @@ static int gather_tile(const int32_t* widx, const int32_t* bidx, const void* W, 
     rc = allow_lds(device);
     if (rc) return rc;
     Sorted S;
-    rc = launch_sort(widx, bidx, B, K, R, L, ws, st, &S);
+    rc = launch_sort(widx, bidx, B, K, R, L, ws, st, &S, ff.us, ff.them);
     if (rc) return rc;
     const uint16_t* lists = S.lists;
     const uint32_t* pidcnt = S.pidcnt;
     const uint16_t* loff = S.loff;
     const Chunk* chunks = S.chunks;
     uint32_t* sched = S.sched;
-    const int ntiles = i16 ? L1 / (2 * kTileCols) : L1 / kTileCols;
+    // what the XCDs share out: tiles, or (ff) pairs of a tile and the one L1/2 columns further on
+    const int ntiles = i16 || ff.l0 ? L1 / (2 * kTileCols) : L1 / kTileCols;
     const int tiles_per_xcd = (ntiles + kXcd - 1) / kXcd;
-    // about three tiles per visit of a chunk: its lists are copied into LDS once per visit, and a batch is
-    // cut into enough units for the CUs of an XCD to finish together
-    int tile_group = (tiles_per_xcd + (tiles_per_xcd + 2) / 3 - 1) / ((tiles_per_xcd + 2) / 3);
+    // about three tiles (two pairs) per visit of a chunk: its lists are copied into LDS once per visit, and a batch
+    // is cut into enough units for the CUs of an XCD to finish together
+    const int per_visit = ff.l0 ? 2 : 3;
+    int tile_group = (tiles_per_xcd + (tiles_per_xcd + per_visit - 1) / per_visit - 1) / ((tiles_per_xcd + per_visit - 1) / per_visit);
 #ifdef NNUEFT_TUNE_ENV
     if (const char* e = getenv("NNUEFT_TILE_GROUP")) tile_group = atoi(e) > 0 ? atoi(e) : tile_group;
 #endif
@@ -780,20 +880,25 @@ static int gather_tile(const int32_t* widx, const int32_t* bidx, const void* W, 
     const float* Wf = (const float*)W;
     float* sf = (float*)sums;
     if (i16 && fz.out)
-        hipLaunchKernelGGL((k_acc_tile<kAccThreads, false, true, true>), dim3(grid), dim3(kAccThreads), kLdsBytes, st, widx,
+        hipLaunchKernelGGL((k_acc_tile<kAccThreads, false, true, kFuse16>), dim3(grid), dim3(kAccThreads), kLdsBytes, st, widx,
                            bidx, lists, pidcnt, loff, chunks, sched, Wf, sf, B, K, R, L1, out_cols, tiles_per_xcd,
-                           tile_group, vt, L.block_rows, fz);
+                           tile_group, vt, L.block_rows, fz, ff);
     else if (i16)
         return NNUEFT_E_ARG;   // the quantized table is only gathered with the fused epilogue
+    else if (ff.l0)
+        hipLaunchKernelGGL((k_acc_tile<kAccThreads, false, false, kFuseF>), dim3(grid), dim3(kAccThreads), kLdsBytes, st,
+                           widx, bidx, lists, pidcnt, loff, chunks, sched, Wf, sf, B, K, R, L1, out_cols, tiles_per_xcd,
+                           tile_group, vt, L.block_rows, fz, ff);
     else if (vt.V)
         hipLaunchKernelGGL((k_acc_tile<kAccThreadsVirtual, true, false>), dim3(grid), dim3(kAccThreadsVirtual), kLdsBytes, st,
                            widx, bidx, lists, pidcnt, loff, chunks, sched, Wf, sf, B, K, R, L1, out_cols, tiles_per_xcd,
-                           tile_group, vt, L.block_rows, fz);
+                           tile_group, vt, L.block_rows, fz, ff);
     else
         hipLaunchKernelGGL((k_acc_tile<kAccThreads, false, false>), dim3(grid), dim3(kAccThreads), kLdsBytes, st, widx, bidx,
                            lists, pidcnt, loff, chunks, sched, Wf, sf, B, K, R, L1, out_cols, tiles_per_xcd,
-                           tile_group, vt, L.block_rows, fz);
+                           tile_group, vt, L.block_rows, fz, ff);
     NNUEFT_LAUNCH_CHECK();
+    if (nonfinite) *nonfinite = sched + kSchedNonFinite;
     return 0;
 }
 
@@ -801,10 +906,27 @@ int double_fwd_tile(const float* us, const float* them, const int32_t* widx, con
                     const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,
                     float* wpsqt, float* bpsqt, float* saved, int B, int K, int R, int L1, int n_psqt, void* ws,
                     hipStream_t st, ActGrid act, VirtualTable vt) {
-    const int rc = gather_tile(widx, bidx, W, saved, B, K, R, L1, L1 + n_psqt, ws, st, vt, false);
+    // The gather finishes the output rows itself where that pays: tiles that come in pairs, four pairs or more for
+    // every XCD (L1 >= 2048: forward 0.25 -> 0.22 ms at L1 = 2048, 0.34 -> 0.31 ms at L1 = 3072, B = 16384; narrower
+    // rows leave the XCD's CUs too few units to share, 0.086 -> 0.092 ms at L1 = 1024, B = 8192), a table that is not
+    // merged on the fly (that variant has no registers to spare).  Else the sums first, then the pass over them.
+    bool pairs = !vt.V && L1 % (2 * kTileCols) == 0 && L1 / (2 * kTileCols) >= 4 * kXcd;
+#ifdef NNUEFT_NO_FWD_FUSE
+    pairs = false;
+#endif
+    if (!pairs) {
+        const int rc = gather_tile(widx, bidx, W, saved, B, K, R, L1, L1 + n_psqt, ws, st, vt, false);
+        if (rc) return rc;
+        return nnueft_blocked::launch_mix(us, them, widx, bidx, psqt_idx, W, bias, saved, max_act, l0, wpsqt, bpsqt, B,
+                                          K, R, L1, n_psqt, st, act, vt, nullptr);
+    }
+    // the gather writes the sums and, where one perspective's sums are all a half row needs, the output row too
+    const uint32_t* nonfinite = nullptr;
+    const int rc = gather_tile(widx, bidx, W, saved, B, K, R, L1, L1 + n_psqt, ws, st, vt, false, kRows,
+                               Fuse16{nullptr, nullptr, nullptr, 0, 0}, FuseF{us, them, bias, l0, max_act, act}, &nonfinite);
     if (rc) return rc;
     return nnueft_blocked::launch_mix(us, them, widx, bidx, psqt_idx, W, bias, saved, max_act, l0, wpsqt, bpsqt, B,
-                                      K, R, L1, n_psqt, st, act, vt);
+                                      K, R, L1, n_psqt, st, act, vt, nonfinite);
 }
 
 bool fits_int16(const nnueft_dev::DeviceInfo& d, int B, int K, int R, int L1, int block_rows) {

@@ -53,12 +53,14 @@ int launch_pair_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int
                      hipStream_t st, const uint32_t** order);
 
 // In-place exclusive scan of data[0..n) (one workgroup); the second half of the forward (bias, mix, clamp,
-// product, psqt chains) over row sums saved[2, B, L1].
+// product, psqt chains) over row sums saved[2, B, L1].  nonfinite != nullptr: the gather has already written the
+// output row of every position whose (us, them) is (1, 0) or (0, 1); only the other positions' rows and the psqt
+// chains are left, unless *nonfinite (device memory) says that some sum was not finite: then every row is redone.
 int launch_scan(uint32_t* data, int n, hipStream_t st);
 int launch_mix(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                const int64_t* psqt_idx, const float* W, const float* bias, const float* saved, float max_act,
                float* l0, float* wpsqt, float* bpsqt, int B, int K, int R, int L1, int n_psqt, hipStream_t st,
-               ActGrid act, VirtualTable vt);
+               ActGrid act, VirtualTable vt, const uint32_t* nonfinite);
 
 int double_fwd_blocked(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                        const int64_t* psqt_idx, const float* W, const float* bias, float max_act, float* l0,

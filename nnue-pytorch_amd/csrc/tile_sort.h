@@ -25,13 +25,22 @@ constexpr int kBins = 2048;                        // LDS counters of the sort (
 static_assert(kMaxBlocks * kLenBins + 1 <= kBins, "sort bins");
 static_assert(kRows == kBlockRows, "rows of a table block");
 constexpr uint32_t kForeign = 63;                  // count field of a list that leaves its block
+// loff[]: a list's place among its chunk's lists in units of 8 entries (12 bits), and, when the sort was given the
+// sides to move, two facts about the pair for the forward that writes the output rows itself
+constexpr uint32_t kLoffMask = 0xfffu;
+constexpr uint32_t kLoffSecondHalf = 0x4000u;      // the pair's sums make the second half of the position's output row
+constexpr uint32_t kLoffOwnRow = 0x8000u;          // (us, them) is (1, 0) or (0, 1): the pair's sums alone make that half
+static_assert(kListCap / 8 <= (int)kLoffMask, "list offsets");
+constexpr int kSchedNonFinite = kXcd * 32 + 1;     // word of Sorted::sched: a gather met a sum that is not finite
 #ifndef NNUEFT_TILE_NT
 #define NNUEFT_TILE_NT 1024
 #endif
 constexpr int kAccThreads = NNUEFT_TILE_NT;
 constexpr int kAccThreadsVirtual = 768;
 constexpr int kSortThreads = 256;
-constexpr int kLdsBytes = kTileBytes + (kListCap + 32) * 2 + kChunk * 4 + kChunk * 2 + 16;
+// tile, lists, pair ids, list offsets, two counters, the bias of two tiles
+constexpr int kLdsBytes = kTileBytes + (kListCap + 32) * 2 + kChunk * 4 + kChunk * 2 + 16 + 2 * kRowBytes;
+static_assert(kLdsBytes <= 160 * 1024, "LDS of a CU");
 
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
@@ -75,12 +84,14 @@ struct Sorted {
     const BlockRec* brec;
     const uint32_t* cpool8;
     const uint32_t* border;   // table blocks, most pairs first
-    uint32_t* sched;          // kXcd unit counters 32 words apart (zero after the sort), [kXcd * 32] = chunks in all
+    uint32_t* sched;          // kXcd unit counters 32 words apart (zero after the sort), [kXcd * 32] = chunks in all,
+                              // [kSchedNonFinite] = 0 after the sort
 };
 
-// k_tl_hist, k_tl_binscan, k_tl_lists on `st`.
+// k_tl_hist, k_tl_binscan, k_tl_lists on `st`.  us, them (both or neither; f32 [B], L.npairs == 2 B): the sides to
+// move, for the kLoff* bits of loff[]; without them those bits are 0.
 int launch_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, const Layout& L, void* ws, hipStream_t st,
-                Sorted* out);
+                Sorted* out, const float* us = nullptr, const float* them = nullptr);
 
 // One wave per bin: hist[bin][0 .. ngroups) becomes its exclusive prefix, total[bin] the sum.
 int launch_binscan(uint32_t* hist, uint32_t* total, int nbins, int ngroups, hipStream_t st);

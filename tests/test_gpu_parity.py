@@ -298,6 +298,66 @@ def test_double_forward(oracle_cpu, B, L1, R, K, kw, with_workspace):
         assert np.array_equal(got, ref)
 
 
+@pytest.mark.parametrize("kind", ["mixed_sides", "a_sum_that_is_not_finite"])
+@pytest.mark.parametrize("B,L1,R,K,kw", [
+    (900, 2112, 24576, 32, dict(halfka=True, weight_scale=0.05, max_act=255 / 256)),  # lists inside their blocks; 33
+                                                                                      # pairs of tiles over 8 XCDs
+    (700, 2048, 2000, 32, dict(allow_holes=True)),                                    # lists that leave them
+    (300, 1024, 24576, 32, dict(halfka=True, weight_scale=0.05, max_act=255 / 256)),  # rows too narrow for it: the sums
+                                                                                      # first, then the pass over them
+])
+def test_double_forward_rows_written_by_the_gather(oracle_cpu, kind, B, L1, R, K, kw):
+    """From L1 = 2048 on the LDS-tiled gather writes a position's output row itself when (us, them) is (1, 0) or
+    (0, 1), and leaves every other position to the pass behind it; the two must not be told apart in the result.  mixed_sides: both
+    kinds of position (and signed zeros, which count as zero) in one batch.  a_sum_that_is_not_finite: an infinite
+    weight makes 0 * inf = NaN in the other perspective's half of the row, as the mix of both perspectives gives it."""
+    c = double_case(470 + B, B, L1, R, K, **kw)
+    rng = np.random.default_rng(9)
+    sides = np.array([(1.0, 0.0), (0.0, 1.0), (1.0, -0.0), (-0.0, 1.0), (0.5, 0.5), (1.0, 1.0), (0.0, 0.0), (1.0, 1e-3),
+                      (2.0, 0.0)], np.float32)
+    pick = sides[rng.integers(0, 4 if kind != "mixed_sides" else len(sides), size=B)]
+    c["us"], c["them"] = np.ascontiguousarray(pick[:, :1]), np.ascontiguousarray(pick[:, 1:])
+    if kind != "mixed_sides":
+        rows = np.unique(c["widx"][c["widx"] >= 0])
+        c["W"][rows[len(rows) // 2], 5] = np.inf
+        c["W"][rows[len(rows) // 3], L1 // 2 + 40] = -np.inf
+    for act in (False, True):
+        nat, lib = _native()
+        n_psqt = c["n_psqt"]
+        d = {k: _t(c[k]) for k in ("us", "them", "widx", "bidx", "psqt_idx", "W", "bias")}
+        l0 = torch.full((B, L1), float("nan"), device=_dev())
+        wp, bp = torch.empty(B, 1, device=_dev()), torch.empty(B, 1, device=_dev())
+        saved = torch.full((2, B, L1), float("nan"), device=_dev())
+        nbytes = lib.nnueft_fwd_workspace_bytes(B, K, R, L1, n_psqt)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=_dev())
+        args = (d["us"].data_ptr(), d["them"].data_ptr(), d["widx"].data_ptr(), d["bidx"].data_ptr(),
+                d["psqt_idx"].data_ptr(), d["W"].data_ptr(), d["bias"].data_ptr(), c["max_act"], l0.data_ptr(),
+                wp.data_ptr(), bp.data_ptr(), saved.data_ptr(), B, K, R, L1, n_psqt, ws.data_ptr(), nbytes)
+        if act:
+            nat.check(lib.nnueft_double_fwd_act(*args, 127.0, 1e-5, 0.75, _stream()), "double_fwd_act")
+        else:
+            nat.check(lib.nnueft_double_fwd(*args, _stream()), "double_fwd")
+        with np.errstate(invalid="ignore"):
+            r_l0, r_wp, r_bp, r_saved = oracle_cpu.double_fwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"],
+                                                              c["W"], c["bias"], c["max_act"], L1)
+            if act:
+                r_l0 = oracle_cpu.act_fake_quantize(r_l0, 127.0, 1e-5, 0.75)
+        if kind != "mixed_sides":
+            assert np.isnan(r_l0).any() and not np.isnan(r_l0).all(axis=1).any()
+        for got, ref in ((l0, r_l0), (wp, r_wp), (bp, r_bp), (saved, r_saved)):
+            assert np.array_equal(got.cpu().numpy(), ref, equal_nan=True)
+        # a second forward over the same workspace, now without the weight: the sign that a sum was not finite is gone
+        if kind != "mixed_sides" and not act:
+            Wf = c["W"].copy()
+            Wf[~np.isfinite(Wf)] = 0.25
+            d["W"].copy_(_t(Wf))
+            nat.check(lib.nnueft_double_fwd(*args, _stream()), "double_fwd")
+            r_l0 = oracle_cpu.double_fwd(c["us"], c["them"], c["widx"], c["bidx"], c["psqt_idx"], Wf, c["bias"],
+                                         c["max_act"], L1)[0]
+            assert np.array_equal(l0.cpu().numpy(), r_l0)
+            d["W"].copy_(_t(c["W"]))
+
+
 def test_double_forward_from_index_lists_that_are_not_16_byte_aligned(oracle_cpu):
     """Index tensors that begin 4 bytes past a 16-byte boundary (a view into a larger buffer): the sort of the
     LDS-tiled forward then reads the lists entry by entry; same bits."""
