@@ -82,7 +82,15 @@ def compulsory_bytes(L1, B, sum_a):
     lists = 2 * B * K_SLOTS * 4
     saved = 2 * B * L1 * 4
     small = B * 24
-    if forward_path(L1) == "tile":
+    if forward_path(L1) == "tile_pairs":
+        fwd = {
+            "list sort": 2 * lists + sum_a * 2 + 2 * B * 6 + B * 8,       # + the sides to move
+            # table once, packed lists, row sums written, output rows written (the sums of a visit's first tile come
+            # back from memory once: they have left the XCD's L2 by the time the second tile's are done)
+            "k_acc_tile": R_ROWS * oc * 4 + sum_a * 2 + 2 * B * 6 + saved + saved // 2 + B * L1 * 4,
+            "k_mix_rest": lists + small,                                  # psqt chains
+        }
+    elif forward_path(L1) == "tile":
         fwd = {
             # 16-bit lists at their own length, pair id and list place per list
             "list sort": 2 * lists + sum_a * 2 + 2 * B * 6,               # lists twice, packed lists written
@@ -146,7 +154,10 @@ def sum_traffic(traffic, kernels):
 
 
 def forward_path(L1):
-    """Which gather nnueft_double_fwd takes with a workspace: out of LDS tiles for wide rows, else blocked for L2."""
+    """Which gather nnueft_double_fwd takes with a workspace: out of LDS tiles for wide rows (from L1 = 2048 on it visits
+    the column tiles in pairs and writes the output rows itself), else blocked for L2."""
+    if L1 >= 2048 and L1 % 64 == 0:
+        return "tile_pairs"
     return "tile" if L1 >= 512 and L1 % 32 == 0 else "blocked"
 
 
@@ -166,8 +177,10 @@ def bwd_kernels(L1, mode):
 
 
 def fwd_kernels(L1):
+    if forward_path(L1) == "tile_pairs":
+        return ("k_tl_hist", "k_tl_binscan", "k_tl_lists", "k_acc_tile", "k_mix_rest")
     if forward_path(L1) == "tile":
-        return ("k_tl_hist", "k_tl_binscan", "k_tl_lists", "k_acc_tile", "k_mix")
+        return ("k_tl_hist", "k_tl_binscan", "k_tl_lists", "k_acc_tile", "k_mix<")
     return ("k_pair_hist", "k_pair_scan", "k_pair_scatter", "k_acc_blocked", "k_mix")
 
 
@@ -791,9 +804,11 @@ def run_ft(args, lib, dev):
                   "lds_nominal_GBs": LDS_PEAK_GBS, "lds_nominal": f"256 CUs x 256 B per clock at {ENGINE_CLOCK_GHZ} GHz",
                   "measured": probes, "traffic_source": traffic_file},
     }
-    if forward_path(L1) == "tile":
+    if forward_path(L1) in ("tile", "tile_pairs"):
         # the gather reads the table out of LDS tiles: its algorithmic bytes are LDS reads
         fwd_block, fwd_comp = bound_block(
+            "nnueft_double_fwd: k_acc_tile (the gather out of LDS tiles; it writes the output rows too) + k_mix_rest "
+            "(psqt chains) + list sort" if forward_path(L1) == "tile_pairs" else
             "nnueft_double_fwd: k_acc_tile (the gather out of LDS tiles, ~2/3 of the time) + k_mix + list sort", fwd_ms,
             fwd_bytes, None, sum(comp_fwd.values()), sum_traffic(traffic, fwd_kernels(L1)), LDS_PEAK_GBS,
             note="the gathered rows are LDS reads: peak = what 16-byte reads of whole 128-byte rows at random rows of a "

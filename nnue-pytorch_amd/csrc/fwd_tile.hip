@@ -19,6 +19,10 @@
 //                 while the current one is summed; waves take tasks of 8 pairs from a counter in LDS
 //   k_mix         as in the L2-blocked path
 //
+// Rows of 2048 columns and more: the gather visits the column tiles in pairs (columns j and j + L1/2) and writes
+// the output rows of the positions whose (us, them) is (1, 0) or (0, 1) itself (see FuseF); k_mix_rest then does
+// the psqt chains and the other positions.
+//
 // A list that names rows of more than one block (the interface allows it) is summed from global
 // memory by the same wave; results are bit-identical to the other forward kernels.
 #include <atomic>
@@ -446,7 +450,7 @@ __device__ __forceinline__ void acc_add(f4& a, const f4& r) {
 // saved[pair, columns of the tile] = chain from +0 over the pair's list, for every pair of the chunk.
 // VIRT: the table is W + V[row % kRows] (see merged4); the tile is merged on its way into LDS.  That variant
 // runs with 768 threads: the tile of V waits in registers beside the tile of W.
-// What the quantized forward does with a pair's sums when the gather finishes them itself (FUSE): + bias, clip,
+// What the quantized forward does with a pair's sums when the gather finishes them itself (FUSE == kFuse16): + bias, clip,
 // product of column j with column j + L1/2, >> shift, one byte per column pair, written to the half of the
 // position's output row that the side to move selects.
 struct Fuse16 {
@@ -482,7 +486,7 @@ __device__ __forceinline__ bool finite4(const f4& x) {
 
 typedef unsigned int u2 __attribute__((ext_vector_type(2)));
 
-// 16 bytes of a row in the FUSE layout: four 16-bit columns at `lo` and the four that pair with them, L1/2 further on
+// 16 bytes of a row in the kFuse16 layout: four 16-bit columns at `lo` and the four that pair with them, L1/2 further on
 __device__ __forceinline__ f4 load_pair8(const char* lo, size_t half_bytes) {
     const u2 a = *reinterpret_cast<const u2*>(lo);
     const u2 b = *reinterpret_cast<const u2*>(lo + half_bytes);
@@ -525,7 +529,7 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
     const size_t w_pitch = I16 ? (size_t)L1 * 2 : (size_t)out_cols * 4;
     const size_t a_pitch = I16 ? (size_t)L1 * 2 : (size_t)L1 * 4;
     const char* Wb = reinterpret_cast<const char*>(W);
-    // FUSE: a tile row is 32 column pairs (j, j + L1/2): lane piece q holds columns 4q .. 4q+3 of the tile's 32 and
+    // F16: a tile row is 32 column pairs (j, j + L1/2): lane piece q holds columns 4q .. 4q+3 of the tile's 32 and
     // their four partners, so the product needs no other lane
     const size_t half_bytes = (size_t)L1;   // L1/2 columns of 2 bytes
     // the column tiles of this XCD, in groups of tile_group; a unit = (chunk, group)
@@ -533,7 +537,7 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
     const int groups = (my_tiles + tile_group - 1) / tile_group;
     // A unit's tiles are `groups` apart, so that the units (chunk, g), (chunk, g + 1), handed to two CUs one after
     // the other, fetch neighbouring tiles at about the same time: a 128-byte tile row straddles two cache lines of
-    // a 12 320-byte table row (FUSE: it is two half lines whose other halves the neighbour tile holds), and the
+    // a 12 320-byte table row (F16: it is two half lines whose other halves the neighbour tile holds), and the
     // second fetch of a shared line then hits the XCD's L2 (forward at L1 = 3072: 0.318 -> 0.306 ms; the
     // quantized table: fetched 0.43 -> 0.26 GB)
     const int qs = groups;
@@ -662,7 +666,7 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
                 const uint32_t field = pc >> 26;
                 const int pair = (int)(pc & 0x3ffffffu);
                 const int mx = __builtin_amdgcn_readfirstlane((int)field);   // lists are sorted longest first
-                // FUSE: which half of the output row the pair's bytes go to (asked for here, used after the sums)
+                // F16: which half of the output row the pair's bytes go to (asked for here, used after the sums)
                 int half = 0;
                 if (F16) {
                     const int persp = pair >= B;
