@@ -269,13 +269,15 @@ def test_reduce_rows_stage_equals_the_sparse_backward(oracle_cpu):
                                                   nbytes, lists.data_ptr(), st) == -1
 
 
-@pytest.mark.parametrize("L1", [256, 1024], ids=["l2_blocked_forward", "lds_tiled_forward"])
+@pytest.mark.parametrize("L1", [256, 1024, 2048],
+                         ids=["l2_blocked_forward", "lds_tiled_forward", "lds_tiled_forward_that_writes_the_output_rows"])
 def test_forward_and_deterministic_backward_under_graph_capture(L1):
     """The launch path of the operator inside one captured HIP graph: forward + deterministic backward (sort
     inline, workspaces allocated before the capture), replayed with eager work and synchronisations between the
     replays; every replay must give the bits of the eager run, also after the inputs changed in place.  Both
     forward gathers: blocked for L2 (narrow rows) and out of LDS tiles (its unit counters live in the workspace
-    and are reset by the sort of every call)."""
+    and are reset by the sort of every call; from L1 = 2048 on it also writes the output rows, and its sign for a sum
+    that is not finite lives there too)."""
     lib = _native.load()
     B, K, R, n_psqt = 4096, 32, hk.NUM_INPUTS, 8
     oc = L1 + n_psqt
