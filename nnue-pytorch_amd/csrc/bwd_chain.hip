@@ -69,6 +69,10 @@ constexpr int kTileB = (kCP + 1) * kRowB;  // + the row of zeros the padding nam
 // units | blocks << 20, bit 31: dense); from byte 256 the row of every chain in task order (a long task has 4 chains,
 // the others 16; chains that fill up a task name row 768, which exists in LDS and nowhere else).
 constexpr int kMaxTasks = 63;
+constexpr int kSortWaves = kRows / 64;             // the list maker sorts a block's rows, a row a thread
+constexpr int kCntBins = 640;                      // chain lengths 0 .. kCP
+static_assert(kCntBins > kCP && kCntBins % 2 == 0, "a counter per chain length");
+static_assert(kSortWaves * kCntBins >= kRows * (kMaskWords / 2) && kMaskWords % 2 == 0, "the prefix table takes the counters' place");
 constexpr int kRowSlots = 832;
 constexpr int kMdB = 256 + kRowSlots * 2;
 constexpr int kMdWords = kMdB / 4;
@@ -330,7 +334,11 @@ __global__ __launch_bounds__(kThreads) void k_cs_expand(const int32_t* __restric
     uint32_t* mdw = reinterpret_cast<uint32_t*>(slot_of_row + kRows);  // [kMdWords]
     uint32_t* small = mdw + kMdWords;                                  // [8] counters
     uint16_t* lent = reinterpret_cast<uint16_t*>(small + 8);           // [kEntCap]
+    // [kSortWaves][kCntBins] rows of a wave by chain length (the sort), then [kRows][kMaskWords / 2] set bits of a row
+    // in front of every second word of its bit map (the lists)
+    uint16_t* whist = lent + kEntCap;
     const int tid = threadIdx.x;
+    const int lane = tid & 63;
     const int c = blockIdx.x;
     if (sched[kFlagWord] != 0 || c >= (int)sched[kChunksWord]) return;
     const RChunk C = chunks[c];
@@ -355,31 +363,57 @@ __global__ __launch_bounds__(kThreads) void k_cs_expand(const int32_t* __restric
         if (twice) atomicOr(&sched[kFlagWord], 2u);   // a row twice in one list: not for the bit map
     }
     __syncthreads();
-    // rows by chain length, longest first (ties: lower row first); a bitonic sort of 1024 keys
-    {
-        uint32_t key = 0;
-        if (tid < kRows) {
-            uint32_t cnt = 0;
-            for (int w = 0; w < kMaskWords; ++w) cnt += (uint32_t)__popc(mask[tid * kMaskWords + w]);
-            key = (cnt << 10) | (uint32_t)(1023 - tid);
+    // Rows by chain length, longest first (ties: lower row first), by counting: a row's place = the rows with longer
+    // chains + the rows of its length in the waves in front + those in front of it in its own wave.  (A bitonic sort
+    // of the 1024 keys, 55 steps with a barrier each, took 10 of the kernel's 33 microseconds.)
+    uint32_t cnt = 0;
+    if (tid < kRows)
+        for (int w = 0; w < kMaskWords; ++w) cnt += (uint32_t)__popc(mask[tid * kMaskWords + w]);
+    for (int i = tid; i < kSortWaves * kCntBins / 2; i += kThreads) reinterpret_cast<uint32_t*>(whist)[i] = 0;
+    __syncthreads();
+    int before = 0;   // rows of the same length in front, in this wave
+    if (tid < kRows) {
+        static_assert(kRows % 64 == 0, "the waves that hold rows are full");
+        u64 todo = ~(u64)0;
+        const u64 lt = ((u64)1 << lane) - 1;
+        while (todo) {
+            const int l = __ffsll((long long)todo) - 1;
+            const uint32_t k = (uint32_t)__builtin_amdgcn_readlane((int)cnt, l);
+            const u64 m = __ballot(cnt == k);
+            if (cnt == k) before = __popcll(m & lt);
+            if (lane == l) whist[(tid >> 6) * kCntBins + k] = (uint16_t)__popcll(m);
+            todo &= ~m;
         }
-        keys[tid] = key;
     }
     __syncthreads();
-    for (int k2 = 2; k2 <= 1024; k2 <<= 1) {
-        for (int j = k2 >> 1; j > 0; j >>= 1) {
-            const int partner = tid ^ j;
-            if (partner > tid) {
-                const uint32_t a = keys[tid], b = keys[partner];
-                const bool desc = (tid & k2) == 0;
-                if (desc ? a < b : a > b) {
-                    keys[tid] = b;
-                    keys[partner] = a;
-                }
-            }
-            __syncthreads();
+    {
+        // thread i has length kCP - i: the rows longer than that (an exclusive scan over the threads), then the place
+        // of every wave's rows of that length
+        const int k = kCP - tid;
+        uint32_t tot = 0;
+        if (k >= 0)
+            for (int w = 0; w < kSortWaves; ++w) tot += whist[w * kCntBins + k];
+        uint32_t incl = tot;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const uint32_t t = __shfl_up(incl, off);
+            if (lane >= off) incl += t;
         }
+        if (lane == 63) keys[tid >> 6] = incl;
+        __syncthreads();
+        uint32_t run = incl - tot;
+        for (int w = 0; w < (tid >> 6); ++w) run += keys[w];
+        __syncthreads();   // keys gets the sorted rows next
+        if (k >= 0)
+            for (int w = 0; w < kSortWaves; ++w) {
+                const uint32_t h = whist[w * kCntBins + k];
+                whist[w * kCntBins + k] = (uint16_t)run;
+                run += h;
+            }
     }
+    __syncthreads();
+    if (tid < kRows) keys[whist[(tid >> 6) * kCntBins + cnt] + before] = (cnt << 10) | (uint32_t)(1023 - tid);
+    __syncthreads();
     uint32_t my_cnt = 0;
     int my_row = kRows;
     if (tid < kRows) {
@@ -414,19 +448,35 @@ __global__ __launch_bounds__(kThreads) void k_cs_expand(const int32_t* __restric
         else if (s >= nl && ((s - nl) & 15) == 0) mdw[1 + nd + nlt + ((s - nl) >> 4)] = ((my_cnt + 3) / 4) << 20;
     }
     __syncthreads();
-    if (tid == 0) {
+    if (tid < 64) {
         // places of the tasks' lists, in 8-byte units: a long task's block is 4 chains x 8 entries, a short task's
-        // 16 chains x 4 entries
-        uint32_t run = 0;
-        for (int t = nd; t < ntasks; ++t) {
-            const uint32_t nb = (mdw[1 + t] >> 20) & 0x7ffu;
-            mdw[1 + t] |= run;
-            run += nb * (t < nd + nlt ? 8u : 16u);
+        // 16 chains x 4 entries; lane t has task t (there are fewer than 64), and the last lane the total
+        static_assert(kMaxTasks < 64, "a lane a task, and one to spare");
+        const bool has_list = tid >= nd && tid < ntasks;
+        uint32_t sz = 0;
+        if (has_list) sz = ((mdw[1 + tid] >> 20) & 0x7ffu) * (tid < nd + nlt ? 8u : 16u);
+        uint32_t incl = sz;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const uint32_t t = __shfl_up(incl, off);
+            if (lane >= off) incl += t;
         }
-        run += run & 1u;
-        small[2] = run;
-        mdw[0] = (uint32_t)(nd + nlt) | ((uint32_t)ntasks << 16);
-        if (run * 4 > (uint32_t)kEntCap) atomicOr(&sched[kFlagWord], 4u);
+        if (has_list) mdw[1 + tid] |= incl - sz;
+        if (tid == 63) {
+            const uint32_t run = incl + (incl & 1u);
+            small[2] = run;
+            if (run * 4 > (uint32_t)kEntCap) atomicOr(&sched[kFlagWord], 4u);
+        }
+        if (tid == 0) mdw[0] = (uint32_t)(nd + nlt) | ((uint32_t)ntasks << 16);
+    }
+    // the set bits of a row in front of every second word of its bit map
+    if (tid < kRows) {
+        uint32_t run = 0;
+#pragma unroll
+        for (int w = 0; w < kMaskWords; w += 2) {
+            whist[tid * (kMaskWords / 2) + (w >> 1)] = (uint16_t)run;
+            run += (uint32_t)(__popc(mask[tid * kMaskWords + w]) + __popc(mask[tid * kMaskWords + w + 1]));
+        }
     }
     __syncthreads();
     const int n4 = (int)small[2];
@@ -441,8 +491,8 @@ __global__ __launch_bounds__(kThreads) void k_cs_expand(const int32_t* __restric
         const int slot = (int)slot_of_row[row];
         if (slot < nd) continue;
         const int s = slot - nd;
-        int pos = 0;
-        for (int w2 = 0; w2 < w; ++w2) pos += __popc(mask[row * kMaskWords + w2]);
+        int pos = (int)whist[row * (kMaskWords / 2) + (w >> 1)];
+        if (w & 1) pos += __popc(mask[item - 1]);
         const bool is_long = s < nl;
         const int task = is_long ? nd + (s >> 2) : nd + nlt + ((s - nl) >> 4);
         const uint32_t base = (mdw[1 + task] & 0xfffffu) * 4;
@@ -466,7 +516,7 @@ __global__ __launch_bounds__(kThreads) void k_cs_expand(const int32_t* __restric
         if (tid == 0) chunks[c].n4 = n4;
     }
 }
-constexpr int kExpandLds = (kRows * kMaskWords + 1024) * 4 + kRows * 2 + kMdB + 32 + kEntCap * 2;
+constexpr int kExpandLds = (kRows * kMaskWords + 1024) * 4 + kRows * 2 + kMdB + 32 + kEntCap * 2 + kSortWaves * kCntBins * 2;
 static_assert(kExpandLds <= 160 * 1024, "LDS of the list maker");
 
 typedef __attribute__((address_space(3))) const f4 lds_f4;
