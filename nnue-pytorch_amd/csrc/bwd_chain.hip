@@ -25,7 +25,7 @@
 //   k_cs_place    pairs to their places, a key's pairs in ascending pair order; the chunk table, the blocks by
 //                 pairs, the counters
 //   k_cs_expand   one workgroup per chunk: a bit per (row, pair) set with LDS atomics (ascending order for free),
-//                 rows sorted by chain length, tasks formed, lists written
+//                 rows ranked by chain length (by counting), tasks formed, lists written
 //   k_chain_tile  persistent workgroups, one per CU: units of (table block, column tile) dealt to the workgroups of
 //                 an XCD round by round; a step is one chunk of a unit; while a step runs, the tile, the lists and
 //                 the facts of the next step are on their way into registers, the pair ids of the one after it and
