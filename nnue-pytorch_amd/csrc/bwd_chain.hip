@@ -244,17 +244,37 @@ __global__ __launch_bounds__(kSortThreads) void k_cs_place(const int32_t* __rest
     __shared__ uint32_t tot[kMaxKeys + 1];
     for (int i = tid; i <= nkeys; i += kSortThreads) tot[i] = total[i];
     __syncthreads();
-    if (tid == 0) {
-        uint32_t run = 0, cr = 0;
-        for (int k = 0; k < nkeys; ++k) {
-            keybase[k] = run;
-            chunk0[k] = cr;
-            run += tot[k];
+    if (tid < 64) {
+        // where a key's pairs and chunks begin: two keys a lane, a scan over the wave
+        static_assert(kMaxKeys <= 128, "two keys a lane");
+        uint32_t np[2], nc[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int k = 2 * tid + h;
+            np[h] = k < nkeys ? tot[k] : 0u;
             // a single list of the batch (n_persp == 1) has no black chunks at all
-            cr += (n_persp == 1 && (k & 1)) ? 0 : chunks_of((int)tot[k]);
+            nc[h] = k < nkeys && !(n_persp == 1 && (k & 1)) ? (uint32_t)chunks_of((int)tot[k]) : 0u;
         }
-        keybase[nkeys] = run;
-        chunk0[nkeys] = cr;
+        uint32_t ip = np[0] + np[1], ic = nc[0] + nc[1];
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const uint32_t tp = __shfl_up(ip, off), tc = __shfl_up(ic, off);
+            if (lane >= off) {
+                ip += tp;
+                ic += tc;
+            }
+        }
+        uint32_t run = ip - np[0] - np[1], cr = ic - nc[0] - nc[1];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int k = 2 * tid + h;
+            if (k <= nkeys) {
+                keybase[k] = run;
+                chunk0[k] = cr;
+            }
+            run += np[h];
+            cr += nc[h];
+        }
     }
     __syncthreads();
     int key = nkeys;
