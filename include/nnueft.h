@@ -136,9 +136,12 @@ size_t nnueft_fwd_workspace_bytes(int B, int K, int R, int L1, int n_psqt);
  * L1 % 8 == 0, (L1+n_psqt) % 4 == 0) the positions are grouped by the 768-row table block their lists
  * name.  Rows of 512 columns and more (L1 % 32 == 0, K <= 32, a table of at most 62 blocks) are then
  * gathered out of LDS: a workgroup holds a tile of one block, 768 rows x 32 columns, and sums it for
- * every list of the block.  Other shapes are blocked for the per-XCD L2 caches: each XCD works through
- * its share of the grouped lists one column slice at a time.  Results are bit-identical with and
- * without the workspace.
+ * every list of the block.  From 2048 columns on (L1 % 64 == 0) the same kernel also writes l0 for every
+ * position whose (us, them) is (1, 0) or (0, 1), what the loaders produce; other values of us and them are
+ * allowed as everywhere and take a pass over `saved`, as does a batch in which a sum is not finite (0 * inf
+ * of the mix is NaN, here as in the reference).  Other shapes are blocked for the per-XCD L2 caches: each
+ * XCD works through its share of the grouped lists one column slice at a time.  Results are bit-identical
+ * with and without the workspace.
  */
 int nnueft_double_fwd(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                       const int64_t* psqt_idx, const float* W, const float* bias, float max_act,
