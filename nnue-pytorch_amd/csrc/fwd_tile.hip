@@ -630,6 +630,10 @@ __global__ __launch_bounds__(NT) void k_acc_tile(const int32_t* __restrict__ wid
             // way to memory, and the waves that read them back after the second are others than those that wrote them,
             // but of this workgroup: the barrier orders the two, and a fence of wider scope would write the XCD's L2
             // back, 0.7 ms a forward.)
+            // (The wait for this wave's stores to be acknowledged is not something the barrier asks for on this
+            // device, whose waves of a workgroup share an L1 that keeps their accesses in order; it costs nothing
+            // measurable and leaves nothing to that order.)
+            if (FF && second) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             if (q != q0 || second) __syncthreads();
 #pragma unroll
             for (int i = 0; i < IT; ++i) {
