@@ -250,25 +250,31 @@ __global__ __launch_bounds__(64) void k_mix(const float* __restrict__ us, const 
     if (s == 0) psqt_chains(b, lane, widx, bidx, psqt_idx, W, bias, wpsqt, bpsqt, K, R, L1, n_psqt, vt);
 }
 
-// What is left per position when the gather has written the output rows itself (it does for a position whose
-// (us, them) is (1, 0) or (0, 1): such a row is one perspective's sums on each half): the two psqt chains, and
+// What is left when the gather has written the output rows itself (it does for a position whose (us, them) is
+// (1, 0) or (0, 1): such a row is one perspective's sums on each half) and the sort in front of it the psqt chains:
 // the whole row of a position with any other (us, them), which needs both perspectives' sums at once; every row
 // when the gather met a sum that is not finite (*nonfinite != 0: 0 * inf of the other perspective's sum is NaN
-// in the mix, which the gather's row does not show).
+// in the mix, which the gather's row does not show).  A lane looks at a position, the wave redoes the ones that
+// need it one after the other.
+constexpr int kRestThreads = 256;
 template <int VW>
-__global__ __launch_bounds__(64) void k_mix_rest(const float* __restrict__ us, const float* __restrict__ them,
-                                                 const int32_t* __restrict__ widx, const int32_t* __restrict__ bidx,
-                                                 const int64_t* __restrict__ psqt_idx, const float* __restrict__ W,
-                                                 const float* __restrict__ bias, const float* __restrict__ saved,
-                                                 float max_act, float* __restrict__ l0, float* __restrict__ wpsqt,
-                                                 float* __restrict__ bpsqt, int B, int K, int R, int L1, int n_psqt,
-                                                 int nslices, ActGrid act, VirtualTable vt,
-                                                 const uint32_t* __restrict__ nonfinite) {
-    const int lane = threadIdx.x;
-    const int b = blockIdx.x;
-    if (!one_sided(us[b], them[b]) || *nonfinite != 0u)
-        for (int s = 0; s < nslices; ++s) mix_slice<VW>(s, b, lane, us, them, bias, saved, max_act, l0, B, L1, act);
-    psqt_chains(b, lane, widx, bidx, psqt_idx, W, bias, wpsqt, bpsqt, K, R, L1, n_psqt, vt);
+__global__ __launch_bounds__(kRestThreads) void k_mix_rest(const float* __restrict__ us, const float* __restrict__ them,
+                                                           const float* __restrict__ bias,
+                                                           const float* __restrict__ saved, float max_act,
+                                                           float* __restrict__ l0, int B, int L1, int nslices,
+                                                           ActGrid act, const uint32_t* __restrict__ nonfinite) {
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * (kRestThreads / 64) + (threadIdx.x >> 6);
+    const int nwaves = gridDim.x * (kRestThreads / 64);
+    const bool all = *nonfinite != 0u;
+    for (int base = wave * 64; base < B; base += nwaves * 64) {
+        const int p = base + lane;
+        u64 todo = __ballot(p < B && (all || !one_sided(us[min(p, B - 1)], them[min(p, B - 1)])));
+        while (todo) {
+            const int b = base + pop_lane(todo);
+            for (int s = 0; s < nslices; ++s) mix_slice<VW>(s, b, lane, us, them, bias, saved, max_act, l0, B, L1, act);
+        }
+    }
 }
 
 static inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -289,8 +295,12 @@ int launch_mix(const float* us, const float* them, const int32_t* widx, const in
     const int mix_slices = (hv + 63) / 64;
     if ((long long)B * mix_slices > 0x7fffffffLL) return NNUEFT_E_UNSUPPORTED;
     if (nonfinite) {
-        hipLaunchKernelGGL(k_mix_rest<4>, dim3((unsigned)B), dim3(64), 0, st, us, them, widx, bidx, psqt_idx, W, bias, saved,
-                           max_act, l0, wpsqt, bpsqt, B, K, R, L1, n_psqt, mix_slices, act, vt, nonfinite);
+        // the rows the gather left alone, nothing else: the psqt chains are the caller's
+        if (wpsqt || bpsqt) return NNUEFT_E_ARG;
+        const int waves = (B + 63) / 64;
+        const int blocks = min((waves + kRestThreads / 64 - 1) / (kRestThreads / 64), 1024);
+        hipLaunchKernelGGL(k_mix_rest<4>, dim3((unsigned)blocks), dim3(kRestThreads), 0, st, us, them, bias, saved, max_act,
+                           l0, B, L1, mix_slices, act, nonfinite);
         NNUEFT_LAUNCH_CHECK();
         return 0;
     }

@@ -196,8 +196,9 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
                                                            BlockRec* __restrict__ brec, uint32_t* __restrict__ cpool8,
                                                            uint32_t* __restrict__ border, int npairs, int B, int K,
                                                            int R, int nblocks, int nbins, int vec, int block_rows,
-                                                           const float* __restrict__ us,
-                                                           const float* __restrict__ them) {
+                                                           SortExtras ex) {
+    const float* __restrict__ us = ex.us;
+    const float* __restrict__ them = ex.them;
     __shared__ uint32_t cursor[kBins];      // next slot of this workgroup in every bin
     __shared__ uint32_t bin_base[kBins];    // first slot of every bin
     __shared__ uint32_t bin_eoff[kBins];    // list entries of its block before the bin's lists
@@ -326,6 +327,19 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
     }
     if (n >= npairs) return;
     const ListRegs l = load_list(pair_list(widx, bidx, n, B, K), K, vec);
+    // The pair's psqt chain, while its list is in registers: the entries of the list's valid rows are asked for here
+    // and summed at the end of the kernel, so that they are on their way during the rest.
+    float psv[kSlots];
+    int64_t psqt_col = -1;
+    if (ex.wpsqt) {
+        const int64_t pi = ex.psqt_idx[n >= B ? n - B : n];
+        if (pi >= 0 && pi < ex.n_psqt) psqt_col = pi;
+    }
+#pragma unroll
+    for (int k = 0; k < kSlots; ++k) {
+        const int r = l.v[k];
+        psv[k] = psqt_col >= 0 && r >= 0 && r < R ? ex.W[(size_t)r * ((size_t)ex.L1 + ex.n_psqt) + ex.L1 + psqt_col] : 0.0f;
+    }
     const ListFacts f = list_facts(l, R, block_rows);
     const int bin = sort_key(f);
     const uint32_t slot = atomicAdd(&cursor[bin], 1u);
@@ -391,6 +405,14 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
                 ++m;
             }
         }
+    }
+    if (ex.wpsqt) {
+        // in slot order; a slot without a row adds +0, which leaves a sum that began at +0 as it is
+        float ps = 0.0f;
+#pragma unroll
+        for (int k = 0; k < kSlots; ++k) ps = ps + psv[k];
+        if (psqt_col >= 0) ps = ps + ex.bias[ex.L1 + psqt_col];
+        (n >= B ? ex.bpsqt : ex.wpsqt)[n >= B ? n - B : n] = ps;
     }
     if (ci >= (uint32_t)kMaxChunks) return;   // (the launcher takes this path only when the table is long enough)
     u4* out = reinterpret_cast<u4*>(lists + ((size_t)chunk_pool8[ci] << 3) + off);
@@ -476,6 +498,10 @@ struct FuseF {
     float* l0;
     float max_act;
     ActGrid act;
+    // what the sort needs to sum the psqt chains on its way (it has every list in registers anyway)
+    const int64_t* psqt_idx;
+    float* wpsqt;
+    float* bpsqt;
 };
 constexpr int kFuse16 = 1, kFuseF = 2;
 
@@ -822,8 +848,9 @@ int launch_binscan(uint32_t* hist, uint32_t* total, int nbins, int ngroups, hipS
 }
 
 int launch_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, const Layout& L, void* ws, hipStream_t st,
-                Sorted* out, const float* us, const float* them) {
-    if ((us != nullptr) != (them != nullptr) || (us && L.npairs != 2 * B)) return NNUEFT_E_ARG;
+                Sorted* out, SortExtras ex) {
+    if ((ex.us != nullptr) != (ex.them != nullptr) || ((ex.us || ex.wpsqt) && L.npairs != 2 * B)) return NNUEFT_E_ARG;
+    if (ex.wpsqt && !(ex.bpsqt && ex.psqt_idx && ex.W && ex.bias)) return NNUEFT_E_ARG;
     char* base = (char*)ws;
     uint32_t* hist = (uint32_t*)(base + L.hist);
     uint16_t* lists = (uint16_t*)(base + L.lists);
@@ -844,7 +871,7 @@ int launch_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, c
     NNUEFT_LAUNCH_CHECK();
     hipLaunchKernelGGL(k_tl_lists, dim3(L.ngroups), dim3(kSortThreads), 0, st, widx, bidx, hist, total, lists, pidcnt,
                        loff, chunks, sched, brec, cpool8, border, L.npairs, B, K, R, L.nblocks, L.nbins, vec, L.block_rows,
-                       us, them);
+                       ex);
     NNUEFT_LAUNCH_CHECK();
     *out = Sorted{lists, pidcnt, loff, chunks, brec, cpool8, border, sched};
     return 0;
@@ -855,7 +882,8 @@ int launch_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, c
 static int gather_tile(const int32_t* widx, const int32_t* bidx, const void* W, void* sums, int B, int K, int R, int L1,
                        int out_cols, void* ws, hipStream_t st, VirtualTable vt, bool i16, int block_rows = kRows,
                        Fuse16 fz = Fuse16{nullptr, nullptr, nullptr, 0, 0},
-                       FuseF ff = FuseF{nullptr, nullptr, nullptr, nullptr, 0.0f, ActGrid{1.0f, 0.0f, 1.0f, 0}},
+                       FuseF ff = FuseF{nullptr, nullptr, nullptr, nullptr, 0.0f, ActGrid{1.0f, 0.0f, 1.0f, 0}, nullptr, nullptr,
+                                        nullptr},
                        const uint32_t** nonfinite = nullptr) {
     if (ff.l0 && (i16 || vt.V || L1 % (2 * kTileCols) != 0)) return NNUEFT_E_ARG;   // the tiles must come in pairs
     Layout L;
@@ -867,7 +895,20 @@ static int gather_tile(const int32_t* widx, const int32_t* bidx, const void* W, 
     rc = allow_lds(device);
     if (rc) return rc;
     Sorted S;
-    rc = launch_sort(widx, bidx, B, K, R, L, ws, st, &S, ff.us, ff.them);
+    SortExtras ex{};
+    ex.us = ff.us;
+    ex.them = ff.them;
+    if (ff.l0) {
+        // the forward that writes the output rows: the sort sums the psqt chains on its way
+        ex.psqt_idx = ff.psqt_idx;
+        ex.W = (const float*)W;
+        ex.bias = ff.bias;
+        ex.wpsqt = ff.wpsqt;
+        ex.bpsqt = ff.bpsqt;
+        ex.L1 = L1;
+        ex.n_psqt = out_cols - L1;
+    }
+    rc = launch_sort(widx, bidx, B, K, R, L, ws, st, &S, ex);
     if (rc) return rc;
     const uint16_t* lists = S.lists;
     const uint32_t* pidcnt = S.pidcnt;
@@ -931,9 +972,11 @@ int double_fwd_tile(const float* us, const float* them, const int32_t* widx, con
     // the gather writes the sums and, where one perspective's sums are all a half row needs, the output row too
     const uint32_t* nonfinite = nullptr;
     const int rc = gather_tile(widx, bidx, W, saved, B, K, R, L1, L1 + n_psqt, ws, st, vt, false, kRows,
-                               Fuse16{nullptr, nullptr, nullptr, 0, 0}, FuseF{us, them, bias, l0, max_act, act}, &nonfinite);
+                               Fuse16{nullptr, nullptr, nullptr, 0, 0},
+                               FuseF{us, them, bias, l0, max_act, act, psqt_idx, wpsqt, bpsqt}, &nonfinite);
     if (rc) return rc;
-    return nnueft_blocked::launch_mix(us, them, widx, bidx, psqt_idx, W, bias, saved, max_act, l0, wpsqt, bpsqt, B,
+    // (the psqt chains are done: no psqt outputs for the pass)
+    return nnueft_blocked::launch_mix(us, them, widx, bidx, psqt_idx, W, bias, saved, max_act, l0, nullptr, nullptr, B,
                                       K, R, L1, n_psqt, st, act, vt, nonfinite);
 }
 

@@ -54,8 +54,9 @@ int launch_pair_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int
 
 // In-place exclusive scan of data[0..n) (one workgroup); the second half of the forward (bias, mix, clamp,
 // product, psqt chains) over row sums saved[2, B, L1].  nonfinite != nullptr: the gather has already written the
-// output row of every position whose (us, them) is (1, 0) or (0, 1); only the other positions' rows and the psqt
-// chains are left, unless *nonfinite (device memory) says that some sum was not finite: then every row is redone.
+// output row of every position whose (us, them) is (1, 0) or (0, 1), and the psqt chains are done (wpsqt and bpsqt
+// must be nullptr); only the other positions' rows are left, unless *nonfinite (device memory) says that some sum was
+// not finite: then every row is redone.
 int launch_scan(uint32_t* data, int n, hipStream_t st);
 int launch_mix(const float* us, const float* them, const int32_t* widx, const int32_t* bidx,
                const int64_t* psqt_idx, const float* W, const float* bias, const float* saved, float max_act,

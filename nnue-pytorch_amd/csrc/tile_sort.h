@@ -88,10 +88,24 @@ struct Sorted {
                               // [kSchedNonFinite] = 0 after the sort
 };
 
-// k_tl_hist, k_tl_binscan, k_tl_lists on `st`.  us, them (both or neither; f32 [B], L.npairs == 2 B): the sides to
-// move, for the kLoff* bits of loff[]; without them those bits are 0.
+// What the sort can do on its way for the forward that calls it (all of it optional; L.npairs == 2 B):
+//   us, them (both or neither; f32 [B]): the sides to move, for the kLoff* bits of loff[]; without them those bits are 0;
+//   wpsqt, bpsqt (f32 [B], with psqt_idx, W [R, L1 + n_psqt], bias): every list's psqt chain, W[row, L1 + psqt_idx] over
+//   the list's valid rows in slot order + bias[L1 + psqt_idx] (0 for a psqt_idx outside [0, n_psqt)).
+struct SortExtras {
+    const float* us;
+    const float* them;
+    const int64_t* psqt_idx;
+    const float* W;
+    const float* bias;
+    float* wpsqt;
+    float* bpsqt;
+    int L1, n_psqt;
+};
+
+// k_tl_hist, k_tl_binscan, k_tl_lists on `st`.
 int launch_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, const Layout& L, void* ws, hipStream_t st,
-                Sorted* out, const float* us = nullptr, const float* them = nullptr);
+                Sorted* out, SortExtras ex = SortExtras{});
 
 // One wave per bin: hist[bin][0 .. ngroups) becomes its exclusive prefix, total[bin] the sum.
 int launch_binscan(uint32_t* hist, uint32_t* total, int nbins, int ngroups, hipStream_t st);
