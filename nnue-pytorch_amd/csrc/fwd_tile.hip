@@ -340,6 +340,21 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
         const int r = l.v[k];
         psv[k] = psqt_col >= 0 && r >= 0 && r < R ? ex.W[(size_t)r * ((size_t)ex.L1 + ex.n_psqt) + ex.L1 + psqt_col] : 0.0f;
     }
+    // The quantized forward's psqt difference of the position whose white list this is: both lists' entries asked
+    // for here, summed at the end of the kernel.
+    uint32_t qw[kSlots], qb[kSlots];
+    const bool q_psqt = ex.psqt_out != nullptr && n < B;
+    if (q_psqt) {
+        const int64_t pi = ex.psqt_idx[n];
+        const bool ok = pi >= 0 && pi < ex.n_psqt;
+        const ListRegs lb = load_list(pair_list(widx, bidx, n + B, B, K), K, vec);
+#pragma unroll
+        for (int k = 0; k < kSlots; ++k) {
+            const int rw = l.v[k], rb = lb.v[k];
+            qw[k] = ok && rw >= 0 && rw < R ? (uint32_t)ex.psqt32[(size_t)rw * ex.n_psqt + pi] : 0u;
+            qb[k] = ok && rb >= 0 && rb < R ? (uint32_t)ex.psqt32[(size_t)rb * ex.n_psqt + pi] : 0u;
+        }
+    }
     const ListFacts f = list_facts(l, R, block_rows);
     const int bin = sort_key(f);
     const uint32_t slot = atomicAdd(&cursor[bin], 1u);
@@ -414,6 +429,16 @@ __global__ __launch_bounds__(kSortThreads) void k_tl_lists(const int32_t* __rest
         if (psqt_col >= 0) ps = ps + ex.bias[ex.L1 + psqt_col];
         (n >= B ? ex.bpsqt : ex.wpsqt)[n >= B ? n - B : n] = ps;
     }
+    if (q_psqt) {
+        uint32_t white = 0u, black = 0u;
+#pragma unroll
+        for (int k = 0; k < kSlots; ++k) {
+            white += qw[k];
+            black += qb[k];
+        }
+        // (sum over the mover's list - sum over the other list) / 2
+        ex.psqt_out[n] = (int32_t)(ex.stm[n] ? black - white : white - black) / 2;
+    }
     if (ci >= (uint32_t)kMaxChunks) return;   // (the launcher takes this path only when the table is long enough)
     u4* out = reinterpret_cast<u4*>(lists + ((size_t)chunk_pool8[ci] << 3) + off);
 #pragma unroll
@@ -480,6 +505,11 @@ struct Fuse16 {
     const int16_t* b16;
     uint8_t* out;
     int clip_max, shift;
+    // what the sort needs for the psqt difference (it has every list in registers anyway)
+    const int32_t* psqt32;
+    const int64_t* psqt_idx;
+    int32_t* psqt_out;
+    int n_psqt;
 };
 
 // What the float forward does with a pair's sums when the gather finishes them itself (FUSE == kFuseF).  A unit then
@@ -851,6 +881,7 @@ int launch_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, c
                 Sorted* out, SortExtras ex) {
     if ((ex.us != nullptr) != (ex.them != nullptr) || ((ex.us || ex.wpsqt) && L.npairs != 2 * B)) return NNUEFT_E_ARG;
     if (ex.wpsqt && !(ex.bpsqt && ex.psqt_idx && ex.W && ex.bias)) return NNUEFT_E_ARG;
+    if (ex.psqt_out && (L.npairs != 2 * B || !ex.psqt_idx || !ex.stm || (ex.n_psqt > 0 && !ex.psqt32))) return NNUEFT_E_ARG;
     char* base = (char*)ws;
     uint32_t* hist = (uint32_t*)(base + L.hist);
     uint16_t* lists = (uint16_t*)(base + L.lists);
@@ -881,7 +912,7 @@ int launch_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int R, c
 // integers over a table W of [R, L1] int16).
 static int gather_tile(const int32_t* widx, const int32_t* bidx, const void* W, void* sums, int B, int K, int R, int L1,
                        int out_cols, void* ws, hipStream_t st, VirtualTable vt, bool i16, int block_rows = kRows,
-                       Fuse16 fz = Fuse16{nullptr, nullptr, nullptr, 0, 0},
+                       Fuse16 fz = Fuse16{nullptr, nullptr, nullptr, 0, 0, nullptr, nullptr, nullptr, 0},
                        FuseF ff = FuseF{nullptr, nullptr, nullptr, nullptr, 0.0f, ActGrid{1.0f, 0.0f, 1.0f, 0}, nullptr, nullptr,
                                         nullptr},
                        const uint32_t** nonfinite = nullptr) {
@@ -907,6 +938,13 @@ static int gather_tile(const int32_t* widx, const int32_t* bidx, const void* W, 
         ex.bpsqt = ff.bpsqt;
         ex.L1 = L1;
         ex.n_psqt = out_cols - L1;
+    }
+    if (fz.psqt_out) {
+        ex.psqt_idx = fz.psqt_idx;
+        ex.n_psqt = fz.n_psqt;
+        ex.psqt32 = fz.psqt32;
+        ex.stm = fz.stm;
+        ex.psqt_out = fz.psqt_out;
     }
     rc = launch_sort(widx, bidx, B, K, R, L, ws, st, &S, ex);
     if (rc) return rc;
@@ -972,7 +1010,7 @@ int double_fwd_tile(const float* us, const float* them, const int32_t* widx, con
     // the gather writes the sums and, where one perspective's sums are all a half row needs, the output row too
     const uint32_t* nonfinite = nullptr;
     const int rc = gather_tile(widx, bidx, W, saved, B, K, R, L1, L1 + n_psqt, ws, st, vt, false, kRows,
-                               Fuse16{nullptr, nullptr, nullptr, 0, 0},
+                               Fuse16{nullptr, nullptr, nullptr, 0, 0, nullptr, nullptr, nullptr, 0},
                                FuseF{us, them, bias, l0, max_act, act, psqt_idx, wpsqt, bpsqt}, &nonfinite);
     if (rc) return rc;
     // (the psqt chains are done: no psqt outputs for the pass)
@@ -992,10 +1030,10 @@ size_t workspace_int16(int B, int R, int block_rows) {
 }
 
 int int16_fused_tile(const int32_t* widx, const int32_t* bidx, const uint8_t* stm, const int16_t* W16, const int16_t* b16,
-                     uint8_t* out_u8, int B, int K, int R, int L1, int clip_max, int shift, int block_rows, void* ws,
-                     hipStream_t st) {
+                     const int32_t* psqt32, const int64_t* psqt_idx, uint8_t* out_u8, int32_t* psqt_out, int B, int K, int R,
+                     int L1, int n_psqt, int clip_max, int shift, int block_rows, void* ws, hipStream_t st) {
     return gather_tile(widx, bidx, W16, nullptr, B, K, R, L1, L1, ws, st, VirtualTable{nullptr, 1.0f, 1.0f, 0, 0.0f}, true,
-                       block_rows, Fuse16{stm, b16, out_u8, clip_max, shift});
+                       block_rows, Fuse16{stm, b16, out_u8, clip_max, shift, psqt32, psqt_idx, psqt_out, n_psqt});
 }
 
 }  // namespace nnueft_tile

@@ -14,7 +14,7 @@
 //                         forward's gather out of LDS tiles (fwd_tile.hip) over the int16 table
 //       k_acc_tile        a tile is 32 column pairs (j, j + L1/2): the sums of a pair and tile stay in registers and
 //                         leave as 32 output bytes (+ b16, clip, product >> shift) in the half the side to move selects
-//       k_psqt16          the psqt difference of every position
+//       k_tl_lists        (the sort in front of it) the psqt difference of every position, while it has the lists
 #include "internal.h"
 
 namespace {
@@ -284,32 +284,6 @@ __global__ __launch_bounds__(64) void k_black_mix16(const int32_t* __restrict__ 
     }
 }
 
-// psqt_out of a position on its own (the LDS-tiled path finishes the output bytes inside its gather): four
-// positions a workgroup, a wave each, the white list on lanes 0 .. 31 and the black one on lanes 32 .. 63.
-__global__ __launch_bounds__(256) void k_psqt16(const int32_t* __restrict__ widx, const int32_t* __restrict__ bidx,
-                                                const uint8_t* __restrict__ stm, const int32_t* __restrict__ psqt32,
-                                                const int64_t* __restrict__ psqt_idx, int32_t* __restrict__ psqt_out,
-                                                int B, int K, int R, int n_psqt) {
-    const int lane = threadIdx.x & 63;
-    const int b = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (b >= B) return;
-    const int64_t pi = psqt_idx[b];
-    const int p = lane >> 5;
-    uint32_t ps = 0u;
-    if (pi >= 0 && pi < n_psqt) {
-        const int32_t* ix = (p ? bidx : widx) + (size_t)b * K;
-        for (int k = lane & 31; k < K; k += 32) {
-            const int r = ix[k];
-            if (r >= 0 && r < R) ps += (uint32_t)psqt32[(size_t)r * n_psqt + pi];
-        }
-    }
-#pragma unroll
-    for (int off = 16; off > 0; off >>= 1) ps += (uint32_t)__shfl_xor((int)ps, off);
-    const uint32_t white = (uint32_t)__shfl((int)ps, 0), black = (uint32_t)__shfl((int)ps, 32);
-    // (sum over the mover's list - sum over the other list) / 2
-    if (lane == 0) psqt_out[b] = (int32_t)(stm[b] ? black - white : white - black) / 2;
-}
-
 struct Int16Layout {
     size_t accW, sort, end;
     size_t tile_sort;              // the LDS-tiled path's view of the same bytes: its sort scratch
@@ -383,12 +357,9 @@ extern "C" int nnueft_ft_int16_fwd(const int32_t* widx, const int32_t* bidx, con
         if (vec && L.tile_ok && nnueft_tile::fits_int16(*info, B, K, R, L1, br)) {
             char* ws = (char*)workspace;
             // an output half depends on one list's sums only, so the gather finishes the bytes itself (32 column
-            // pairs a tile) and no sums pass through memory; the psqt difference is a kernel of its own
-            hipLaunchKernelGGL(k_psqt16, dim3((unsigned)((B + 3) / 4)), dim3(256), 0, st, widx, bidx, stm, psqt32, psqt_idx,
-                               psqt_out, B, K, R, n_psqt);
-            NNUEFT_LAUNCH_CHECK();
-            return nnueft_tile::int16_fused_tile(widx, bidx, stm, W16, b16, out_u8, B, K, R, L1, clip_max, shift, br,
-                                                 ws + L.tile_sort, st);
+            // pairs a tile) and no sums pass through memory; the psqt difference comes out of the sort of the lists
+            return nnueft_tile::int16_fused_tile(widx, bidx, stm, W16, b16, psqt32, psqt_idx, out_u8, psqt_out, B, K, R, L1,
+                                                 n_psqt, clip_max, shift, br, ws + L.tile_sort, st);
         }
         if (vec && (long long)B <= 0x3fffffffLL && nnueft_blocked::blocked_layout_fits(*info)) {
             char* ws = (char*)workspace;

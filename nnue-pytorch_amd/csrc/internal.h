@@ -84,13 +84,14 @@ int double_fwd_tile(const float* us, const float* them, const int32_t* widx, con
 // The same gather over the quantized table W16 [R, L1] int16 (wrapping 16-bit sums), finishing the quantized forward
 // itself: a tile is 32 column pairs (j, j + L1/2), and a pair's sums leave the kernel as
 // out_u8[b, half * L1/2 + j] = (clip(sum_j + b16_j) * clip(sum_{j+L1/2} + b16_{j+L1/2})) >> shift, half 0 for the list of the
-// side to move (stm[b] != 0: the black list).  No sums pass through memory.  block_rows <= 768: the rows of a table
-// block (704 for an exported net).  workspace_int16(): bytes of its scratch (0: the shape cannot take it).
+// side to move (stm[b] != 0: the black list).  No sums pass through memory.  The sort in front of the gather also
+// writes psqt_out[b] = (sum of psqt32[row, psqt_idx[b]] over the mover's list - the same over the other list) / 2.
+// block_rows <= 768: the rows of a table block (704 for an exported net).  workspace_int16(): bytes of its scratch (0: the shape cannot take it).
 bool fits_int16(const nnueft_dev::DeviceInfo& d, int B, int K, int R, int L1, int block_rows);
 size_t workspace_int16(int B, int R, int block_rows);
 int int16_fused_tile(const int32_t* widx, const int32_t* bidx, const uint8_t* stm, const int16_t* W16, const int16_t* b16,
-                     uint8_t* out_u8, int B, int K, int R, int L1, int clip_max, int shift, int block_rows, void* ws,
-                     hipStream_t st);
+                     const int32_t* psqt32, const int64_t* psqt_idx, uint8_t* out_u8, int32_t* psqt_out, int B, int K, int R,
+                     int L1, int n_psqt, int clip_max, int shift, int block_rows, void* ws, hipStream_t st);
 }  // namespace nnueft_tile
 
 namespace nnueft_chain {

@@ -92,6 +92,9 @@ struct Sorted {
 //   us, them (both or neither; f32 [B]): the sides to move, for the kLoff* bits of loff[]; without them those bits are 0;
 //   wpsqt, bpsqt (f32 [B], with psqt_idx, W [R, L1 + n_psqt], bias): every list's psqt chain, W[row, L1 + psqt_idx] over
 //   the list's valid rows in slot order + bias[L1 + psqt_idx] (0 for a psqt_idx outside [0, n_psqt)).
+//   psqt_out (int32 [B], with psqt_idx, psqt32 [R, n_psqt] int32, stm u8 [B]): the quantized forward's psqt difference,
+//   (sum of psqt32[row, psqt_idx] over the mover's list - the same over the other list) / 2 with wrapping sums (the
+//   thread that has a position's white list fetches its black list too).
 struct SortExtras {
     const float* us;
     const float* them;
@@ -101,6 +104,9 @@ struct SortExtras {
     float* wpsqt;
     float* bpsqt;
     int L1, n_psqt;
+    const int32_t* psqt32;
+    const uint8_t* stm;
+    int32_t* psqt_out;
 };
 
 // k_tl_hist, k_tl_binscan, k_tl_lists on `st`.
