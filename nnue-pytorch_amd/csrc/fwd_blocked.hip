@@ -247,7 +247,8 @@ __global__ __launch_bounds__(64) void k_mix(const float* __restrict__ us, const 
     const int s = blockIdx.x % nslices;
     const int b = blockIdx.x / nslices;
     mix_slice<VW>(s, b, lane, us, them, bias, saved, max_act, l0, B, L1, act);
-    if (s == 0) psqt_chains(b, lane, widx, bidx, psqt_idx, W, bias, wpsqt, bpsqt, K, R, L1, n_psqt, vt);
+    // (no psqt outputs: the sort in front of the gather has summed the psqt chains already)
+    if (s == 0 && wpsqt) psqt_chains(b, lane, widx, bidx, psqt_idx, W, bias, wpsqt, bpsqt, K, R, L1, n_psqt, vt);
 }
 
 // What is left when the gather has written the output rows itself (it does for a position whose (us, them) is

@@ -929,8 +929,8 @@ static int gather_tile(const int32_t* widx, const int32_t* bidx, const void* W, 
     SortExtras ex{};
     ex.us = ff.us;
     ex.them = ff.them;
-    if (ff.l0) {
-        // the forward that writes the output rows: the sort sums the psqt chains on its way
+    if (ff.wpsqt) {
+        // the sort sums the psqt chains on its way
         ex.psqt_idx = ff.psqt_idx;
         ex.W = (const float*)W;
         ex.bias = ff.bias;
@@ -1002,10 +1002,21 @@ int double_fwd_tile(const float* us, const float* them, const int32_t* widx, con
     pairs = false;
 #endif
     if (!pairs) {
-        const int rc = gather_tile(widx, bidx, W, saved, B, K, R, L1, L1 + n_psqt, ws, st, vt, false);
+        // (the psqt chains out of the sort here too, unless the table is merged on the fly: the sort does not merge)
+        const bool sort_psqt = !vt.V;
+        FuseF none{};
+        if (sort_psqt) {
+            none.bias = bias;
+            none.psqt_idx = psqt_idx;
+            none.wpsqt = wpsqt;
+            none.bpsqt = bpsqt;
+        }
+        const int rc = gather_tile(widx, bidx, W, saved, B, K, R, L1, L1 + n_psqt, ws, st, vt, false, kRows,
+                                   Fuse16{nullptr, nullptr, nullptr, 0, 0, nullptr, nullptr, nullptr, 0}, none);
         if (rc) return rc;
-        return nnueft_blocked::launch_mix(us, them, widx, bidx, psqt_idx, W, bias, saved, max_act, l0, wpsqt, bpsqt, B,
-                                          K, R, L1, n_psqt, st, act, vt, nullptr);
+        return nnueft_blocked::launch_mix(us, them, widx, bidx, psqt_idx, W, bias, saved, max_act, l0,
+                                          sort_psqt ? nullptr : wpsqt, sort_psqt ? nullptr : bpsqt, B, K, R, L1, n_psqt, st,
+                                          act, vt, nullptr);
     }
     // the gather writes the sums and, where one perspective's sums are all a half row needs, the output row too
     const uint32_t* nonfinite = nullptr;

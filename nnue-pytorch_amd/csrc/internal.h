@@ -53,7 +53,8 @@ int launch_pair_sort(const int32_t* widx, const int32_t* bidx, int B, int K, int
                      hipStream_t st, const uint32_t** order);
 
 // In-place exclusive scan of data[0..n) (one workgroup); the second half of the forward (bias, mix, clamp,
-// product, psqt chains) over row sums saved[2, B, L1].  nonfinite != nullptr: the gather has already written the
+// product, psqt chains) over row sums saved[2, B, L1]; wpsqt == nullptr (with bpsqt): without the psqt chains (the
+// caller has them from elsewhere).  nonfinite != nullptr: the gather has already written the
 // output row of every position whose (us, them) is (1, 0) or (0, 1), and the psqt chains are done (wpsqt and bpsqt
 // must be nullptr); only the other positions' rows are left, unless *nonfinite (device memory) says that some sum was
 // not finite: then every row is redone.
