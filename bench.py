@@ -84,11 +84,12 @@ def compulsory_bytes(L1, B, sum_a):
     small = B * 24
     if forward_path(L1) == "tile_pairs":
         fwd = {
-            "list sort": 2 * lists + sum_a * 2 + 2 * B * 6 + B * 8,       # + the sides to move
+            # + the sides to move and the psqt chains (4 bytes per list entry out of the table's psqt columns)
+            "list sort": 2 * lists + sum_a * 2 + 2 * B * 6 + B * 8 + sum_a * 4 + small,
             # table once, packed lists, row sums written, output rows written (the sums of a visit's first tile come
             # back from memory once: they have left the XCD's L2 by the time the second tile's are done)
             "k_acc_tile": R_ROWS * oc * 4 + sum_a * 2 + 2 * B * 6 + saved + saved // 2 + B * L1 * 4,
-            "k_mix_rest": lists + small,                                  # psqt chains
+            "k_mix_rest": B * 8,                                          # a look at the sides to move
         }
     elif forward_path(L1) == "tile":
         fwd = {
@@ -386,7 +387,7 @@ def run_int16(args, lib, dev):
                    "active_rows_per_position": sum_a / B,
                    "with_int8_layer_stacks_ms": ms_chain, "with_int8_layer_stacks_positions_per_s": B / (ms_chain * 1e-3)},
         "roofline": {"kernel": "nnueft_ft_int16_fwd: k_acc_tile over the int16 table (the gather out of LDS tiles) + "
-                               "k_mix16 + list sort", "bound": "lds",
+                               "list sort (with the psqt difference)", "bound": "lds",
                      "achieved": gbs, "peak": lds_peak, "unit": "GB/s", "frac": gbs / lds_peak, "traffic": None,
                      "algorithmic_bytes_per_launch": alg, "avg_launch_ms": ms,
                      "achieved_over_hbm_peak": gbs / HBM_PEAK_GBS,
@@ -807,8 +808,8 @@ def run_ft(args, lib, dev):
     if forward_path(L1) in ("tile", "tile_pairs"):
         # the gather reads the table out of LDS tiles: its algorithmic bytes are LDS reads
         fwd_block, fwd_comp = bound_block(
-            "nnueft_double_fwd: k_acc_tile (the gather out of LDS tiles; it writes the output rows too) + k_mix_rest "
-            "(psqt chains) + list sort" if forward_path(L1) == "tile_pairs" else
+            "nnueft_double_fwd: k_acc_tile (the gather out of LDS tiles; it writes the output rows too) + list sort (with the "
+            "psqt chains) + k_mix_rest" if forward_path(L1) == "tile_pairs" else
             "nnueft_double_fwd: k_acc_tile (the gather out of LDS tiles, ~2/3 of the time) + k_mix + list sort", fwd_ms,
             fwd_bytes, None, sum(comp_fwd.values()), sum_traffic(traffic, fwd_kernels(L1)), LDS_PEAK_GBS,
             note="the gathered rows are LDS reads: peak = what 16-byte reads of whole 128-byte rows at random rows of a "
