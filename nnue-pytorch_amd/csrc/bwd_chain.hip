@@ -72,7 +72,7 @@ constexpr int kMaxTasks = 63;
 constexpr int kSortWaves = kRows / 64;             // the list maker sorts a block's rows, a row a thread
 constexpr int kCntBins = 640;                      // chain lengths 0 .. kCP
 static_assert(kCntBins > kCP && kCntBins % 2 == 0, "a counter per chain length");
-static_assert(kSortWaves * kCntBins >= kRows * (kMaskWords / 2) && kMaskWords % 2 == 0, "the prefix table takes the counters' place");
+
 constexpr int kRowSlots = 832;
 constexpr int kMdB = 256 + kRowSlots * 2;
 constexpr int kMdWords = kMdB / 4;
@@ -350,13 +350,10 @@ __global__ __launch_bounds__(kThreads) void k_cs_expand(const int32_t* __restric
     extern __shared__ float4 lds_raw[];
     uint32_t* mask = reinterpret_cast<uint32_t*>(lds_raw);             // [kRows][kMaskWords]
     uint32_t* keys = mask + kRows * kMaskWords;                        // [1024] sort keys, then the rows in slot order
-    uint16_t* slot_of_row = reinterpret_cast<uint16_t*>(keys + 1024);  // [kRows]
-    uint32_t* mdw = reinterpret_cast<uint32_t*>(slot_of_row + kRows);  // [kMdWords]
+    uint32_t* mdw = keys + 1024;                                       // [kMdWords]
     uint32_t* small = mdw + kMdWords;                                  // [8] counters
     uint16_t* lent = reinterpret_cast<uint16_t*>(small + 8);           // [kEntCap]
-    // [kSortWaves][kCntBins] rows of a wave by chain length (the sort), then [kRows][kMaskWords / 2] set bits of a row
-    // in front of every second word of its bit map (the lists)
-    uint16_t* whist = lent + kEntCap;
+    uint16_t* whist = lent + kEntCap;   // [kSortWaves][kCntBins] rows of a wave by chain length (the sort)
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int c = blockIdx.x;
@@ -450,7 +447,6 @@ __global__ __launch_bounds__(kThreads) void k_cs_expand(const int32_t* __restric
     const int nshort = (kRows - nd - nl + kTaskChains - 1) / kTaskChains;
     const int ntasks = nd + nlt + nshort;
     // slot s of the sorted rows: dense (s < nd), else place s - nd among the long and short chains
-    if (tid < kRows) slot_of_row[my_row] = (uint16_t)tid;
     for (int i = tid; i < kMdWords; i += kThreads) mdw[i] = 0;
     __syncthreads();
     {
@@ -489,40 +485,33 @@ __global__ __launch_bounds__(kThreads) void k_cs_expand(const int32_t* __restric
         }
         if (tid == 0) mdw[0] = (uint32_t)(nd + nlt) | ((uint32_t)ntasks << 16);
     }
-    // the set bits of a row in front of every second word of its bit map
-    if (tid < kRows) {
-        uint32_t run = 0;
-#pragma unroll
-        for (int w = 0; w < kMaskWords; w += 2) {
-            whist[tid * (kMaskWords / 2) + (w >> 1)] = (uint16_t)run;
-            run += (uint32_t)(__popc(mask[tid * kMaskWords + w]) + __popc(mask[tid * kMaskWords + w + 1]));
-        }
-    }
     __syncthreads();
     const int n4 = (int)small[2];
     if (n4 * 4 > kEntCap) return;
     for (int i = tid; i < n4 * 4; i += kThreads) lent[i] = (uint16_t)kCP;
     __syncthreads();
-    // every (row, word of its bit map): the set bits go to the row's list, behind those of the words in front
-    for (int item = tid; item < kRows * kMaskWords; item += kThreads) {
-        const int row = item / kMaskWords, w = item - row * kMaskWords;
-        uint32_t bits = mask[item];
-        if (!bits) continue;
-        const int slot = (int)slot_of_row[row];
-        if (slot < nd) continue;
-        const int s = slot - nd;
-        int pos = (int)whist[row * (kMaskWords / 2) + (w >> 1)];
-        if (w & 1) pos += __popc(mask[item - 1]);
+    // A thread a chain: its row's bit map word by word, the set bits to the row's list in order.  The slots are in
+    // order of chain length, so the lanes of a wave have about as much to do.  (A thread per (row, word), which has
+    // to find the set bits in front of its word and a third of whose words are empty, took 8.7 of the kernel's 19
+    // microseconds.)
+    if (tid < kRows && tid >= nd && my_cnt > 0) {
+        const int s = tid - nd;
         const bool is_long = s < nl;
         const int task = is_long ? nd + (s >> 2) : nd + nlt + ((s - nl) >> 4);
         const uint32_t base = (mdw[1 + task] & 0xfffffu) * 4;
-        while (bits) {
-            const int bit = __ffs((int)bits) - 1;
-            bits &= bits - 1;
-            const uint32_t dest = is_long ? base + (uint32_t)(((pos >> 3) * 4 + (s & 3)) * 8 + (pos & 7))
-                                          : base + (uint32_t)(((pos >> 2) * 16 + ((s - nl) & 15)) * 4 + (pos & 3));
-            lent[dest] = (uint16_t)(w * 32 + bit);
-            ++pos;
+        // entry `pos` of the chain: a long task's block is 4 chains x 8 entries, a short task's 16 chains x 4 entries
+        const uint32_t first = is_long ? base + (uint32_t)(s & 3) * 8 : base + (uint32_t)((s - nl) & 15) * 4;
+        const int sh = is_long ? 3 : 2;
+        const uint32_t stride = is_long ? 32u : 64u, in_block = is_long ? 7u : 3u;
+        uint32_t pos = 0;
+        for (int w = 0; w < kMaskWords; ++w) {
+            uint32_t bits = mask[my_row * kMaskWords + w];
+            while (bits) {
+                const int bit = __ffs((int)bits) - 1;
+                bits &= bits - 1;
+                lent[first + (pos >> sh) * stride + (pos & in_block)] = (uint16_t)(w * 32 + bit);
+                ++pos;
+            }
         }
     }
     __syncthreads();
@@ -536,7 +525,7 @@ __global__ __launch_bounds__(kThreads) void k_cs_expand(const int32_t* __restric
         if (tid == 0) chunks[c].n4 = n4;
     }
 }
-constexpr int kExpandLds = (kRows * kMaskWords + 1024) * 4 + kRows * 2 + kMdB + 32 + kEntCap * 2 + kSortWaves * kCntBins * 2;
+constexpr int kExpandLds = (kRows * kMaskWords + 1024) * 4 + kMdB + 32 + kEntCap * 2 + kSortWaves * kCntBins * 2;
 static_assert(kExpandLds <= 160 * 1024, "LDS of the list maker");
 
 typedef __attribute__((address_space(3))) const f4 lds_f4;
