@@ -303,6 +303,7 @@ def test_double_forward(oracle_cpu, B, L1, R, K, kw, with_workspace):
     (900, 2112, 24576, 32, dict(halfka=True, weight_scale=0.05, max_act=255 / 256)),  # lists inside their blocks; 33
                                                                                       # pairs of tiles over 8 XCDs
     (700, 2048, 2000, 32, dict(allow_holes=True)),                                    # lists that leave them
+    (400, 2048, 1000, 20, dict(allow_holes=True, n_psqt=0)),                          # short lists, no psqt columns
     (300, 1024, 24576, 32, dict(halfka=True, weight_scale=0.05, max_act=255 / 256)),  # rows too narrow for it: the sums
                                                                                       # first, then the pass over them
 ])
